@@ -1,0 +1,89 @@
+/* Thin C-ABI launch layer between host C++ and the HIP kernels (gfx950).
+ *
+ * Plain pointers, sizes and ints only: no HIP, C++ or torch types cross this
+ * boundary, so the calculator classes above it (include/sphericart_cuda.hpp)
+ * and any foreign-function binding can be built by an ordinary host compiler.
+ *
+ * Each entry point below names the piece of the reference it stands in for
+ * (paths relative to the reference checkout).
+ */
+#ifndef SPHX_LAUNCH_H
+#define SPHX_LAUNCH_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SPHX_EXPORT __attribute__((visibility("default")))
+
+/* Status codes returned by every function of this layer. */
+#define SPHX_OK 0
+#define SPHX_ERR_ARGUMENT 1    /* null pointer, negative l_max, unknown selector */
+#define SPHX_ERR_UNSUPPORTED 2 /* l_max beyond the device tables / LDS capacity */
+#define SPHX_ERR_HIP 3         /* a HIP runtime call failed; see sphx_last_error() */
+
+/* What to evaluate next to the values. */
+#define SPHX_VALUES 0
+#define SPHX_GRADIENTS 1
+#define SPHX_HESSIANS 2
+
+/* Largest l_max the constant-memory prefactor tables cover. */
+#define SPHX_TABLE_LMAX 64
+
+/* Evaluate real spherical (normalized != 0) or solid (normalized == 0)
+ * harmonics up to l_max for n_samples points, enqueued on `stream`.
+ *
+ *   xyz    device, [n_samples][3]
+ *   sph    device, [n_samples][(l_max+1)^2]
+ *   dsph   device, [n_samples][3][(l_max+1)^2]     (derivatives >= SPHX_GRADIENTS)
+ *   ddsph  device, [n_samples][3][3][(l_max+1)^2]  (derivatives == SPHX_HESSIANS)
+ *   stream the hipStream_t value itself (not a pointer to it); NULL = default stream
+ *
+ * The call returns after enqueueing; it does not synchronise. n_samples == 0
+ * returns SPHX_OK before looking at any pointer. The device is taken from the
+ * xyz pointer and the caller's current device is restored on return.
+ *
+ * Replaces sphericart::cuda::spherical_harmonics_cuda_base<T>
+ * (sphericart/src/cuda_base.cpp:69-120, declared sphericart/include/cuda_base.hpp)
+ * together with the pointer-to-device switch and prefactor upload of
+ * SphericalHarmonics<T>::compute_internal (sphericart/src/sphericart_cuda.cpp:115-159).
+ */
+SPHX_EXPORT int sphx_forward_f32(const float* xyz, size_t n_samples, int l_max, int normalized,
+                                 int derivatives, float* sph, float* dsph, float* ddsph,
+                                 void* stream);
+SPHX_EXPORT int sphx_forward_f64(const double* xyz, size_t n_samples, int l_max, int normalized,
+                                 int derivatives, double* sph, double* dsph, double* ddsph,
+                                 void* stream);
+
+/* Host copy of the prefactor table the kernels use for this l_max: the F_l^m
+ * block followed by the Q_l^m-recursion block, (l_max+1)(l_max+2) numbers.
+ * Replaces compute_sph_prefactors<T> (sphericart/include/templates.hpp:54-97)
+ * as called from the device class (sphericart/src/sphericart_cuda.cpp:57). */
+SPHX_EXPORT int sphx_prefactors_f32(int l_max, float* out);
+SPHX_EXPORT int sphx_prefactors_f64(int l_max, double* out);
+
+/* Number of visible GPUs, or a negative value when the HIP runtime reports an
+ * error. Replaces the cudaGetDeviceCount probe of the device-class constructor
+ * (sphericart/src/sphericart_cuda.cpp:54). */
+SPHX_EXPORT int sphx_device_count(void);
+
+/* Message of the last failure on the calling thread ("" if none). No
+ * counterpart in the reference, which throws from inside its launcher
+ * (sphericart/src/cuda_base.cpp:75-84); the classes above this layer turn the
+ * message into the same std::runtime_error. */
+SPHX_EXPORT const char* sphx_last_error(void);
+
+/* Launch geometry chosen for a call of this shape (for benchmarks and tests):
+ * samples per workgroup tile, threads per workgroup, LDS bytes per workgroup,
+ * number of workgroups. Returns a status code. No counterpart in the reference
+ * (its geometry is fixed at 8 x 8 threads, sphericart/src/cuda_base.cpp:89-94). */
+SPHX_EXPORT int sphx_plan(size_t n_samples, int l_max, int derivatives, int is_f64,
+                          int* tile_samples, int* threads, int* lds_bytes, int* workgroups);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

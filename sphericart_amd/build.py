@@ -1,0 +1,57 @@
+"""Build the HIP library in-tree: ``python -m sphericart_amd.build``.
+
+One ``hipcc`` call compiles the kernels for gfx950 together with the host-side
+C and C++ API into ``sphericart_amd/libsphericart_amd.so``. hipcc cross-compiles,
+so this works on a machine without a GPU.
+"""
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIBRARY = os.path.join(HERE, "libsphericart_amd.so")
+
+SOURCES = ["sphx_kernels.hip", "sphx_tables.cpp", "device_api.cpp", "capi.cpp"]
+
+# -ffp-contract=off: one rounding per source-level operation, on device and
+#   host alike; results then match the reference CPU evaluator built the same
+#   way bit for bit instead of merely within tolerance.
+# -packed-fp32-ops off: no v_pk_*_f32 code generation.
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-fPIC",
+    "-shared",
+    "-fvisibility=hidden",
+]
+
+
+def hipcc():
+    found = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(found):
+        raise RuntimeError("hipcc not found; a ROCm toolchain is required to build sphericart_amd")
+    return found
+
+
+def build(verbose=False, extra_flags=()):
+    """Compile ``libsphericart_amd.so``; raises ``RuntimeError`` with the compiler output on failure."""
+    command = [hipcc(), *FLAGS, *extra_flags, *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIBRARY]
+    if verbose:
+        print(" ".join(command), flush=True)
+    done = subprocess.run(command, capture_output=True, text=True)
+    if done.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({done.returncode}):\n{done.stdout}\n{done.stderr}")
+    if verbose and done.stderr:
+        # hipcc's host pass does not know the packed-fp32 feature and says so
+        print(done.stderr, file=sys.stderr)
+    return LIBRARY
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

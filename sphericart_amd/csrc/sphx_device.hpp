@@ -1,0 +1,476 @@
+// Device-side building blocks of the spherical / solid harmonics evaluator for
+// gfx950 (wave64, LDS-staged stores). Three jobs run inside one workgroup tile:
+//
+//   closed_form_job  one lane = one point, l = 0..H in registers
+//                    (sphericart/include/templates.hpp:156-265 with the closed
+//                    forms of macros.hpp; same split as the reference CPU
+//                    classes, sphericart/src/sphericart.cpp:45-92)
+//   azimuth_job      one lane = one point: c_m, s_m, 2(m+1)z into LDS
+//                    (sphericart/include/templates.hpp:451-466)
+//   channel_job      one lane = one (point, l) pair: the downward-in-m Q_l^m
+//                    recursion with first and second derivatives
+//                    (sphericart/include/templates_core.hpp:35-427)
+//
+// plus the unit-sphere chain rule (templates.hpp:553-614) applied in registers
+// right before an entry is staged, and copy_out, which streams a finished tile
+// from LDS to HBM as contiguous 16-byte stores.
+//
+// All arithmetic keeps the reference's operation order; the library is built
+// with -ffp-contract=off so that each source-level operation rounds once.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "sphx_lowl.hpp"
+
+namespace sphx {
+
+// ---- small helpers --------------------------------------------------------
+
+__device__ __forceinline__ float root(float v) { return sqrtf(v); }
+__device__ __forceinline__ double root(double v) { return sqrt(v); }
+
+template <typename T> struct Pack;
+template <> struct Pack<float> {
+    typedef float type __attribute__((ext_vector_type(4)));
+    static constexpr unsigned width = 4;
+};
+template <> struct Pack<double> {
+    typedef double type __attribute__((ext_vector_type(2)));
+    static constexpr unsigned width = 2;
+};
+
+// Where the staged outputs of one point live in LDS. Element (component a,
+// index k) of the point's gradient row is at dsph[a * ny + k], and so on; the
+// rows mirror the layout of the output arrays in HBM.
+template <typename T> struct Rows {
+    T* sph;
+    T* dsph;
+    T* ddsph;
+    int ny;
+};
+
+// Normalised coordinates of one point as every job needs them.
+template <typename T> struct Point {
+    T x, y, z, x2, y2, z2, ir;
+};
+
+// templates.hpp:156-173 / :386-400
+template <typename T, bool NORM> __device__ __forceinline__ Point<T> load_point(const T* xyz) {
+    Point<T> p;
+    p.x = xyz[0];
+    p.y = xyz[1];
+    p.z = xyz[2];
+    p.x2 = p.x * p.x;
+    p.y2 = p.y * p.y;
+    p.z2 = p.z * p.z;
+    p.ir = 0.0;
+    if constexpr (NORM) {
+        p.ir = 1 / root(p.x2 + p.y2 + p.z2);
+        p.x *= p.ir;
+        p.y *= p.ir;
+        p.z *= p.ir;
+        p.x2 = p.x * p.x;
+        p.y2 = p.y * p.y;
+        p.z2 = p.z * p.z;
+    }
+    return p;
+}
+
+// One (l, m) entry on its way to LDS: value, gradient, the six distinct second
+// derivatives (the reference assigns the symmetric partners the same number).
+template <typename T> struct Entry {
+    T v, gx, gy, gz, hxx, hxy, hxz, hyy, hyz, hzz;
+};
+
+// Chain rule for the polynomials evaluated at (x, y, z)/r, then store.
+// templates.hpp:572-613: the Hessian is corrected first, from the uncorrected
+// gradient; then the gradient.
+template <typename T, int MODE, bool NORM>
+__device__ __forceinline__ void stage(const Rows<T>& out, int k, const Point<T>& p, Entry<T> e) {
+    out.sph[k] = e.v;
+    if constexpr (MODE >= 1) {
+        if constexpr (NORM) {
+            const T x = p.x, y = p.y, z = p.z, ir = p.ir;
+            auto tmp = (e.gx * x + e.gy * y + e.gz * z);
+            if constexpr (MODE == 2) {
+                auto irsq = ir * ir;
+                auto tmpx = x * e.hxx + y * e.hxy + z * e.hxz;
+                auto tmpy = x * e.hxy + y * e.hyy + z * e.hyz;
+                auto tmpz = x * e.hxz + y * e.hyz + z * e.hzz;
+                auto tmp2 = x * x * e.hxx + y * y * e.hyy + z * z * e.hzz + 2 * x * y * e.hxy +
+                            2 * x * z * e.hxz + 2 * y * z * e.hyz;
+                T nxx = (-2 * x * tmpx + e.hxx + 3 * x * x * tmp - tmp - 2 * x * e.gx + x * x * tmp2) *
+                        irsq;
+                T nyy = (-2 * y * tmpy + e.hyy + 3 * y * y * tmp - tmp - 2 * y * e.gy + y * y * tmp2) *
+                        irsq;
+                T nzz = (-2 * z * tmpz + e.hzz + 3 * z * z * tmp - tmp - 2 * z * e.gz + z * z * tmp2) *
+                        irsq;
+                T nxy = (-x * tmpy - y * tmpx + e.hxy + 3 * x * y * tmp - x * e.gy - y * e.gx +
+                         x * y * tmp2) *
+                        irsq;
+                T nxz = (-x * tmpz - z * tmpx + e.hxz + 3 * x * z * tmp - x * e.gz - z * e.gx +
+                         x * z * tmp2) *
+                        irsq;
+                T nyz = (-z * tmpy - y * tmpz + e.hyz + 3 * y * z * tmp - z * e.gy - y * e.gz +
+                         y * z * tmp2) *
+                        irsq;
+                e.hxx = nxx;
+                e.hyy = nyy;
+                e.hzz = nzz;
+                e.hxy = nxy;
+                e.hxz = nxz;
+                e.hyz = nyz;
+            }
+            e.gx = (e.gx - x * tmp) * ir;
+            e.gy = (e.gy - y * tmp) * ir;
+            e.gz = (e.gz - z * tmp) * ir;
+        }
+        const int ny = out.ny;
+        out.dsph[k] = e.gx;
+        out.dsph[ny + k] = e.gy;
+        out.dsph[2 * ny + k] = e.gz;
+        if constexpr (MODE == 2) {
+            out.ddsph[k] = e.hxx;
+            out.ddsph[ny + k] = e.hxy;
+            out.ddsph[2 * ny + k] = e.hxz;
+            out.ddsph[3 * ny + k] = e.hxy;
+            out.ddsph[4 * ny + k] = e.hyy;
+            out.ddsph[5 * ny + k] = e.hyz;
+            out.ddsph[6 * ny + k] = e.hxz;
+            out.ddsph[7 * ny + k] = e.hyz;
+            out.ddsph[8 * ny + k] = e.hzz;
+        }
+    }
+}
+
+// ---- l = 0..H in closed form, one point per lane ---------------------------
+//
+// All (H+1)^2 values and, if asked, their gradients stay in VGPRs until they
+// are staged. Second derivatives of l <= 1 vanish identically
+// (macros.hpp:56-131), which is the only case MODE == 2 reaches here.
+template <typename T, int MODE, bool NORM, int H>
+__device__ __forceinline__ void closed_form_job(const Point<T>& p, const Rows<T>& out) {
+    static_assert(MODE < 2 || H <= 1, "second derivatives in closed form stop at l = 1");
+    constexpr int NH = (H + 1) * (H + 1);
+    T Y[NH];
+    low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
+    if constexpr (MODE == 0) {
+#pragma unroll
+        for (int k = 0; k < NH; ++k) {
+            out.sph[k] = Y[k];
+        }
+    } else {
+        T DX[NH], DY[NH], DZ[NH];
+        low_gradients<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y, DX, DY, DZ);
+#pragma unroll
+        for (int k = 0; k < NH; ++k) {
+            Entry<T> e;
+            e.v = Y[k];
+            e.gx = DX[k];
+            e.gy = DY[k];
+            e.gz = DZ[k];
+            e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = static_cast<T>(0.0);
+            stage<T, MODE, NORM>(out, k, p, e);
+        }
+    }
+}
+
+// ---- c_m, s_m, 2(m+1)z for one point ---------------------------------------
+// templates.hpp:451-466. The running sum for 2(m+1)z is kept as a sum: it
+// rounds differently from a product.
+template <typename T>
+__device__ __forceinline__ void azimuth_job(const Point<T>& p, int L, T* c, T* s, T* tmz) {
+    T twoz = p.z + p.z;
+    T cm = 1.0, sm = 0.0, tz = twoz;
+    c[0] = cm;
+    s[0] = sm;
+    tmz[0] = tz;
+    for (int m = 1; m <= L; ++m) {
+        T cn = cm * p.x - sm * p.y;
+        T sn = cm * p.y + sm * p.x;
+        tz = tz + twoz;
+        cm = cn;
+        sm = sn;
+        c[m] = cm;
+        s[m] = sm;
+        tmz[m] = tz;
+    }
+}
+
+// ---- one l channel for one point -------------------------------------------
+//
+// templates_core.hpp:35-427. F and Q are the two triangular prefactor blocks
+// (entry (l, m) at l(l+1)/2 + m); c, s, tmz the point's azimuthal tables. The
+// three-term recursion runs downward in m for Q_l, and alongside for Q_{l-1}
+// (first derivatives) and Q_{l-2} (second derivatives).
+template <typename T, int MODE, bool NORM>
+__device__ __forceinline__ void channel_job(int l, const Point<T>& p, T rxy, const T* F,
+                                            const T* Q, const T* c, const T* s, const T* tmz,
+                                            const Rows<T>& out) {
+    constexpr bool GRAD = MODE >= 1;
+    constexpr bool HESS = MODE == 2;
+    const T x = p.x, y = p.y, z = p.z;
+    const int tri = l * (l + 1) / 2;
+    const int mid = l * (l + 1);
+    const T* pk = F + tri;
+    const T* qk = Q + tri;
+    const T zero = static_cast<T>(0.0);
+
+    T qlm_2, qlm_1, qlm_0;
+    [[maybe_unused]] T ql1m_2 = 0, ql1m_1 = 0, ql1m_0 = 0;
+    [[maybe_unused]] T ql2m_2 = 0, ql2m_1 = 0, ql2m_0 = 0;
+    [[maybe_unused]] T x2 = 0, y2 = 0, xy = 0;
+    if constexpr (HESS) {
+        x2 = x * x;
+        y2 = y * y;
+        xy = x * y;
+    }
+
+    // |m| = l (:122-152)
+    {
+        qlm_2 = qk[l];
+        auto pq = qlm_2 * pk[l];
+        Entry<T> neg, pos;
+        neg.v = pq * s[l];
+        pos.v = pq * c[l];
+        neg.gx = neg.gy = neg.gz = pos.gx = pos.gy = pos.gz = zero;
+        neg.hxx = neg.hxy = neg.hxz = neg.hyy = neg.hyz = neg.hzz = zero;
+        pos.hxx = pos.hxy = pos.hxz = pos.hyy = pos.hyz = pos.hzz = zero;
+        if constexpr (GRAD) {
+            pq *= l;
+            neg.gx = pq * s[l - 1];
+            neg.gy = pos.gx = pq * c[l - 1];
+            pos.gy = -neg.gx;
+            ql1m_2 = 0;
+            if constexpr (HESS) {
+                pq *= (l - 1);
+                pos.hxx = pq * c[l - 2];
+                neg.hxx = pq * s[l - 2];
+                pos.hxy = neg.hyy = -neg.hxx;
+                neg.hxy = pos.hxx;
+                pos.hyy = -pos.hxx;
+                ql2m_2 = 0.0;
+            }
+        }
+        stage<T, MODE, NORM>(out, mid - l, p, neg);
+        stage<T, MODE, NORM>(out, mid + l, p, pos);
+    }
+
+    // |m| = l - 1 (:154-198)
+    {
+        qlm_1 = -z * qlm_2;
+        auto pq = qlm_1 * pk[l - 1];
+        Entry<T> neg, pos;
+        neg.v = pq * s[l - 1];
+        pos.v = pq * c[l - 1];
+        neg.gx = neg.gy = neg.gz = pos.gx = pos.gy = pos.gz = zero;
+        neg.hxx = neg.hxy = neg.hxz = neg.hyy = neg.hyz = neg.hzz = zero;
+        pos.hxx = pos.hxy = pos.hxz = pos.hyy = pos.hyz = pos.hzz = zero;
+        if constexpr (GRAD) {
+            pq *= (l - 1);
+            neg.gx = pq * s[l - 2];
+            neg.gy = pos.gx = pq * c[l - 2];
+            pos.gy = -neg.gx;
+            ql1m_1 = qk[-1];
+            auto pdq = pk[l - 1] * (l + l - 1) * ql1m_1;
+            neg.gz = pdq * s[l - 1];
+            pos.gz = pdq * c[l - 1];
+            if constexpr (HESS) {
+                pq *= (l - 2);
+                if (l == 2) {
+                    pos.hxx = 0;
+                    neg.hxx = 0;
+                } else {
+                    pos.hxx = pq * c[l - 3];
+                    neg.hxx = pq * s[l - 3];
+                }
+                pos.hxy = neg.hyy = -neg.hxx;
+                neg.hxy = pos.hxx;
+                auto temp = -pk[l - 1] * (l - 1) * qlm_2;
+                pos.hxz = temp * c[l - 2];
+                neg.hxz = temp * s[l - 2];
+                pos.hyy = -pos.hxx;
+                pos.hyz = -neg.hxz;
+                neg.hyz = pos.hxz;
+                ql2m_1 = 0.0;
+            }
+        }
+        stage<T, MODE, NORM>(out, mid - l + 1, p, neg);
+        stage<T, MODE, NORM>(out, mid + l - 1, p, pos);
+    }
+
+    // l - 2 >= |m| >= 1 (:201-390; the reference's two loops share one body)
+    for (auto m = l - 2; m > 0; --m) {
+        const T cm = c[m], sm = s[m], tz = tmz[m], pkm = pk[m];
+        qlm_0 = qk[m] * (tz * qlm_1 + rxy * qlm_2);
+        qlm_2 = qlm_1;
+        qlm_1 = qlm_0;
+        auto pq = qlm_0 * pkm;
+        Entry<T> neg, pos;
+        neg.v = pq * sm;
+        pos.v = pq * cm;
+        neg.gx = neg.gy = neg.gz = pos.gx = pos.gy = pos.gz = zero;
+        neg.hxx = neg.hxy = neg.hxz = neg.hyy = neg.hyz = neg.hzz = zero;
+        pos.hxx = pos.hxy = pos.hxz = pos.hyy = pos.hyz = pos.hzz = zero;
+
+        if constexpr (GRAD) {
+            const T cm1 = c[m - 1], sm1 = s[m - 1];
+            ql1m_0 = qk[m - l] * (tz * ql1m_1 + rxy * ql1m_2);
+            ql1m_2 = ql1m_1;
+            ql1m_1 = ql1m_0;
+
+            pq *= m;
+            auto pqs = pq * sm1, pqc = pq * cm1;
+            auto pdq = pkm * ql1m_2;
+            auto pdqx = pdq * x;
+            neg.gx = (pdqx * sm + pqs);
+            pos.gx = (pdqx * cm + pqc);
+            auto pdqy = pdq * y;
+            neg.gy = (pdqy * sm + pqc);
+            pos.gy = (pdqy * cm - pqs);
+            pdq = pkm * (l + m) * ql1m_1;
+            neg.gz = pdq * sm;
+            pos.gz = pdq * cm;
+
+            if constexpr (HESS) {
+                if (m == l - 2) {
+                    ql2m_0 = qk[-l - 1];
+                } else {
+                    ql2m_0 = qk[m - 2 * l + 1] * (tz * ql2m_1 + rxy * ql2m_2);
+                }
+
+                pq /= m;
+                // ql1m_2 / ql1m_1 were shifted above: they are Q_{l-1}^{m+1} and Q_{l-1}^{m}
+                auto pql1m_1 = pkm * ql1m_2;
+                auto pql2m_2 = pkm * ql2m_2;
+                auto pql2m_0 = pkm * ql2m_0;
+                auto pql1m_0 = pkm * ql1m_1;
+                auto pql2m_1 = pkm * ql2m_1;
+
+                T mmpqc2 = 0.0;
+                T mmpqs2 = 0.0;
+                if (m != 1) {
+                    mmpqc2 = m * (m - 1) * pq * c[m - 2];
+                    mmpqs2 = m * (m - 1) * pq * s[m - 2];
+                }
+
+                pos.hxx = pql1m_1 * cm + x2 * pql2m_2 * cm + 2 * m * x * pql1m_1 * cm1 + mmpqc2;
+                neg.hxx = pql1m_1 * sm + x2 * pql2m_2 * sm + 2 * m * x * pql1m_1 * sm1 + mmpqs2;
+                pos.hyy = pql1m_1 * cm + y2 * pql2m_2 * cm - 2 * m * y * pql1m_1 * sm1 - mmpqc2;
+                neg.hyy = pql1m_1 * sm + y2 * pql2m_2 * sm + 2 * m * y * pql1m_1 * cm1 - mmpqs2;
+                pos.hzz = (l + m) * (l + m - 1) * pql2m_0 * cm;
+                neg.hzz = (l + m) * (l + m - 1) * pql2m_0 * sm;
+
+                pos.hxy = xy * pql2m_2 * cm + y * pql1m_1 * m * cm1 - x * pql1m_1 * m * sm1 - mmpqs2;
+                neg.hxy = xy * pql2m_2 * sm + y * pql1m_1 * m * sm1 + x * pql1m_1 * m * cm1 + mmpqc2;
+                pos.hxz = x * (l + m) * pql2m_1 * cm + (l + m) * pql1m_0 * m * cm1;
+                neg.hxz = x * (l + m) * pql2m_1 * sm + (l + m) * pql1m_0 * m * sm1;
+                pos.hyz = y * (l + m) * pql2m_1 * cm - (l + m) * pql1m_0 * m * sm1;
+                neg.hyz = y * (l + m) * pql2m_1 * sm + (l + m) * pql1m_0 * m * cm1;
+
+                ql2m_2 = ql2m_1;
+                ql2m_1 = ql2m_0;
+            }
+        }
+        stage<T, MODE, NORM>(out, mid - m, p, neg);
+        stage<T, MODE, NORM>(out, mid + m, p, pos);
+    }
+
+    // m = 0 (:392-426)
+    {
+        const T tz = tmz[0];
+        qlm_0 = qk[0] * (tz * qlm_1 + rxy * qlm_2);
+        Entry<T> e;
+        e.v = qlm_0 * pk[0];
+        e.gx = e.gy = e.gz = zero;
+        e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = zero;
+        if constexpr (GRAD) {
+            ql1m_0 = qk[-l] * (tz * ql1m_1 + rxy * ql1m_2);
+            e.gx = pk[0] * x * ql1m_1;
+            e.gy = pk[0] * y * ql1m_1;
+            e.gz = pk[0] * l * ql1m_0;
+            if constexpr (HESS) {
+                if (l == 2) {
+                    ql2m_0 = qk[-2 * l + 1];
+                } else {
+                    ql2m_0 = qk[-2 * l + 1] * (tz * ql2m_1 + rxy * ql2m_2);
+                }
+                auto pql1m_1 = pk[0] * ql1m_1;
+                auto pql2m_2 = pk[0] * ql2m_2;
+                auto pql2m_0 = pk[0] * ql2m_0;
+                auto pql2m_1 = pk[0] * ql2m_1;
+                e.hxx = pql1m_1 + x2 * pql2m_2;
+                e.hyy = pql1m_1 + y2 * pql2m_2;
+                e.hzz = (l) * (l - 1) * pql2m_0;
+                e.hxy = xy * pql2m_2;
+                e.hxz = x * l * pql2m_1;
+                e.hyz = y * l * pql2m_1;
+            }
+        }
+        stage<T, MODE, NORM>(out, mid, p, e);
+    }
+}
+
+// ---- LDS -> HBM ------------------------------------------------------------
+//
+// A tile of consecutive points is one contiguous run of `len` elements in an
+// output array; in LDS the same run is stored point after point with `pad`
+// spare elements after every `row` elements (row = what one point contributes;
+// the pad keeps the per-point stride odd so that lanes staging the same entry
+// of different points hit different banks). `magic` = ceil(2^32 / row) turns the
+// division by `row` into a multiply-high; it is exact here because an LDS tile
+// holds fewer than 2^16 elements.
+template <typename T>
+__device__ __forceinline__ unsigned staged_index(unsigned g, unsigned row, unsigned pad,
+                                                 unsigned magic) {
+    return g + pad * __umulhi(g, magic);
+}
+
+template <typename T, bool STREAMING>
+__device__ __forceinline__ void copy_out(const T* staged, T* dst, unsigned len, unsigned row,
+                                         unsigned pad, unsigned magic, bool wide, unsigned tid,
+                                         unsigned nthreads) {
+    using V = typename Pack<T>::type;
+    constexpr unsigned W = Pack<T>::width;
+    unsigned done = 0;
+    if (wide) {
+        const unsigned nvec = len / W;
+        V* dst_v = reinterpret_cast<V*>(dst);
+        if (pad == 0) {
+            const V* src_v = reinterpret_cast<const V*>(staged);
+            for (unsigned g = tid; g < nvec; g += nthreads) {
+                V v = src_v[g];
+                if constexpr (STREAMING) {
+                    __builtin_nontemporal_store(v, dst_v + g);
+                } else {
+                    dst_v[g] = v;
+                }
+            }
+        } else {
+            for (unsigned g = tid; g < nvec; g += nthreads) {
+                V v;
+#pragma unroll
+                for (unsigned e = 0; e < W; ++e) {
+                    v[e] = staged[staged_index<T>(g * W + e, row, pad, magic)];
+                }
+                if constexpr (STREAMING) {
+                    __builtin_nontemporal_store(v, dst_v + g);
+                } else {
+                    dst_v[g] = v;
+                }
+            }
+        }
+        done = nvec * W;
+    }
+    for (unsigned g = done + tid; g < len; g += nthreads) {
+        T v = staged[pad ? staged_index<T>(g, row, pad, magic) : g];
+        if constexpr (STREAMING) {
+            __builtin_nontemporal_store(v, dst + g);
+        } else {
+            dst[g] = v;
+        }
+    }
+}
+
+} // namespace sphx

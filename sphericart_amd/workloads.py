@@ -1,0 +1,145 @@
+"""Seeded synthetic point clouds for the five benchmark / parity configurations.
+
+Points are generated on the host in float64 from a counter-based generator
+(SplitMix64 over the point index, so any slice of a cloud can be produced on its
+own and the numbers do not depend on the numpy version), rounded once to the
+working precision, and that one array is what both the GPU path and any CPU
+checker are fed with.
+"""
+
+from dataclasses import dataclass
+
+import numpy as np
+
+_MASK = np.uint64(0xFFFFFFFFFFFFFFFF)
+
+
+def _splitmix64(x):
+    """Vectorised SplitMix64 finaliser on uint64 arrays."""
+    with np.errstate(over="ignore"):
+        x = (x + np.uint64(0x9E3779B97F4A7C15)) & _MASK
+        x = ((x ^ (x >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)) & _MASK
+        x = ((x ^ (x >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)) & _MASK
+        return x ^ (x >> np.uint64(31))
+
+
+def uniform(seed, n, stream, first=0):
+    """n doubles in (0, 1), stream-th sequence of the seed, starting at index `first`."""
+    idx = np.arange(first, first + n, dtype=np.uint64)
+    with np.errstate(over="ignore"):
+        key = _splitmix64(np.uint64(seed) * np.uint64(0x100000001B3) + np.uint64(stream))
+        bits = _splitmix64(idx * np.uint64(0xD1342543DE82EF95) + key)
+    return ((bits >> np.uint64(11)).astype(np.float64) + 0.5) * (1.0 / 9007199254740992.0)
+
+
+def normal(seed, n, stream, first=0):
+    """Standard normal deviates by Box-Muller from two uniform streams."""
+    u1 = uniform(seed, n, 2 * stream, first)
+    u2 = uniform(seed, n, 2 * stream + 1, first)
+    return np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
+
+
+def _directions(seed, n, first):
+    v = np.stack([normal(seed, n, 10 + a, first) for a in range(3)], axis=1)
+    return v / np.linalg.norm(v, axis=1, keepdims=True)
+
+
+def _on_axis(xyz, radius, every, first):
+    """Every `every`-th point (by global index) exactly on the z axis, sign alternating."""
+    idx = np.arange(first, first + xyz.shape[0])
+    hit = idx % every == 0
+    sign = np.where((idx // every) % 2 == 0, 1.0, -1.0)
+    xyz[hit, 0] = 0.0
+    xyz[hit, 1] = 0.0
+    xyz[hit, 2] = (sign * radius)[hit]
+    return xyz
+
+
+@dataclass(frozen=True)
+class Workload:
+    name: str
+    description: str
+    l_max: int
+    dtype: str          # "f32" or "f64"
+    normalized: bool    # spherical (True) or solid (False) harmonics
+    derivatives: str    # "values", "gradients" or "hessians"
+    n_samples: int
+    seed: int
+
+    @property
+    def numpy_dtype(self):
+        return np.float32 if self.dtype == "f32" else np.float64
+
+    @property
+    def n_components(self):
+        return {"values": 1, "gradients": 4, "hessians": 13}[self.derivatives]
+
+    @property
+    def bytes_per_point(self):
+        """Algorithmic traffic: 3 coordinates read, (l_max+1)^2 (1 + 3 + 9) numbers written."""
+        size = 4 if self.dtype == "f32" else 8
+        return size * (3 + (self.l_max + 1) ** 2 * self.n_components)
+
+    def points(self, n=None, first=0):
+        """`n` points of the cloud starting at global index `first` (default: all of it)."""
+        n = self.n_samples if n is None else n
+        return _GENERATORS[self.name](self.seed, n, first).astype(self.numpy_dtype)
+
+
+def _cfg1(seed, n, first):
+    return np.stack([normal(seed, n, a, first) for a in range(3)], axis=1)
+
+
+def _shell(seed, n, first):
+    radius = 0.5 + 4.5 * uniform(seed, n, 20, first)
+    return _directions(seed, n, first) * radius[:, None], radius
+
+
+def _cfg2(seed, n, first):
+    return _shell(seed, n, first)[0]
+
+
+def _cfg3(seed, n, first):
+    xyz, radius = _shell(seed, n, first)
+    return _on_axis(xyz, radius, 100, first)
+
+
+def _cfg4(seed, n, first):
+    return np.stack([-3.0 + 6.0 * uniform(seed, n, a, first) for a in range(3)], axis=1)
+
+
+def _cfg5(seed, n, first):
+    lo, hi = np.log(1e-2), np.log(1e2)
+    radius = np.exp(lo + (hi - lo) * uniform(seed, n, 20, first))
+    xyz = _directions(seed, n, first) * radius[:, None]
+    return _on_axis(xyz, radius, 200, first)
+
+
+_GENERATORS = {"cfg1": _cfg1, "cfg2": _cfg2, "cfg3": _cfg3, "cfg4": _cfg4, "cfg5": _cfg5}
+
+WORKLOADS = {
+    "cfg1": Workload(
+        "cfg1", "spherical, l_max=8, f64, values+gradients, 10k points, xyz ~ N(0,1)",
+        8, "f64", True, "gradients", 10_000, 1001,
+    ),
+    "cfg2": Workload(
+        "cfg2", "spherical, l_max=3, f32, values, 1M points, uniform directions, r ~ U[0.5,5)",
+        3, "f32", True, "values", 1_000_000, 1002,
+    ),
+    "cfg3": Workload(
+        "cfg3",
+        "spherical, l_max=6, f32, values+gradients, 1M points, uniform directions, r ~ U[0.5,5), "
+        "1% of the points exactly on the +-z axis",
+        6, "f32", True, "gradients", 1_000_000, 1003,
+    ),
+    "cfg4": Workload(
+        "cfg4", "solid, l_max=16, f64, values+gradients+Hessians, 100k points, xyz ~ U[-3,3)^3",
+        16, "f64", False, "hessians", 100_000, 1004,
+    ),
+    "cfg5": Workload(
+        "cfg5",
+        "spherical, l_max=32, f32, values+gradients, 200k points, uniform directions, "
+        "r log-uniform in [1e-2,1e2), 0.5% of the points on the +-z axis",
+        32, "f32", True, "gradients", 200_000, 1005,
+    ),
+}
