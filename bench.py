@@ -1,0 +1,203 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3]
+
+A step is one evaluation of one batch of synthetic points that already sit in
+HBM: one kernel launch through the C launch layer (sphx_forward_*) writing
+preallocated outputs. The default workload is the configuration the headline
+metric is quoted on: real spherical harmonics, l_max = 6, float32, values and
+gradients, 1,000,000 points.
+
+One JSON line is printed. Next to the contract fields it carries
+
+  roofline      achieved HBM bandwidth of the kernel: algorithmic bytes per
+                launch (sizeof(T) * (3 + (l_max+1)^2 * components) per point)
+                divided by the average launch duration, measured with events
+                on the launch stream around every timed launch, against the
+                8 TB/s peak of MI355X;
+  cpu_baseline  the reference CPU implementation (oracle/_ref, built from the
+                reference's own sources; the repository's restatement when that
+                is absent) timed on the host cores on a bounded number of
+                passes over the same points.
+"""
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBPS = 8000.0
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script (profiles/), scaled by what the same counters read for a plain copy of
+# known size. None until measured for a workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--workload", default="cfg3")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    return p.parse_args()
+
+
+def cpu_baseline(workload, xyz):
+    """Reference CPU path on the host cores: best-of timing over a bounded number of passes."""
+    import numpy as np
+
+    import oracle  # the CPU checker: used here only as the baseline being reported
+
+    if oracle.available("ref_fma"):
+        flavour, kind = "ref_fma", "reference"
+    else:
+        flavour, kind = "oracle", "port"
+    n = workload.n_samples
+    ny = (workload.l_max + 1) ** 2
+    mode = workload.derivatives
+    out = (
+        np.empty((n, ny), dtype=xyz.dtype),
+        np.empty((n, 3, ny), dtype=xyz.dtype) if mode != "values" else None,
+        np.empty((n, 3, 3, ny), dtype=xyz.dtype) if mode == "hessians" else None,
+    )
+    for o in out:
+        if o is not None:
+            o.fill(0)  # touch the pages once
+    times = []
+    started = time.perf_counter()
+    passes = 0
+    while passes < 3 or (time.perf_counter() - started < 2.0 and passes < 40):
+        t0 = time.perf_counter()
+        oracle.compute(xyz, workload.l_max, workload.normalized, mode, flavour, out=out)
+        times.append(time.perf_counter() - t0)
+        passes += 1
+    timed = times[2:] if len(times) > 4 else times
+    best = min(timed)
+    cores = oracle.max_threads(flavour)
+    return {
+        "value": n / best,
+        "unit": "points/s",
+        "cores": cores,
+        "kind": kind,
+        "sample": f"{passes} passes over all {n} points of the workload, best pass "
+        f"{best * 1e3:.2f} ms, median {statistics.median(timed) * 1e3:.2f} ms; "
+        f"{'compiled reference sources (-O3, AVX2/FMA)' if kind == 'reference' else 'restatement (-O2, no FMA)'}, "
+        f"OpenMP over {cores} threads",
+        "GBps": workload.bytes_per_point * n / best / 1e9,
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(
+            "bench.py measures one GPU: the evaluator shards by giving each GPU its own slice of "
+            "points and needs no exchange, so there is no multi-GPU figure to report (--gpus 1 only).",
+            file=sys.stderr,
+        )
+        return 2
+
+    import torch
+
+    import sphericart_amd
+    from sphericart_amd.workloads import WORKLOADS
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    w = WORKLOADS[args.workload]
+    lib = sphericart_amd.get_library()
+    torch.cuda.set_device(0)
+
+    xyz_host = w.points()
+    xyz = torch.from_numpy(xyz_host).cuda()
+    n, ny = w.n_samples, (w.l_max + 1) ** 2
+    opts = dict(dtype=xyz.dtype, device=xyz.device)
+    mode = {"values": 0, "gradients": 1, "hessians": 2}[w.derivatives]
+    sph = torch.empty((n, ny), **opts)
+    dsph = torch.empty((n, 3, ny), **opts) if mode >= 1 else None
+    ddsph = torch.empty((n, 3, 3, ny), **opts) if mode >= 2 else None
+    forward = lib.sphx_forward_f32 if w.dtype == "f32" else lib.sphx_forward_f64
+    stream = torch.cuda.current_stream()
+    pointers = (
+        xyz.data_ptr(), n, w.l_max, int(w.normalized), mode, sph.data_ptr(),
+        dsph.data_ptr() if dsph is not None else None,
+        ddsph.data_ptr() if ddsph is not None else None, stream.cuda_stream,
+    )
+
+    def step():
+        status = forward(*pointers)
+        if status != 0:
+            raise RuntimeError(lib.sphx_last_error().decode())
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for begin, end in events:
+        begin.record(stream)
+        step()
+        end.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    launch_ms = [b.elapsed_time(e) for b, e in events]
+    avg_launch_s = sum(launch_ms) / len(launch_ms) / 1e3
+    bytes_per_launch = w.bytes_per_point * n
+    achieved = bytes_per_launch / avg_launch_s / 1e9
+
+    result = {
+        "metric": "points/sec + achieved HBM GB/s (% peak), l_max=6 fp32 w/ gradients, 1M pts"
+        if args.workload == "cfg3"
+        else f"points/sec + achieved HBM GB/s (% peak), {w.description}",
+        "value": n * args.steps / wall,
+        "unit": "points/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": w.dtype,
+        "data": "synthetic",
+        "config": {
+            "workload": f"{w.name}: {w.description}",
+            "l_max": w.l_max,
+            "n_samples": n,
+            "derivatives": w.derivatives,
+            "harmonics": "spherical" if w.normalized else "solid",
+            "seed": w.seed,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": PEAK_HBM_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / PEAK_HBM_GBPS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "algorithmic_bytes_per_launch": bytes_per_launch,
+            "avg_launch_us": avg_launch_s * 1e6,
+            "median_launch_us": statistics.median(launch_ms) * 1e3,
+            "min_launch_us": min(launch_ms) * 1e3,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(w, xyz_host)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

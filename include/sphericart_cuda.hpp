@@ -18,6 +18,10 @@
 
 #include <cstddef>
 
+#ifndef SPHERICART_EXPORT
+#define SPHERICART_EXPORT __attribute__((visibility("default")))
+#endif
+
 namespace sphericart {
 namespace cuda {
 
@@ -28,7 +32,7 @@ namespace cuda {
  *
  * Reference: sphericart/include/sphericart_cuda.hpp:33-170.
  */
-template <typename T> class SphericalHarmonics {
+template <typename T> class SPHERICART_EXPORT SphericalHarmonics {
   public:
     /** @param l_max largest degree to evaluate.
      *  Throws std::runtime_error when no HIP device is usable or l_max
@@ -74,7 +78,7 @@ template <typename T> class SphericalHarmonics {
  * Solid harmonics r^l Y_l^m: the same polynomials evaluated at (x, y, z)
  * itself. Reference: sphericart/include/sphericart_cuda.hpp:179-187.
  */
-template <typename T> class SolidHarmonics : public SphericalHarmonics<T> {
+template <typename T> class SPHERICART_EXPORT SolidHarmonics : public SphericalHarmonics<T> {
   public:
     SolidHarmonics(size_t l_max);
 };

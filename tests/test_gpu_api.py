@@ -1,0 +1,160 @@
+"""Behaviour of the boundary on a real GPU: sizes, alignment, streams, error conventions."""
+
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import sphericart_amd
+from gpu_utils import announce, run_calculator, run_launch_layer
+from helpers import MODES, same_numbers, special_points
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize("l_max,mode", [(3, "values"), (6, "gradients"), (1, "hessians"), (9, "gradients"), (5, "hessians")])
+def test_ragged_sizes(oracle, l_max, mode):
+    """Point counts around the tile sizes, including a single point (tail tiles are partial)."""
+    rng = np.random.default_rng(0)
+    for n in (1, 2, 3, 7, 63, 64, 65, 127, 129, 255, 1000, 4099):
+        for dtype in (np.float32, np.float64):
+            announce("ragged", l_max, mode, n, np.dtype(dtype).name)
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, True, mode)
+            got = run_calculator(xyz, l_max, True, mode)
+            for g, w in zip(got, want):
+                if w is not None:
+                    assert same_numbers(g, w).all(), (n, dtype)
+
+
+def test_zero_points():
+    """Reference: python/tests/test_corner_cases.py:7-32 and
+    sphericart-torch/python/tests/test_no_points.py:32-45."""
+    for l_max in (0, 3, 7, 10, 20, 50):
+        for cls in (sphericart_amd.SphericalHarmonics, sphericart_amd.SolidHarmonics):
+            calc = cls(l_max)
+            for dtype in (torch.float32, torch.float64):
+                xyz = torch.empty((0, 3), dtype=dtype, device="cuda")
+                sph, dsph, ddsph = calc.compute_with_hessians(xyz)
+                assert sph.shape == (0, (l_max + 1) ** 2)
+                assert dsph.shape == (0, 3, (l_max + 1) ** 2)
+                assert ddsph.shape == (0, 3, 3, (l_max + 1) ** 2)
+            del calc  # double delete must be harmless
+    calc = sphericart_amd.SphericalHarmonics(2)
+    calc._ensure_cuda_calculators()
+    calc.__del__()
+    calc.__del__()
+
+
+def test_unaligned_outputs_take_the_narrow_store_path(oracle, library):
+    """Output pointers that are not 16-byte aligned still give the same numbers."""
+    rng = np.random.default_rng(1)
+    for dtype, tdtype in ((np.float32, torch.float32), (np.float64, torch.float64)):
+        for l_max, mode in ((6, "gradients"), (7, "gradients"), (3, "hessians"), (3, "values")):
+            announce("unaligned", np.dtype(dtype).name, l_max, mode)
+            n, ny = 333, (l_max + 1) ** 2
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, True, mode)
+            sizes = (n * ny, 3 * n * ny, 9 * n * ny)
+            shapes = ((n, ny), (n, 3, ny), (n, 3, 3, ny))
+            raw = [torch.zeros(s + 1, dtype=tdtype, device="cuda") for s in sizes]
+            out = tuple(raw[i][1:].view(shapes[i]) if w is not None else None for i, w in enumerate(want))
+            assert out[0].data_ptr() % 16 != 0
+            status, _ = run_launch_layer(library, torch.from_numpy(xyz).cuda(), l_max, True, mode, out=out)
+            assert status == 0, library.sphx_last_error()
+            torch.cuda.synchronize()
+            for o, w in zip(out, want):
+                if w is not None:
+                    assert same_numbers(o.cpu().numpy(), w).all()
+
+
+def test_non_contiguous_input(oracle):
+    """Reference: sphericart-torch/python/tests/test_autograd.py:88-124 (inputs are made contiguous)."""
+    rng = np.random.default_rng(2)
+    wide = torch.from_numpy(rng.normal(size=(100, 6))).cuda()
+    xyz = wide[:, ::2]
+    assert not xyz.is_contiguous()
+    calc = sphericart_amd.SolidHarmonics(5)
+    sph, dsph = calc.compute_with_gradients(xyz)
+    want = oracle.compute(xyz.cpu().numpy().copy(), 5, False, "gradients")
+    assert same_numbers(sph.cpu().numpy(), want[0]).all()
+    assert same_numbers(dsph.cpu().numpy(), want[1]).all()
+
+
+def test_user_streams(oracle):
+    """Work goes to the caller's stream; two streams give the same numbers
+    (reference: sphericart-torch/python/tests/test_cuda_stream.py:15-29)."""
+    rng = np.random.default_rng(3)
+    xyz_host = rng.normal(size=(5000, 3)).astype(np.float32)
+    want = oracle.compute(xyz_host, 8, True, "gradients")
+    calc = sphericart_amd.SphericalHarmonics(8)
+    results = []
+    for _ in range(2):
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            xyz = torch.from_numpy(xyz_host).cuda()
+            sph, dsph = calc.compute_with_gradients(xyz)
+        stream.synchronize()
+        results.append((sph.cpu().numpy(), dsph.cpu().numpy()))
+    for sph, dsph in results:
+        assert same_numbers(sph, want[0]).all() and same_numbers(dsph, want[1]).all()
+
+
+def test_offsets_beyond_32_bits(oracle, library):
+    """Element offsets past 2^31 (the reference's device kernel indexes with int,
+    sphericart/src/sphericart_impl.cu:159,195): check the last rows of a 2.4e9-element dsph."""
+    l_max, n = 32, 740_000
+    ny = (l_max + 1) ** 2
+    assert 3 * n * ny > 2**31
+    announce("large offsets", n, l_max)
+    rng = np.random.default_rng(4)
+    tail = rng.normal(size=(2000, 3)).astype(np.float32)
+    xyz = torch.ones((n, 3), dtype=torch.float32, device="cuda")
+    xyz[-2000:] = torch.from_numpy(tail).cuda()
+    status, (sph, dsph, _) = run_launch_layer(library, xyz, l_max, True, "gradients")
+    assert status == 0, library.sphx_last_error()
+    torch.cuda.synchronize()
+    want = oracle.compute(tail, l_max, True, "gradients")
+    assert same_numbers(sph[-2000:].cpu().numpy(), want[0]).all()
+    assert same_numbers(dsph[-2000:].cpu().numpy(), want[1]).all()
+    first = oracle.compute(np.ones((1, 3), dtype=np.float32), l_max, True, "gradients")
+    assert same_numbers(dsph[:1].cpu().numpy(), first[1]).all()
+
+
+def test_unsupported_l_max():
+    calc = sphericart_amd.SphericalHarmonics(65)
+    with pytest.raises(RuntimeError, match="failed to initialize"):
+        calc.compute(torch.zeros((4, 3), device="cuda"))
+
+
+def test_rows_too_large_for_lds_are_reported(library):
+    xyz = torch.ones((4, 3), dtype=torch.float64, device="cuda")
+    status, _ = run_launch_layer(library, xyz, 60, True, "hessians")
+    assert status == 2
+    assert b"LDS" in library.sphx_last_error()
+
+
+def test_c_api_aborts_on_null_output():
+    """compute_* print `fatal error: ...` and abort (reference: sphericart-capi.cpp:653-666);
+    the check happens on the host before any device work."""
+    code = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "import torch, sphericart_amd\n"
+        "lib = sphericart_amd.get_library()\n"
+        "calc = lib.sphericart_cuda_spherical_harmonics_new_f(3)\n"
+        "assert calc\n"
+        "xyz = torch.ones((4, 3), dtype=torch.float32, device='cuda')\n"
+        "sph = torch.empty((4, 16), dtype=torch.float32, device='cuda')\n"
+        "print('before', flush=True)\n"
+        "lib.sphericart_cuda_spherical_harmonics_compute_array_with_gradients_f(calc, xyz.data_ptr(), 4, sph.data_ptr(), None, None)\n"
+        "print('after', flush=True)\n"
+    ) % ROOT
+    done = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert done.returncode == -6, (done.returncode, done.stdout, done.stderr)
+    assert "before" in done.stdout and "after" not in done.stdout
+    assert "fatal error:" in done.stdout and "dsph != nullptr" in done.stdout

@@ -1,0 +1,136 @@
+"""GPU results against the CPU oracle and the golden vectors, through the C entry points.
+
+Bar (reference: python/tests/test_cupy.py:22-49): |gpu - cpu| <= 1e-5 max(1, |cpu|) in float32,
+1e-12 max(1, |cpu|) in float64, and non-finite exactly where the reference is non-finite
+(float32 prefactors overflow from l = 29). Because library and oracle are both built without
+FMA contraction and follow the same operation order, the tests also demand the stronger
+property that every number is identical.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from golden_io import CONFIGS, config_case, edge_cases
+from gpu_utils import announce, run_calculator, run_launch_layer
+from helpers import MODES, same_numbers, special_points, within_tolerance
+from sphericart_amd.workloads import WORKLOADS
+
+pytestmark = pytest.mark.gpu
+
+L_MAX_SWEEP = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 16, 20, 25, 32]
+
+
+def check(got, want, what):
+    for g, w, label in zip(got, want, ("sph", "dsph", "ddsph")):
+        assert (g is None) == (w is None), (what, label)
+        if w is None:
+            continue
+        assert g.shape == w.shape and g.dtype == w.dtype, (what, label)
+        ok = within_tolerance(g, w)
+        assert ok.all(), (what, label, "outside tolerance:", int((~ok).sum()))
+        same = same_numbers(g, w)
+        assert same.all(), (what, label, "not identical:", int((~same).sum()))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("normalized", [True, False])
+@pytest.mark.parametrize("mode", MODES)
+def test_sweep_against_oracle(oracle, dtype, normalized, mode):
+    rng = np.random.default_rng(42)
+    for l_max in L_MAX_SWEEP:
+        announce("sweep", np.dtype(dtype).name, "normalized" if normalized else "solid", mode, "l_max", l_max)
+        xyz = special_points(dtype, rng, 777)
+        want = oracle.compute(xyz, l_max, normalized, mode)
+        got = run_calculator(xyz, l_max, normalized, mode)
+        check(got, want, (l_max, normalized, mode))
+
+
+@pytest.mark.parametrize("name", CONFIGS)
+def test_golden_benchmark_configurations(name):
+    xyz, l_max, normalized, mode, want = config_case(name)
+    announce("golden", name)
+    check(run_calculator(xyz, l_max, normalized, mode), want, name)
+
+
+@pytest.mark.parametrize("tag", ["f32", "f64"])
+def test_golden_edge_cases(tag):
+    for xyz, l_max, normalized, mode, want in edge_cases(tag):
+        announce("golden edge", tag, l_max, normalized, mode)
+        check(run_calculator(xyz, l_max, normalized, mode), want, (tag, l_max, normalized, mode))
+
+
+@pytest.mark.parametrize("name", CONFIGS)
+def test_benchmark_configurations_at_full_size(oracle, library, name):
+    """The five configurations at their real sizes: every number against the oracle, in slabs."""
+    w = WORKLOADS[name]
+    announce("full size", name, w.description)
+    xyz = w.points()
+    xyz_dev = torch.from_numpy(xyz).cuda()
+    status, out = run_launch_layer(library, xyz_dev, w.l_max, w.normalized, w.derivatives)
+    assert status == 0, library.sphx_last_error()
+    torch.cuda.synchronize()
+    slab = max(1, min(w.n_samples, (256 << 20) // w.bytes_per_point))
+    for first in range(0, w.n_samples, slab):
+        last = min(w.n_samples, first + slab)
+        want = oracle.compute(xyz[first:last], w.l_max, w.normalized, w.derivatives)
+        got = tuple(o[first:last].cpu().numpy() if o is not None else None for o in out)
+        check(got, want, (name, first))
+
+
+@pytest.mark.parametrize("name", ["cfg3", "cfg4", "cfg5"])
+def test_size_independent_properties_at_full_size(library, name):
+    """Identities that need no reference at all, evaluated on the device over the whole output:
+    Unsold's sum rule, Euler homogeneity, harmonicity and symmetry of the Hessian."""
+    w = WORKLOADS[name]
+    announce("properties", name)
+    xyz = torch.from_numpy(w.points()).cuda()
+    status, (sph, dsph, ddsph) = run_launch_layer(library, xyz, w.l_max, w.normalized, w.derivatives)
+    assert status == 0, library.sphx_last_error()
+    torch.cuda.synchronize()
+    l_top = min(w.l_max, 16)  # float32 loses the high-|m| prefactors beyond l ~ 18
+    r = xyz.double().norm(dim=1)
+    eps = 3e-4 if w.dtype == "f32" else 1e-10
+    for l in range(l_top + 1):
+        block = slice(l * l, (l + 1) ** 2)
+        total = (sph[:, block].double() ** 2).sum(dim=1)
+        want = (2 * l + 1) / (4 * np.pi) * (torch.ones_like(r) if w.normalized else r ** (2 * l))
+        assert torch.allclose(total, want, rtol=eps * (l + 1), atol=0), (name, "sum rule", l)
+        radial = torch.einsum("ia,iak->ik", xyz.double(), dsph[:, :, block].double())
+        scale = (dsph[:, :, block].double().abs().amax(dim=(1, 2)) * r).clamp_min(1e-30)
+        if w.normalized:
+            assert ((radial.abs().amax(dim=1) / scale) < eps * (l + 1)).all(), (name, "r.grad = 0", l)
+        else:
+            diff = (radial - l * sph[:, block].double()).abs().amax(dim=1)
+            assert ((diff / scale) < eps * (l + 1)).all(), (name, "r.grad = l", l)
+    if ddsph is not None:
+        assert torch.equal(ddsph, ddsph.transpose(1, 2))
+        if not w.normalized:
+            trace = (ddsph[:, 0, 0] + ddsph[:, 1, 1] + ddsph[:, 2, 2]).abs().amax(dim=1)
+            top = ddsph.abs().amax(dim=(1, 2, 3))
+            assert (trace <= 1e-9 * top).all(), (name, "harmonicity")
+
+
+def test_finite_differences_through_the_device():
+    """Same pattern as the reference's device-side derivative test
+    (sphericart/tests/test_derivatives_sycl.cpp:262-312): analytic gradients and Hessians from the
+    device against central differences of device values, float64, delta = 1e-4, tolerance 1e-4."""
+    delta, tol = 1e-4, 1e-4
+    rng = np.random.default_rng(8)
+    xyz = rng.normal(size=(16, 3))
+    xyz *= (rng.uniform(0.8, 1.5, size=16) / np.linalg.norm(xyz, axis=1))[:, None]
+    for normalized in (True, False):
+        for l_max in (1, 4, 6, 9, 14):
+            announce("finite differences", normalized, l_max)
+            _, dsph, ddsph = run_calculator(xyz, l_max, normalized, "hessians")
+            gscale = 1e-2 * np.abs(dsph).max()
+            hscale = 1e-2 * np.abs(ddsph).max() + 1e-9
+            for a in range(3):
+                step = np.zeros(3)
+                step[a] = delta
+                plus = run_calculator(xyz + step, l_max, normalized, "hessians")
+                minus = run_calculator(xyz - step, l_max, normalized, "hessians")
+                fd1 = (plus[0] - minus[0]) / (2 * delta)
+                fd2 = (plus[1] - minus[1]) / (2 * delta)
+                assert (np.abs(dsph[:, a] - fd1) <= tol * np.maximum(np.abs(fd1), gscale)).all()
+                assert (np.abs(ddsph[:, a] - fd2) <= tol * np.maximum(np.abs(fd2), hscale)).all()

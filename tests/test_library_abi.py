@@ -1,0 +1,121 @@
+"""Host-side checks that need no GPU: the shared library loads, exports every symbol the headers
+declare, plans launches sensibly, and the Python calculators validate their input."""
+
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import sphericart_amd
+from sphericart_amd import _c_lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sphx_[a-z0-9_]+|sphericart_cuda_[a-z_]+harmonics_[a-z_]+?(?:_f)?)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(library):
+    c_api = [s for s in _declared("sphericart.h") if not s.endswith("_t")]
+    launch = _declared("sphx_launch.h")
+    assert sorted(c_api) == sorted(_c_lib.C_API_SYMBOLS)
+    assert len(c_api) == 20
+    for name in c_api + launch:
+        assert hasattr(library, name), name
+    assert set(_c_lib.LAUNCH_SYMBOLS) <= set(launch)
+
+
+def test_cxx_classes_are_exported(library):
+    out = subprocess.run(["nm", "-DC", _c_lib.LIBRARY_PATH], capture_output=True, text=True, check=True).stdout
+    for cls in ("SphericalHarmonics", "SolidHarmonics"):
+        for t in ("float", "double"):
+            assert f"sphericart::cuda::{cls}<{t}>::{cls}(unsigned long)" in out
+    for method in ("compute", "compute_with_gradients", "compute_with_hessians"):
+        assert f"sphericart::cuda::SphericalHarmonics<double>::{method}(" in out
+
+
+def test_header_compiles_as_c_and_cxx(tmp_path):
+    """include/sphericart.h is a C header and a C++ header; sphx_launch.h is plain C."""
+    c_file = tmp_path / "probe.c"
+    c_file.write_text('#include "sphericart.h"\n#include "sphx_launch.h"\nint main(void) { return 0; }\n')
+    subprocess.run(["gcc", "-std=c99", "-fsyntax-only", f"-I{ROOT}/include", str(c_file)], check=True)
+    cxx_file = tmp_path / "probe.cpp"
+    cxx_file.write_text(
+        '#include "sphericart.h"\n#include "sphericart_cuda.hpp"\n'
+        "int main() { sphericart::cuda::SolidHarmonics<float>* p = nullptr; (void)p; return 0; }\n"
+    )
+    subprocess.run(["g++", "-std=c++17", "-fsyntax-only", f"-I{ROOT}/include", str(cxx_file)], check=True)
+
+
+def _plan(library, n, l_max, mode, f64):
+    out = [ctypes.c_int() for _ in range(4)]
+    status = library.sphx_plan(n, l_max, mode, int(f64), *[ctypes.byref(v) for v in out])
+    return status, [v.value for v in out]
+
+
+def test_launch_plans(library):
+    status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 6, 1, False)
+    assert status == 0 and tile == 64 and threads == 64
+    assert lds == 64 * 4 * 49 * 4 and groups == 15625
+    for n, l_max, mode, f64 in ((10_000, 8, 1, True), (100_000, 16, 2, True), (200_000, 32, 1, False), (5, 20, 2, False)):
+        status, (tile, threads, lds, groups) = _plan(library, n, l_max, mode, f64)
+        assert status == 0
+        assert 1 <= tile <= 64 and threads == 256 and lds <= 160 * 1024
+        assert groups % 8 == 0 and groups >= 8
+    assert _plan(library, 10, 65, 0, False)[0] == 2       # beyond the tables
+    assert _plan(library, 10, 64, 2, True)[0] == 2        # one point's rows no longer fit in LDS
+    assert b"LDS" in library.sphx_last_error()
+    assert _plan(library, 10, -1, 0, False)[0] == 1
+    assert _plan(library, 10, 3, 7, False)[0] == 1
+
+
+def test_zero_samples_is_a_no_op(library):
+    # returns before touching pointers or the GPU (reference: sphericart_cuda.cpp:85-89)
+    assert library.sphx_forward_f32(None, 0, 4, 1, 2, None, None, None, None) == 0
+    assert library.sphx_forward_f64(None, 0, 4, 0, 0, None, None, None, None) == 0
+
+
+def test_null_pointers_are_rejected(library):
+    assert library.sphx_forward_f32(None, 3, 4, 1, 0, None, None, None, None) == 1
+    assert b"null" in library.sphx_last_error()
+
+
+def test_python_calculators_validate_input():
+    calc = sphericart_amd.SphericalHarmonics(4)
+    with pytest.raises(TypeError):
+        calc.compute(np.zeros((3, 3)))
+    with pytest.raises(TypeError):
+        calc.compute(torch.zeros((3, 3), dtype=torch.float16))
+    with pytest.raises(ValueError):
+        calc.compute(torch.zeros((3, 4)))
+    with pytest.raises(ValueError, match="no CPU evaluation path"):
+        calc.compute(torch.zeros((3, 3)))
+    with pytest.raises(ValueError):
+        sphericart_amd.SolidHarmonics(-1)
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    """Without the built library there is nothing to fall back to."""
+    code = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "from sphericart_amd import _c_lib\n"
+        "_c_lib.LIBRARY_PATH = %r\n"
+        "try:\n    _c_lib.get_library()\nexcept RuntimeError as e:\n    print('RuntimeError', e)\n"
+    ) % (ROOT, str(tmp_path / "absent.so"))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, check=True).stdout
+    assert "RuntimeError" in out and "no CPU or pure-Python evaluation path" in out
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="only meaningful without a GPU")
+def test_no_gpu_means_no_calculator(library):
+    """`new` maps the constructor's exception to NULL (reference: sphericart-capi.cpp:637-643)."""
+    assert library.sphericart_cuda_spherical_harmonics_new(3) is None
+    assert library.sphericart_cuda_solid_harmonics_new_f(3) is None
