@@ -46,7 +46,21 @@ def parse():
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--workload", default="cfg3")
+    p.add_argument(
+        "--settle-seconds",
+        type=float,
+        default=0.5,
+        help="untimed launches before the warm-up steps until the GPU has been busy this long: the "
+        "memory and fabric clocks of an idle MI355X take tens of milliseconds of load to ramp up "
+        "(the same launch takes 160 us right after idle and 136 us once settled)",
+    )
     p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument(
+        "--calibrate-copy",
+        action="store_true",
+        help="instead of the hot path, launch plain device-to-device copies of as many bytes as "
+        "the workload writes per launch: the yardstick for the FETCH_SIZE / WRITE_SIZE counters",
+    )
     return p.parse_args()
 
 
@@ -138,6 +152,30 @@ def main():
         if status != 0:
             raise RuntimeError(lib.sphx_last_error().decode())
 
+    if args.calibrate_copy:
+        nbytes = w.bytes_per_point * n
+        src = torch.zeros(nbytes // 4, dtype=torch.float32, device=xyz.device)
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        print(json.dumps({
+            "calibration": "device-to-device copy", "bytes_read_per_launch": src.numel() * 4,
+            "bytes_written_per_launch": src.numel() * 4, "steps": args.steps,
+            "us_per_launch": wall / args.steps * 1e6,
+        }))
+        return 0
+
+    settle_until = time.perf_counter() + args.settle_seconds
+    while time.perf_counter() < settle_until:
+        for _ in range(50):
+            step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -174,6 +212,7 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": f"{w.name}: {w.description}",
+            "settle_seconds": args.settle_seconds,
             "l_max": w.l_max,
             "n_samples": n,
             "derivatives": w.derivatives,

@@ -83,49 +83,55 @@ template <typename T> struct Entry {
     T v, gx, gy, gz, hxx, hxy, hxz, hyy, hyz, hzz;
 };
 
-// Chain rule for the polynomials evaluated at (x, y, z)/r, then store.
+// Chain rule for the polynomials evaluated at (x, y, z)/r.
 // templates.hpp:572-613: the Hessian is corrected first, from the uncorrected
 // gradient; then the gradient.
 template <typename T, int MODE, bool NORM>
-__device__ __forceinline__ void stage(const Rows<T>& out, int k, const Point<T>& p, Entry<T> e) {
+__device__ __forceinline__ Entry<T> finish(const Point<T>& p, Entry<T> e) {
+    if constexpr (MODE >= 1 && NORM) {
+        const T x = p.x, y = p.y, z = p.z, ir = p.ir;
+        auto tmp = (e.gx * x + e.gy * y + e.gz * z);
+        if constexpr (MODE == 2) {
+            auto irsq = ir * ir;
+            auto tmpx = x * e.hxx + y * e.hxy + z * e.hxz;
+            auto tmpy = x * e.hxy + y * e.hyy + z * e.hyz;
+            auto tmpz = x * e.hxz + y * e.hyz + z * e.hzz;
+            auto tmp2 = x * x * e.hxx + y * y * e.hyy + z * z * e.hzz + 2 * x * y * e.hxy +
+                        2 * x * z * e.hxz + 2 * y * z * e.hyz;
+            T nxx = (-2 * x * tmpx + e.hxx + 3 * x * x * tmp - tmp - 2 * x * e.gx + x * x * tmp2) *
+                    irsq;
+            T nyy = (-2 * y * tmpy + e.hyy + 3 * y * y * tmp - tmp - 2 * y * e.gy + y * y * tmp2) *
+                    irsq;
+            T nzz = (-2 * z * tmpz + e.hzz + 3 * z * z * tmp - tmp - 2 * z * e.gz + z * z * tmp2) *
+                    irsq;
+            T nxy = (-x * tmpy - y * tmpx + e.hxy + 3 * x * y * tmp - x * e.gy - y * e.gx +
+                     x * y * tmp2) *
+                    irsq;
+            T nxz = (-x * tmpz - z * tmpx + e.hxz + 3 * x * z * tmp - x * e.gz - z * e.gx +
+                     x * z * tmp2) *
+                    irsq;
+            T nyz = (-z * tmpy - y * tmpz + e.hyz + 3 * y * z * tmp - z * e.gy - y * e.gz +
+                     y * z * tmp2) *
+                    irsq;
+            e.hxx = nxx;
+            e.hyy = nyy;
+            e.hzz = nzz;
+            e.hxy = nxy;
+            e.hxz = nxz;
+            e.hyz = nyz;
+        }
+        e.gx = (e.gx - x * tmp) * ir;
+        e.gy = (e.gy - y * tmp) * ir;
+        e.gz = (e.gz - z * tmp) * ir;
+    }
+    return e;
+}
+
+// Store a finished entry into the point's staged rows.
+template <typename T, int MODE>
+__device__ __forceinline__ void put(const Rows<T>& out, int k, const Entry<T>& e) {
     out.sph[k] = e.v;
     if constexpr (MODE >= 1) {
-        if constexpr (NORM) {
-            const T x = p.x, y = p.y, z = p.z, ir = p.ir;
-            auto tmp = (e.gx * x + e.gy * y + e.gz * z);
-            if constexpr (MODE == 2) {
-                auto irsq = ir * ir;
-                auto tmpx = x * e.hxx + y * e.hxy + z * e.hxz;
-                auto tmpy = x * e.hxy + y * e.hyy + z * e.hyz;
-                auto tmpz = x * e.hxz + y * e.hyz + z * e.hzz;
-                auto tmp2 = x * x * e.hxx + y * y * e.hyy + z * z * e.hzz + 2 * x * y * e.hxy +
-                            2 * x * z * e.hxz + 2 * y * z * e.hyz;
-                T nxx = (-2 * x * tmpx + e.hxx + 3 * x * x * tmp - tmp - 2 * x * e.gx + x * x * tmp2) *
-                        irsq;
-                T nyy = (-2 * y * tmpy + e.hyy + 3 * y * y * tmp - tmp - 2 * y * e.gy + y * y * tmp2) *
-                        irsq;
-                T nzz = (-2 * z * tmpz + e.hzz + 3 * z * z * tmp - tmp - 2 * z * e.gz + z * z * tmp2) *
-                        irsq;
-                T nxy = (-x * tmpy - y * tmpx + e.hxy + 3 * x * y * tmp - x * e.gy - y * e.gx +
-                         x * y * tmp2) *
-                        irsq;
-                T nxz = (-x * tmpz - z * tmpx + e.hxz + 3 * x * z * tmp - x * e.gz - z * e.gx +
-                         x * z * tmp2) *
-                        irsq;
-                T nyz = (-z * tmpy - y * tmpz + e.hyz + 3 * y * z * tmp - z * e.gy - y * e.gz +
-                         y * z * tmp2) *
-                        irsq;
-                e.hxx = nxx;
-                e.hyy = nyy;
-                e.hzz = nzz;
-                e.hxy = nxy;
-                e.hxz = nxz;
-                e.hyz = nyz;
-            }
-            e.gx = (e.gx - x * tmp) * ir;
-            e.gy = (e.gy - y * tmp) * ir;
-            e.gz = (e.gz - z * tmp) * ir;
-        }
         const int ny = out.ny;
         out.dsph[k] = e.gx;
         out.dsph[ny + k] = e.gy;
@@ -142,6 +148,11 @@ __device__ __forceinline__ void stage(const Rows<T>& out, int k, const Point<T>&
             out.ddsph[8 * ny + k] = e.hzz;
         }
     }
+}
+
+template <typename T, int MODE, bool NORM>
+__device__ __forceinline__ void stage(const Rows<T>& out, int k, const Point<T>& p, Entry<T> e) {
+    put<T, MODE>(out, k, finish<T, MODE, NORM>(p, e));
 }
 
 // ---- l = 0..H in closed form, one point per lane ---------------------------
@@ -172,6 +183,36 @@ __device__ __forceinline__ void closed_form_job(const Point<T>& p, const Rows<T>
             e.gz = DZ[k];
             e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = static_cast<T>(0.0);
             stage<T, MODE, NORM>(out, k, p, e);
+        }
+    }
+}
+
+// Same, but the finished entries are handed back in registers so that the
+// caller can stage them in several passes through a small LDS buffer.
+template <typename T, int MODE, bool NORM, int H>
+__device__ __forceinline__ void closed_form_entries(const Point<T>& p,
+                                                    Entry<T> (&E)[(H + 1) * (H + 1)]) {
+    static_assert(MODE < 2 || H <= 1, "second derivatives in closed form stop at l = 1");
+    constexpr int NH = (H + 1) * (H + 1);
+    T Y[NH];
+    low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
+    if constexpr (MODE == 0) {
+#pragma unroll
+        for (int k = 0; k < NH; ++k) {
+            E[k].v = Y[k];
+        }
+    } else {
+        T DX[NH], DY[NH], DZ[NH];
+        low_gradients<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y, DX, DY, DZ);
+#pragma unroll
+        for (int k = 0; k < NH; ++k) {
+            Entry<T> e;
+            e.v = Y[k];
+            e.gx = DX[k];
+            e.gy = DY[k];
+            e.gz = DZ[k];
+            e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = static_cast<T>(0.0);
+            E[k] = finish<T, MODE, NORM>(p, e);
         }
     }
 }
