@@ -21,6 +21,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
+
 #include "sphx_lowl.hpp"
 
 namespace sphx {
@@ -245,10 +247,18 @@ __device__ __forceinline__ void azimuth_job(const Point<T>& p, int L, T* c, T* s
 // (entry (l, m) at l(l+1)/2 + m); c, s, tmz the point's azimuthal tables. The
 // three-term recursion runs downward in m for Q_l, and alongside for Q_{l-1}
 // (first derivatives) and Q_{l-2} (second derivatives).
+//
+// A job emits the entries with m_lo <= |m| <= m_hi only. The recursion itself
+// costs a handful of operations per m while an emitted pair of entries costs
+// hundreds, so a channel is cut into segments of consecutive m that different
+// lanes work on: a lane first runs the bare recursion from m = l down to its
+// segment (the same operations in the same order, hence the same numbers),
+// then does the full work inside it. m_hi == l marks the top segment, which
+// must reach down to l - 1 at least; m_lo == 0 the bottom one.
 template <typename T, int MODE, bool NORM>
-__device__ __forceinline__ void channel_job(int l, const Point<T>& p, T rxy, const T* F,
-                                            const T* Q, const T* c, const T* s, const T* tmz,
-                                            const Rows<T>& out) {
+__device__ __forceinline__ void channel_job(int l, int m_hi, int m_lo, const Point<T>& p, T rxy,
+                                            const T* F, const T* Q, const T* c, const T* s,
+                                            const T* tmz, const Rows<T>& out) {
     constexpr bool GRAD = MODE >= 1;
     constexpr bool HESS = MODE == 2;
     const T x = p.x, y = p.y, z = p.z;
@@ -268,9 +278,17 @@ __device__ __forceinline__ void channel_job(int l, const Point<T>& p, T rxy, con
         xy = x * y;
     }
 
+    const bool top = m_hi == l;
+
     // |m| = l (:122-152)
-    {
-        qlm_2 = qk[l];
+    qlm_2 = qk[l];
+    if constexpr (GRAD) {
+        ql1m_2 = 0;
+    }
+    if constexpr (HESS) {
+        ql2m_2 = 0.0;
+    }
+    if (top) {
         auto pq = qlm_2 * pk[l];
         Entry<T> neg, pos;
         neg.v = pq * s[l];
@@ -283,7 +301,6 @@ __device__ __forceinline__ void channel_job(int l, const Point<T>& p, T rxy, con
             neg.gx = pq * s[l - 1];
             neg.gy = pos.gx = pq * c[l - 1];
             pos.gy = -neg.gx;
-            ql1m_2 = 0;
             if constexpr (HESS) {
                 pq *= (l - 1);
                 pos.hxx = pq * c[l - 2];
@@ -291,7 +308,6 @@ __device__ __forceinline__ void channel_job(int l, const Point<T>& p, T rxy, con
                 pos.hxy = neg.hyy = -neg.hxx;
                 neg.hxy = pos.hxx;
                 pos.hyy = -pos.hxx;
-                ql2m_2 = 0.0;
             }
         }
         stage<T, MODE, NORM>(out, mid - l, p, neg);
@@ -299,8 +315,14 @@ __device__ __forceinline__ void channel_job(int l, const Point<T>& p, T rxy, con
     }
 
     // |m| = l - 1 (:154-198)
-    {
-        qlm_1 = -z * qlm_2;
+    qlm_1 = -z * qlm_2;
+    if constexpr (GRAD) {
+        ql1m_1 = qk[-1];
+    }
+    if constexpr (HESS) {
+        ql2m_1 = 0.0;
+    }
+    if (top) {
         auto pq = qlm_1 * pk[l - 1];
         Entry<T> neg, pos;
         neg.v = pq * s[l - 1];
@@ -313,7 +335,6 @@ __device__ __forceinline__ void channel_job(int l, const Point<T>& p, T rxy, con
             neg.gx = pq * s[l - 2];
             neg.gy = pos.gx = pq * c[l - 2];
             pos.gy = -neg.gx;
-            ql1m_1 = qk[-1];
             auto pdq = pk[l - 1] * (l + l - 1) * ql1m_1;
             neg.gz = pdq * s[l - 1];
             pos.gz = pdq * c[l - 1];
@@ -334,15 +355,38 @@ __device__ __forceinline__ void channel_job(int l, const Point<T>& p, T rxy, con
                 pos.hyy = -pos.hxx;
                 pos.hyz = -neg.hxz;
                 neg.hyz = pos.hxz;
-                ql2m_1 = 0.0;
             }
         }
         stage<T, MODE, NORM>(out, mid - l + 1, p, neg);
         stage<T, MODE, NORM>(out, mid + l - 1, p, pos);
     }
 
+    // bare recursion down to the segment: the Q updates of :202-204, :210-212, :228-235, :289-290
+    for (auto m = l - 2; m > m_hi; --m) {
+        const T tz = tmz[m];
+        qlm_0 = qk[m] * (tz * qlm_1 + rxy * qlm_2);
+        qlm_2 = qlm_1;
+        qlm_1 = qlm_0;
+        if constexpr (GRAD) {
+            ql1m_0 = qk[m - l] * (tz * ql1m_1 + rxy * ql1m_2);
+            ql1m_2 = ql1m_1;
+            ql1m_1 = ql1m_0;
+        }
+        if constexpr (HESS) {
+            if (m == l - 2) {
+                ql2m_0 = qk[-l - 1];
+            } else {
+                ql2m_0 = qk[m - 2 * l + 1] * (tz * ql2m_1 + rxy * ql2m_2);
+            }
+            ql2m_2 = ql2m_1;
+            ql2m_1 = ql2m_0;
+        }
+    }
+
     // l - 2 >= |m| >= 1 (:201-390; the reference's two loops share one body)
-    for (auto m = l - 2; m > 0; --m) {
+    const int m_first = m_hi < l - 2 ? m_hi : l - 2;
+    const int m_last = m_lo > 1 ? m_lo : 1;
+    for (auto m = m_first; m >= m_last; --m) {
         const T cm = c[m], sm = s[m], tz = tmz[m], pkm = pk[m];
         qlm_0 = qk[m] * (tz * qlm_1 + rxy * qlm_2);
         qlm_2 = qlm_1;
@@ -419,7 +463,7 @@ __device__ __forceinline__ void channel_job(int l, const Point<T>& p, T rxy, con
     }
 
     // m = 0 (:392-426)
-    {
+    if (m_lo == 0) {
         const T tz = tmz[0];
         qlm_0 = qk[0] * (tz * qlm_1 + rxy * qlm_2);
         Entry<T> e;
@@ -468,49 +512,51 @@ __device__ __forceinline__ unsigned staged_index(unsigned g, unsigned row, unsig
     return g + pad * __umulhi(g, magic);
 }
 
+template <typename T, bool STREAMING, typename V>
+__device__ __forceinline__ void emit(V v, V* dst) {
+    if constexpr (STREAMING) {
+        __builtin_nontemporal_store(v, dst);
+    } else {
+        *dst = v;
+    }
+}
+
+// Copy `len` staged elements to dst[0 .. len). Whatever the alignment of dst, the bulk goes out
+// as 16-byte stores at 16-byte aligned addresses, consecutive lanes to consecutive addresses;
+// at most three (float) or one (double) leading and trailing elements are stored one by one.
 template <typename T, bool STREAMING>
 __device__ __forceinline__ void copy_out(const T* staged, T* dst, unsigned len, unsigned row,
-                                         unsigned pad, unsigned magic, bool wide, unsigned tid,
+                                         unsigned pad, unsigned magic, unsigned tid,
                                          unsigned nthreads) {
     using V = typename Pack<T>::type;
     constexpr unsigned W = Pack<T>::width;
-    unsigned done = 0;
-    if (wide) {
-        const unsigned nvec = len / W;
-        V* dst_v = reinterpret_cast<V*>(dst);
-        if (pad == 0) {
-            const V* src_v = reinterpret_cast<const V*>(staged);
-            for (unsigned g = tid; g < nvec; g += nthreads) {
-                V v = src_v[g];
-                if constexpr (STREAMING) {
-                    __builtin_nontemporal_store(v, dst_v + g);
-                } else {
-                    dst_v[g] = v;
-                }
-            }
-        } else {
-            for (unsigned g = tid; g < nvec; g += nthreads) {
-                V v;
+    const unsigned misalign = static_cast<unsigned>(reinterpret_cast<uintptr_t>(dst) & 15u);
+    unsigned head = ((16u - misalign) & 15u) / static_cast<unsigned>(sizeof(T));
+    if (head > len) head = len;
+    const unsigned nvec = (len - head) / W;
+    V* dst_v = reinterpret_cast<V*>(dst + head);
+    if (pad == 0 && head == 0) {
+        const V* src_v = reinterpret_cast<const V*>(staged);
+        for (unsigned g = tid; g < nvec; g += nthreads) {
+            emit<T, STREAMING>(src_v[g], dst_v + g);
+        }
+    } else {
+        for (unsigned g = tid; g < nvec; g += nthreads) {
+            V v;
 #pragma unroll
-                for (unsigned e = 0; e < W; ++e) {
-                    v[e] = staged[staged_index<T>(g * W + e, row, pad, magic)];
-                }
-                if constexpr (STREAMING) {
-                    __builtin_nontemporal_store(v, dst_v + g);
-                } else {
-                    dst_v[g] = v;
-                }
+            for (unsigned e = 0; e < W; ++e) {
+                const unsigned at = head + g * W + e;
+                v[e] = staged[pad ? staged_index<T>(at, row, pad, magic) : at];
             }
+            emit<T, STREAMING>(v, dst_v + g);
         }
-        done = nvec * W;
     }
-    for (unsigned g = done + tid; g < len; g += nthreads) {
-        T v = staged[pad ? staged_index<T>(g, row, pad, magic) : g];
-        if constexpr (STREAMING) {
-            __builtin_nontemporal_store(v, dst + g);
-        } else {
-            dst[g] = v;
-        }
+    // leading and trailing elements
+    const unsigned tail_first = head + nvec * W;
+    const unsigned loose = head + (len - tail_first);
+    if (tid < loose) {
+        const unsigned at = tid < head ? tid : tail_first + (tid - head);
+        emit<T, STREAMING>(staged[pad ? staged_index<T>(at, row, pad, magic) : at], dst + at);
     }
 }
 

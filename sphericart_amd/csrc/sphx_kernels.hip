@@ -63,9 +63,11 @@ struct Tiling {
     int tile;        // points per tile (S)
     unsigned pad;    // spare LDS elements after each point's block (0 or 1)
     unsigned magic[3]; // ceil(2^32 / row) for row = ny, 3 ny, 9 ny
-    unsigned wide;   // bit a: array a (0 sph, 1 dsph, 2 ddsph) may be written 16 bytes at a time
     // LDS carve-up, in elements of T from the start of dynamic LDS
-    unsigned off_dsph, off_ddsph, off_F, off_Q, off_c, off_s, off_tmz, off_pts;
+    unsigned off_dsph, off_ddsph, off_F, off_Q, off_pts, off_jobs;
+    // every l channel above the closed-form limit is cut into segments of `segment`
+    // consecutive m; one point has `jobs_per_point` (channel, segment) jobs in all
+    unsigned segment, jobs_per_point;
     // persistent-workgroup walk: workgroups of one XCD take consecutive tiles
     unsigned tiles_per_group;
 };
@@ -85,15 +87,15 @@ __device__ __forceinline__ void flush_run(const Tiling& g, T* lds, unsigned long
                                           unsigned valid, T* sph, T* dsph, T* ddsph,
                                           unsigned tid, unsigned nthreads) {
     const unsigned ny = g.ny;
-    copy_out<T, SPHX_STREAMING_STORES>(lds, sph + first * ny, valid * ny, ny, g.pad, g.magic[0], g.wide & 1u, tid,
-                      nthreads);
+    copy_out<T, SPHX_STREAMING_STORES>(lds, sph + first * ny, valid * ny, ny, g.pad, g.magic[0], tid,
+                                       nthreads);
     if constexpr (MODE >= 1) {
-        copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_dsph, dsph + first * 3 * ny, valid * 3 * ny, 3 * ny, g.pad,
-                          g.magic[1], g.wide & 2u, tid, nthreads);
+        copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_dsph, dsph + first * 3 * ny, valid * 3 * ny,
+                                           3 * ny, g.pad, g.magic[1], tid, nthreads);
     }
     if constexpr (MODE == 2) {
-        copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_ddsph, ddsph + first * 9 * ny, valid * 9 * ny, 9 * ny, g.pad,
-                          g.magic[2], g.wide & 4u, tid, nthreads);
+        copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_ddsph, ddsph + first * 9 * ny, valid * 9 * ny,
+                                           9 * ny, g.pad, g.magic[2], tid, nthreads);
     }
 }
 
@@ -201,6 +203,7 @@ __global__ __launch_bounds__(256) void recursion_kernel(Tiling g, const T* __res
 
     T* F = lds + g.off_F;
     T* Q = lds + g.off_Q;
+    unsigned short* job_table = reinterpret_cast<unsigned short*>(lds + g.off_jobs);
     {
         const unsigned nq = (L + 1) * (L + 2) / 2;
         const T* cF = table_F<T>();
@@ -208,6 +211,18 @@ __global__ __launch_bounds__(256) void recursion_kernel(Tiling g, const T* __res
         for (unsigned i = tid; i < nq; i += nthreads) {
             F[i] = cF[i];
             Q[i] = cQ[i];
+        }
+        // (l, segment) pairs, top segments of all channels first, longest channels first:
+        // neighbouring lanes then run loops of the same length
+        if (tid == 0) {
+            unsigned n = 0;
+            for (unsigned seg = 0; seg * g.segment <= static_cast<unsigned>(L); ++seg) {
+                for (int l = L; l > H; --l) {
+                    if (seg * g.segment <= static_cast<unsigned>(l)) {
+                        job_table[n++] = static_cast<unsigned short>((l << 8) | seg);
+                    }
+                }
+            }
         }
     }
 
@@ -221,53 +236,106 @@ __global__ __launch_bounds__(256) void recursion_kernel(Tiling g, const T* __res
     unsigned xcd_last = xcd_first + g.tiles_per_group;
     if (xcd_last > g.n_tiles) xcd_last = g.n_tiles;
 
-    for (unsigned tile_idx = xcd_first + lane_in_xcd; tile_idx < xcd_last;
-         tile_idx += groups_per_xcd) {
+    // Per-point data (normalised coordinates, c_m, s_m, 2(m+1)z) is double buffered: while the
+    // recursion jobs of one tile run, wave 0 prepares the next tile, so that the LDS rows are
+    // only held from the first staged entry to the end of the flush.
+    const unsigned per_point_tables = 3 * (L + 1) + 8;
+    auto tables_of = [&](unsigned parity, unsigned s) -> T* {
+        return lds + g.off_pts + (parity * S + s) * per_point_tables;
+    };
+    auto prepare = [&](unsigned tile_idx, unsigned parity, T rx, T ry, T rz) {
+        // templates.hpp:386-400 and :451-466 for point `tid` of the tile
+        (void)tile_idx;
+        T* rec = tables_of(parity, tid);
+        Point<T> p;
+        p.x = rx;
+        p.y = ry;
+        p.z = rz;
+        p.x2 = p.x * p.x;
+        p.y2 = p.y * p.y;
+        p.z2 = p.z * p.z;
+        p.ir = 0.0;
+        if constexpr (NORM) {
+            p.ir = 1 / root(p.x2 + p.y2 + p.z2);
+            p.x *= p.ir;
+            p.y *= p.ir;
+            p.z *= p.ir;
+            p.x2 = p.x * p.x;
+            p.y2 = p.y * p.y;
+            p.z2 = p.z * p.z;
+        }
+        rec[0] = p.x;
+        rec[1] = p.y;
+        rec[2] = p.z;
+        rec[3] = p.x2;
+        rec[4] = p.y2;
+        rec[5] = p.z2;
+        rec[6] = p.ir;
+        azimuth_job<T>(p, L, rec + 8, rec + 8 + (L + 1), rec + 8 + 2 * (L + 1));
+    };
+    auto point_of = [&](const T* rec) {
+        Point<T> q;
+        q.x = rec[0];
+        q.y = rec[1];
+        q.z = rec[2];
+        q.x2 = rec[3];
+        q.y2 = rec[4];
+        q.z2 = rec[5];
+        q.ir = rec[6];
+        return q;
+    };
+    auto valid_in = [&](unsigned tile_idx) -> unsigned {
         const unsigned long long first = static_cast<unsigned long long>(tile_idx) * S;
         const unsigned long long left = g.n_samples - first;
-        const unsigned valid = left < S ? static_cast<unsigned>(left) : S;
+        return left < S ? static_cast<unsigned>(left) : S;
+    };
 
-        __syncthreads(); // previous tile fully flushed (and tables in place)
+    unsigned tile_idx = xcd_first + lane_in_xcd;
+    unsigned parity = 0;
+    if (tile_idx < xcd_last && tid < valid_in(tile_idx)) {
+        const T* src = xyz + (static_cast<unsigned long long>(tile_idx) * S + tid) * 3;
+        prepare(tile_idx, 0, src[0], src[1], src[2]);
+    }
 
-        Point<T> p;
-        if (tid < valid) {
-            p = load_point<T, NORM>(xyz + (first + tid) * 3);
-            T* rec = lds + g.off_pts + tid * 8;
-            rec[0] = p.x;
-            rec[1] = p.y;
-            rec[2] = p.z;
-            rec[3] = p.x2;
-            rec[4] = p.y2;
-            rec[5] = p.z2;
-            rec[6] = p.ir;
-            azimuth_job<T>(p, L, lds + g.off_c + tid * (L + 1), lds + g.off_s + tid * (L + 1),
-                           lds + g.off_tmz + tid * (L + 1));
-        }
-        __syncthreads();
+    for (; tile_idx < xcd_last; tile_idx += groups_per_xcd, parity ^= 1u) {
+        const unsigned long long first = static_cast<unsigned long long>(tile_idx) * S;
+        const unsigned valid = valid_in(tile_idx);
+        const unsigned next_idx = tile_idx + groups_per_xcd;
+        const unsigned next_valid = next_idx < xcd_last ? valid_in(next_idx) : 0u;
+
+        __syncthreads(); // rows free again (previous flush done); this tile's point data in place
 
         if (tid < 64) {
+            // fetch the next tile's coordinates now, use them after the closed-form work
+            T nx = 0, ny_ = 0, nz = 0;
+            if (tid < next_valid) {
+                const T* src = xyz + (static_cast<unsigned long long>(next_idx) * S + tid) * 3;
+                nx = src[0];
+                ny_ = src[1];
+                nz = src[2];
+            }
             if (tid < valid) {
+                const Point<T> p = point_of(tables_of(parity, tid));
                 closed_form_job<T, MODE, NORM, H>(p, rows_of<T, MODE>(g, lds, tid));
             }
+            if (tid < next_valid) {
+                prepare(next_idx, parity ^ 1u, nx, ny_, nz);
+            }
         } else {
-            const unsigned jobs = valid * (L - H);
+            const unsigned jobs = valid * g.jobs_per_point;
             for (unsigned j = tid - 64; j < jobs; j += nthreads - 64) {
                 const unsigned s = j % valid;
-                const int l = L - static_cast<int>(j / valid); // longest recursions first
-                const T* rec = lds + g.off_pts + s * 8;
-                Point<T> q;
-                q.x = rec[0];
-                q.y = rec[1];
-                q.z = rec[2];
-                q.x2 = rec[3];
-                q.y2 = rec[4];
-                q.z2 = rec[5];
-                q.ir = rec[6];
+                const unsigned entry = job_table[j / valid];
+                const int l = static_cast<int>(entry >> 8);
+                const int m_hi = l - static_cast<int>((entry & 0xffu) * g.segment);
+                const int m_lo = m_hi - static_cast<int>(g.segment) + 1 > 0
+                                     ? m_hi - static_cast<int>(g.segment) + 1
+                                     : 0;
+                const T* rec = tables_of(parity, s);
+                const Point<T> q = point_of(rec);
                 const T rxy = q.x2 + q.y2;
-                channel_job<T, MODE, NORM>(l, q, rxy, F, Q, lds + g.off_c + s * (L + 1),
-                                           lds + g.off_s + s * (L + 1),
-                                           lds + g.off_tmz + s * (L + 1),
-                                           rows_of<T, MODE>(g, lds, s));
+                channel_job<T, MODE, NORM>(l, m_hi, m_lo, q, rxy, F, Q, rec + 8, rec + 8 + (L + 1),
+                                           rec + 8 + 2 * (L + 1), rows_of<T, MODE>(g, lds, s));
             }
         }
         __syncthreads();
@@ -377,7 +445,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     } else {
         plan->threads = 256;
         const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", 36 * 1024));
-        const unsigned per_point = (row_elems + 3 * (l_max + 1) + 8) * elem;
+        const unsigned per_point = (row_elems + 2 * (3 * (l_max + 1) + 8)) * elem;
         unsigned fit = budget / per_point;
         S = fit >= 1 ? pow2_floor(fit) : 1;
         if (S > 64) S = 64;
@@ -403,14 +471,28 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
         at += nq;
         g.off_Q = at;
         at += nq;
-        g.off_c = at;
-        at += S * (l_max + 1);
-        g.off_s = at;
-        at += S * (l_max + 1);
-        g.off_tmz = at;
-        at += S * (l_max + 1);
-        g.off_pts = at;
-        at += S * 8;
+        g.off_pts = at; // per point: 8 coordinates-and-such, then c, s, 2(m+1)z; two buffers
+        at += 2 * S * (3 * (l_max + 1) + 8);
+        // segment length: the shortest that still gives every job its own lane (192 lanes run
+        // the recursion jobs), so that the longest chain of dependent work is as short as possible
+        const int hard = mode == 2 ? 1 : 6;
+        static const unsigned candidates[] = {2, 3, 4, 6, 8, 12, 16, 24, 32, 65};
+        unsigned chosen = 65, jobs = 0;
+        const int forced_segment = env_int("SPHX_SEGMENT", 0);
+        for (unsigned cand : candidates) {
+            unsigned count = 0;
+            for (int l = hard + 1; l <= l_max; ++l) count += static_cast<unsigned>(l) / cand + 1;
+            if ((forced_segment > 1 && cand >= static_cast<unsigned>(forced_segment)) ||
+                (forced_segment <= 1 && S * count <= 192) || cand == 65) {
+                chosen = cand;
+                jobs = count;
+                break;
+            }
+        }
+        g.segment = chosen;
+        g.jobs_per_point = jobs;
+        g.off_jobs = at;
+        at += (jobs * 2 + static_cast<unsigned>(elem) - 1) / static_cast<unsigned>(elem);
     }
     plan->lds_bytes = at * static_cast<unsigned>(elem);
     if (plan->lds_bytes > static_cast<unsigned>(lds_limit)) {
@@ -443,20 +525,6 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
         g.tiles_per_group = (g.n_tiles + 7u) / 8u;
     }
     return SPHX_OK;
-}
-
-template <typename T>
-static unsigned wide_mask(const Tiling& g, int mode, const T* sph, const T* dsph, const T* ddsph) {
-    unsigned mask = 0;
-    const T* ptr[3] = {sph, dsph, ddsph};
-    for (int a = 0; a <= mode; ++a) {
-        const unsigned long long row = (a == 0 ? 1ull : (a == 1 ? 3ull : 9ull)) * g.ny;
-        const unsigned long long tile_bytes = row * g.tile * sizeof(T);
-        if ((reinterpret_cast<uintptr_t>(ptr[a]) % 16 == 0) && (tile_bytes % 16 == 0)) {
-            mask |= 1u << a;
-        }
-    }
-    return mask;
 }
 
 template <typename T, int MODE, bool NORM, int H>
@@ -551,7 +619,6 @@ static int forward(const T* xyz, size_t n_samples, int l_max, int normalized, in
                            g_compute_units[device], &plan);
     }
     if (status == SPHX_OK) {
-        plan.g.wide = wide_mask<T>(plan.g, mode, sph, dsph, ddsph);
         hipStream_t s = reinterpret_cast<hipStream_t>(stream);
         hipError_t e;
         if (normalized) {
