@@ -7,9 +7,11 @@
 //                    classes, sphericart/src/sphericart.cpp:45-92)
 //   azimuth_job      one lane = one point: c_m, s_m, 2(m+1)z into LDS
 //                    (sphericart/include/templates.hpp:451-466)
-//   channel_job      one lane = one (point, l) pair: the downward-in-m Q_l^m
-//                    recursion with first and second derivatives
-//                    (sphericart/include/templates_core.hpp:35-427)
+//   sequence_job     one lane = one (point, l, sequence) triple: one of the downward-in-m
+//                    three-term recursions of Q_l, Q_{l-1}, Q_{l-2}, iterates to LDS
+//   entry_job        one lane = one (point, l, m) triple: the entries (l, +-m)
+//                    with first and second derivatives from those iterates
+//                    (together: sphericart/include/templates_core.hpp:35-427)
 //
 // plus the unit-sphere chain rule (templates.hpp:553-614) applied in registers
 // right before an entry is staged, and copy_out, which streams a finished tile
@@ -241,61 +243,105 @@ __device__ __forceinline__ void azimuth_job(const Point<T>& p, int L, T* c, T* s
     }
 }
 
-// ---- one l channel for one point -------------------------------------------
+// ---- one bare recursion of one l channel -----------------------------------
 //
-// templates_core.hpp:35-427. F and Q are the two triangular prefactor blocks
-// (entry (l, m) at l(l+1)/2 + m); c, s, tmz the point's azimuthal tables. The
-// three-term recursion runs downward in m for Q_l, and alongside for Q_{l-1}
-// (first derivatives) and Q_{l-2} (second derivatives).
+// For one point and one l the reference runs three three-term recursions
+// downward in m side by side (templates_core.hpp:202-204, :210-212, :228-235
+// with the start values of :122-123,135,150,155,167,196 and the m = 0 steps of
+// :393,397,404-409):
+//   which = 0:  A[m] = Q_l^m                 (its qlm_0 at step m)
+//   which = 1:  B[m] = the Q_{l-1} sequence  (ql1m_0; B[l] = 0, B[l-1] = Q_{l-1}^{l-1})
+//   which = 2:  C[m] = the Q_{l-2} sequence  (ql2m_0; C[l] = C[l-1] = 0, C[l-2] = Q_{l-2}^{l-2})
+// They share the form v_m = k_m (2(m+1)z v_{m+1} + (x^2+y^2) v_{m+2}) and differ in
+// start values and in which row of the constant table k_m comes from, so each
+// is one job here, every iterate written to LDS. A recursion step is a handful
+// of operations while turning an iterate into output entries costs a hundred
+// or more: the iterates are computed once by a few lanes and the entries are
+// then independent jobs (entry_job) for all lanes of the workgroup. Same
+// operations in the same order as the reference's fused loop, hence the same
+// numbers.
+template <typename T>
+__device__ __forceinline__ void sequence_job(int l, int which, T z, T rxy,
+                                             const T* __restrict__ Q,
+                                             const T* __restrict__ tmz, T* __restrict__ out) {
+    const T* qk = Q + l * (l + 1) / 2;
+    // row of the constant table: (l, m) for A, (l-1, m) for B, (l-2, m) for C
+    const T* k = which == 0 ? qk : (which == 1 ? qk - l : qk - 2 * l + 1);
+    T v2, v1;
+    if (which == 0) {
+        v2 = qk[l];
+        v1 = -z * v2;
+    } else if (which == 1) {
+        v2 = 0;
+        v1 = qk[-1];
+    } else {
+        v2 = 0.0;
+        v1 = 0.0;
+    }
+    out[l] = v2;
+    out[l - 1] = v1;
+    int m = l - 2;
+    if (which == 2) {
+        // first step of the Q_{l-2} sequence: its start value itself (:228-231, :404-406)
+        const T v0 = qk[-l - 1];
+        out[m] = v0;
+        v2 = v1;
+        v1 = v0;
+        --m;
+    }
+    if (m < 0) return;
+    // the constants of a step do not depend on the iterates: fetch them one step ahead so that
+    // the chain of dependent operations never waits for LDS
+    T tz_next = tmz[m];
+    T k_next = k[m];
+    for (; m >= 0; --m) {
+        const T tz = tz_next;
+        const T km = k_next;
+        const int ahead = m > 0 ? m - 1 : 0;
+        tz_next = tmz[ahead];
+        k_next = k[ahead];
+        const T v0 = km * (tz * v1 + rxy * v2);
+        out[m] = v0;
+        v2 = v1;
+        v1 = v0;
+    }
+}
+
+// ---- the entries (l, +m) and (l, -m) of one point ---------------------------
 //
-// A job emits the entries with m_lo <= |m| <= m_hi only. The recursion itself
-// costs a handful of operations per m while an emitted pair of entries costs
-// hundreds, so a channel is cut into segments of consecutive m that different
-// lanes work on: a lane first runs the bare recursion from m = l down to its
-// segment (the same operations in the same order, hence the same numbers),
-// then does the full work inside it. m_hi == l marks the top segment, which
-// must reach down to l - 1 at least; m_lo == 0 the bottom one.
+// templates_core.hpp:122-152 (|m| = l), :154-198 (|m| = l - 1), :201-390
+// (l - 2 >= |m| >= 1) and :392-426 (m = 0), with the Q iterates read from the
+// arrays the sequence jobs left in LDS. F is the prefactor block, c / s the point's
+// azimuthal tables.
 template <typename T, int MODE, bool NORM>
-__device__ __forceinline__ void channel_job(int l, int m_hi, int m_lo, const Point<T>& p, T rxy,
-                                            const T* F, const T* Q, const T* c, const T* s,
-                                            const T* tmz, const Rows<T>& out) {
+__device__ __forceinline__ void entry_job(int l, int m, const Point<T>& p, const T* F, const T* c,
+                                          const T* s, const T* A, [[maybe_unused]] const T* B,
+                                          [[maybe_unused]] const T* C, const Rows<T>& out) {
     constexpr bool GRAD = MODE >= 1;
     constexpr bool HESS = MODE == 2;
     const T x = p.x, y = p.y, z = p.z;
-    const int tri = l * (l + 1) / 2;
     const int mid = l * (l + 1);
-    const T* pk = F + tri;
-    const T* qk = Q + tri;
+    const T* pk = F + l * (l + 1) / 2;
     const T zero = static_cast<T>(0.0);
-
-    T qlm_2, qlm_1, qlm_0;
-    [[maybe_unused]] T ql1m_2 = 0, ql1m_1 = 0, ql1m_0 = 0;
-    [[maybe_unused]] T ql2m_2 = 0, ql2m_1 = 0, ql2m_0 = 0;
     [[maybe_unused]] T x2 = 0, y2 = 0, xy = 0;
     if constexpr (HESS) {
         x2 = x * x;
         y2 = y * y;
         xy = x * y;
     }
+    (void)z;
 
-    const bool top = m_hi == l;
+    Entry<T> neg, pos;
+    neg.gx = neg.gy = neg.gz = pos.gx = pos.gy = pos.gz = zero;
+    neg.hxx = neg.hxy = neg.hxz = neg.hyy = neg.hyz = neg.hzz = zero;
+    pos.hxx = pos.hxy = pos.hxz = pos.hyy = pos.hyz = pos.hzz = zero;
 
-    // |m| = l (:122-152)
-    qlm_2 = qk[l];
-    if constexpr (GRAD) {
-        ql1m_2 = 0;
-    }
-    if constexpr (HESS) {
-        ql2m_2 = 0.0;
-    }
-    if (top) {
+    if (m == l) {
+        // :122-152
+        const T qlm_2 = A[l];
         auto pq = qlm_2 * pk[l];
-        Entry<T> neg, pos;
         neg.v = pq * s[l];
         pos.v = pq * c[l];
-        neg.gx = neg.gy = neg.gz = pos.gx = pos.gy = pos.gz = zero;
-        neg.hxx = neg.hxy = neg.hxz = neg.hyy = neg.hyz = neg.hzz = zero;
-        pos.hxx = pos.hxy = pos.hxz = pos.hyy = pos.hyz = pos.hzz = zero;
         if constexpr (GRAD) {
             pq *= l;
             neg.gx = pq * s[l - 1];
@@ -310,31 +356,19 @@ __device__ __forceinline__ void channel_job(int l, int m_hi, int m_lo, const Poi
                 pos.hyy = -pos.hxx;
             }
         }
-        stage<T, MODE, NORM>(out, mid - l, p, neg);
-        stage<T, MODE, NORM>(out, mid + l, p, pos);
-    }
-
-    // |m| = l - 1 (:154-198)
-    qlm_1 = -z * qlm_2;
-    if constexpr (GRAD) {
-        ql1m_1 = qk[-1];
-    }
-    if constexpr (HESS) {
-        ql2m_1 = 0.0;
-    }
-    if (top) {
+    } else if (m == l - 1) {
+        // :154-198
+        const T qlm_2 = A[l];
+        const T qlm_1 = A[l - 1];
         auto pq = qlm_1 * pk[l - 1];
-        Entry<T> neg, pos;
         neg.v = pq * s[l - 1];
         pos.v = pq * c[l - 1];
-        neg.gx = neg.gy = neg.gz = pos.gx = pos.gy = pos.gz = zero;
-        neg.hxx = neg.hxy = neg.hxz = neg.hyy = neg.hyz = neg.hzz = zero;
-        pos.hxx = pos.hxy = pos.hxz = pos.hyy = pos.hyz = pos.hzz = zero;
         if constexpr (GRAD) {
             pq *= (l - 1);
             neg.gx = pq * s[l - 2];
             neg.gy = pos.gx = pq * c[l - 2];
             pos.gy = -neg.gx;
+            const T ql1m_1 = B[l - 1];
             auto pdq = pk[l - 1] * (l + l - 1) * ql1m_1;
             neg.gz = pdq * s[l - 1];
             pos.gz = pdq * c[l - 1];
@@ -357,54 +391,19 @@ __device__ __forceinline__ void channel_job(int l, int m_hi, int m_lo, const Poi
                 neg.hyz = pos.hxz;
             }
         }
-        stage<T, MODE, NORM>(out, mid - l + 1, p, neg);
-        stage<T, MODE, NORM>(out, mid + l - 1, p, pos);
-    }
-
-    // bare recursion down to the segment: the Q updates of :202-204, :210-212, :228-235, :289-290
-    for (auto m = l - 2; m > m_hi; --m) {
-        const T tz = tmz[m];
-        qlm_0 = qk[m] * (tz * qlm_1 + rxy * qlm_2);
-        qlm_2 = qlm_1;
-        qlm_1 = qlm_0;
-        if constexpr (GRAD) {
-            ql1m_0 = qk[m - l] * (tz * ql1m_1 + rxy * ql1m_2);
-            ql1m_2 = ql1m_1;
-            ql1m_1 = ql1m_0;
-        }
-        if constexpr (HESS) {
-            if (m == l - 2) {
-                ql2m_0 = qk[-l - 1];
-            } else {
-                ql2m_0 = qk[m - 2 * l + 1] * (tz * ql2m_1 + rxy * ql2m_2);
-            }
-            ql2m_2 = ql2m_1;
-            ql2m_1 = ql2m_0;
-        }
-    }
-
-    // l - 2 >= |m| >= 1 (:201-390; the reference's two loops share one body)
-    const int m_first = m_hi < l - 2 ? m_hi : l - 2;
-    const int m_last = m_lo > 1 ? m_lo : 1;
-    for (auto m = m_first; m >= m_last; --m) {
-        const T cm = c[m], sm = s[m], tz = tmz[m], pkm = pk[m];
-        qlm_0 = qk[m] * (tz * qlm_1 + rxy * qlm_2);
-        qlm_2 = qlm_1;
-        qlm_1 = qlm_0;
+    } else if (m > 0) {
+        // :201-390
+        const T cm = c[m], sm = s[m], pkm = pk[m];
+        const T qlm_0 = A[m];
         auto pq = qlm_0 * pkm;
-        Entry<T> neg, pos;
         neg.v = pq * sm;
         pos.v = pq * cm;
-        neg.gx = neg.gy = neg.gz = pos.gx = pos.gy = pos.gz = zero;
-        neg.hxx = neg.hxy = neg.hxz = neg.hyy = neg.hyz = neg.hzz = zero;
-        pos.hxx = pos.hxy = pos.hxz = pos.hyy = pos.hyz = pos.hzz = zero;
-
         if constexpr (GRAD) {
             const T cm1 = c[m - 1], sm1 = s[m - 1];
-            ql1m_0 = qk[m - l] * (tz * ql1m_1 + rxy * ql1m_2);
-            ql1m_2 = ql1m_1;
-            ql1m_1 = ql1m_0;
-
+            // the reference reads these after its shift: ql1m_2 is the iterate of step m + 1
+            // (or the start value), ql1m_1 the iterate of step m
+            const T ql1m_2 = B[m + 1];
+            const T ql1m_1 = B[m];
             pq *= m;
             auto pqs = pq * sm1, pqc = pq * cm1;
             auto pdq = pkm * ql1m_2;
@@ -419,14 +418,11 @@ __device__ __forceinline__ void channel_job(int l, int m_hi, int m_lo, const Poi
             pos.gz = pdq * cm;
 
             if constexpr (HESS) {
-                if (m == l - 2) {
-                    ql2m_0 = qk[-l - 1];
-                } else {
-                    ql2m_0 = qk[m - 2 * l + 1] * (tz * ql2m_1 + rxy * ql2m_2);
-                }
-
+                // ... and these before its shift: the iterates of steps m + 2, m + 1 and m
+                const T ql2m_2 = C[m + 2];
+                const T ql2m_1 = C[m + 1];
+                const T ql2m_0 = C[m];
                 pq /= m;
-                // ql1m_2 / ql1m_1 were shifted above: they are Q_{l-1}^{m+1} and Q_{l-1}^{m}
                 auto pql1m_1 = pkm * ql1m_2;
                 auto pql2m_2 = pkm * ql2m_2;
                 auto pql2m_0 = pkm * ql2m_0;
@@ -453,47 +449,38 @@ __device__ __forceinline__ void channel_job(int l, int m_hi, int m_lo, const Poi
                 neg.hxz = x * (l + m) * pql2m_1 * sm + (l + m) * pql1m_0 * m * sm1;
                 pos.hyz = y * (l + m) * pql2m_1 * cm - (l + m) * pql1m_0 * m * sm1;
                 neg.hyz = y * (l + m) * pql2m_1 * sm + (l + m) * pql1m_0 * m * cm1;
-
-                ql2m_2 = ql2m_1;
-                ql2m_1 = ql2m_0;
             }
         }
-        stage<T, MODE, NORM>(out, mid - m, p, neg);
-        stage<T, MODE, NORM>(out, mid + m, p, pos);
-    }
-
-    // m = 0 (:392-426)
-    if (m_lo == 0) {
-        const T tz = tmz[0];
-        qlm_0 = qk[0] * (tz * qlm_1 + rxy * qlm_2);
-        Entry<T> e;
-        e.v = qlm_0 * pk[0];
-        e.gx = e.gy = e.gz = zero;
-        e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = zero;
+    } else {
+        // m = 0, :392-426
+        const T qlm_0 = A[0];
+        pos.v = qlm_0 * pk[0];
         if constexpr (GRAD) {
-            ql1m_0 = qk[-l] * (tz * ql1m_1 + rxy * ql1m_2);
-            e.gx = pk[0] * x * ql1m_1;
-            e.gy = pk[0] * y * ql1m_1;
-            e.gz = pk[0] * l * ql1m_0;
+            const T ql1m_1 = B[1];
+            const T ql1m_0 = B[0];
+            pos.gx = pk[0] * x * ql1m_1;
+            pos.gy = pk[0] * y * ql1m_1;
+            pos.gz = pk[0] * l * ql1m_0;
             if constexpr (HESS) {
-                if (l == 2) {
-                    ql2m_0 = qk[-2 * l + 1];
-                } else {
-                    ql2m_0 = qk[-2 * l + 1] * (tz * ql2m_1 + rxy * ql2m_2);
-                }
+                const T ql2m_2 = C[2];
+                const T ql2m_1 = C[1];
+                const T ql2m_0 = C[0];
                 auto pql1m_1 = pk[0] * ql1m_1;
                 auto pql2m_2 = pk[0] * ql2m_2;
                 auto pql2m_0 = pk[0] * ql2m_0;
                 auto pql2m_1 = pk[0] * ql2m_1;
-                e.hxx = pql1m_1 + x2 * pql2m_2;
-                e.hyy = pql1m_1 + y2 * pql2m_2;
-                e.hzz = (l) * (l - 1) * pql2m_0;
-                e.hxy = xy * pql2m_2;
-                e.hxz = x * l * pql2m_1;
-                e.hyz = y * l * pql2m_1;
+                pos.hxx = pql1m_1 + x2 * pql2m_2;
+                pos.hyy = pql1m_1 + y2 * pql2m_2;
+                pos.hzz = (l) * (l - 1) * pql2m_0;
+                pos.hxy = xy * pql2m_2;
+                pos.hxz = x * l * pql2m_1;
+                pos.hyz = y * l * pql2m_1;
             }
         }
-        stage<T, MODE, NORM>(out, mid, p, e);
+    }
+    stage<T, MODE, NORM>(out, mid + m, p, pos);
+    if (m > 0) {
+        stage<T, MODE, NORM>(out, mid - m, p, neg);
     }
 }
 
@@ -537,10 +524,12 @@ __device__ __forceinline__ void copy_out(const T* staged, T* dst, unsigned len, 
     V* dst_v = reinterpret_cast<V*>(dst + head);
     if (pad == 0 && head == 0) {
         const V* src_v = reinterpret_cast<const V*>(staged);
+#pragma unroll 4
         for (unsigned g = tid; g < nvec; g += nthreads) {
             emit<T, STREAMING>(src_v[g], dst_v + g);
         }
     } else {
+#pragma unroll 4
         for (unsigned g = tid; g < nvec; g += nthreads) {
             V v;
 #pragma unroll
@@ -557,6 +546,21 @@ __device__ __forceinline__ void copy_out(const T* staged, T* dst, unsigned len, 
     if (tid < loose) {
         const unsigned at = tid < head ? tid : tail_first + (tid - head);
         emit<T, STREAMING>(staged[pad ? staged_index<T>(at, row, pad, magic) : at], dst + at);
+    }
+}
+
+// The first NY entries of `count` points' component rows, staged as [count][MULT * NY + pad],
+// to rows that are `ny` apart in HBM (4- or 8-byte stores, consecutive lanes to consecutive
+// entries).
+template <typename T, bool STREAMING, unsigned NY, unsigned MULT>
+__device__ __forceinline__ void copy_prefixes(const T* staged, T* dst, unsigned count, unsigned ny,
+                                              unsigned pad, unsigned tid, unsigned nthreads) {
+    const unsigned total = count * MULT * NY;
+    for (unsigned g = tid; g < total; g += nthreads) {
+        const unsigned row = g / NY;
+        const unsigned k = g - row * NY;
+        const unsigned s = row / MULT;
+        emit<T, STREAMING>(staged[g + pad * s], dst + static_cast<unsigned long long>(row) * ny + k);
     }
 }
 

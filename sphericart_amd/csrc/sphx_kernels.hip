@@ -57,19 +57,16 @@ template <> __device__ __forceinline__ const double* table_Q<double>() { return 
 // Everything a kernel needs to know about the tiling; filled in on the host.
 struct Tiling {
     unsigned long long n_samples;
-    unsigned n_tiles;
+    unsigned n_tiles;       // tiles of `tile` points (recursion) or groups of 64 points (closed form)
+    unsigned tiles_per_xcd; // workgroups of one XCD walk one contiguous stretch of tiles
     int l_max;
-    int ny;          // (l_max + 1)^2
-    int tile;        // points per tile (S)
-    unsigned pad;    // spare LDS elements after each point's block (0 or 1)
-    unsigned magic[3]; // ceil(2^32 / row) for row = ny, 3 ny, 9 ny
+    int ny;                 // (l_max + 1)^2: length of one component row in HBM
+    int tile;               // points whose rows are staged in LDS at a time
+    unsigned magic_jobs;    // ceil(2^32 / jobs_per_point)
+    unsigned jobs_per_point; // (l, m >= 0) pairs above the closed-form limit
+    unsigned sequence_waves; // waves that run the bare recursions (1 or 2)
     // LDS carve-up, in elements of T from the start of dynamic LDS
-    unsigned off_dsph, off_ddsph, off_F, off_Q, off_pts, off_jobs;
-    // every l channel above the closed-form limit is cut into segments of `segment`
-    // consecutive m; one point has `jobs_per_point` (channel, segment) jobs in all
-    unsigned segment, jobs_per_point;
-    // persistent-workgroup walk: workgroups of one XCD take consecutive tiles
-    unsigned tiles_per_group;
+    unsigned off_dsph, off_ddsph, off_F, off_Q, off_pts, off_iter, off_jobs;
 };
 
 extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -80,45 +77,24 @@ extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 #define SPHX_STREAMING_STORES true
 #endif
 
-// Stream the staged rows of `valid` consecutive points, the first of which is
-// point number `first`, from LDS to the output arrays.
-template <typename T, int MODE>
-__device__ __forceinline__ void flush_run(const Tiling& g, T* lds, unsigned long long first,
-                                          unsigned valid, T* sph, T* dsph, T* ddsph,
-                                          unsigned tid, unsigned nthreads) {
-    const unsigned ny = g.ny;
-    copy_out<T, SPHX_STREAMING_STORES>(lds, sph + first * ny, valid * ny, ny, g.pad, g.magic[0], tid,
-                                       nthreads);
-    if constexpr (MODE >= 1) {
-        copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_dsph, dsph + first * 3 * ny, valid * 3 * ny,
-                                           3 * ny, g.pad, g.magic[1], tid, nthreads);
-    }
-    if constexpr (MODE == 2) {
-        copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_ddsph, ddsph + first * 9 * ny, valid * 9 * ny,
-                                           9 * ny, g.pad, g.magic[2], tid, nthreads);
-    }
-}
-
-template <typename T, int MODE>
-__device__ __forceinline__ Rows<T> rows_of(const Tiling& g, T* lds, unsigned s) {
-    Rows<T> r;
-    r.ny = g.ny;
-    r.sph = lds + s * (g.ny + g.pad);
-    r.dsph = MODE >= 1 ? lds + g.off_dsph + s * (3 * g.ny + g.pad) : nullptr;
-    r.ddsph = MODE == 2 ? lds + g.off_ddsph + s * (9 * g.ny + g.pad) : nullptr;
-    return r;
+__host__ __device__ constexpr unsigned magic_of(unsigned long long divisor) {
+    return static_cast<unsigned>(((1ull << 32) + divisor - 1) / divisor);
 }
 
 // ---------------------------------------------------------------------------
-// l_max = H, everything in closed form. One wave per workgroup, one point per
-// lane, 64 points per workgroup.
+// l <= H in closed form. One wave per workgroup, one point per lane, 64 points
+// per workgroup.
 //
 // The finished numbers of a point stay in the lane's VGPRs; LDS is only the
 // transposition buffer between "one point per lane" and "consecutive addresses
-// per lane". To keep many waves resident per CU (the register file, not LDS,
-// then bounds the bytes in flight) the 64 points go through the buffer in
-// PHASES passes of 64 / PHASES points each; the slice of every output array
-// that a pass covers is still one contiguous run.
+// per lane". The 64 points go through the buffer in PHASES passes of
+// 64 / PHASES points each when all of them do not fit.
+//
+// PREFIX == false: l_max == H. The slice of every output array that a pass
+// covers is one contiguous run, streamed out with 16-byte stores.
+// PREFIX == true: l_max > H; only the first (H+1)^2 entries of every component
+// row are produced here (the recursion kernel fills in the rest), so the runs
+// are (H+1)^2 long and ny apart.
 // ---------------------------------------------------------------------------
 // Bytes of LDS one pass may use: 52 KB lets three workgroups share a CU. Measured on MI355X,
 // l_max = 6 float32 with gradients runs fastest with a single pass (50 KB).
@@ -126,11 +102,20 @@ __device__ __forceinline__ Rows<T> rows_of(const Tiling& g, T* lds, unsigned s) 
 #define SPHX_PHASE_LDS_BUDGET (52 * 1024)
 #endif
 
+__host__ __device__ constexpr unsigned components_of(int mode) {
+    return mode == 0 ? 1u : (mode == 1 ? 4u : 13u);
+}
+
+// LDS elements per point in the closed-form kernel: the rows of all arrays, each array padded
+// by one element when (H+1)^2 is even so that the per-point stride is odd (lanes staging the
+// same entry of different points then hit different banks).
+__host__ __device__ constexpr unsigned closed_form_pad(int H) {
+    return ((H + 1) * (H + 1)) % 2 == 0 ? 1u : 0u;
+}
+
 __host__ __device__ constexpr unsigned closed_form_phases(unsigned elem, int mode, int H) {
     const unsigned ny = (H + 1) * (H + 1);
-    const unsigned arrays = mode + 1;
-    const unsigned mult = mode == 0 ? 1 : (mode == 1 ? 4 : 13);
-    const unsigned per_point = (mult * ny + arrays * (ny % 2 == 0 ? 1u : 0u)) * elem;
+    const unsigned per_point = (components_of(mode) * ny + (mode + 1) * closed_form_pad(H)) * elem;
     unsigned phases = 1;
     while (phases < 16 && (64 / phases) * per_point > SPHX_PHASE_LDS_BUDGET) {
         phases *= 2;
@@ -138,31 +123,27 @@ __host__ __device__ constexpr unsigned closed_form_phases(unsigned elem, int mod
     return phases;
 }
 
-template <typename T, int MODE, bool NORM, int H>
+template <typename T, int MODE, bool NORM, int H, bool PREFIX>
 __global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __restrict__ xyz,
                                                         T* __restrict__ sph, T* __restrict__ dsph,
                                                         T* __restrict__ ddsph) {
     constexpr unsigned PHASES = closed_form_phases(sizeof(T), MODE, H);
     constexpr unsigned PER = 64 / PHASES;
     constexpr unsigned NY = (H + 1) * (H + 1);
+    constexpr unsigned PAD = closed_form_pad(H);
+    // LDS: [PER][NY + PAD] values, then [PER][3 NY + PAD] gradients, then [PER][9 NY + PAD]
+    constexpr unsigned OFF_D = (PER * (NY + PAD) + 3u) & ~3u;
+    constexpr unsigned OFF_DD = (OFF_D + PER * (3 * NY + PAD) + 3u) & ~3u;
     T* lds = reinterpret_cast<T*>(lds_raw);
     const unsigned tid = threadIdx.x;
     // Workgroups are handed to the 8 XCDs round-robin; give each XCD one contiguous stretch of
     // points, so that what one XCD writes at any moment is a compact window of each array
     // (measured: 6 % faster than the identity mapping).
-    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_group + (blockIdx.x >> 3);
+    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
     if (group >= g.n_tiles) return;
     const unsigned long long first = static_cast<unsigned long long>(group) * 64;
     const unsigned long long left = g.n_samples - first;
     const unsigned valid = left < 64ull ? static_cast<unsigned>(left) : 64u;
-    // the row length is a compile-time constant here: rebuild the geometry with it
-    Tiling gc = g;
-    gc.ny = NY;
-    gc.tile = PER;
-    gc.pad = (NY % 2 == 0) ? 1u : 0u;
-    gc.magic[0] = static_cast<unsigned>(((1ull << 32) + NY - 1) / NY);
-    gc.magic[1] = static_cast<unsigned>(((1ull << 32) + 3 * NY - 1) / (3 * NY));
-    gc.magic[2] = static_cast<unsigned>(((1ull << 32) + 9 * NY - 1) / (9 * NY));
 
     Entry<T> E[NY];
     if (tid < valid) {
@@ -175,7 +156,12 @@ __global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __re
         if (base >= valid) break; // uniform across the wave
         if (phase > 0) __syncthreads();
         if (tid >= base && tid < base + PER && tid < valid) {
-            const Rows<T> rows = rows_of<T, MODE>(gc, lds, tid - base);
+            const unsigned s = tid - base;
+            Rows<T> rows;
+            rows.ny = NY;
+            rows.sph = lds + s * (NY + PAD);
+            rows.dsph = lds + OFF_D + s * (3 * NY + PAD);
+            rows.ddsph = lds + OFF_DD + s * (9 * NY + PAD);
 #pragma unroll
             for (unsigned k = 0; k < NY; ++k) {
                 put<T, MODE>(rows, k, E[k]);
@@ -183,163 +169,293 @@ __global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __re
         }
         __syncthreads();
         const unsigned count = valid - base < PER ? valid - base : PER;
-        flush_run<T, MODE>(gc, lds, first + base, count, sph, dsph, ddsph, tid, 64);
+        const unsigned long long at = first + base;
+        if constexpr (!PREFIX) {
+            copy_out<T, SPHX_STREAMING_STORES>(lds, sph + at * NY, count * NY, NY, PAD,
+                                               magic_of(NY), tid, 64);
+            if constexpr (MODE >= 1) {
+                copy_out<T, SPHX_STREAMING_STORES>(lds + OFF_D, dsph + at * 3 * NY, count * 3 * NY,
+                                                   3 * NY, PAD, magic_of(3 * NY), tid, 64);
+            }
+            if constexpr (MODE == 2) {
+                copy_out<T, SPHX_STREAMING_STORES>(lds + OFF_DD, ddsph + at * 9 * NY,
+                                                   count * 9 * NY, 9 * NY, PAD, magic_of(9 * NY),
+                                                   tid, 64);
+            }
+        } else {
+            const unsigned ny = g.ny;
+            copy_prefixes<T, SPHX_STREAMING_STORES, NY, 1>(lds, sph + at * ny, count, ny, PAD, tid, 64);
+            if constexpr (MODE >= 1) {
+                copy_prefixes<T, SPHX_STREAMING_STORES, NY, 3>(lds + OFF_D, dsph + at * 3 * ny, count,
+                                                              ny, PAD, tid, 64);
+            }
+            if constexpr (MODE == 2) {
+                copy_prefixes<T, SPHX_STREAMING_STORES, NY, 9>(lds + OFF_DD, ddsph + at * 9 * ny,
+                                                              count, ny, PAD, tid, 64);
+            }
+        }
     }
 }
 
 // ---------------------------------------------------------------------------
-// General case: closed form up to H, recursion above. 256 threads; wave 0
-// hosts the per-point lanes, waves 1..3 the (point, l) jobs.
+// l > H through the recursion. 512 threads, persistent workgroups that walk
+// over tiles of `tile` consecutive points, three tiles in flight per workgroup:
+//
+//   wave 0       tile i+2, one lane per point: normalised coordinates, c_m,
+//                s_m, 2(m+1)z into LDS (azimuth_job);
+//   wave 1 (, 2) tile i+1, one lane per (point, l, sequence): the bare Q recursions,
+//                every iterate into LDS (sequence_job);
+//   the others   tile i, one job per (point, l, m >= 0): the entries (l, +-m) of
+//                every requested array, chain rule included, staged in LDS in
+//                HBM layout (entry_job). Neighbouring lanes take neighbouring m
+//                of one (point, l), so their LDS traffic falls on neighbouring
+//                banks;
+//   all waves    stream the staged rows of tile i to HBM with 16-byte stores.
+//
+// The first two stages are short chains of dependent operations that only a
+// few lanes can share; running them one and two tiles ahead of the wide stage
+// takes them off the critical path. The point tables are kept in three
+// buffers, the iterates in two; the staged rows, by far the largest part of
+// LDS, exist once.
+//
+// WHOLE == true: the closed forms of l <= H are evaluated here too (one lane
+// per point) and the tile's rows are complete, one contiguous run per array.
+// WHOLE == false: the rows start at l = H + 1 (closed_form_kernel<PREFIX>
+// writes the part below); every (point, component) row is its own run.
 // ---------------------------------------------------------------------------
-template <typename T, int MODE, bool NORM, int H>
-__global__ __launch_bounds__(256) void recursion_kernel(Tiling g, const T* __restrict__ xyz,
-                                                       T* __restrict__ sph, T* __restrict__ dsph,
-                                                       T* __restrict__ ddsph) {
+constexpr unsigned kRecursionThreads = 512;
+
+template <typename T, int MODE, bool NORM, bool WHOLE>
+__global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, const T* __restrict__ xyz,
+                                                                     T* __restrict__ sph,
+                                                                     T* __restrict__ dsph,
+                                                                     T* __restrict__ ddsph) {
+    constexpr int H = MODE == 2 ? 1 : 6;
+    constexpr unsigned NYH = (H + 1) * (H + 1);
+    constexpr unsigned ARRAYS = MODE + 1; // iterate arrays per point: A, B, C
+    constexpr unsigned NT = kRecursionThreads;
     T* lds = reinterpret_cast<T*>(lds_raw);
     const unsigned tid = threadIdx.x;
-    const unsigned nthreads = blockDim.x;
+    const unsigned lane = tid & 63u;
+    const unsigned wave = tid >> 6;
     const int L = g.l_max;
     const unsigned S = g.tile;
+    const unsigned ny = g.ny;
+    const unsigned nrow = WHOLE ? ny : ny - NYH; // staged elements per component row
+    const unsigned skip = WHOLE ? 0u : NYH;      // first staged entry of a row
+    const unsigned tri_all = (L + 1) * (L + 2) / 2;
 
     T* F = lds + g.off_F;
     T* Q = lds + g.off_Q;
     unsigned short* job_table = reinterpret_cast<unsigned short*>(lds + g.off_jobs);
     {
-        const unsigned nq = (L + 1) * (L + 2) / 2;
         const T* cF = table_F<T>();
         const T* cQ = table_Q<T>();
-        for (unsigned i = tid; i < nq; i += nthreads) {
+        for (unsigned i = tid; i < tri_all; i += NT) {
             F[i] = cF[i];
             Q[i] = cQ[i];
         }
-        // (l, segment) pairs, top segments of all channels first, longest channels first:
-        // neighbouring lanes then run loops of the same length
+        // (l, m) pairs: the bulk 1 <= m <= l - 2 first, then the special cases m = l, l - 1 and
+        // 0 each as one block, so that the lanes of a wave mostly share one branch of entry_job
         if (tid == 0) {
             unsigned n = 0;
-            for (unsigned seg = 0; seg * g.segment <= static_cast<unsigned>(L); ++seg) {
-                for (int l = L; l > H; --l) {
-                    if (seg * g.segment <= static_cast<unsigned>(l)) {
-                        job_table[n++] = static_cast<unsigned short>((l << 8) | seg);
-                    }
-                }
+            for (int l = L; l > H; --l) {
+                for (int m = l - 2; m >= 1; --m) job_table[n++] = static_cast<unsigned short>((l << 8) | m);
             }
+            for (int l = L; l > H; --l) job_table[n++] = static_cast<unsigned short>((l << 8) | l);
+            for (int l = L; l > H; --l) job_table[n++] = static_cast<unsigned short>((l << 8) | (l - 1));
+            for (int l = L; l > H; --l) job_table[n++] = static_cast<unsigned short>(l << 8);
         }
     }
 
-    // Workgroups are handed to the 8 XCDs round-robin; give each XCD one
-    // contiguous stretch of tiles so that lines shared by neighbouring tiles
-    // meet in one L2.
-    const unsigned xcd = blockIdx.x & 7u;
-    const unsigned lane_in_xcd = blockIdx.x >> 3;
-    const unsigned groups_per_xcd = gridDim.x >> 3;
-    const unsigned xcd_first = xcd * g.tiles_per_group;
-    unsigned xcd_last = xcd_first + g.tiles_per_group;
-    if (xcd_last > g.n_tiles) xcd_last = g.n_tiles;
+    // per point: 8 numbers (x, y, z, x^2, y^2, z^2, 1/r, x^2 + y^2), then c, s, 2(m+1)z
+    const unsigned point_stride = 8 + 3 * (L + 1);
+    auto point_data = [&](unsigned buffer, unsigned s) -> T* {
+        return lds + g.off_pts + (buffer * S + s) * point_stride;
+    };
+    auto iterates = [&](unsigned buffer, unsigned s, unsigned which, int l) -> T* {
+        return lds + g.off_iter + ((buffer * S + s) * ARRAYS + which) * tri_all + l * (l + 1) / 2;
+    };
 
-    // Per-point data (normalised coordinates, c_m, s_m, 2(m+1)z) is double buffered: while the
-    // recursion jobs of one tile run, wave 0 prepares the next tile, so that the LDS rows are
-    // only held from the first staged entry to the end of the flush.
-    const unsigned per_point_tables = 3 * (L + 1) + 8;
-    auto tables_of = [&](unsigned parity, unsigned s) -> T* {
-        return lds + g.off_pts + (parity * S + s) * per_point_tables;
-    };
-    auto prepare = [&](unsigned tile_idx, unsigned parity, T rx, T ry, T rz) {
-        // templates.hpp:386-400 and :451-466 for point `tid` of the tile
-        (void)tile_idx;
-        T* rec = tables_of(parity, tid);
-        Point<T> p;
-        p.x = rx;
-        p.y = ry;
-        p.z = rz;
-        p.x2 = p.x * p.x;
-        p.y2 = p.y * p.y;
-        p.z2 = p.z * p.z;
-        p.ir = 0.0;
-        if constexpr (NORM) {
-            p.ir = 1 / root(p.x2 + p.y2 + p.z2);
-            p.x *= p.ir;
-            p.y *= p.ir;
-            p.z *= p.ir;
-            p.x2 = p.x * p.x;
-            p.y2 = p.y * p.y;
-            p.z2 = p.z * p.z;
-        }
-        rec[0] = p.x;
-        rec[1] = p.y;
-        rec[2] = p.z;
-        rec[3] = p.x2;
-        rec[4] = p.y2;
-        rec[5] = p.z2;
-        rec[6] = p.ir;
-        azimuth_job<T>(p, L, rec + 8, rec + 8 + (L + 1), rec + 8 + 2 * (L + 1));
-    };
-    auto point_of = [&](const T* rec) {
-        Point<T> q;
-        q.x = rec[0];
-        q.y = rec[1];
-        q.z = rec[2];
-        q.x2 = rec[3];
-        q.y2 = rec[4];
-        q.z2 = rec[5];
-        q.ir = rec[6];
-        return q;
-    };
-    auto valid_in = [&](unsigned tile_idx) -> unsigned {
-        const unsigned long long first = static_cast<unsigned long long>(tile_idx) * S;
+    // same XCD-contiguous walk as the closed-form kernel
+    const unsigned xcd = blockIdx.x & 7u;
+    const unsigned rank_in_xcd = blockIdx.x >> 3;
+    const unsigned groups_per_xcd = gridDim.x >> 3;
+    const unsigned xcd_first = xcd * g.tiles_per_xcd;
+    unsigned xcd_last = xcd_first + g.tiles_per_xcd;
+    if (xcd_last > g.n_tiles) xcd_last = g.n_tiles;
+    if (xcd_first + rank_in_xcd >= xcd_last) return; // whole workgroup
+
+    // the n-th tile of this workgroup, and how many points it has (0 past the end)
+    auto tile_of = [&](unsigned n) -> unsigned { return xcd_first + rank_in_xcd + n * groups_per_xcd; };
+    auto valid_in = [&](unsigned n) -> unsigned {
+        const unsigned t = tile_of(n);
+        if (t >= xcd_last) return 0u;
+        const unsigned long long first = static_cast<unsigned long long>(t) * S;
         const unsigned long long left = g.n_samples - first;
         return left < S ? static_cast<unsigned>(left) : S;
     };
+    auto fetch = [&](unsigned n, T& rx, T& ry, T& rz) {
+        rx = ry = rz = 0;
+        if (lane < valid_in(n)) {
+            const T* src = xyz + (static_cast<unsigned long long>(tile_of(n)) * S + lane) * 3;
+            rx = src[0];
+            ry = src[1];
+            rz = src[2];
+        }
+    };
+    // stage one of tile n (wave 0; lane == tid there)
+    auto azimuth_stage = [&](unsigned n, T rx, T ry, T rz) {
+        if (lane < valid_in(n)) {
+            T* rec = point_data(n % 3u, lane);
+            Point<T> p;
+            p.x = rx;
+            p.y = ry;
+            p.z = rz;
+            p.x2 = p.x * p.x;
+            p.y2 = p.y * p.y;
+            p.z2 = p.z * p.z;
+            p.ir = 0.0;
+            if constexpr (NORM) {
+                p.ir = 1 / root(p.x2 + p.y2 + p.z2);
+                p.x *= p.ir;
+                p.y *= p.ir;
+                p.z *= p.ir;
+                p.x2 = p.x * p.x;
+                p.y2 = p.y * p.y;
+                p.z2 = p.z * p.z;
+            }
+            rec[0] = p.x;
+            rec[1] = p.y;
+            rec[2] = p.z;
+            rec[3] = p.x2;
+            rec[4] = p.y2;
+            rec[5] = p.z2;
+            rec[6] = p.ir;
+            rec[7] = p.x2 + p.y2;
+            azimuth_job<T>(p, L, rec + 8, rec + 8 + (L + 1), rec + 8 + 2 * (L + 1));
+        }
+    };
+    // stage two of tile n (waves 1 .. g.sequence_waves)
+    auto recursion_stage = [&](unsigned n) {
+        const unsigned count = valid_in(n);
+        const unsigned per_l = count * ARRAYS;
+        const unsigned jobs = per_l * static_cast<unsigned>(L - H);
+        for (unsigned j = tid - 64; j < jobs; j += 64 * g.sequence_waves) {
+            const unsigned step = j / per_l;
+            const unsigned rest = j - step * per_l;
+            const int l = L - static_cast<int>(step); // longest recursions first
+            const unsigned s = rest / ARRAYS;
+            const unsigned which = rest - s * ARRAYS;
+            const T* rec = point_data(n % 3u, s);
+            sequence_job<T>(l, static_cast<int>(which), rec[2], rec[7], Q, rec + 8 + 2 * (L + 1),
+                            iterates(n & 1u, s, which, l));
+        }
+    };
 
-    unsigned tile_idx = xcd_first + lane_in_xcd;
-    unsigned parity = 0;
-    if (tile_idx < xcd_last && tid < valid_in(tile_idx)) {
-        const T* src = xyz + (static_cast<unsigned long long>(tile_idx) * S + tid) * 3;
-        prepare(tile_idx, 0, src[0], src[1], src[2]);
+    // fill the pipeline: tables of tiles 0 and 1, iterates of tile 0
+    T rx = 0, ry = 0, rz = 0;
+    if (wave == 0) {
+        fetch(0, rx, ry, rz);
+        azimuth_stage(0, rx, ry, rz);
+        fetch(1, rx, ry, rz);
+    }
+    __syncthreads(); // prefactor tables, job table, tables of tile 0
+    if (wave == 0) {
+        azimuth_stage(1, rx, ry, rz);
+        fetch(2, rx, ry, rz);
+    } else if (wave <= g.sequence_waves) {
+        recursion_stage(0);
     }
 
-    for (; tile_idx < xcd_last; tile_idx += groups_per_xcd, parity ^= 1u) {
-        const unsigned long long first = static_cast<unsigned long long>(tile_idx) * S;
-        const unsigned valid = valid_in(tile_idx);
-        const unsigned next_idx = tile_idx + groups_per_xcd;
-        const unsigned next_valid = next_idx < xcd_last ? valid_in(next_idx) : 0u;
+    for (unsigned n = 0; valid_in(n) != 0; ++n) {
+        const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
+        const unsigned valid = valid_in(n);
 
-        __syncthreads(); // rows free again (previous flush done); this tile's point data in place
+        __syncthreads(); // tables of tile n+1, iterates of tile n in place; rows of tile n-1 flushed
 
-        if (tid < 64) {
-            // fetch the next tile's coordinates now, use them after the closed-form work
-            T nx = 0, ny_ = 0, nz = 0;
-            if (tid < next_valid) {
-                const T* src = xyz + (static_cast<unsigned long long>(next_idx) * S + tid) * 3;
-                nx = src[0];
-                ny_ = src[1];
-                nz = src[2];
-            }
-            if (tid < valid) {
-                const Point<T> p = point_of(tables_of(parity, tid));
-                closed_form_job<T, MODE, NORM, H>(p, rows_of<T, MODE>(g, lds, tid));
-            }
-            if (tid < next_valid) {
-                prepare(next_idx, parity ^ 1u, nx, ny_, nz);
-            }
+        if (wave == 0) {
+            azimuth_stage(n + 2, rx, ry, rz);
+            fetch(n + 3, rx, ry, rz); // needed one round from now
+        } else if (wave <= g.sequence_waves) {
+            recursion_stage(n + 1);
         } else {
+            const unsigned wide_first = 64 * (1 + g.sequence_waves);
+            const unsigned t = tid - wide_first;
+            if constexpr (WHOLE) {
+                if (t < valid) {
+                    const T* rec = point_data(n % 3u, t);
+                    Point<T> p;
+                    p.x = rec[0];
+                    p.y = rec[1];
+                    p.z = rec[2];
+                    p.x2 = rec[3];
+                    p.y2 = rec[4];
+                    p.z2 = rec[5];
+                    p.ir = rec[6];
+                    Rows<T> rows;
+                    rows.ny = static_cast<int>(ny);
+                    rows.sph = lds + t * ny;
+                    rows.dsph = lds + g.off_dsph + t * 3 * ny;
+                    rows.ddsph = lds + g.off_ddsph + t * 9 * ny;
+                    closed_form_job<T, MODE, NORM, H>(p, rows);
+                }
+            }
             const unsigned jobs = valid * g.jobs_per_point;
-            for (unsigned j = tid - 64; j < jobs; j += nthreads - 64) {
-                const unsigned s = j % valid;
-                const unsigned entry = job_table[j / valid];
+            for (unsigned j = t; j < jobs; j += NT - wide_first) {
+                const unsigned s = __umulhi(j, g.magic_jobs);
+                const unsigned entry = job_table[j - s * g.jobs_per_point];
                 const int l = static_cast<int>(entry >> 8);
-                const int m_hi = l - static_cast<int>((entry & 0xffu) * g.segment);
-                const int m_lo = m_hi - static_cast<int>(g.segment) + 1 > 0
-                                     ? m_hi - static_cast<int>(g.segment) + 1
-                                     : 0;
-                const T* rec = tables_of(parity, s);
-                const Point<T> q = point_of(rec);
-                const T rxy = q.x2 + q.y2;
-                channel_job<T, MODE, NORM>(l, m_hi, m_lo, q, rxy, F, Q, rec + 8, rec + 8 + (L + 1),
-                                           rec + 8 + 2 * (L + 1), rows_of<T, MODE>(g, lds, s));
+                const int m = static_cast<int>(entry & 0xffu);
+                const T* rec = point_data(n % 3u, s);
+                Point<T> p;
+                p.x = rec[0];
+                p.y = rec[1];
+                p.z = rec[2];
+                p.x2 = rec[3];
+                p.y2 = rec[4];
+                p.z2 = rec[5];
+                p.ir = rec[6];
+                // rows are addressed with the entry's index in the full row; shift the bases when
+                // the staged rows start at l = H + 1
+                Rows<T> rows;
+                rows.ny = static_cast<int>(nrow);
+                rows.sph = lds + s * nrow - skip;
+                rows.dsph = lds + g.off_dsph + s * 3 * nrow - skip;
+                rows.ddsph = lds + g.off_ddsph + s * 9 * nrow - skip;
+                entry_job<T, MODE, NORM>(l, m, p, F, rec + 8, rec + 8 + (L + 1), iterates(n & 1u, s, 0, l),
+                                         iterates(n & 1u, s, MODE >= 1 ? 1 : 0, l),
+                                         iterates(n & 1u, s, MODE == 2 ? 2 : 0, l), rows);
             }
         }
-        __syncthreads();
-        flush_run<T, MODE>(g, lds, first, valid, sph, dsph, ddsph, tid, nthreads);
+        __syncthreads(); // rows of tile n complete
+
+        if constexpr (WHOLE) {
+            copy_out<T, SPHX_STREAMING_STORES>(lds, sph + first * ny, valid * ny, ny, 0, 0, tid, NT);
+            if constexpr (MODE >= 1) {
+                copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_dsph, dsph + first * 3 * ny,
+                                                   valid * 3 * ny, 3 * ny, 0, 0, tid, NT);
+            }
+            if constexpr (MODE == 2) {
+                copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_ddsph, ddsph + first * 9 * ny,
+                                                   valid * 9 * ny, 9 * ny, 0, 0, tid, NT);
+            }
+        } else {
+            // one run per (point, component) row, dealt to the waves in turn
+            constexpr unsigned NW = NT / 64;
+            for (unsigned r = wave; r < valid * components_of(MODE); r += NW) {
+                // rows [0, valid) are values, the next 3 * valid are gradients
+                if (r < valid) {
+                    copy_out<T, SPHX_STREAMING_STORES>(lds + r * nrow, sph + (first + r) * ny + skip, nrow,
+                                                       nrow, 0, 0, lane, 64);
+                } else {
+                    const unsigned q = r - valid;
+                    copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_dsph + q * nrow,
+                                                       dsph + (first * 3 + q) * ny + skip, nrow, nrow, 0,
+                                                       0, lane, 64);
+                }
+            }
+        }
     }
 }
 
@@ -398,13 +514,19 @@ static int env_int(const char* name, int fallback) {
     return std::atoi(v);
 }
 
-struct Plan {
+struct Launch {
     Tiling g;
-    bool closed_form;
-    unsigned points_per_group;
-    int threads;
-    unsigned lds_bytes;
     unsigned workgroups;
+    unsigned threads;
+    unsigned lds_bytes;
+};
+
+struct Plan {
+    bool closed_only; // l_max within the closed forms: one launch of closed_form_kernel
+    bool whole;       // recursion_kernel evaluates the closed forms too: one launch
+                      // otherwise closed_form_kernel<PREFIX> + recursion_kernel: two launches
+    Launch closed;
+    Launch rec;
 };
 
 static unsigned pow2_floor(unsigned v) {
@@ -413,7 +535,95 @@ static unsigned pow2_floor(unsigned v) {
     return p;
 }
 
-// Choose tile size and LDS layout. `lds_limit` / `cus` describe the device.
+static unsigned align4(unsigned v) { return (v + 3u) & ~3u; }
+
+static void plan_closed(size_t n_samples, int l_max, int hard, int mode, size_t elem, Launch* out) {
+    Tiling& g = out->g;
+    std::memset(&g, 0, sizeof(g));
+    g.n_samples = n_samples;
+    g.l_max = l_max;
+    g.ny = (l_max + 1) * (l_max + 1);
+    g.tile = 64;
+    g.n_tiles = static_cast<unsigned>((n_samples + 63) / 64);
+    g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
+    out->workgroups = g.tiles_per_xcd * 8u;
+    out->threads = 64;
+    const unsigned nyh = static_cast<unsigned>(hard + 1) * (hard + 1);
+    const unsigned pad = closed_form_pad(hard);
+    const unsigned per = 64 / closed_form_phases(static_cast<unsigned>(elem), mode, hard);
+    unsigned at = align4(per * (nyh + pad));
+    if (mode >= 1) at = align4(at + per * (3 * nyh + pad));
+    if (mode == 2) at = align4(at + per * (9 * nyh + pad));
+    out->lds_bytes = at * static_cast<unsigned>(elem);
+}
+
+// Tile size and LDS layout of the recursion kernel. Returns false when not even one point fits.
+static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, size_t elem,
+                           unsigned budget, int lds_limit, int cus, Launch* out) {
+    Tiling& g = out->g;
+    std::memset(&g, 0, sizeof(g));
+    const int hard = mode == 2 ? 1 : 6;
+    const unsigned ny = static_cast<unsigned>(l_max + 1) * (l_max + 1);
+    const unsigned nyh = static_cast<unsigned>(hard + 1) * (hard + 1);
+    const unsigned nrow = whole ? ny : ny - nyh;
+    const unsigned tri_all = static_cast<unsigned>(l_max + 1) * (l_max + 2) / 2;
+    const unsigned arrays = mode + 1;
+    unsigned jobs = 0;
+    for (int l = hard + 1; l <= l_max; ++l) jobs += l + 1;
+    // rows once, point tables three times, iterates twice (see recursion_kernel)
+    const unsigned per_point =
+        components_of(mode) * nrow + 3 * (8 + 3 * (l_max + 1)) + 2 * arrays * tri_all;
+    const unsigned fixed = 2 * tri_all + (jobs * 2 + static_cast<unsigned>(elem) - 1) / static_cast<unsigned>(elem) + 16;
+    auto bytes_for = [&](unsigned S) { return (S * per_point + fixed) * static_cast<unsigned>(elem); };
+    if (bytes_for(1) > static_cast<unsigned>(lds_limit)) return false;
+    unsigned S = 1;
+    if (bytes_for(1) <= budget) {
+        S = pow2_floor((budget / static_cast<unsigned>(elem) - fixed) / per_point);
+        if (S > 64) S = 64;
+    }
+    const int forced = env_int("SPHX_TILE", 0);
+    if (forced > 0 && forced <= 64 && bytes_for(forced) <= static_cast<unsigned>(lds_limit)) {
+        S = static_cast<unsigned>(forced);
+    }
+
+    g.n_samples = n_samples;
+    g.l_max = l_max;
+    g.ny = static_cast<int>(ny);
+    g.tile = static_cast<int>(S);
+    g.jobs_per_point = jobs;
+    g.magic_jobs = magic_of(jobs);
+    g.sequence_waves = S * arrays * static_cast<unsigned>(l_max - hard) > 64 ? 2u : 1u;
+    unsigned at = align4(S * nrow);
+    g.off_dsph = at;
+    if (mode >= 1) at = align4(at + S * 3 * nrow);
+    g.off_ddsph = at;
+    if (mode == 2) at = align4(at + S * 9 * nrow);
+    g.off_F = at;
+    at += tri_all;
+    g.off_Q = at;
+    at += tri_all;
+    g.off_pts = at;
+    at += 3 * S * (8 + 3 * (l_max + 1));
+    g.off_iter = at;
+    at += 2 * S * arrays * tri_all;
+    g.off_jobs = at;
+    at += (jobs * 2 + static_cast<unsigned>(elem) - 1) / static_cast<unsigned>(elem);
+    out->lds_bytes = at * static_cast<unsigned>(elem);
+    out->threads = kRecursionThreads;
+
+    g.n_tiles = static_cast<unsigned>((n_samples + S - 1) / S);
+    g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
+    unsigned per_cu = static_cast<unsigned>(lds_limit) / out->lds_bytes;
+    if (per_cu < 1) per_cu = 1;
+    if (per_cu > 4) per_cu = 4; // 512 threads each: 2048 lanes per CU
+    unsigned want = (static_cast<unsigned>(cus) * per_cu + 7u) & ~7u;
+    unsigned need = g.tiles_per_xcd * 8u;
+    out->workgroups = want < need ? want : need;
+    if (out->workgroups < 8) out->workgroups = 8;
+    return true;
+}
+
+// Choose kernels, tile sizes and LDS layouts. `lds_limit` / `cus` describe the device.
 static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit, int cus,
                      Plan* plan) {
     if (l_max < 0) return fail(SPHX_ERR_ARGUMENT, "l_max must be non-negative");
@@ -423,166 +633,107 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
                     "l_max = " + std::to_string(l_max) + " exceeds the device prefactor tables (" +
                         std::to_string(SPHX_TABLE_LMAX) + ")");
     }
-    Tiling& g = plan->g;
-    std::memset(&g, 0, sizeof(g));
-    const int hard_cap = mode == 2 ? 1 : 6;
-    plan->closed_form = l_max <= hard_cap;
-    const unsigned ny = static_cast<unsigned>(l_max + 1) * (l_max + 1);
-    const unsigned mult = mode == 0 ? 1 : (mode == 1 ? 4 : 13); // elements per point = mult * ny
-    g.n_samples = n_samples;
-    g.l_max = l_max;
-    g.ny = static_cast<int>(ny);
-    g.pad = (ny % 2 == 0) ? 1u : 0u;
-    const unsigned arrays = mode + 1;
-    const unsigned row_elems = mult * ny + arrays * g.pad; // LDS elements per point
-
-    unsigned S;         // points whose rows are staged in LDS at a time
-    unsigned per_group; // points one workgroup handles before it moves on (or ends)
-    if (plan->closed_form) {
-        plan->threads = 64;
-        per_group = 64;
-        S = 64 / closed_form_phases(static_cast<unsigned>(elem), mode, l_max);
-    } else {
-        plan->threads = 256;
-        const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", 36 * 1024));
-        const unsigned per_point = (row_elems + 2 * (3 * (l_max + 1) + 8)) * elem;
-        unsigned fit = budget / per_point;
-        S = fit >= 1 ? pow2_floor(fit) : 1;
-        if (S > 64) S = 64;
-        const int forced = env_int("SPHX_TILE", 0);
-        if (forced > 0 && forced <= 64) S = static_cast<unsigned>(forced);
-        per_group = S;
+    if ((n_samples + 63) / 64 > 0x7fffffffull) {
+        return fail(SPHX_ERR_UNSUPPORTED, "too many samples for one launch");
     }
-    g.tile = static_cast<int>(S);
-    plan->points_per_group = per_group;
-
-    // LDS carve-up (elements)
-    unsigned at = S * (ny + g.pad);
-    at = (at + 3u) & ~3u;
-    g.off_dsph = at;
-    if (mode >= 1) at += S * (3 * ny + g.pad);
-    at = (at + 3u) & ~3u;
-    g.off_ddsph = at;
-    if (mode == 2) at += S * (9 * ny + g.pad);
-    at = (at + 3u) & ~3u;
-    if (!plan->closed_form) {
-        const unsigned nq = static_cast<unsigned>(l_max + 1) * (l_max + 2) / 2;
-        g.off_F = at;
-        at += nq;
-        g.off_Q = at;
-        at += nq;
-        g.off_pts = at; // per point: 8 coordinates-and-such, then c, s, 2(m+1)z; two buffers
-        at += 2 * S * (3 * (l_max + 1) + 8);
-        // segment length: the shortest that still gives every job its own lane (192 lanes run
-        // the recursion jobs), so that the longest chain of dependent work is as short as possible
-        const int hard = mode == 2 ? 1 : 6;
-        static const unsigned candidates[] = {2, 3, 4, 6, 8, 12, 16, 24, 32, 65};
-        unsigned chosen = 65, jobs = 0;
-        const int forced_segment = env_int("SPHX_SEGMENT", 0);
-        for (unsigned cand : candidates) {
-            unsigned count = 0;
-            for (int l = hard + 1; l <= l_max; ++l) count += static_cast<unsigned>(l) / cand + 1;
-            if ((forced_segment > 1 && cand >= static_cast<unsigned>(forced_segment)) ||
-                (forced_segment <= 1 && S * count <= 192) || cand == 65) {
-                chosen = cand;
-                jobs = count;
-                break;
-            }
+    const int hard = mode == 2 ? 1 : 6;
+    plan->closed_only = l_max <= hard;
+    plan->whole = true;
+    if (plan->closed_only) {
+        plan_closed(n_samples, l_max, l_max, mode, elem, &plan->closed);
+        return SPHX_OK;
+    }
+    const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", 76 * 1024));
+    bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec);
+    // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of
+    // a wave idle for a thousand instructions per tile: hand them to the closed-form kernel,
+    // which runs them 64 points at a time, and let the recursion kernel stage l >= 7 only.
+    const int split_below = env_int("SPHX_SPLIT_BELOW", 16);
+    if (mode < 2 && (!fits || plan->rec.g.tile < split_below)) {
+        Launch split;
+        if (plan_recursion(n_samples, l_max, mode, false, elem, budget, lds_limit, cus, &split)) {
+            plan->whole = false;
+            plan->rec = split;
+            plan_closed(n_samples, l_max, hard, mode, elem, &plan->closed);
+            fits = true;
         }
-        g.segment = chosen;
-        g.jobs_per_point = jobs;
-        g.off_jobs = at;
-        at += (jobs * 2 + static_cast<unsigned>(elem) - 1) / static_cast<unsigned>(elem);
     }
-    plan->lds_bytes = at * static_cast<unsigned>(elem);
-    if (plan->lds_bytes > static_cast<unsigned>(lds_limit)) {
+    if (!fits) {
         return fail(SPHX_ERR_UNSUPPORTED,
-                    "l_max = " + std::to_string(l_max) + " with this many derivatives needs " +
-                        std::to_string(plan->lds_bytes) + " bytes of LDS per point tile; the device offers " +
-                        std::to_string(lds_limit));
-    }
-
-    const unsigned long long tiles = (n_samples + per_group - 1) / per_group;
-    if (tiles > 0x7fffffffull) return fail(SPHX_ERR_UNSUPPORTED, "too many samples for one launch");
-    g.n_tiles = static_cast<unsigned>(tiles);
-    for (int a = 0; a < 3; ++a) {
-        const unsigned long long row = (a == 0 ? 1ull : (a == 1 ? 3ull : 9ull)) * ny;
-        g.magic[a] = static_cast<unsigned>(((1ull << 32) + row - 1) / row); // unused when row == 1
-    }
-
-    if (plan->closed_form) {
-        g.tiles_per_group = (g.n_tiles + 7u) / 8u;
-        plan->workgroups = g.tiles_per_group * 8u;
-    } else {
-        unsigned per_cu = static_cast<unsigned>(lds_limit) / (plan->lds_bytes ? plan->lds_bytes : 1u);
-        if (per_cu < 1) per_cu = 1;
-        if (per_cu > 8) per_cu = 8; // 256 threads each: 2048 lanes per CU
-        unsigned want = static_cast<unsigned>(cus) * per_cu;
-        want = (want + 7u) & ~7u;
-        unsigned need = (g.n_tiles + 7u) & ~7u;
-        plan->workgroups = want < need ? want : need;
-        if (plan->workgroups < 8) plan->workgroups = 8;
-        g.tiles_per_group = (g.n_tiles + 7u) / 8u;
+                    "l_max = " + std::to_string(l_max) +
+                        " with this many derivatives needs more LDS for the rows of one point than "
+                        "the device offers (" + std::to_string(lds_limit) + " bytes)");
     }
     return SPHX_OK;
 }
 
-template <typename T, int MODE, bool NORM, int H>
-static hipError_t launch_closed(const Plan& plan, const T* xyz, T* sph, T* dsph, T* ddsph,
+template <typename T, int MODE, bool NORM, int H, bool PREFIX>
+static hipError_t launch_closed(const Launch& l, const T* xyz, T* sph, T* dsph, T* ddsph,
                                 hipStream_t stream) {
-    auto kernel = closed_form_kernel<T, MODE, NORM, H>;
-    if (plan.lds_bytes > 64u * 1024u) {
+    auto kernel = closed_form_kernel<T, MODE, NORM, H, PREFIX>;
+    if (l.lds_bytes > 64u * 1024u) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(plan.lds_bytes));
+                                           static_cast<int>(l.lds_bytes));
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL(kernel, dim3(plan.workgroups), dim3(plan.threads), plan.lds_bytes, stream,
-                       plan.g, xyz, sph, dsph, ddsph);
+    hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz,
+                       sph, dsph, ddsph);
     return hipGetLastError();
 }
 
-template <typename T, int MODE, bool NORM, int H>
-static hipError_t launch_recursion(const Plan& plan, const T* xyz, T* sph, T* dsph, T* ddsph,
+template <typename T, int MODE, bool NORM, bool WHOLE>
+static hipError_t launch_recursion(const Launch& l, const T* xyz, T* sph, T* dsph, T* ddsph,
                                    hipStream_t stream) {
-    auto kernel = recursion_kernel<T, MODE, NORM, H>;
-    if (plan.lds_bytes > 64u * 1024u) {
+    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE>;
+    if (l.lds_bytes > 64u * 1024u) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(plan.lds_bytes));
+                                           static_cast<int>(l.lds_bytes));
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL(kernel, dim3(plan.workgroups), dim3(plan.threads), plan.lds_bytes, stream,
-                       plan.g, xyz, sph, dsph, ddsph);
+    hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz,
+                       sph, dsph, ddsph);
     return hipGetLastError();
 }
 
 template <typename T, int MODE, bool NORM>
 static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* ddsph,
                            hipStream_t stream) {
-    if (!plan.closed_form) {
-        return launch_recursion<T, MODE, NORM, (MODE == 2 ? 1 : 6)>(plan, xyz, sph, dsph, ddsph, stream);
+    if (!plan.closed_only) {
+        if constexpr (MODE == 2) {
+            return launch_recursion<T, MODE, NORM, true>(plan.rec, xyz, sph, dsph, ddsph, stream);
+        } else {
+            if (plan.whole) {
+                return launch_recursion<T, MODE, NORM, true>(plan.rec, xyz, sph, dsph, ddsph, stream);
+            }
+            // the two kernels write disjoint parts of every row
+            hipError_t e = launch_closed<T, MODE, NORM, 6, true>(plan.closed, xyz, sph, dsph, ddsph, stream);
+            if (e != hipSuccess) return e;
+            return launch_recursion<T, MODE, NORM, false>(plan.rec, xyz, sph, dsph, ddsph, stream);
+        }
     }
-    switch (plan.g.l_max) {
+    const Launch& l = plan.closed;
+    switch (l.g.l_max) {
     case 0:
-        return launch_closed<T, MODE, NORM, 0>(plan, xyz, sph, dsph, ddsph, stream);
+        return launch_closed<T, MODE, NORM, 0, false>(l, xyz, sph, dsph, ddsph, stream);
     case 1:
-        return launch_closed<T, MODE, NORM, 1>(plan, xyz, sph, dsph, ddsph, stream);
+        return launch_closed<T, MODE, NORM, 1, false>(l, xyz, sph, dsph, ddsph, stream);
     default:
         break;
     }
     if constexpr (MODE < 2) {
-        switch (plan.g.l_max) {
+        switch (l.g.l_max) {
         case 2:
-            return launch_closed<T, MODE, NORM, 2>(plan, xyz, sph, dsph, ddsph, stream);
+            return launch_closed<T, MODE, NORM, 2, false>(l, xyz, sph, dsph, ddsph, stream);
         case 3:
-            return launch_closed<T, MODE, NORM, 3>(plan, xyz, sph, dsph, ddsph, stream);
+            return launch_closed<T, MODE, NORM, 3, false>(l, xyz, sph, dsph, ddsph, stream);
         case 4:
-            return launch_closed<T, MODE, NORM, 4>(plan, xyz, sph, dsph, ddsph, stream);
+            return launch_closed<T, MODE, NORM, 4, false>(l, xyz, sph, dsph, ddsph, stream);
         case 5:
-            return launch_closed<T, MODE, NORM, 5>(plan, xyz, sph, dsph, ddsph, stream);
+            return launch_closed<T, MODE, NORM, 5, false>(l, xyz, sph, dsph, ddsph, stream);
         case 6:
-            return launch_closed<T, MODE, NORM, 6>(plan, xyz, sph, dsph, ddsph, stream);
+            return launch_closed<T, MODE, NORM, 6, false>(l, xyz, sph, dsph, ddsph, stream);
         default:
             break;
         }
@@ -687,10 +838,11 @@ int sphx_plan(size_t n_samples, int l_max, int derivatives, int is_f64, int* til
     int status = sphx::make_plan(n_samples ? n_samples : 1, l_max, derivatives,
                                  is_f64 ? sizeof(double) : sizeof(float), lds, cus, &plan);
     if (status != SPHX_OK) return status;
-    if (tile_samples) *tile_samples = static_cast<int>(plan.points_per_group);
-    if (threads) *threads = plan.threads;
-    if (lds_bytes) *lds_bytes = static_cast<int>(plan.lds_bytes);
-    if (workgroups) *workgroups = static_cast<int>(plan.workgroups);
+    const sphx::Launch& main = plan.closed_only ? plan.closed : plan.rec;
+    if (tile_samples) *tile_samples = main.g.tile;
+    if (threads) *threads = static_cast<int>(main.threads);
+    if (lds_bytes) *lds_bytes = static_cast<int>(main.lds_bytes);
+    if (workgroups) *workgroups = static_cast<int>(main.workgroups);
     return SPHX_OK;
 }
 
