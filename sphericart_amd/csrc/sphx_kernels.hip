@@ -171,16 +171,17 @@ __global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __re
         const unsigned count = valid - base < PER ? valid - base : PER;
         const unsigned long long at = first + base;
         if constexpr (!PREFIX) {
-            copy_out<T, SPHX_STREAMING_STORES>(lds, sph + at * NY, count * NY, NY, PAD,
-                                               magic_of(NY), tid, 64);
+            copy_out<T, SPHX_STREAMING_STORES, PAD != 0>(lds, sph + at * NY, count * NY, NY, PAD,
+                                                         magic_of(NY), tid, 64);
             if constexpr (MODE >= 1) {
-                copy_out<T, SPHX_STREAMING_STORES>(lds + OFF_D, dsph + at * 3 * NY, count * 3 * NY,
-                                                   3 * NY, PAD, magic_of(3 * NY), tid, 64);
+                copy_out<T, SPHX_STREAMING_STORES, PAD != 0>(lds + OFF_D, dsph + at * 3 * NY,
+                                                             count * 3 * NY, 3 * NY, PAD,
+                                                             magic_of(3 * NY), tid, 64);
             }
             if constexpr (MODE == 2) {
-                copy_out<T, SPHX_STREAMING_STORES>(lds + OFF_DD, ddsph + at * 9 * NY,
-                                                   count * 9 * NY, 9 * NY, PAD, magic_of(9 * NY),
-                                                   tid, 64);
+                copy_out<T, SPHX_STREAMING_STORES, PAD != 0>(lds + OFF_DD, ddsph + at * 9 * NY,
+                                                             count * 9 * NY, 9 * NY, PAD,
+                                                             magic_of(9 * NY), tid, 64);
             }
         } else {
             const unsigned ny = g.ny;
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
 
     T* F = lds + g.off_F;
     T* Q = lds + g.off_Q;
-    unsigned short* job_table = reinterpret_cast<unsigned short*>(lds + g.off_jobs);
+    unsigned* job_table = reinterpret_cast<unsigned*>(lds + g.off_jobs);
     {
         const T* cF = table_F<T>();
         const T* cQ = table_Q<T>();
@@ -257,14 +258,19 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         }
         // (l, m) pairs: the bulk 1 <= m <= l - 2 first, then the special cases m = l, l - 1 and
         // 0 each as one block, so that the lanes of a wave mostly share one branch of entry_job
+        // one word per job: m in bits 0-7, l in bits 8-15, l(l+1)/2 above
+        auto pack = [](int l, int m) -> unsigned {
+            return (static_cast<unsigned>(l * (l + 1) / 2) << 16) | (static_cast<unsigned>(l) << 8) |
+                   static_cast<unsigned>(m);
+        };
         if (tid == 0) {
             unsigned n = 0;
             for (int l = L; l > H; --l) {
-                for (int m = l - 2; m >= 1; --m) job_table[n++] = static_cast<unsigned short>((l << 8) | m);
+                for (int m = l - 2; m >= 1; --m) job_table[n++] = pack(l, m);
             }
-            for (int l = L; l > H; --l) job_table[n++] = static_cast<unsigned short>((l << 8) | l);
-            for (int l = L; l > H; --l) job_table[n++] = static_cast<unsigned short>((l << 8) | (l - 1));
-            for (int l = L; l > H; --l) job_table[n++] = static_cast<unsigned short>(l << 8);
+            for (int l = L; l > H; --l) job_table[n++] = pack(l, l);
+            for (int l = L; l > H; --l) job_table[n++] = pack(l, l - 1);
+            for (int l = L; l > H; --l) job_table[n++] = pack(l, 0);
         }
     }
 
@@ -401,12 +407,7 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
                     closed_form_job<T, MODE, NORM, H>(p, rows);
                 }
             }
-            const unsigned jobs = valid * g.jobs_per_point;
-            for (unsigned j = t; j < jobs; j += NT - wide_first) {
-                const unsigned s = __umulhi(j, g.magic_jobs);
-                const unsigned entry = job_table[j - s * g.jobs_per_point];
-                const int l = static_cast<int>(entry >> 8);
-                const int m = static_cast<int>(entry & 0xffu);
+            for (unsigned s = 0; s < valid; ++s) {
                 const T* rec = point_data(n % 3u, s);
                 Point<T> p;
                 p.x = rec[0];
@@ -416,6 +417,11 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
                 p.y2 = rec[4];
                 p.z2 = rec[5];
                 p.ir = rec[6];
+                const T* c = rec + 8;
+                const T* sn = rec + 8 + (L + 1);
+                const T* itA = iterates(n & 1u, s, 0, 0);
+                const T* itB = iterates(n & 1u, s, MODE >= 1 ? 1 : 0, 0);
+                const T* itC = iterates(n & 1u, s, MODE == 2 ? 2 : 0, 0);
                 // rows are addressed with the entry's index in the full row; shift the bases when
                 // the staged rows start at l = H + 1
                 Rows<T> rows;
@@ -423,22 +429,27 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
                 rows.sph = lds + s * nrow - skip;
                 rows.dsph = lds + g.off_dsph + s * 3 * nrow - skip;
                 rows.ddsph = lds + g.off_ddsph + s * 9 * nrow - skip;
-                entry_job<T, MODE, NORM>(l, m, p, F, rec + 8, rec + 8 + (L + 1), iterates(n & 1u, s, 0, l),
-                                         iterates(n & 1u, s, MODE >= 1 ? 1 : 0, l),
-                                         iterates(n & 1u, s, MODE == 2 ? 2 : 0, l), rows);
+                for (unsigned e = t; e < g.jobs_per_point; e += NT - wide_first) {
+                    const unsigned packed = job_table[e];
+                    const int m = static_cast<int>(packed & 0xffu);
+                    const int l = static_cast<int>((packed >> 8) & 0xffu);
+                    const int tri = static_cast<int>(packed >> 16);
+                    entry_job<T, MODE, NORM>(l, m, tri, p, F + tri, c, sn, itA + tri, itB + tri,
+                                             itC + tri, rows);
+                }
             }
         }
         __syncthreads(); // rows of tile n complete
 
         if constexpr (WHOLE) {
-            copy_out<T, SPHX_STREAMING_STORES>(lds, sph + first * ny, valid * ny, ny, 0, 0, tid, NT);
+            copy_out<T, SPHX_STREAMING_STORES, false>(lds, sph + first * ny, valid * ny, ny, 0, 0, tid, NT);
             if constexpr (MODE >= 1) {
-                copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_dsph, dsph + first * 3 * ny,
+                copy_out<T, SPHX_STREAMING_STORES, false>(lds + g.off_dsph, dsph + first * 3 * ny,
                                                    valid * 3 * ny, 3 * ny, 0, 0, tid, NT);
             }
             if constexpr (MODE == 2) {
-                copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_ddsph, ddsph + first * 9 * ny,
-                                                   valid * 9 * ny, 9 * ny, 0, 0, tid, NT);
+                copy_out<T, SPHX_STREAMING_STORES, false>(lds + g.off_ddsph, ddsph + first * 9 * ny,
+                                                          valid * 9 * ny, 9 * ny, 0, 0, tid, NT);
             }
         } else {
             // one run per (point, component) row, dealt to the waves in turn
@@ -446,11 +457,11 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
             for (unsigned r = wave; r < valid * components_of(MODE); r += NW) {
                 // rows [0, valid) are values, the next 3 * valid are gradients
                 if (r < valid) {
-                    copy_out<T, SPHX_STREAMING_STORES>(lds + r * nrow, sph + (first + r) * ny + skip, nrow,
+                    copy_out<T, SPHX_STREAMING_STORES, false>(lds + r * nrow, sph + (first + r) * ny + skip, nrow,
                                                        nrow, 0, 0, lane, 64);
                 } else {
                     const unsigned q = r - valid;
-                    copy_out<T, SPHX_STREAMING_STORES>(lds + g.off_dsph + q * nrow,
+                    copy_out<T, SPHX_STREAMING_STORES, false>(lds + g.off_dsph + q * nrow,
                                                        dsph + (first * 3 + q) * ny + skip, nrow, nrow, 0,
                                                        0, lane, 64);
                 }
@@ -573,7 +584,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // rows once, point tables three times, iterates twice (see recursion_kernel)
     const unsigned per_point =
         components_of(mode) * nrow + 3 * (8 + 3 * (l_max + 1)) + 2 * arrays * tri_all;
-    const unsigned fixed = 2 * tri_all + (jobs * 2 + static_cast<unsigned>(elem) - 1) / static_cast<unsigned>(elem) + 16;
+    const unsigned fixed = 2 * tri_all + (jobs * 4 + static_cast<unsigned>(elem) - 1) / static_cast<unsigned>(elem) + 16;
     auto bytes_for = [&](unsigned S) { return (S * per_point + fixed) * static_cast<unsigned>(elem); };
     if (bytes_for(1) > static_cast<unsigned>(lds_limit)) return false;
     unsigned S = 1;
@@ -607,7 +618,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.off_iter = at;
     at += 2 * S * arrays * tri_all;
     g.off_jobs = at;
-    at += (jobs * 2 + static_cast<unsigned>(elem) - 1) / static_cast<unsigned>(elem);
+    at += (jobs * 4 + static_cast<unsigned>(elem) - 1) / static_cast<unsigned>(elem);
     out->lds_bytes = at * static_cast<unsigned>(elem);
     out->threads = kRecursionThreads;
 
@@ -692,7 +703,20 @@ static hipError_t launch_recursion(const Launch& l, const T* xyz, T* sph, T* dsp
                                            static_cast<int>(l.lds_bytes));
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz,
+    // The workgroups are persistent: launch exactly as many as are resident at once (registers
+    // may allow fewer per CU than LDS does), or the last ones would run alone after the rest.
+    unsigned workgroups = l.workgroups;
+    int resident = 0, device = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kernel, static_cast<int>(l.threads),
+                                                     l.lds_bytes) == hipSuccess &&
+        resident > 0 && hipGetDevice(&device) == hipSuccess &&
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess) {
+        const unsigned cap = (static_cast<unsigned>(resident) * static_cast<unsigned>(cus)) & ~7u;
+        if (cap >= 8 && cap < workgroups) workgroups = cap;
+    } else {
+        (void)hipGetLastError();
+    }
+    hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz,
                        sph, dsph, ddsph);
     return hipGetLastError();
 }
