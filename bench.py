@@ -35,9 +35,16 @@ sys.path.insert(0, ROOT)
 PEAK_HBM_GBPS = 8000.0
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script (profiles/), scaled by what the same counters read for a plain copy of
-# known size. None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {}
+# script (summaries under profiles/), each counter scaled by what it reads for a
+# plain device-to-device copy of known size (`--calibrate-copy`: WRITE_SIZE
+# reads the copied bytes exactly, FETCH_SIZE half of them, so fetches are
+# doubled). KiB per dispatch * 1024 * factor, fetch + write, all kernels of one
+# call added up.
+MEASURED_TRAFFIC_BYTES = {
+    "cfg3": int((5932.6 * 2.0 + 765883.9) * 1024),
+    "cfg4": int((1304.2 * 2.0 + 3063197.6) * 1024),
+    "cfg5": int(((1239.9 + 1279.8) * 2.0 + 184231.9 + 3427561.4) * 1024),
+}
 
 
 def parse():
