@@ -290,20 +290,46 @@ __device__ __forceinline__ void sequence_job(int l, int which, T z, T rxy,
         --m;
     }
     if (m < 0) return;
-    // the constants of a step do not depend on the iterates: fetch them one step ahead so that
-    // the chain of dependent operations never waits for LDS
-    T tz_next = tmz[m];
-    T k_next = k[m];
-    for (; m >= 0; --m) {
-        const T tz = tz_next;
-        const T km = k_next;
-        const int ahead = m > 0 ? m - 1 : 0;
-        tz_next = tmz[ahead];
-        k_next = k[ahead];
-        const T v0 = km * (tz * v1 + rxy * v2);
+    // The constants of a step (2(m+1)z and k_m) do not depend on the iterates, the steps do
+    // depend on one another: a step that waited for its own constants would take one LDS round
+    // trip, several times the arithmetic. So the constants are fetched DEPTH steps ahead, a
+    // block of DEPTH at a time, while the block before is being worked through.
+    constexpr int DEPTH = 4;
+    for (int odd = (m + 1) & (DEPTH - 1); odd > 0; --odd, --m) {
+        const T v0 = k[m] * (tmz[m] * v1 + rxy * v2);
         out[m] = v0;
         v2 = v1;
         v1 = v0;
+    }
+    if (m < 0) return;
+    // m + 1 is a multiple of DEPTH from here on; element j of a block belongs to step base + j
+    T tz[DEPTH], km[DEPTH];
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) {
+        tz[j] = tmz[m - (DEPTH - 1) + j];
+        km[j] = k[m - (DEPTH - 1) + j];
+    }
+    for (; m >= 0; m -= DEPTH) {
+        const int base = m - (DEPTH - 1);
+        const int next = base >= DEPTH ? base - DEPTH : 0; // the last block fetches, unused, from 0
+        T tz_next[DEPTH], km_next[DEPTH];
+#pragma unroll
+        for (int j = 0; j < DEPTH; ++j) {
+            tz_next[j] = tmz[next + j];
+            km_next[j] = k[next + j];
+        }
+#pragma unroll
+        for (int j = DEPTH - 1; j >= 0; --j) {
+            const T v0 = km[j] * (tz[j] * v1 + rxy * v2);
+            out[base + j] = v0;
+            v2 = v1;
+            v1 = v0;
+        }
+#pragma unroll
+        for (int j = 0; j < DEPTH; ++j) {
+            tz[j] = tz_next[j];
+            km[j] = km_next[j];
+        }
     }
 }
 
@@ -313,8 +339,17 @@ __device__ __forceinline__ void sequence_job(int l, int which, T z, T rxy,
 // (l - 2 >= |m| >= 1) and :392-426 (m = 0), with the Q iterates read from the
 // arrays the sequence jobs left in LDS. pk is the (l, .) row of the prefactor block, c / s the
 // point's azimuthal tables.
-template <typename T, int MODE, bool NORM>
-__device__ __forceinline__ void entry_job(int l, int m, int tri, const Point<T>& p,
+//
+// The reference writes the entry (l, +m) with c_m, c_{m-1}, c_{m-2} and the entry (l, -m) with
+// s_m, s_{m-1}, s_{m-2} in their place; where the two formulas differ beyond that, one has
+// "+ t c_{m-1}" where the other has "- t s_{m-1}" (same for m - 2). Both are written here once,
+// as a function of the side: u_k stands for c_k or s_k, w_k for -s_k or c_k. Negating a factor
+// negates the rounded product exactly and a + (-b) is a - b, so the numbers are the
+// reference's. SPLIT == false: one job computes both sides (the common factors are shared).
+// SPLIT == true: one job computes the side it is given, so that a tile with few (l, m) pairs
+// still spreads over all lanes.
+template <typename T, int MODE, bool NORM, bool SPLIT>
+__device__ __forceinline__ void entry_job(int l, int m, int tri, int side, const Point<T>& p,
                                           const T* __restrict__ pk, const T* __restrict__ c,
                                           const T* __restrict__ s, const T* __restrict__ A,
                                           [[maybe_unused]] const T* __restrict__ B,
@@ -323,7 +358,7 @@ __device__ __forceinline__ void entry_job(int l, int m, int tri, const Point<T>&
     // tri = l(l+1)/2; pk, A, B, C already point at the (l, 0) entries of their triangular arrays
     constexpr bool GRAD = MODE >= 1;
     constexpr bool HESS = MODE == 2;
-    const T x = p.x, y = p.y, z = p.z;
+    const T x = p.x, y = p.y;
     const int mid = 2 * tri;
     const T zero = static_cast<T>(0.0);
     [[maybe_unused]] T x2 = 0, y2 = 0, xy = 0;
@@ -332,130 +367,168 @@ __device__ __forceinline__ void entry_job(int l, int m, int tri, const Point<T>&
         y2 = y * y;
         xy = x * y;
     }
-    (void)z;
-
-    Entry<T> neg, pos;
-    neg.gx = neg.gy = neg.gz = pos.gx = pos.gy = pos.gz = zero;
-    neg.hxx = neg.hxy = neg.hxz = neg.hyy = neg.hyz = neg.hzz = zero;
-    pos.hxx = pos.hxy = pos.hxz = pos.hyy = pos.hyz = pos.hzz = zero;
+    auto blank = [&]() {
+        Entry<T> e;
+        e.v = e.gx = e.gy = e.gz = zero;
+        e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = zero;
+        return e;
+    };
+    // stage what `make(side)` returns: both sides, or the one this job was given
+    auto emit_sides = [&](auto make) {
+        if constexpr (SPLIT) {
+            stage<T, MODE, NORM>(out, side ? mid - m : mid + m, p, make(side != 0));
+        } else {
+            stage<T, MODE, NORM>(out, mid + m, p, make(false));
+            stage<T, MODE, NORM>(out, mid - m, p, make(true));
+        }
+    };
 
     if (m == l) {
         // :122-152
         const T qlm_2 = A[l];
-        auto pq = qlm_2 * pk[l];
-        neg.v = pq * s[l];
-        pos.v = pq * c[l];
+        const T cl = c[l], sl = s[l];
+        [[maybe_unused]] T cl1 = 0, sl1 = 0, cl2 = 0, sl2 = 0;
         if constexpr (GRAD) {
-            pq *= l;
-            neg.gx = pq * s[l - 1];
-            neg.gy = pos.gx = pq * c[l - 1];
-            pos.gy = -neg.gx;
-            if constexpr (HESS) {
-                pq *= (l - 1);
-                pos.hxx = pq * c[l - 2];
-                neg.hxx = pq * s[l - 2];
-                pos.hxy = neg.hyy = -neg.hxx;
-                neg.hxy = pos.hxx;
-                pos.hyy = -pos.hxx;
-            }
+            cl1 = c[l - 1];
+            sl1 = s[l - 1];
         }
+        if constexpr (HESS) {
+            cl2 = c[l - 2];
+            sl2 = s[l - 2];
+        }
+        emit_sides([&](bool minus) {
+            Entry<T> e = blank();
+            auto pq = qlm_2 * pk[l];
+            e.v = pq * (minus ? sl : cl);
+            if constexpr (GRAD) {
+                pq *= l;
+                e.gx = pq * (minus ? sl1 : cl1);
+                e.gy = pq * (minus ? cl1 : -sl1);
+                if constexpr (HESS) {
+                    pq *= (l - 1);
+                    e.hxx = pq * (minus ? sl2 : cl2);
+                    e.hxy = pq * (minus ? cl2 : -sl2);
+                    e.hyy = -e.hxx;
+                }
+            }
+            return e;
+        });
     } else if (m == l - 1) {
         // :154-198
-        const T qlm_2 = A[l];
+        [[maybe_unused]] const T qlm_2 = A[l];
         const T qlm_1 = A[l - 1];
-        auto pq = qlm_1 * pk[l - 1];
-        neg.v = pq * s[l - 1];
-        pos.v = pq * c[l - 1];
+        const T pkm = pk[l - 1];
+        const T cm = c[l - 1], sm = s[l - 1];
+        [[maybe_unused]] T cm1 = 0, sm1 = 0, cm2 = 0, sm2 = 0, ql1m_1 = 0;
         if constexpr (GRAD) {
-            pq *= (l - 1);
-            neg.gx = pq * s[l - 2];
-            neg.gy = pos.gx = pq * c[l - 2];
-            pos.gy = -neg.gx;
-            const T ql1m_1 = B[l - 1];
-            auto pdq = pk[l - 1] * (l + l - 1) * ql1m_1;
-            neg.gz = pdq * s[l - 1];
-            pos.gz = pdq * c[l - 1];
-            if constexpr (HESS) {
-                pq *= (l - 2);
-                if (l == 2) {
-                    pos.hxx = 0;
-                    neg.hxx = 0;
-                } else {
-                    pos.hxx = pq * c[l - 3];
-                    neg.hxx = pq * s[l - 3];
-                }
-                pos.hxy = neg.hyy = -neg.hxx;
-                neg.hxy = pos.hxx;
-                auto temp = -pk[l - 1] * (l - 1) * qlm_2;
-                pos.hxz = temp * c[l - 2];
-                neg.hxz = temp * s[l - 2];
-                pos.hyy = -pos.hxx;
-                pos.hyz = -neg.hxz;
-                neg.hyz = pos.hxz;
+            cm1 = c[l - 2];
+            sm1 = s[l - 2];
+            ql1m_1 = B[l - 1];
+        }
+        if constexpr (HESS) {
+            if (l != 2) {
+                cm2 = c[l - 3];
+                sm2 = s[l - 3];
             }
         }
+        emit_sides([&](bool minus) {
+            Entry<T> e = blank();
+            auto pq = qlm_1 * pkm;
+            e.v = pq * (minus ? sm : cm);
+            if constexpr (GRAD) {
+                pq *= (l - 1);
+                e.gx = pq * (minus ? sm1 : cm1);
+                e.gy = pq * (minus ? cm1 : -sm1);
+                auto pdq = pkm * (l + l - 1) * ql1m_1;
+                e.gz = pdq * (minus ? sm : cm);
+                if constexpr (HESS) {
+                    pq *= (l - 2);
+                    if (l == 2) {
+                        // the reference sets xx to zero and derives the rest from it by negation
+                        e.hxx = zero;
+                        e.hxy = minus ? zero : -zero;
+                    } else {
+                        e.hxx = pq * (minus ? sm2 : cm2);
+                        e.hxy = pq * (minus ? cm2 : -sm2);
+                    }
+                    e.hyy = -e.hxx;
+                    auto temp = -pkm * (l - 1) * qlm_2;
+                    e.hxz = temp * (minus ? sm1 : cm1);
+                    e.hyz = temp * (minus ? cm1 : -sm1);
+                }
+            }
+            return e;
+        });
     } else if (m > 0) {
         // :201-390
         const T cm = c[m], sm = s[m], pkm = pk[m];
         const T qlm_0 = A[m];
-        auto pq = qlm_0 * pkm;
-        neg.v = pq * sm;
-        pos.v = pq * cm;
+        [[maybe_unused]] T cm1 = 0, sm1 = 0, cm2 = 0, sm2 = 0, ql1m_2 = 0, ql1m_1 = 0;
+        [[maybe_unused]] T ql2m_2 = 0, ql2m_1 = 0, ql2m_0 = 0;
         if constexpr (GRAD) {
-            const T cm1 = c[m - 1], sm1 = s[m - 1];
+            cm1 = c[m - 1];
+            sm1 = s[m - 1];
             // the reference reads these after its shift: ql1m_2 is the iterate of step m + 1
             // (or the start value), ql1m_1 the iterate of step m
-            const T ql1m_2 = B[m + 1];
-            const T ql1m_1 = B[m];
-            pq *= m;
-            auto pqs = pq * sm1, pqc = pq * cm1;
-            auto pdq = pkm * ql1m_2;
-            auto pdqx = pdq * x;
-            neg.gx = (pdqx * sm + pqs);
-            pos.gx = (pdqx * cm + pqc);
-            auto pdqy = pdq * y;
-            neg.gy = (pdqy * sm + pqc);
-            pos.gy = (pdqy * cm - pqs);
-            pdq = pkm * (l + m) * ql1m_1;
-            neg.gz = pdq * sm;
-            pos.gz = pdq * cm;
-
-            if constexpr (HESS) {
-                // ... and these before its shift: the iterates of steps m + 2, m + 1 and m
-                const T ql2m_2 = C[m + 2];
-                const T ql2m_1 = C[m + 1];
-                const T ql2m_0 = C[m];
-                pq /= m;
-                auto pql1m_1 = pkm * ql1m_2;
-                auto pql2m_2 = pkm * ql2m_2;
-                auto pql2m_0 = pkm * ql2m_0;
-                auto pql1m_0 = pkm * ql1m_1;
-                auto pql2m_1 = pkm * ql2m_1;
-
-                T mmpqc2 = 0.0;
-                T mmpqs2 = 0.0;
-                if (m != 1) {
-                    mmpqc2 = m * (m - 1) * pq * c[m - 2];
-                    mmpqs2 = m * (m - 1) * pq * s[m - 2];
-                }
-
-                pos.hxx = pql1m_1 * cm + x2 * pql2m_2 * cm + 2 * m * x * pql1m_1 * cm1 + mmpqc2;
-                neg.hxx = pql1m_1 * sm + x2 * pql2m_2 * sm + 2 * m * x * pql1m_1 * sm1 + mmpqs2;
-                pos.hyy = pql1m_1 * cm + y2 * pql2m_2 * cm - 2 * m * y * pql1m_1 * sm1 - mmpqc2;
-                neg.hyy = pql1m_1 * sm + y2 * pql2m_2 * sm + 2 * m * y * pql1m_1 * cm1 - mmpqs2;
-                pos.hzz = (l + m) * (l + m - 1) * pql2m_0 * cm;
-                neg.hzz = (l + m) * (l + m - 1) * pql2m_0 * sm;
-
-                pos.hxy = xy * pql2m_2 * cm + y * pql1m_1 * m * cm1 - x * pql1m_1 * m * sm1 - mmpqs2;
-                neg.hxy = xy * pql2m_2 * sm + y * pql1m_1 * m * sm1 + x * pql1m_1 * m * cm1 + mmpqc2;
-                pos.hxz = x * (l + m) * pql2m_1 * cm + (l + m) * pql1m_0 * m * cm1;
-                neg.hxz = x * (l + m) * pql2m_1 * sm + (l + m) * pql1m_0 * m * sm1;
-                pos.hyz = y * (l + m) * pql2m_1 * cm - (l + m) * pql1m_0 * m * sm1;
-                neg.hyz = y * (l + m) * pql2m_1 * sm + (l + m) * pql1m_0 * m * cm1;
+            ql1m_2 = B[m + 1];
+            ql1m_1 = B[m];
+        }
+        if constexpr (HESS) {
+            // ... and these before its shift: the iterates of steps m + 2, m + 1 and m
+            ql2m_2 = C[m + 2];
+            ql2m_1 = C[m + 1];
+            ql2m_0 = C[m];
+            if (m != 1) {
+                cm2 = c[m - 2];
+                sm2 = s[m - 2];
             }
         }
+        emit_sides([&](bool minus) {
+            Entry<T> e = blank();
+            const T u = minus ? sm : cm;
+            auto pq = qlm_0 * pkm;
+            e.v = pq * u;
+            if constexpr (GRAD) {
+                const T u1 = minus ? sm1 : cm1;
+                const T w1 = minus ? cm1 : -sm1;
+                pq *= m;
+                auto pdq = pkm * ql1m_2;
+                auto pdqx = pdq * x;
+                e.gx = (pdqx * u + pq * u1);
+                auto pdqy = pdq * y;
+                e.gy = (pdqy * u + pq * w1);
+                pdq = pkm * (l + m) * ql1m_1;
+                e.gz = pdq * u;
+
+                if constexpr (HESS) {
+                    pq /= m;
+                    auto pql1m_1 = pkm * ql1m_2;
+                    auto pql2m_2 = pkm * ql2m_2;
+                    auto pql2m_0 = pkm * ql2m_0;
+                    auto pql1m_0 = pkm * ql1m_1;
+                    auto pql2m_1 = pkm * ql2m_1;
+
+                    // m (m-1) pq u_{m-2} and m (m-1) pq w_{m-2}
+                    T mmpqu2 = 0.0;
+                    T mmpqw2 = 0.0;
+                    if (m != 1) {
+                        mmpqu2 = m * (m - 1) * pq * (minus ? sm2 : cm2);
+                        mmpqw2 = m * (m - 1) * pq * (minus ? cm2 : -sm2);
+                    }
+
+                    e.hxx = pql1m_1 * u + x2 * pql2m_2 * u + 2 * m * x * pql1m_1 * u1 + mmpqu2;
+                    e.hyy = pql1m_1 * u + y2 * pql2m_2 * u + 2 * m * y * pql1m_1 * w1 - mmpqu2;
+                    e.hzz = (l + m) * (l + m - 1) * pql2m_0 * u;
+                    e.hxy = xy * pql2m_2 * u + y * pql1m_1 * m * u1 + x * pql1m_1 * m * w1 + mmpqw2;
+                    e.hxz = x * (l + m) * pql2m_1 * u + (l + m) * pql1m_0 * m * u1;
+                    e.hyz = y * (l + m) * pql2m_1 * u + (l + m) * pql1m_0 * m * w1;
+                }
+            }
+            return e;
+        });
     } else {
         // m = 0, :392-426
+        Entry<T> pos = blank();
         const T qlm_0 = A[0];
         pos.v = qlm_0 * pk[0];
         if constexpr (GRAD) {
@@ -480,10 +553,7 @@ __device__ __forceinline__ void entry_job(int l, int m, int tri, const Point<T>&
                 pos.hyz = y * l * pql2m_1;
             }
         }
-    }
-    stage<T, MODE, NORM>(out, mid + m, p, pos);
-    if (m > 0) {
-        stage<T, MODE, NORM>(out, mid - m, p, neg);
+        stage<T, MODE, NORM>(out, mid, p, pos);
     }
 }
 
@@ -515,7 +585,7 @@ __device__ __forceinline__ void emit(V v, V* dst) {
 // as 16-byte stores at 16-byte aligned addresses, consecutive lanes to consecutive addresses;
 // at most three (float) or one (double) leading and trailing elements are stored one by one.
 // PADDED: the staged run has `pad` spare elements after every `row` elements (see staged_index).
-template <typename T, bool STREAMING, bool PADDED>
+template <typename T, bool STREAMING, bool PADDED, int UNROLL = 1>
 __device__ __forceinline__ void copy_out(const T* __restrict__ staged, T* __restrict__ dst,
                                          unsigned len, unsigned row, unsigned pad, unsigned magic,
                                          unsigned tid, unsigned nthreads) {
@@ -527,17 +597,43 @@ __device__ __forceinline__ void copy_out(const T* __restrict__ staged, T* __rest
     const unsigned nvec = (len - head) / W;
     V* out = reinterpret_cast<V*>(dst + head) + tid;
     if (!PADDED && head == 0) {
-        // not unrolled on purpose: loads and stores alternating one by one measured 3 % faster
-        // than batches of four on the closed-form kernel
+        // UNROLL == 1 where many waves share the copy: loads and stores alternating one by one
+        // measured 3 % faster than batches of four on the closed-form kernel. A lone flushing
+        // wave needs several loads in flight to keep its stores coming.
         const V* in = reinterpret_cast<const V*>(staged);
         V* aligned = reinterpret_cast<V*>(dst);
-        for (unsigned g = tid; g < nvec; g += nthreads) {
+        unsigned g = tid;
+        if constexpr (UNROLL > 1) {
+            for (; g + (UNROLL - 1) * nthreads < nvec; g += UNROLL * nthreads) {
+                V v[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) v[u] = in[g + u * nthreads];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) emit<T, STREAMING>(v[u], aligned + g + u * nthreads);
+            }
+        }
+        for (; g < nvec; g += nthreads) {
             emit<T, STREAMING>(in[g], aligned + g);
         }
     } else if (!PADDED) {
+        // staged data and destination differ in their position within 16 bytes: the LDS side
+        // is read element by element
         const T* in = staged + head + tid * W;
-#pragma unroll 4
-        for (unsigned g = tid; g < nvec; g += nthreads, in += nthreads * W, out += nthreads) {
+        unsigned g = tid;
+        if constexpr (UNROLL > 1) {
+            for (; g + (UNROLL - 1) * nthreads < nvec;
+                 g += UNROLL * nthreads, in += UNROLL * nthreads * W, out += UNROLL * nthreads) {
+                V v[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+#pragma unroll
+                    for (unsigned e = 0; e < W; ++e) v[u][e] = in[u * nthreads * W + e];
+                }
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) emit<T, STREAMING>(v[u], out + u * nthreads);
+            }
+        }
+        for (; g < nvec; g += nthreads, in += nthreads * W, out += nthreads) {
             V v;
 #pragma unroll
             for (unsigned e = 0; e < W; ++e) {

@@ -33,6 +33,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <type_traits>
 
 #include "../../include/sphx_launch.h"
 #include "sphx_device.hpp"
@@ -63,10 +64,16 @@ struct Tiling {
     int ny;                 // (l_max + 1)^2: length of one component row in HBM
     int tile;               // points whose rows are staged in LDS at a time
     unsigned magic_jobs;    // ceil(2^32 / jobs_per_point)
-    unsigned jobs_per_point; // (l, m >= 0) pairs above the closed-form limit
+    unsigned jobs_per_point; // entry jobs per point: (l, m >= 0) pairs above the closed-form
+                             // limit, or (l, m, side) triples when the sides are split
     unsigned sequence_waves; // waves that run the bare recursions (1 or 2)
-    // LDS carve-up, in elements of T from the start of dynamic LDS
-    unsigned off_dsph, off_ddsph, off_F, off_Q, off_pts, off_iter, off_jobs;
+    unsigned points_per_pass; // points whose entry jobs fit side by side in the wide waves (>= 1)
+    unsigned row_buffers;   // 2: tile n is flushed while tile n+1 is computed; 1: one after the other
+    unsigned flush_waves;   // waves that do nothing but flush (row_buffers == 2)
+    // LDS carve-up, in elements of T: the row buffers come first, rows_elems each, with the
+    // gradient and second-derivative rows at off_dsph and off_ddsph inside a buffer; the other
+    // offsets count from the start of dynamic LDS
+    unsigned rows_elems, off_dsph, off_ddsph, off_F, off_Q, off_pts, off_iter, off_jobs;
 };
 
 extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -75,6 +82,11 @@ extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 // non-temporal hint (measured 10-20 % faster than plain stores here).
 #ifndef SPHX_STREAMING_STORES
 #define SPHX_STREAMING_STORES true
+#endif
+
+// LDS loads a flushing wave of the recursion kernel keeps in flight
+#ifndef SPHX_FLUSH_UNROLL
+#define SPHX_FLUSH_UNROLL 4
 #endif
 
 __host__ __device__ constexpr unsigned magic_of(unsigned long long divisor) {
@@ -200,24 +212,32 @@ __global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __re
 
 // ---------------------------------------------------------------------------
 // l > H through the recursion. 512 threads, persistent workgroups that walk
-// over tiles of `tile` consecutive points, three tiles in flight per workgroup:
+// over tiles of `tile` consecutive points, four tiles in flight per workgroup,
+// every wave with a role of its own and one barrier per tile:
 //
 //   wave 0       tile i+2, one lane per point: normalised coordinates, c_m,
 //                s_m, 2(m+1)z into LDS (azimuth_job);
 //   wave 1 (, 2) tile i+1, one lane per (point, l, sequence): the bare Q recursions,
 //                every iterate into LDS (sequence_job);
-//   the others   tile i, one job per (point, l, m >= 0): the entries (l, +-m) of
+//   entry waves  tile i, one job per (point, l, m >= 0): the entries (l, +-m) of
 //                every requested array, chain rule included, staged in LDS in
 //                HBM layout (entry_job). Neighbouring lanes take neighbouring m
 //                of one (point, l), so their LDS traffic falls on neighbouring
 //                banks;
-//   all waves    stream the staged rows of tile i to HBM with 16-byte stores.
+//   flush waves  tile i-1: stream its staged rows to HBM with 16-byte stores.
 //
 // The first two stages are short chains of dependent operations that only a
 // few lanes can share; running them one and two tiles ahead of the wide stage
-// takes them off the critical path. The point tables are kept in three
-// buffers, the iterates in two; the staged rows, by far the largest part of
-// LDS, exist once.
+// takes them off the critical path. The last stage is bound by HBM, the entry
+// stage by the vector ALUs: side by side, neither waits for the other. The
+// point tables are kept in three buffers, the iterates and the staged rows in
+// two. When the rows of a single point are too long for two row buffers there
+// is one, no wave is set aside for flushing, and all waves flush tile i after
+// a second barrier.
+//
+// SPLIT == true (second derivatives, so few points per tile that the (l, m)
+// pairs of a tile leave lanes idle): the entries (l, +m) and (l, -m) are two
+// jobs.
 //
 // WHOLE == true: the closed forms of l <= H are evaluated here too (one lane
 // per point) and the tile's rows are complete, one contiguous run per array.
@@ -226,7 +246,7 @@ __global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __re
 // ---------------------------------------------------------------------------
 constexpr unsigned kRecursionThreads = 512;
 
-template <typename T, int MODE, bool NORM, bool WHOLE>
+template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT>
 __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, const T* __restrict__ xyz,
                                                                      T* __restrict__ sph,
                                                                      T* __restrict__ dsph,
@@ -258,19 +278,25 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         }
         // (l, m) pairs: the bulk 1 <= m <= l - 2 first, then the special cases m = l, l - 1 and
         // 0 each as one block, so that the lanes of a wave mostly share one branch of entry_job
-        // one word per job: m in bits 0-7, l in bits 8-15, l(l+1)/2 above
-        auto pack = [](int l, int m) -> unsigned {
+        // one word per job: m in bits 0-6, the side in bit 7, l in bits 8-15, l(l+1)/2 above
+        auto pack = [](int l, int m, int side) -> unsigned {
             return (static_cast<unsigned>(l * (l + 1) / 2) << 16) | (static_cast<unsigned>(l) << 8) |
-                   static_cast<unsigned>(m);
+                   (static_cast<unsigned>(side) << 7) | static_cast<unsigned>(m);
         };
         if (tid == 0) {
             unsigned n = 0;
-            for (int l = L; l > H; --l) {
-                for (int m = l - 2; m >= 1; --m) job_table[n++] = pack(l, m);
+            for (int side = 0; side < (SPLIT ? 2 : 1); ++side) {
+                for (int l = L; l > H; --l) {
+                    for (int m = l - 2; m >= 1; --m) job_table[n++] = pack(l, m, side);
+                }
             }
-            for (int l = L; l > H; --l) job_table[n++] = pack(l, l);
-            for (int l = L; l > H; --l) job_table[n++] = pack(l, l - 1);
-            for (int l = L; l > H; --l) job_table[n++] = pack(l, 0);
+            for (int side = 0; side < (SPLIT ? 2 : 1); ++side) {
+                for (int l = L; l > H; --l) job_table[n++] = pack(l, l, side);
+            }
+            for (int side = 0; side < (SPLIT ? 2 : 1); ++side) {
+                for (int l = L; l > H; --l) job_table[n++] = pack(l, l - 1, side);
+            }
+            for (int l = L; l > H; --l) job_table[n++] = pack(l, 0, 0);
         }
     }
 
@@ -347,7 +373,7 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         const unsigned count = valid_in(n);
         const unsigned per_l = count * ARRAYS;
         const unsigned jobs = per_l * static_cast<unsigned>(L - H);
-        for (unsigned j = tid - 64; j < jobs; j += 64 * g.sequence_waves) {
+        for (unsigned j = tid - 64; j < jobs; j += 64 * g.sequence_waves) { // waves 1 .. sequence_waves
             const unsigned step = j / per_l;
             const unsigned rest = j - step * per_l;
             const int l = L - static_cast<int>(step); // longest recursions first
@@ -356,6 +382,120 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
             const T* rec = point_data(n % 3u, s);
             sequence_job<T>(l, static_cast<int>(which), rec[2], rec[7], Q, rec + 8 + 2 * (L + 1),
                             iterates(n & 1u, s, which, l));
+        }
+    };
+
+    // The waves between the sequence waves and the flush waves compute entries.
+    const bool streaming = g.row_buffers == 2;
+    const unsigned entry_first_wave = 1 + g.sequence_waves;
+    const unsigned entry_end_wave = NT / 64 - (streaming ? g.flush_waves : 0u);
+    const unsigned wide_first = 64 * entry_first_wave;
+    const unsigned wide_lanes = 64 * (entry_end_wave - entry_first_wave);
+
+    // stage three of tile n, into row buffer `buffer` (the entry waves)
+    auto entry_stage = [&](unsigned n, unsigned buffer) {
+        const unsigned valid = valid_in(n);
+        T* staged = lds + buffer * g.rows_elems;
+        const unsigned t = tid - wide_first;
+        if constexpr (WHOLE) {
+            if (t < valid) {
+                const T* rec = point_data(n % 3u, t);
+                Point<T> p;
+                p.x = rec[0];
+                p.y = rec[1];
+                p.z = rec[2];
+                p.x2 = rec[3];
+                p.y2 = rec[4];
+                p.z2 = rec[5];
+                p.ir = rec[6];
+                Rows<T> rows;
+                rows.ny = static_cast<int>(ny);
+                rows.sph = staged + t * ny;
+                rows.dsph = staged + g.off_dsph + t * 3 * ny;
+                rows.ddsph = staged + g.off_ddsph + t * 9 * ny;
+                closed_form_job<T, MODE, NORM, H>(p, rows);
+            }
+        }
+        // One pass takes the jobs of as many points as fit side by side in the wide lanes
+        // (of one point, in several rounds, when it has more jobs than there are lanes);
+        // what depends on the point only is read once per pass.
+        unsigned local = 0, e_first = t;
+        if (g.points_per_pass > 1) {
+            local = __umulhi(t, g.magic_jobs);
+            e_first = t - local * g.jobs_per_point;
+        }
+        for (unsigned s0 = 0; s0 < valid; s0 += g.points_per_pass) {
+            const unsigned s = s0 + local;
+            if (s >= valid || local >= g.points_per_pass) continue;
+            const T* rec = point_data(n % 3u, s);
+            Point<T> p;
+            p.x = rec[0];
+            p.y = rec[1];
+            p.z = rec[2];
+            p.x2 = rec[3];
+            p.y2 = rec[4];
+            p.z2 = rec[5];
+            p.ir = rec[6];
+            const T* c = rec + 8;
+            const T* sn = rec + 8 + (L + 1);
+            const T* itA = iterates(n & 1u, s, 0, 0);
+            const T* itB = iterates(n & 1u, s, MODE >= 1 ? 1 : 0, 0);
+            const T* itC = iterates(n & 1u, s, MODE == 2 ? 2 : 0, 0);
+            // rows are addressed with the entry's index in the full row; shift the bases when
+            // the staged rows start at l = H + 1
+            Rows<T> rows;
+            rows.ny = static_cast<int>(nrow);
+            rows.sph = staged + s * nrow - skip;
+            rows.dsph = staged + g.off_dsph + s * 3 * nrow - skip;
+            rows.ddsph = staged + g.off_ddsph + s * 9 * nrow - skip;
+            for (unsigned e = e_first; e < g.jobs_per_point; e += wide_lanes) {
+                const unsigned packed = job_table[e];
+                const int m = static_cast<int>(packed & 0x7fu);
+                const int side = static_cast<int>((packed >> 7) & 1u);
+                const int l = static_cast<int>((packed >> 8) & 0xffu);
+                const int tri = static_cast<int>(packed >> 16);
+                entry_job<T, MODE, NORM, SPLIT>(l, m, tri, side, p, F + tri, c, sn, itA + tri,
+                                                itB + tri, itC + tri, rows);
+            }
+        }
+    };
+
+    // last stage of tile n: row buffer `buffer` to HBM, by `count` threads of which this is
+    // number `ft`. `lone` (a std::integral_constant): the copy of a run is the work of a single
+    // wave, which then keeps several LDS loads in flight; with all waves of the workgroup on one
+    // run, loads and stores alternating one by one measured faster.
+    auto flush_stage = [&](unsigned n, unsigned buffer, unsigned ft, unsigned count, auto lone) {
+        constexpr int WHOLE_UNROLL = decltype(lone)::value ? SPHX_FLUSH_UNROLL : 1;
+        const unsigned valid = valid_in(n);
+        const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
+        const T* staged = lds + buffer * g.rows_elems;
+        if constexpr (WHOLE) {
+            copy_out<T, SPHX_STREAMING_STORES, false, WHOLE_UNROLL>(staged, sph + first * ny, valid * ny, ny, 0, 0, ft,
+                                                      count);
+            if constexpr (MODE >= 1) {
+                copy_out<T, SPHX_STREAMING_STORES, false, WHOLE_UNROLL>(staged + g.off_dsph, dsph + first * 3 * ny,
+                                                          valid * 3 * ny, 3 * ny, 0, 0, ft, count);
+            }
+            if constexpr (MODE == 2) {
+                copy_out<T, SPHX_STREAMING_STORES, false, WHOLE_UNROLL>(staged + g.off_ddsph, ddsph + first * 9 * ny,
+                                                          valid * 9 * ny, 9 * ny, 0, 0, ft, count);
+            }
+        } else {
+            // one run per (point, component) row, dealt to the waves in turn
+            const unsigned waves = count / 64;
+            for (unsigned r = ft >> 6; r < valid * components_of(MODE); r += waves) {
+                // rows [0, valid) are values, the next 3 * valid are gradients
+                if (r < valid) {
+                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL>(staged + r * nrow,
+                                                              sph + (first + r) * ny + skip, nrow, nrow,
+                                                              0, 0, ft & 63u, 64);
+                } else {
+                    const unsigned q = r - valid;
+                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL>(staged + g.off_dsph + q * nrow,
+                                                              dsph + (first * 3 + q) * ny + skip, nrow,
+                                                              nrow, 0, 0, ft & 63u, 64);
+                }
+            }
         }
     };
 
@@ -370,102 +510,46 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
     if (wave == 0) {
         azimuth_stage(1, rx, ry, rz);
         fetch(2, rx, ry, rz);
-    } else if (wave <= g.sequence_waves) {
+    } else if (wave < entry_first_wave) {
         recursion_stage(0);
     }
 
-    for (unsigned n = 0; valid_in(n) != 0; ++n) {
-        const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
-        const unsigned valid = valid_in(n);
-
-        __syncthreads(); // tables of tile n+1, iterates of tile n in place; rows of tile n-1 flushed
-
-        if (wave == 0) {
-            azimuth_stage(n + 2, rx, ry, rz);
-            fetch(n + 3, rx, ry, rz); // needed one round from now
-        } else if (wave <= g.sequence_waves) {
-            recursion_stage(n + 1);
-        } else {
-            const unsigned wide_first = 64 * (1 + g.sequence_waves);
-            const unsigned t = tid - wide_first;
-            if constexpr (WHOLE) {
-                if (t < valid) {
-                    const T* rec = point_data(n % 3u, t);
-                    Point<T> p;
-                    p.x = rec[0];
-                    p.y = rec[1];
-                    p.z = rec[2];
-                    p.x2 = rec[3];
-                    p.y2 = rec[4];
-                    p.z2 = rec[5];
-                    p.ir = rec[6];
-                    Rows<T> rows;
-                    rows.ny = static_cast<int>(ny);
-                    rows.sph = lds + t * ny;
-                    rows.dsph = lds + g.off_dsph + t * 3 * ny;
-                    rows.ddsph = lds + g.off_ddsph + t * 9 * ny;
-                    closed_form_job<T, MODE, NORM, H>(p, rows);
-                }
-            }
-            for (unsigned s = 0; s < valid; ++s) {
-                const T* rec = point_data(n % 3u, s);
-                Point<T> p;
-                p.x = rec[0];
-                p.y = rec[1];
-                p.z = rec[2];
-                p.x2 = rec[3];
-                p.y2 = rec[4];
-                p.z2 = rec[5];
-                p.ir = rec[6];
-                const T* c = rec + 8;
-                const T* sn = rec + 8 + (L + 1);
-                const T* itA = iterates(n & 1u, s, 0, 0);
-                const T* itB = iterates(n & 1u, s, MODE >= 1 ? 1 : 0, 0);
-                const T* itC = iterates(n & 1u, s, MODE == 2 ? 2 : 0, 0);
-                // rows are addressed with the entry's index in the full row; shift the bases when
-                // the staged rows start at l = H + 1
-                Rows<T> rows;
-                rows.ny = static_cast<int>(nrow);
-                rows.sph = lds + s * nrow - skip;
-                rows.dsph = lds + g.off_dsph + s * 3 * nrow - skip;
-                rows.ddsph = lds + g.off_ddsph + s * 9 * nrow - skip;
-                for (unsigned e = t; e < g.jobs_per_point; e += NT - wide_first) {
-                    const unsigned packed = job_table[e];
-                    const int m = static_cast<int>(packed & 0xffu);
-                    const int l = static_cast<int>((packed >> 8) & 0xffu);
-                    const int tri = static_cast<int>(packed >> 16);
-                    entry_job<T, MODE, NORM>(l, m, tri, p, F + tri, c, sn, itA + tri, itB + tri,
-                                             itC + tri, rows);
-                }
+    if (streaming) {
+        // Two row buffers: while the entry waves fill one with tile n, the flush waves send the
+        // other, tile n - 1, to HBM; one barrier per tile, and the stores never pause for the
+        // arithmetic. One more round after the last tile flushes it.
+        for (unsigned n = 0;; ++n) {
+            __syncthreads(); // tables of tile n+1, iterates of tile n, rows of tile n-1 complete
+            const unsigned valid = valid_in(n);
+            const unsigned before = n > 0 ? valid_in(n - 1) : 0u;
+            if (valid == 0 && before == 0) break;
+            if (wave == 0) {
+                azimuth_stage(n + 2, rx, ry, rz);
+                fetch(n + 3, rx, ry, rz); // needed one round from now
+            } else if (wave < entry_first_wave) {
+                recursion_stage(n + 1);
+            } else if (wave < entry_end_wave) {
+                if (valid != 0) entry_stage(n, n & 1u);
+            } else if (before != 0) {
+                flush_stage(n - 1, (n - 1) & 1u, tid - 64 * entry_end_wave, 64 * g.flush_waves,
+                            std::true_type{});
             }
         }
-        __syncthreads(); // rows of tile n complete
-
-        if constexpr (WHOLE) {
-            copy_out<T, SPHX_STREAMING_STORES, false>(lds, sph + first * ny, valid * ny, ny, 0, 0, tid, NT);
-            if constexpr (MODE >= 1) {
-                copy_out<T, SPHX_STREAMING_STORES, false>(lds + g.off_dsph, dsph + first * 3 * ny,
-                                                   valid * 3 * ny, 3 * ny, 0, 0, tid, NT);
+    } else {
+        // One row buffer (the rows of one point fill most of LDS): every wave takes part in the
+        // flush, after a second barrier.
+        for (unsigned n = 0; valid_in(n) != 0; ++n) {
+            __syncthreads(); // tables of tile n+1, iterates of tile n in place; rows of tile n-1 flushed
+            if (wave == 0) {
+                azimuth_stage(n + 2, rx, ry, rz);
+                fetch(n + 3, rx, ry, rz);
+            } else if (wave < entry_first_wave) {
+                recursion_stage(n + 1);
+            } else {
+                entry_stage(n, 0);
             }
-            if constexpr (MODE == 2) {
-                copy_out<T, SPHX_STREAMING_STORES, false>(lds + g.off_ddsph, ddsph + first * 9 * ny,
-                                                          valid * 9 * ny, 9 * ny, 0, 0, tid, NT);
-            }
-        } else {
-            // one run per (point, component) row, dealt to the waves in turn
-            constexpr unsigned NW = NT / 64;
-            for (unsigned r = wave; r < valid * components_of(MODE); r += NW) {
-                // rows [0, valid) are values, the next 3 * valid are gradients
-                if (r < valid) {
-                    copy_out<T, SPHX_STREAMING_STORES, false>(lds + r * nrow, sph + (first + r) * ny + skip, nrow,
-                                                       nrow, 0, 0, lane, 64);
-                } else {
-                    const unsigned q = r - valid;
-                    copy_out<T, SPHX_STREAMING_STORES, false>(lds + g.off_dsph + q * nrow,
-                                                       dsph + (first * 3 + q) * ny + skip, nrow, nrow, 0,
-                                                       0, lane, 64);
-                }
-            }
+            __syncthreads(); // rows of tile n complete
+            flush_stage(n, 0, tid, NT, std::false_type{});
         }
     }
 }
@@ -536,6 +620,7 @@ struct Plan {
     bool closed_only; // l_max within the closed forms: one launch of closed_form_kernel
     bool whole;       // recursion_kernel evaluates the closed forms too: one launch
                       // otherwise closed_form_kernel<PREFIX> + recursion_kernel: two launches
+    bool split_sides; // recursion_kernel takes the entries (l, +m) and (l, -m) as two jobs
     Launch closed;
     Launch rec;
 };
@@ -570,10 +655,11 @@ static void plan_closed(size_t n_samples, int l_max, int hard, int mode, size_t 
 
 // Tile size and LDS layout of the recursion kernel. Returns false when not even one point fits.
 static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, size_t elem,
-                           unsigned budget, int lds_limit, int cus, Launch* out) {
+                           unsigned budget, int lds_limit, int cus, Launch* out, bool* split_sides) {
     Tiling& g = out->g;
     std::memset(&g, 0, sizeof(g));
     const int hard = mode == 2 ? 1 : 6;
+    const unsigned esize = static_cast<unsigned>(elem);
     const unsigned ny = static_cast<unsigned>(l_max + 1) * (l_max + 1);
     const unsigned nyh = static_cast<unsigned>(hard + 1) * (hard + 1);
     const unsigned nrow = whole ? ny : ny - nyh;
@@ -581,19 +667,46 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     const unsigned arrays = mode + 1;
     unsigned jobs = 0;
     for (int l = hard + 1; l <= l_max; ++l) jobs += l + 1;
-    // rows once, point tables three times, iterates twice (see recursion_kernel)
-    const unsigned per_point =
-        components_of(mode) * nrow + 3 * (8 + 3 * (l_max + 1)) + 2 * arrays * tri_all;
-    const unsigned fixed = 2 * tri_all + (jobs * 4 + static_cast<unsigned>(elem) - 1) / static_cast<unsigned>(elem) + 16;
-    auto bytes_for = [&](unsigned S) { return (S * per_point + fixed) * static_cast<unsigned>(elem); };
-    if (bytes_for(1) > static_cast<unsigned>(lds_limit)) return false;
+    // with the sides split every (l, m > 0) pair is two jobs; the job table is sized for that
+    const unsigned jobs_split = 2 * jobs - static_cast<unsigned>(l_max - hard);
+    bool may_split = mode == 2 && env_int("SPHX_SPLIT_SIDES", 1) != 0;
+    auto table_elems_for = [&](bool split) { return ((split ? jobs_split : jobs) * 4 + esize - 1) / esize; };
+    // per point: the rows in every row buffer, point tables three times, iterates twice
+    const unsigned rows_per_point = components_of(mode) * nrow;
+    const unsigned rest_per_point = 3 * (8 + 3 * (l_max + 1)) + 2 * arrays * tri_all;
+    unsigned fixed = 0;
+    auto bytes_for = [&](unsigned S, unsigned buffers) {
+        return (S * (buffers * rows_per_point + rest_per_point) + fixed) * esize;
+    };
+    const unsigned limit = static_cast<unsigned>(lds_limit);
+    for (;;) {
+        // 24: alignment slack of the row arrays
+        fixed = 2 * tri_all + table_elems_for(may_split) + 24;
+        if (bytes_for(1, 1) <= limit || !may_split) break;
+        may_split = false; // the longer job table is what does not fit
+    }
+    // Two row buffers (tile n flushed by a wave of its own while tile n+1 is computed) pay off
+    // where the rows of a point are so long that a single buffer holds one or two points and
+    // the flush of such a tile is long: measured with second derivatives (l_max = 16, float64:
+    // 770 us against 810 us). With many points per tile, or with the rows cut in two kernels,
+    // one buffer flushed by all waves measured faster.
+    int want_buffers = env_int("SPHX_ROW_BUFFERS", 0);
+    if (want_buffers == 0) {
+        const unsigned single = bytes_for(1, 1) <= budget
+                                    ? (budget / esize - fixed) / (rows_per_point + rest_per_point)
+                                    : 1u;
+        want_buffers = mode == 2 && single <= 2 ? 2 : 1;
+    }
+    unsigned buffers = want_buffers == 2 ? 2u : 1u;
+    if (bytes_for(1, buffers) > limit) buffers = 1;
+    if (bytes_for(1, buffers) > limit) return false;
     unsigned S = 1;
-    if (bytes_for(1) <= budget) {
-        S = pow2_floor((budget / static_cast<unsigned>(elem) - fixed) / per_point);
+    if (bytes_for(1, buffers) <= budget) {
+        S = pow2_floor((budget / esize - fixed) / (buffers * rows_per_point + rest_per_point));
         if (S > 64) S = 64;
     }
     const int forced = env_int("SPHX_TILE", 0);
-    if (forced > 0 && forced <= 64 && bytes_for(forced) <= static_cast<unsigned>(lds_limit)) {
+    if (forced > 0 && forced <= 64 && bytes_for(forced, buffers) <= limit) {
         S = static_cast<unsigned>(forced);
     }
 
@@ -601,14 +714,30 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.l_max = l_max;
     g.ny = static_cast<int>(ny);
     g.tile = static_cast<int>(S);
-    g.jobs_per_point = jobs;
-    g.magic_jobs = magic_of(jobs);
+    g.row_buffers = buffers;
+    g.flush_waves = buffers == 2 ? static_cast<unsigned>(env_int("SPHX_FLUSH_WAVES", 1)) : 0u;
+    if (g.flush_waves > 2) g.flush_waves = 2;
+    if (buffers == 2 && g.flush_waves < 1) g.flush_waves = 1;
     g.sequence_waves = S * arrays * static_cast<unsigned>(l_max - hard) > 64 ? 2u : 1u;
+    // Split the sides when that lets the entries of a tile go through the entry waves in fewer
+    // rounds than it costs: a one-sided job is about 0.6 of a two-sided one.
+    const unsigned wide = kRecursionThreads - 64 * (1 + g.sequence_waves + g.flush_waves);
+    auto per_pass = [&](unsigned j) { return j >= wide ? 1u : wide / j; };
+    auto rounds = [&](unsigned j) {
+        return ((S + per_pass(j) - 1) / per_pass(j)) * ((j + wide - 1) / wide);
+    };
+    *split_sides = may_split && 6 * rounds(jobs_split) < 10 * rounds(jobs);
+    g.jobs_per_point = *split_sides ? jobs_split : jobs;
+    g.magic_jobs = magic_of(g.jobs_per_point);
+    g.points_per_pass = per_pass(g.jobs_per_point);
+
     unsigned at = align4(S * nrow);
     g.off_dsph = at;
     if (mode >= 1) at = align4(at + S * 3 * nrow);
     g.off_ddsph = at;
     if (mode == 2) at = align4(at + S * 9 * nrow);
+    g.rows_elems = at;
+    at *= buffers;
     g.off_F = at;
     at += tri_all;
     g.off_Q = at;
@@ -618,13 +747,14 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.off_iter = at;
     at += 2 * S * arrays * tri_all;
     g.off_jobs = at;
-    at += (jobs * 4 + static_cast<unsigned>(elem) - 1) / static_cast<unsigned>(elem);
-    out->lds_bytes = at * static_cast<unsigned>(elem);
+    at += table_elems_for(may_split);
+    out->lds_bytes = at * esize;
     out->threads = kRecursionThreads;
+    if (out->lds_bytes > limit) return false;
 
     g.n_tiles = static_cast<unsigned>((n_samples + S - 1) / S);
     g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
-    unsigned per_cu = static_cast<unsigned>(lds_limit) / out->lds_bytes;
+    unsigned per_cu = limit / out->lds_bytes;
     if (per_cu < 1) per_cu = 1;
     if (per_cu > 4) per_cu = 4; // 512 threads each: 2048 lanes per CU
     unsigned want = (static_cast<unsigned>(cus) * per_cu + 7u) & ~7u;
@@ -650,21 +780,24 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     const int hard = mode == 2 ? 1 : 6;
     plan->closed_only = l_max <= hard;
     plan->whole = true;
+    plan->split_sides = false;
     if (plan->closed_only) {
         plan_closed(n_samples, l_max, l_max, mode, elem, &plan->closed);
         return SPHX_OK;
     }
     const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", 76 * 1024));
-    bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec);
+    bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
+                               &plan->split_sides);
     // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of
     // a wave idle for a thousand instructions per tile: hand them to the closed-form kernel,
     // which runs them 64 points at a time, and let the recursion kernel stage l >= 7 only.
     const int split_below = env_int("SPHX_SPLIT_BELOW", 16);
     if (mode < 2 && (!fits || plan->rec.g.tile < split_below)) {
-        Launch split;
-        if (plan_recursion(n_samples, l_max, mode, false, elem, budget, lds_limit, cus, &split)) {
+        Launch upper;
+        if (plan_recursion(n_samples, l_max, mode, false, elem, budget, lds_limit, cus, &upper,
+                           &plan->split_sides)) {
             plan->whole = false;
-            plan->rec = split;
+            plan->rec = upper;
             plan_closed(n_samples, l_max, hard, mode, elem, &plan->closed);
             fits = true;
         }
@@ -693,10 +826,10 @@ static hipError_t launch_closed(const Launch& l, const T* xyz, T* sph, T* dsph, 
     return hipGetLastError();
 }
 
-template <typename T, int MODE, bool NORM, bool WHOLE>
+template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT>
 static hipError_t launch_recursion(const Launch& l, const T* xyz, T* sph, T* dsph, T* ddsph,
                                    hipStream_t stream) {
-    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE>;
+    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT>;
     if (l.lds_bytes > 64u * 1024u) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -726,15 +859,18 @@ static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* d
                            hipStream_t stream) {
     if (!plan.closed_only) {
         if constexpr (MODE == 2) {
-            return launch_recursion<T, MODE, NORM, true>(plan.rec, xyz, sph, dsph, ddsph, stream);
+            if (plan.split_sides) {
+                return launch_recursion<T, MODE, NORM, true, true>(plan.rec, xyz, sph, dsph, ddsph, stream);
+            }
+            return launch_recursion<T, MODE, NORM, true, false>(plan.rec, xyz, sph, dsph, ddsph, stream);
         } else {
             if (plan.whole) {
-                return launch_recursion<T, MODE, NORM, true>(plan.rec, xyz, sph, dsph, ddsph, stream);
+                return launch_recursion<T, MODE, NORM, true, false>(plan.rec, xyz, sph, dsph, ddsph, stream);
             }
             // the two kernels write disjoint parts of every row
             hipError_t e = launch_closed<T, MODE, NORM, 6, true>(plan.closed, xyz, sph, dsph, ddsph, stream);
             if (e != hipSuccess) return e;
-            return launch_recursion<T, MODE, NORM, false>(plan.rec, xyz, sph, dsph, ddsph, stream);
+            return launch_recursion<T, MODE, NORM, false, false>(plan.rec, xyz, sph, dsph, ddsph, stream);
         }
     }
     const Launch& l = plan.closed;
