@@ -61,6 +61,13 @@ def parse():
         "memory and fabric clocks of an idle MI355X take tens of milliseconds of load to ramp up "
         "(the same launch takes 160 us right after idle and 136 us once settled)",
     )
+    p.add_argument(
+        "--op",
+        choices=("forward", "backward"),
+        default="forward",
+        help="backward: time the vector-Jacobian product xyz_grad = sum_k dsph * sph_grad "
+        "(sphx_backward_*) on the gradients of the workload instead of the forward pass",
+    )
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument(
         "--calibrate-copy",
@@ -116,6 +123,26 @@ def cpu_baseline(workload, xyz):
     }
 
 
+def cpu_backward_baseline(dsph, sph_grad):
+    """The checker's contraction loop, one thread, timed on a bounded slice of the points."""
+    import oracle  # reported baseline only
+
+    n = min(dsph.shape[0], 200_000)
+    best = None
+    for _ in range(5):
+        t0 = time.perf_counter()
+        oracle.backward(dsph[:n], sph_grad[:n])
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return {
+        "value": n / best,
+        "unit": "points/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"5 passes over the first {n} points, best pass {best * 1e3:.2f} ms; plain C loop, one thread",
+    }
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -159,6 +186,26 @@ def main():
         if status != 0:
             raise RuntimeError(lib.sphx_last_error().decode())
 
+    bytes_per_launch = w.bytes_per_point * n
+    if args.op == "backward":
+        if mode < 1:
+            print("--op backward needs a workload with gradients", file=sys.stderr)
+            return 2
+        step()  # fill dsph
+        torch.manual_seed(w.seed)
+        sph_grad = torch.randn((n, ny), **opts)
+        xyz_grad = torch.empty((n, 3), **opts)
+        backward = lib.sphx_backward_f32 if w.dtype == "f32" else lib.sphx_backward_f64
+        backward_args = (dsph.data_ptr(), sph_grad.data_ptr(), n, ny, xyz_grad.data_ptr(), 0, stream.cuda_stream)
+
+        def step():  # noqa: F811
+            status = backward(*backward_args)
+            if status != 0:
+                raise RuntimeError(lib.sphx_last_error().decode())
+
+        # reads dsph and sph_grad once, writes three numbers per point
+        bytes_per_launch = xyz.element_size() * n * (4 * ny + 3)
+
     if args.calibrate_copy:
         nbytes = w.bytes_per_point * n
         src = torch.zeros(nbytes // 4, dtype=torch.float32, device=xyz.device)
@@ -199,13 +246,12 @@ def main():
 
     launch_ms = [b.elapsed_time(e) for b, e in events]
     avg_launch_s = sum(launch_ms) / len(launch_ms) / 1e3
-    bytes_per_launch = w.bytes_per_point * n
     achieved = bytes_per_launch / avg_launch_s / 1e9
 
     result = {
         "metric": "points/sec + achieved HBM GB/s (% peak), l_max=6 fp32 w/ gradients, 1M pts"
-        if args.workload == "cfg3"
-        else f"points/sec + achieved HBM GB/s (% peak), {w.description}",
+        if args.workload == "cfg3" and args.op == "forward"
+        else f"points/sec + achieved HBM GB/s (% peak), {args.op} pass, {w.description}",
         "value": n * args.steps / wall,
         "unit": "points/s",
         "n_gpus": 1,
@@ -219,6 +265,7 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": f"{w.name}: {w.description}",
+            "op": args.op,
             "settle_seconds": args.settle_seconds,
             "l_max": w.l_max,
             "n_samples": n,
@@ -232,7 +279,7 @@ def main():
             "peak": PEAK_HBM_GBPS,
             "unit": "GB/s",
             "frac": achieved / PEAK_HBM_GBPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.op == "forward" else None,
             "algorithmic_bytes_per_launch": bytes_per_launch,
             "avg_launch_us": avg_launch_s * 1e6,
             "median_launch_us": statistics.median(launch_ms) * 1e3,
@@ -240,7 +287,10 @@ def main():
         },
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(w, xyz_host)
+        if args.op == "forward":
+            result["cpu_baseline"] = cpu_baseline(w, xyz_host)
+        else:
+            result["cpu_baseline"] = cpu_backward_baseline(dsph.cpu().numpy(), sph_grad.cpu().numpy())
     print(json.dumps(result))
     return 0
 

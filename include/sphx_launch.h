@@ -57,6 +57,42 @@ SPHX_EXPORT int sphx_forward_f64(const double* xyz, size_t n_samples, int l_max,
                                  int derivatives, double* sph, double* dsph, double* ddsph,
                                  void* stream);
 
+/* Vector-Jacobian product of the forward pass for reverse-mode callers:
+ *
+ *   xyz_grad[i][a] (+)= sum_k dsph[i][a][k] * sph_grad[i][k]
+ *
+ *   dsph      device, [n_samples][3][n_total]   (as written by sphx_forward_*)
+ *   sph_grad  device, [n_samples][n_total]      gradient of the caller's scalar w.r.t. sph
+ *   xyz_grad  device, [n_samples][3]
+ *   n_total   row length, (l_max+1)^2
+ *   accumulate  0: overwrite xyz_grad; otherwise add to what it holds
+ *
+ * Enqueued on `stream` like the forward pass; n_samples == 0 returns SPHX_OK.
+ * Replaces spherical_harmonics_backward_cuda_base<T>
+ * (sphericart/src/cuda_base.cpp:156-183) and its backward_kernel
+ * (sphericart/src/sphericart_impl.cu:650-684); same arguments plus `accumulate`. */
+SPHX_EXPORT int sphx_backward_f32(const float* dsph, const float* sph_grad, size_t n_samples,
+                                  int n_total, float* xyz_grad, int accumulate, void* stream);
+SPHX_EXPORT int sphx_backward_f64(const double* dsph, const double* sph_grad, size_t n_samples,
+                                  int n_total, double* xyz_grad, int accumulate, void* stream);
+
+/* The same one order up, for callers that differentiate through the gradients:
+ *
+ *   xyz_grad[i][b] (+)= sum_a sum_k ddsph[i][a][b][k] * dsph_grad[i][a][k]
+ *
+ *   ddsph      device, [n_samples][3][3][n_total]
+ *   dsph_grad  device, [n_samples][3][n_total]   gradient of the caller's scalar w.r.t. dsph
+ *
+ * The reference has no kernel for this; its torch binding evaluates it as
+ * torch.sum(grad.unsqueeze(2) * ddsph, dim=(1, 3))
+ * (sphericart-torch/python/sphericart/torch/register.py:106-110). */
+SPHX_EXPORT int sphx_backward_second_f32(const float* ddsph, const float* dsph_grad,
+                                         size_t n_samples, int n_total, float* xyz_grad,
+                                         int accumulate, void* stream);
+SPHX_EXPORT int sphx_backward_second_f64(const double* ddsph, const double* dsph_grad,
+                                         size_t n_samples, int n_total, double* xyz_grad,
+                                         int accumulate, void* stream);
+
 /* Host copy of the prefactor table the kernels use for this l_max: the F_l^m
  * block followed by the Q_l^m-recursion block, (l_max+1)(l_max+2) numbers.
  * Replaces compute_sph_prefactors<T> (sphericart/include/templates.hpp:54-97)

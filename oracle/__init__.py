@@ -70,6 +70,11 @@ def _lib(flavour):
         fn = getattr(lib, f"{pre}_prefactors_{suffix}")
         fn.restype = None
         fn.argtypes = [ctypes.c_int, ptr]
+        if flavour == "oracle":
+            for name in ("backward", "backward_second"):
+                fn = getattr(lib, f"{pre}_{name}_{suffix}")
+                fn.restype = None
+                fn.argtypes = [ptr, ptr, ctypes.c_size_t, ctypes.c_int, ptr]
     getattr(lib, f"{pre}_max_threads").restype = ctypes.c_int
     _LIBS[flavour] = lib
     return lib
@@ -139,3 +144,33 @@ def recursion_route(xyz, l_max, normalized, mode="values", flavour="oracle"):
     if status != 0:
         raise RuntimeError(f"{flavour} recursion route failed with status {status}")
     return sph, dsph
+
+
+def backward(dsph, sph_grad):
+    """``xyz_grad[i, a] = sum_k dsph[i, a, k] * sph_grad[i, k]`` in the arrays' precision."""
+    dsph = np.ascontiguousarray(dsph)
+    sph_grad = np.ascontiguousarray(sph_grad, dtype=dsph.dtype)
+    suffix, ct = _suffix(dsph.dtype)
+    n, three, n_total = dsph.shape
+    if three != 3 or sph_grad.shape != (n, n_total):
+        raise ValueError("dsph must be N x 3 x n_total and sph_grad N x n_total")
+    out = np.empty((n, 3), dtype=dsph.dtype)
+    getattr(_lib("oracle"), f"sphx_oracle_backward_{suffix}")(
+        _ptr(dsph, ct), _ptr(sph_grad, ct), n, n_total, _ptr(out, ct)
+    )
+    return out
+
+
+def backward_second(ddsph, dsph_grad):
+    """``xyz_grad[i, b] = sum_a sum_k ddsph[i, a, b, k] * dsph_grad[i, a, k]``."""
+    ddsph = np.ascontiguousarray(ddsph)
+    dsph_grad = np.ascontiguousarray(dsph_grad, dtype=ddsph.dtype)
+    suffix, ct = _suffix(ddsph.dtype)
+    n, n_total = ddsph.shape[0], ddsph.shape[3]
+    if ddsph.shape[1:3] != (3, 3) or dsph_grad.shape != (n, 3, n_total):
+        raise ValueError("ddsph must be N x 3 x 3 x n_total and dsph_grad N x 3 x n_total")
+    out = np.empty((n, 3), dtype=ddsph.dtype)
+    getattr(_lib("oracle"), f"sphx_oracle_backward_second_{suffix}")(
+        _ptr(ddsph, ct), _ptr(dsph_grad, ct), n, n_total, _ptr(out, ct)
+    )
+    return out

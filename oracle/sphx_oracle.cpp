@@ -20,13 +20,18 @@
 //   one_sample()          sphericart/include/templates.hpp:99-267,333-615
 //   hardcoded_limit()     sphericart/src/sphericart.cpp:45-92,428-475
 //   many_samples()        sphericart/include/templates.hpp:269-331,617-710
+//   backward()            sphericart/src/sphericart_impl.cu:650-684 (the sum it forms; the
+//                         reference adds in sub-warp order, this loop in index order)
+//   backward_second()     sphericart-torch/python/sphericart/torch/register.py:106-110
 //
 // Pinned by (tests/test_oracle_*.py): closed-form prefactors, scipy's
 // sph_harm_y up to l = 20, the Unsold sum rule, finite differences, Euler
 // homogeneity, harmonicity and symmetry of the Hessian, the +-z axis values,
 // the hardcoded-vs-recursion route check, bit-for-bit comparison with the
 // compiled reference (oracle/_ref) where that is built, and the committed
-// golden vectors written by the compiled reference.
+// golden vectors written by the compiled reference. backward() and
+// backward_second() are dot products: pinned against numpy's einsum in extended
+// precision (tests/test_oracle_backward.py).
 
 #include <cmath>
 #include <cstddef>
@@ -737,6 +742,37 @@ int run(const T* xyz, size_t n, int L, int normalized, int mode, int hard, T* sp
 
 #undef K
 
+// xyz_grad[i][a] = sum_k dsph[i][a][k] * sph_grad[i][k]
+template <typename T>
+void backward(const T* dsph, const T* sph_grad, size_t n, int n_total, T* xyz_grad) {
+    for (size_t i = 0; i < n; ++i) {
+        for (int a = 0; a < 3; ++a) {
+            T sum = 0;
+            for (int k = 0; k < n_total; ++k) {
+                sum += dsph[(i * 3 + a) * n_total + k] * sph_grad[i * n_total + k];
+            }
+            xyz_grad[i * 3 + a] = sum;
+        }
+    }
+}
+
+// xyz_grad[i][b] = sum_a sum_k ddsph[i][a][b][k] * dsph_grad[i][a][k]
+template <typename T>
+void backward_second(const T* ddsph, const T* dsph_grad, size_t n, int n_total, T* xyz_grad) {
+    for (size_t i = 0; i < n; ++i) {
+        for (int b = 0; b < 3; ++b) {
+            T sum = 0;
+            for (int a = 0; a < 3; ++a) {
+                for (int k = 0; k < n_total; ++k) {
+                    sum += ddsph[((i * 3 + a) * 3 + b) * n_total + k] *
+                           dsph_grad[(i * 3 + a) * n_total + k];
+                }
+            }
+            xyz_grad[i * 3 + b] = sum;
+        }
+    }
+}
+
 } // namespace
 
 extern "C" {
@@ -770,6 +806,26 @@ void sphx_oracle_prefactors_f32(int l_max, float* out) { prefactors<float>(l_max
 
 int sphx_oracle_hardcoded_limit(int l_max, int with_hessians) {
     return hardcoded_limit(l_max, with_hessians != 0);
+}
+
+void sphx_oracle_backward_f64(const double* dsph, const double* sph_grad, size_t n, int n_total,
+                              double* xyz_grad) {
+    backward<double>(dsph, sph_grad, n, n_total, xyz_grad);
+}
+
+void sphx_oracle_backward_f32(const float* dsph, const float* sph_grad, size_t n, int n_total,
+                              float* xyz_grad) {
+    backward<float>(dsph, sph_grad, n, n_total, xyz_grad);
+}
+
+void sphx_oracle_backward_second_f64(const double* ddsph, const double* dsph_grad, size_t n,
+                                     int n_total, double* xyz_grad) {
+    backward_second<double>(ddsph, dsph_grad, n, n_total, xyz_grad);
+}
+
+void sphx_oracle_backward_second_f32(const float* ddsph, const float* dsph_grad, size_t n,
+                                     int n_total, float* xyz_grad) {
+    backward_second<float>(ddsph, dsph_grad, n, n_total, xyz_grad);
 }
 
 int sphx_oracle_max_threads(void) {

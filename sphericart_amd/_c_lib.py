@@ -24,6 +24,10 @@ C_API_SYMBOLS = [
 LAUNCH_SYMBOLS = [
     "sphx_forward_f32",
     "sphx_forward_f64",
+    "sphx_backward_f32",
+    "sphx_backward_f64",
+    "sphx_backward_second_f32",
+    "sphx_backward_second_f64",
     "sphx_prefactors_f32",
     "sphx_prefactors_f64",
     "sphx_device_count",
@@ -56,6 +60,10 @@ def _declare(lib):
         fn = getattr(lib, f"sphx_forward_{suffix}")
         fn.restype = c_int
         fn.argtypes = [c_void_p, c_size_t, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]
+        for name in ("sphx_backward", "sphx_backward_second"):
+            fn = getattr(lib, f"{name}_{suffix}")
+            fn.restype = c_int
+            fn.argtypes = [c_void_p, c_void_p, c_size_t, c_int, c_void_p, c_int, c_void_p]
         fn = getattr(lib, f"sphx_prefactors_{suffix}")
         fn.restype = c_int
         fn.argtypes = [c_int, c_void_p]

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBRARY = os.path.join(HERE, "libsphericart_amd.so")
 
-SOURCES = ["sphx_kernels.hip", "sphx_tables.cpp", "device_api.cpp", "capi.cpp"]
+SOURCES = ["sphx_kernels.hip", "sphx_backward.hip", "sphx_tables.cpp", "device_api.cpp", "capi.cpp"]
 
 # -ffp-contract=off: one rounding per source-level operation, on device and
 #   host alike; results then match the reference CPU evaluator built the same

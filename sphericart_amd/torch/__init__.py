@@ -1,0 +1,52 @@
+"""``torch.nn.Module`` calculators with autograd, as ``sphericart.torch`` has them.
+
+Same two classes and methods as the reference's
+sphericart-torch/python/sphericart/torch/spherical_hamonics.py (``forward``,
+``compute``, ``compute_with_gradients``, ``compute_with_hessians``, ``l_max``);
+the operators behind them are registered in :mod:`sphericart_amd.torch.ops`.
+Tensors must live on the GPU. ``omp_num_threads`` has no meaning here (there is
+no host evaluator) and is not offered.
+"""
+
+from typing import Tuple
+
+import torch
+from torch import Tensor
+
+from . import ops  # noqa: F401  (registers the operators)
+
+
+class SphericalHarmonics(torch.nn.Module):
+    """Real spherical harmonics of the directions of ``xyz`` up to ``l_max``, differentiable."""
+
+    _prefix = "spherical_harmonics"
+
+    def __init__(self, l_max: int):
+        super().__init__()
+        if l_max < 0:
+            raise ValueError("l_max must be non-negative")
+        self._l_max = int(l_max)
+
+    def forward(self, xyz: Tensor) -> Tensor:
+        return getattr(torch.ops.sphericart_amd, self._prefix)(xyz, self._l_max)
+
+    def compute(self, xyz: Tensor) -> Tensor:
+        return self.forward(xyz)
+
+    def compute_with_gradients(self, xyz: Tensor) -> Tuple[Tensor, Tensor]:
+        return getattr(torch.ops.sphericart_amd, f"{self._prefix}_with_gradients")(xyz, self._l_max)
+
+    def compute_with_hessians(self, xyz: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+        return getattr(torch.ops.sphericart_amd, f"{self._prefix}_with_hessians")(xyz, self._l_max)
+
+    def l_max(self) -> int:
+        return self._l_max
+
+
+class SolidHarmonics(SphericalHarmonics):
+    """Solid harmonics ``r^l Y_l^m`` of ``xyz`` up to ``l_max``, differentiable."""
+
+    _prefix = "solid_harmonics"
+
+
+__all__ = ["SphericalHarmonics", "SolidHarmonics"]
