@@ -68,6 +68,7 @@ struct Tiling {
                              // limit, or (l, m, side) triples when the sides are split
     unsigned sequence_waves; // waves that run the bare recursions (1 or 2)
     unsigned points_per_pass; // points whose entry jobs fit side by side in the wide waves (>= 1)
+    unsigned chunk_shift;   // a workgroup takes 2^chunk_shift consecutive tiles at a time
     unsigned row_buffers;   // 2: tile n is flushed while tile n+1 is computed; 1: one after the other
     unsigned flush_waves;   // waves that do nothing but flush (row_buffers == 2)
     // LDS carve-up, in elements of T: the row buffers come first, rows_elems each, with the
@@ -316,10 +317,18 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
     const unsigned xcd_first = xcd * g.tiles_per_xcd;
     unsigned xcd_last = xcd_first + g.tiles_per_xcd;
     if (xcd_last > g.n_tiles) xcd_last = g.n_tiles;
-    if (xcd_first + rank_in_xcd >= xcd_last) return; // whole workgroup
+    // A workgroup takes chunks of C consecutive tiles; the chunks of an XCD's workgroups lie
+    // side by side. Consecutive tiles in one workgroup share the 128-byte lines in which one
+    // ends and the next begins (see flush_run); C stays small so that what the XCD writes at any
+    // moment remains a compact window.
+    const unsigned chunk_mask = (1u << g.chunk_shift) - 1u;
+    if (xcd_first + (rank_in_xcd << g.chunk_shift) >= xcd_last) return; // whole workgroup
 
     // the n-th tile of this workgroup, and how many points it has (0 past the end)
-    auto tile_of = [&](unsigned n) -> unsigned { return xcd_first + rank_in_xcd + n * groups_per_xcd; };
+    auto tile_of = [&](unsigned n) -> unsigned {
+        return xcd_first + ((((n >> g.chunk_shift) * groups_per_xcd + rank_in_xcd)) << g.chunk_shift) +
+               (n & chunk_mask);
+    };
     auto valid_in = [&](unsigned n) -> unsigned {
         const unsigned t = tile_of(n);
         if (t >= xcd_last) return 0u;
@@ -392,11 +401,23 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
     const unsigned wide_first = 64 * entry_first_wave;
     const unsigned wide_lanes = 64 * (entry_end_wave - entry_first_wave);
 
+    constexpr unsigned LINE = 128u / static_cast<unsigned>(sizeof(T)); // elements per 128-byte line
+    // position within its 128-byte line of element `element` of an output array
+    auto phase_of = [](const T* array, unsigned long long element) -> unsigned {
+        return static_cast<unsigned>((reinterpret_cast<uintptr_t>(array) / sizeof(T) + element) % LINE);
+    };
+
     // stage three of tile n, into row buffer `buffer` (the entry waves)
     auto entry_stage = [&](unsigned n, unsigned buffer) {
         const unsigned valid = valid_in(n);
         T* staged = lds + buffer * g.rows_elems;
         const unsigned t = tid - wide_first;
+        // WHOLE: element 0 of a staging region stands for the start of the 128-byte line in
+        // which the tile's run begins in HBM, so the run itself starts `phase` elements in
+        const unsigned long long first_point = static_cast<unsigned long long>(tile_of(n)) * S;
+        const unsigned phase_sph = WHOLE ? phase_of(sph, first_point * ny) : 0u;
+        const unsigned phase_dsph = WHOLE && MODE >= 1 ? phase_of(dsph, first_point * 3 * ny) : 0u;
+        const unsigned phase_ddsph = WHOLE && MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
         if constexpr (WHOLE) {
             if (t < valid) {
                 const T* rec = point_data(n % 3u, t);
@@ -410,9 +431,9 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
                 p.ir = rec[6];
                 Rows<T> rows;
                 rows.ny = static_cast<int>(ny);
-                rows.sph = staged + t * ny;
-                rows.dsph = staged + g.off_dsph + t * 3 * ny;
-                rows.ddsph = staged + g.off_ddsph + t * 9 * ny;
+                rows.sph = staged + phase_sph + t * ny;
+                rows.dsph = staged + g.off_dsph + phase_dsph + t * 3 * ny;
+                rows.ddsph = staged + g.off_ddsph + phase_ddsph + t * 9 * ny;
                 closed_form_job<T, MODE, NORM, H>(p, rows);
             }
         }
@@ -445,9 +466,9 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
             // the staged rows start at l = H + 1
             Rows<T> rows;
             rows.ny = static_cast<int>(nrow);
-            rows.sph = staged + s * nrow - skip;
-            rows.dsph = staged + g.off_dsph + s * 3 * nrow - skip;
-            rows.ddsph = staged + g.off_ddsph + s * 9 * nrow - skip;
+            rows.sph = staged + phase_sph + s * nrow - skip;
+            rows.dsph = staged + g.off_dsph + phase_dsph + s * 3 * nrow - skip;
+            rows.ddsph = staged + g.off_ddsph + phase_ddsph + s * 9 * nrow - skip;
             for (unsigned e = e_first; e < g.jobs_per_point; e += wide_lanes) {
                 const unsigned packed = job_table[e];
                 const int m = static_cast<int>(packed & 0x7fu);
@@ -470,16 +491,65 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
         const T* staged = lds + buffer * g.rows_elems;
         if constexpr (WHOLE) {
-            copy_out<T, SPHX_STREAMING_STORES, false, WHOLE_UNROLL>(staged, sph + first * ny, valid * ny, ny, 0, 0, ft,
-                                                      count);
-            if constexpr (MODE >= 1) {
-                copy_out<T, SPHX_STREAMING_STORES, false, WHOLE_UNROLL>(staged + g.off_dsph, dsph + first * 3 * ny,
-                                                          valid * 3 * ny, 3 * ny, 0, 0, ft, count);
-            }
-            if constexpr (MODE == 2) {
-                copy_out<T, SPHX_STREAMING_STORES, false, WHOLE_UNROLL>(staged + g.off_ddsph, ddsph + first * 9 * ny,
-                                                          valid * 9 * ny, 9 * ny, 0, 0, ft, count);
-            }
+            // The tile's run of `len` elements of one output array starts at element `at` of that
+            // array. Only whole 128-byte lines go out with vector stores. The line in which the
+            // run ends is completed by the next tile: when that tile is this workgroup's next one
+            // (same chunk), the unfinished part is carried over into the region the next tile is
+            // staged in; at the ends of a chunk the partial lines are stored element by element.
+            const bool starts = (n & chunk_mask) == 0;
+            const bool ends = (n & chunk_mask) == chunk_mask || valid_in(n + 1) == 0;
+            T* carry_to = lds + (streaming ? (buffer ^ 1u) : buffer) * g.rows_elems;
+            auto flush_run = [&](unsigned region_offset, T* array, unsigned long long at, unsigned len) {
+                using V = typename Pack<T>::type;
+                constexpr unsigned W = Pack<T>::width;
+                T* region = lds + buffer * g.rows_elems + region_offset;
+                const unsigned phase = phase_of(array, at);
+                T* line0 = array + (at - phase); // HBM address of region element 0
+                const unsigned lo = starts ? phase : 0u; // first element that holds data
+                const unsigned hi = phase + len;
+                const unsigned full_lo = (lo + LINE - 1u) / LINE * LINE;
+                const unsigned full_hi = hi / LINE * LINE;
+                unsigned tail_from; // what follows the head and the whole lines
+                if (full_hi > full_lo) {
+                    const unsigned nvec = (full_hi - full_lo) / W;
+                    const V* in = reinterpret_cast<const V*>(region + full_lo);
+                    V* out = reinterpret_cast<V*>(line0 + full_lo);
+                    unsigned v = ft;
+                    if constexpr (WHOLE_UNROLL > 1) {
+                        for (; v + (WHOLE_UNROLL - 1) * count < nvec; v += WHOLE_UNROLL * count) {
+                            V hold[WHOLE_UNROLL];
+#pragma unroll
+                            for (int u = 0; u < WHOLE_UNROLL; ++u) hold[u] = in[v + u * count];
+#pragma unroll
+                            for (int u = 0; u < WHOLE_UNROLL; ++u) {
+                                emit<T, SPHX_STREAMING_STORES>(hold[u], out + v + u * count);
+                            }
+                        }
+                    }
+                    for (; v < nvec; v += count) {
+                        emit<T, SPHX_STREAMING_STORES>(in[v], out + v);
+                    }
+                    tail_from = full_hi;
+                } else {
+                    tail_from = full_lo < hi ? full_lo : hi;
+                }
+                // head: the part of the first line that belongs to this chunk
+                const unsigned head_end = full_lo < hi ? full_lo : hi;
+                if (lo + ft < head_end) line0[lo + ft] = region[lo + ft];
+                // tail: stored if the chunk ends here, else handed to the next tile
+                const unsigned tail = hi - tail_from;
+                if (ft < tail) {
+                    const T value = region[tail_from + ft];
+                    if (ends) {
+                        line0[tail_from + ft] = value;
+                    } else if (carry_to + region_offset != region || tail_from != 0) {
+                        carry_to[region_offset + ft] = value;
+                    }
+                }
+            };
+            flush_run(0, sph, first * ny, valid * ny);
+            if constexpr (MODE >= 1) flush_run(g.off_dsph, dsph, first * 3 * ny, valid * 3 * ny);
+            if constexpr (MODE == 2) flush_run(g.off_ddsph, ddsph, first * 9 * ny, valid * 9 * ny);
         } else {
             // one run per (point, component) row, dealt to the waves in turn
             const unsigned waves = count / 64;
@@ -681,7 +751,8 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     const unsigned limit = static_cast<unsigned>(lds_limit);
     for (;;) {
         // 24: alignment slack of the row arrays
-        fixed = 2 * tri_all + table_elems_for(may_split) + 24;
+        // + 3 lines: a staging region starts at a line boundary of its output array
+        fixed = 2 * tri_all + table_elems_for(may_split) + 24 + 2 * 3 * (128u / esize);
         if (bytes_for(1, 1) <= limit || !may_split) break;
         may_split = false; // the longer job table is what does not fit
     }
@@ -731,11 +802,14 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.magic_jobs = magic_of(g.jobs_per_point);
     g.points_per_pass = per_pass(g.jobs_per_point);
 
-    unsigned at = align4(S * nrow);
+    // in front of every staging region, room for the part of a 128-byte line that precedes the
+    // tile's run (recursion_kernel, flush_run)
+    const unsigned line = whole ? 128u / esize : 0u;
+    unsigned at = align4(S * nrow + line);
     g.off_dsph = at;
-    if (mode >= 1) at = align4(at + S * 3 * nrow);
+    if (mode >= 1) at = align4(at + S * 3 * nrow + line);
     g.off_ddsph = at;
-    if (mode == 2) at = align4(at + S * 9 * nrow);
+    if (mode == 2) at = align4(at + S * 9 * nrow + line);
     g.rows_elems = at;
     at *= buffers;
     g.off_F = at;
@@ -754,11 +828,19 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
 
     g.n_tiles = static_cast<unsigned>((n_samples + S - 1) / S);
     g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
+    // Chunks of consecutive tiles per workgroup: only where a tile is one run per array, and a
+    // run is at least a line long (so that a carried part never spans two tiles).
+    g.chunk_shift = 0;
+    if (whole && S * nrow * esize >= 128u) {
+        const int want = env_int("SPHX_CHUNK_SHIFT", 3);
+        g.chunk_shift = want < 0 ? 0u : (want > 10 ? 10u : static_cast<unsigned>(want));
+    }
+    const unsigned chunks_per_xcd = (g.tiles_per_xcd + (1u << g.chunk_shift) - 1u) >> g.chunk_shift;
     unsigned per_cu = limit / out->lds_bytes;
     if (per_cu < 1) per_cu = 1;
     if (per_cu > 4) per_cu = 4; // 512 threads each: 2048 lanes per CU
     unsigned want = (static_cast<unsigned>(cus) * per_cu + 7u) & ~7u;
-    unsigned need = g.tiles_per_xcd * 8u;
+    unsigned need = chunks_per_xcd * 8u;
     out->workgroups = want < need ? want : need;
     if (out->workgroups < 8) out->workgroups = 8;
     return true;
