@@ -41,9 +41,10 @@ PEAK_HBM_GBPS = 8000.0
 # doubled). KiB per dispatch * 1024 * factor, fetch + write, all kernels of one
 # call added up.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg3": int((5932.6 * 2.0 + 765883.9) * 1024),
-    "cfg4": int((1304.2 * 2.0 + 3063197.6) * 1024),
-    "cfg5": int(((1239.9 + 1279.8) * 2.0 + 184231.9 + 3427561.4) * 1024),
+    "cfg3": int((5930.6 * 2.0 + 765861.1) * 1024),
+    "cfg4": int((1329.7 * 2.0 + 2935184.4) * 1024),
+    "cfg5": int(((1239.9 + 1308.3) * 2.0 + 184101.3 + 3404931.8) * 1024),
+    "cfg3:backward": int((394551.2 * 2.0 + 11719.3) * 1024),
 }
 
 
@@ -279,7 +280,7 @@ def main():
             "peak": PEAK_HBM_GBPS,
             "unit": "GB/s",
             "frac": achieved / PEAK_HBM_GBPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.op == "forward" else None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload if args.op == "forward" else f"{args.workload}:backward"),
             "algorithmic_bytes_per_launch": bytes_per_launch,
             "avg_launch_us": avg_launch_s * 1e6,
             "median_launch_us": statistics.median(launch_ms) * 1e3,
