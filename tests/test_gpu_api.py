@@ -73,6 +73,35 @@ def test_unaligned_outputs_take_the_narrow_store_path(oracle, library):
                     assert same_numbers(o.cpu().numpy(), w).all()
 
 
+@pytest.mark.parametrize("shift", [0, 1, 5])
+def test_many_tiles_per_workgroup_with_shifted_outputs(oracle, library, shift):
+    """Enough points that every workgroup of the recursion kernel walks several chunks of tiles,
+    with outputs that start `shift` elements into a 128-byte line: the lines that consecutive
+    tiles share are carried from one tile to the next and must come out complete."""
+    rng = np.random.default_rng(7 + shift)
+    cases = ((np.float32, torch.float32, 7, "gradients"), (np.float64, torch.float64, 10, "gradients"),
+             (np.float32, torch.float32, 3, "hessians"), (np.float64, torch.float64, 12, "hessians"),
+             (np.float32, torch.float32, 9, "values"))
+    for dtype, tdtype, l_max, mode in cases:
+        announce("many tiles", np.dtype(dtype).name, l_max, mode, "shift", shift)
+        n, ny = 40_003, (l_max + 1) ** 2
+        xyz = special_points(dtype, rng, n)
+        want = oracle.compute(xyz, l_max, False, mode)
+        sizes = (n * ny, 3 * n * ny, 9 * n * ny)
+        shapes = ((n, ny), (n, 3, ny), (n, 3, 3, ny))
+        raw = [torch.full((s + 64,), float("nan"), dtype=tdtype, device="cuda") for s in sizes]
+        out = tuple(raw[i][shift:shift + sizes[i]].view(shapes[i]) if w is not None else None
+                    for i, w in enumerate(want))
+        status, _ = run_launch_layer(library, torch.from_numpy(xyz).cuda(), l_max, False, mode, out=out)
+        assert status == 0, library.sphx_last_error()
+        torch.cuda.synchronize()
+        for i, (o, w) in enumerate(zip(out, want)):
+            if w is not None:
+                assert same_numbers(o.cpu().numpy(), w).all()
+                # nothing written outside the arrays
+                assert torch.isnan(raw[i][:shift]).all() and torch.isnan(raw[i][shift + sizes[i]:]).all()
+
+
 def test_non_contiguous_input(oracle):
     """Reference: sphericart-torch/python/tests/test_autograd.py:88-124 (inputs are made contiguous)."""
     rng = np.random.default_rng(2)
