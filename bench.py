@@ -64,10 +64,11 @@ def parse():
     )
     p.add_argument(
         "--op",
-        choices=("forward", "backward"),
+        choices=("forward", "backward", "vjp"),
         default="forward",
         help="backward: time the vector-Jacobian product xyz_grad = sum_k dsph * sph_grad "
-        "(sphx_backward_*) on the gradients of the workload instead of the forward pass",
+        "(sphx_backward_*) on the gradients of the workload instead of the forward pass; "
+        "vjp: the same product fused with the evaluation of the gradients (sphx_vjp_*, l_max <= 6)",
     )
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument(
@@ -144,6 +145,29 @@ def cpu_backward_baseline(dsph, sph_grad):
     }
 
 
+def cpu_vjp_baseline(workload, xyz, sph_grad):
+    """Gradients by the CPU evaluator (all cores), contracted by the checker's loop (one thread)."""
+    import oracle  # reported baseline only
+
+    flavour, kind = ("ref_fma", "reference") if oracle.available("ref_fma") else ("oracle", "port")
+    n = min(xyz.shape[0], 200_000)
+    best = None
+    for _ in range(5):
+        t0 = time.perf_counter()
+        _, dsph, _ = oracle.compute(xyz[:n], workload.l_max, workload.normalized, "gradients", flavour)
+        oracle.backward(dsph, sph_grad[:n])
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return {
+        "value": n / best,
+        "unit": "points/s",
+        "cores": oracle.max_threads(flavour),
+        "kind": kind,
+        "sample": f"5 passes over the first {n} points, best pass {best * 1e3:.2f} ms; gradients by the CPU "
+        "evaluator (OpenMP), then the contraction loop on one thread",
+    }
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -206,6 +230,25 @@ def main():
 
         # reads dsph and sph_grad once, writes three numbers per point
         bytes_per_launch = xyz.element_size() * n * (4 * ny + 3)
+
+    if args.op == "vjp":
+        if w.l_max > 6:
+            print("--op vjp covers workloads with l_max <= 6", file=sys.stderr)
+            return 2
+        torch.manual_seed(w.seed)
+        sph_grad = torch.randn((n, ny), **opts)
+        xyz_grad = torch.empty((n, 3), **opts)
+        fused = lib.sphx_vjp_f32 if w.dtype == "f32" else lib.sphx_vjp_f64
+        fused_args = (xyz.data_ptr(), sph_grad.data_ptr(), n, w.l_max, int(w.normalized),
+                      xyz_grad.data_ptr(), 0, stream.cuda_stream)
+
+        def step():  # noqa: F811
+            status = fused(*fused_args)
+            if status != 0:
+                raise RuntimeError(lib.sphx_last_error().decode())
+
+        # reads xyz and sph_grad, writes xyz_grad
+        bytes_per_launch = xyz.element_size() * n * (3 + ny + 3)
 
     if args.calibrate_copy:
         nbytes = w.bytes_per_point * n
@@ -280,7 +323,7 @@ def main():
             "peak": PEAK_HBM_GBPS,
             "unit": "GB/s",
             "frac": achieved / PEAK_HBM_GBPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload if args.op == "forward" else f"{args.workload}:backward"),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload if args.op == "forward" else f"{args.workload}:{args.op}"),
             "algorithmic_bytes_per_launch": bytes_per_launch,
             "avg_launch_us": avg_launch_s * 1e6,
             "median_launch_us": statistics.median(launch_ms) * 1e3,
@@ -290,6 +333,8 @@ def main():
     if not args.no_cpu_baseline:
         if args.op == "forward":
             result["cpu_baseline"] = cpu_baseline(w, xyz_host)
+        elif args.op == "vjp":
+            result["cpu_baseline"] = cpu_vjp_baseline(w, xyz_host, sph_grad.cpu().numpy())
         else:
             result["cpu_baseline"] = cpu_backward_baseline(dsph.cpu().numpy(), sph_grad.cpu().numpy())
     print(json.dumps(result))

@@ -93,6 +93,23 @@ SPHX_EXPORT int sphx_backward_second_f64(const double* ddsph, const double* dsph
                                          size_t n_samples, int n_total, double* xyz_grad,
                                          int accumulate, void* stream);
 
+/* Forward and backward pass fused, for callers that only need the gradient of a
+ * scalar with respect to the coordinates (training):
+ *
+ *   xyz_grad[i][a] (+)= sum_k (d sph[i][k] / d xyz[i][a]) * sph_grad[i][k]
+ *
+ * without dsph ever reaching memory: reads xyz and sph_grad, writes xyz_grad.
+ * Covers l_max <= 6 (the closed forms); beyond that returns SPHX_ERR_UNSUPPORTED
+ * and the caller combines sphx_forward_* with sphx_backward_*. The numbers are
+ * those of that combination summed over k in index order.
+ * No counterpart in the reference, whose torch binding recomputes dsph in
+ * memory for its backward pass
+ * (sphericart-torch/python/sphericart/torch/register.py:96-103). */
+SPHX_EXPORT int sphx_vjp_f32(const float* xyz, const float* sph_grad, size_t n_samples, int l_max,
+                             int normalized, float* xyz_grad, int accumulate, void* stream);
+SPHX_EXPORT int sphx_vjp_f64(const double* xyz, const double* sph_grad, size_t n_samples, int l_max,
+                             int normalized, double* xyz_grad, int accumulate, void* stream);
+
 /* Host copy of the prefactor table the kernels use for this l_max: the F_l^m
  * block followed by the Q_l^m-recursion block, (l_max+1)(l_max+2) numbers.
  * Replaces compute_sph_prefactors<T> (sphericart/include/templates.hpp:54-97)

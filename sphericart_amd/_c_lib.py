@@ -28,6 +28,8 @@ LAUNCH_SYMBOLS = [
     "sphx_backward_f64",
     "sphx_backward_second_f32",
     "sphx_backward_second_f64",
+    "sphx_vjp_f32",
+    "sphx_vjp_f64",
     "sphx_prefactors_f32",
     "sphx_prefactors_f64",
     "sphx_device_count",
@@ -64,6 +66,9 @@ def _declare(lib):
             fn = getattr(lib, f"{name}_{suffix}")
             fn.restype = c_int
             fn.argtypes = [c_void_p, c_void_p, c_size_t, c_int, c_void_p, c_int, c_void_p]
+        fn = getattr(lib, f"sphx_vjp_{suffix}")
+        fn.restype = c_int
+        fn.argtypes = [c_void_p, c_void_p, c_size_t, c_int, c_int, c_void_p, c_int, c_void_p]
         fn = getattr(lib, f"sphx_prefactors_{suffix}")
         fn.restype = c_int
         fn.argtypes = [c_int, c_void_p]

@@ -212,6 +212,81 @@ __global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __re
 }
 
 // ---------------------------------------------------------------------------
+// Vector-Jacobian product without the Jacobian in memory, l_max <= 6:
+//
+//   xyz_grad[i][a] (+)= sum_k d sph[i][k] / d xyz[i][a] * sph_grad[i][k]
+//
+// Same evaluation as closed_form_kernel with gradients (one point per lane, the
+// finished entries in VGPRs), but instead of staging 4 (l_max+1)^2 numbers per
+// point for HBM the lane multiplies its gradient entries with the point's row of
+// sph_grad and keeps three sums: (l_max+1)^2 + 3 numbers read and 3 written per
+// point instead of 4 (l_max+1)^2 written and read again. LDS only turns the
+// coalesced load of the tile's sph_grad rows into one row per lane (row stride
+// odd, so the lanes hit different banks). The sums run over k in index order
+// with one rounding per operation: the result is what contracting the
+// gradients of the forward pass in that order gives, bit for bit.
+// ---------------------------------------------------------------------------
+template <typename T, bool NORM, int H>
+__global__ __launch_bounds__(64) void closed_form_vjp_kernel(Tiling g, const T* __restrict__ xyz,
+                                                            const T* __restrict__ sph_grad,
+                                                            T* __restrict__ xyz_grad, int accumulate) {
+    constexpr unsigned NY = (H + 1) * (H + 1);
+    constexpr unsigned STRIDE = NY + closed_form_pad(H);
+    T* weights = reinterpret_cast<T*>(lds_raw);
+    const unsigned tid = threadIdx.x;
+    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
+    if (group >= g.n_tiles) return;
+    const unsigned long long first = static_cast<unsigned long long>(group) * 64;
+    const unsigned long long left = g.n_samples - first;
+    const unsigned valid = left < 64ull ? static_cast<unsigned>(left) : 64u;
+
+    // the tile's rows of sph_grad are one contiguous run: consecutive lanes, consecutive addresses
+    const T* run = sph_grad + first * NY;
+    using V = typename Pack<T>::type;
+    constexpr unsigned W = Pack<T>::width;
+    const unsigned total = valid * NY;
+    if ((reinterpret_cast<uintptr_t>(run) & 15u) == 0 && total % W == 0) {
+        const V* in = reinterpret_cast<const V*>(run);
+        for (unsigned v = tid; v < total / W; v += 64) {
+            const V four = in[v];
+#pragma unroll
+            for (unsigned e = 0; e < W; ++e) {
+                const unsigned i = v * W + e;
+                weights[i + (STRIDE - NY) * (i / NY)] = four[e];
+            }
+        }
+    } else {
+        for (unsigned i = tid; i < total; i += 64) {
+            weights[i + (STRIDE - NY) * (i / NY)] = run[i];
+        }
+    }
+    __syncthreads();
+    if (tid >= valid) return;
+
+    Entry<T> E[NY];
+    const Point<T> p = load_point<T, NORM>(xyz + (first + tid) * 3);
+    closed_form_entries<T, 1, NORM, H>(p, E);
+    const T* mine = weights + tid * STRIDE;
+    T sum_x = 0, sum_y = 0, sum_z = 0;
+#pragma unroll
+    for (unsigned k = 0; k < NY; ++k) {
+        const T wk = mine[k];
+        sum_x += E[k].gx * wk;
+        sum_y += E[k].gy * wk;
+        sum_z += E[k].gz * wk;
+    }
+    T* out = xyz_grad + (first + tid) * 3;
+    if (accumulate) {
+        sum_x += out[0];
+        sum_y += out[1];
+        sum_z += out[2];
+    }
+    out[0] = sum_x;
+    out[1] = sum_y;
+    out[2] = sum_z;
+}
+
+// ---------------------------------------------------------------------------
 // l > H through the recursion. 512 threads, persistent workgroups that walk
 // over tiles of `tile` consecutive points, four tiles in flight per workgroup,
 // every wave with a role of its own and one barrier per tile:
@@ -1037,6 +1112,77 @@ static int forward(const T* xyz, size_t n_samples, int l_max, int normalized, in
     return status;
 }
 
+template <typename T, bool NORM, int H>
+static hipError_t launch_vjp(const Launch& l, const T* xyz, const T* sph_grad, T* xyz_grad,
+                             int accumulate, hipStream_t stream) {
+    constexpr unsigned NY = (H + 1) * (H + 1);
+    const unsigned lds_bytes = 64u * (NY + closed_form_pad(H)) * static_cast<unsigned>(sizeof(T));
+    hipLaunchKernelGGL((closed_form_vjp_kernel<T, NORM, H>), dim3(l.workgroups), dim3(64), lds_bytes,
+                       stream, l.g, xyz, sph_grad, xyz_grad, accumulate);
+    return hipGetLastError();
+}
+
+template <typename T, bool NORM>
+static hipError_t dispatch_vjp(const Launch& l, int l_max, const T* xyz, const T* sph_grad,
+                               T* xyz_grad, int accumulate, hipStream_t stream) {
+    switch (l_max) {
+    case 0: return launch_vjp<T, NORM, 0>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
+    case 1: return launch_vjp<T, NORM, 1>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
+    case 2: return launch_vjp<T, NORM, 2>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
+    case 3: return launch_vjp<T, NORM, 3>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
+    case 4: return launch_vjp<T, NORM, 4>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
+    case 5: return launch_vjp<T, NORM, 5>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
+    case 6: return launch_vjp<T, NORM, 6>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template <typename T>
+static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int normalized,
+               T* xyz_grad, int accumulate, void* stream) {
+    t_error.clear();
+    if (n_samples == 0) return SPHX_OK;
+    if (l_max < 0) return fail(SPHX_ERR_ARGUMENT, "l_max must be non-negative");
+    if (l_max > 6) {
+        return fail(SPHX_ERR_UNSUPPORTED,
+                    "the fused vector-Jacobian product covers l_max <= 6; beyond that evaluate the "
+                    "gradients (sphx_forward_*) and contract them (sphx_backward_*)");
+    }
+    if (xyz == nullptr || sph_grad == nullptr || xyz_grad == nullptr) {
+        return fail(SPHX_ERR_ARGUMENT, "null pointer passed to the vector-Jacobian product");
+    }
+    if ((n_samples + 63) / 64 > 0x7fffffffull) {
+        return fail(SPHX_ERR_UNSUPPORTED, "too many samples for one launch");
+    }
+    hipPointerAttribute_t attr;
+    SPHX_HIP(hipPointerGetAttributes(&attr, xyz));
+    int current = 0;
+    SPHX_HIP(hipGetDevice(&current));
+    const int device = attr.device;
+    if (device != current) {
+        SPHX_HIP(hipSetDevice(device));
+    }
+    int status = ensure_device_ready(device);
+    if (status == SPHX_OK) {
+        Launch l;
+        plan_closed(n_samples, l_max, l_max, 1, sizeof(T), &l);
+        hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+        const hipError_t e = normalized
+                                 ? dispatch_vjp<T, true>(l, l_max, xyz, sph_grad, xyz_grad, accumulate, s)
+                                 : dispatch_vjp<T, false>(l, l_max, xyz, sph_grad, xyz_grad, accumulate, s);
+        if (e != hipSuccess) {
+            status = fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
+        }
+    }
+    if (device != current) {
+        hipError_t e = hipSetDevice(current);
+        if (e != hipSuccess && status == SPHX_OK) {
+            status = fail(SPHX_ERR_HIP, std::string("hipSetDevice: ") + hipGetErrorString(e));
+        }
+    }
+    return status;
+}
+
 } // namespace sphx
 
 extern "C" {
@@ -1051,6 +1197,16 @@ int sphx_forward_f64(const double* xyz, size_t n_samples, int l_max, int normali
                      int derivatives, double* sph, double* dsph, double* ddsph, void* stream) {
     return sphx::forward<double>(xyz, n_samples, l_max, normalized, derivatives, sph, dsph, ddsph,
                                  stream);
+}
+
+int sphx_vjp_f32(const float* xyz, const float* sph_grad, size_t n_samples, int l_max, int normalized,
+                 float* xyz_grad, int accumulate, void* stream) {
+    return sphx::vjp<float>(xyz, sph_grad, n_samples, l_max, normalized, xyz_grad, accumulate, stream);
+}
+
+int sphx_vjp_f64(const double* xyz, const double* sph_grad, size_t n_samples, int l_max,
+                 int normalized, double* xyz_grad, int accumulate, void* stream) {
+    return sphx::vjp<double>(xyz, sph_grad, n_samples, l_max, normalized, xyz_grad, accumulate, stream);
 }
 
 int sphx_device_count(void) {

@@ -11,9 +11,13 @@ The backward formulas are the reference's (register.py:82-175). Where it writes
 the vector-Jacobian products as ``torch.sum(grad.unsqueeze(1) * dsph, dim=2)``,
 two more operators, ``contract_gradients`` and ``contract_hessians``, do the
 same sums in one pass over ``dsph`` / ``ddsph`` (``sphx_backward_*``) without
-the product array; they are differentiable themselves, so double backward works
-as it does in the reference.
+the product array. For ``l_max <= 6`` the backward pass of the value operators
+does not build ``dsph`` at all: ``*_vjp`` (``sphx_vjp_*``) evaluates the
+gradients in registers and contracts them on the fly. All of these are
+differentiable themselves, so double backward works as it does in the reference.
 """
+
+FUSED_VJP_LMAX = 6  # what sphx_vjp_* covers
 
 import ctypes
 
@@ -29,6 +33,7 @@ for _prefix in ("spherical_harmonics", "solid_harmonics"):
     _lib.define(f"{_prefix}(Tensor xyz, int l_max) -> Tensor")
     _lib.define(f"{_prefix}_with_gradients(Tensor xyz, int l_max) -> (Tensor, Tensor)")
     _lib.define(f"{_prefix}_with_hessians(Tensor xyz, int l_max) -> (Tensor, Tensor, Tensor)")
+    _lib.define(f"{_prefix}_vjp(Tensor xyz, Tensor sph_grad, int l_max) -> Tensor")
 _lib.define("contract_gradients(Tensor dsph, Tensor sph_grad) -> Tensor")
 _lib.define("contract_hessians(Tensor ddsph, Tensor dsph_grad) -> Tensor")
 
@@ -96,6 +101,26 @@ def _contract(name, derivatives, upstream):
     return out
 
 
+def _vjp(xyz, sph_grad, l_max, normalized):
+    suffix = _suffix(xyz)
+    if sph_grad.dtype != xyz.dtype or sph_grad.device != xyz.device:
+        raise ValueError("xyz and sph_grad must share dtype and device")
+    if sph_grad.shape != (xyz.shape[0], (l_max + 1) ** 2):
+        raise ValueError(f"sph_grad must have shape {(xyz.shape[0], (l_max + 1) ** 2)}")
+    xyz = xyz.detach().contiguous()
+    sph_grad = sph_grad.detach().contiguous()
+    out = torch.empty_like(xyz)
+    library = get_library()
+    with torch.cuda.device(xyz.device):
+        stream = torch.cuda.current_stream(xyz.device).cuda_stream
+        status = getattr(library, f"sphx_vjp_{suffix}")(
+            _pointer(xyz), _pointer(sph_grad), xyz.shape[0], l_max, int(normalized), _pointer(out), 0,
+            ctypes.c_void_p(stream),
+        )
+    _check(status, library)
+    return out
+
+
 def _no_cpu(*args, **kwargs):
     raise RuntimeError(
         "sphericart_amd evaluates on AMD GPUs only: move the tensor to the device "
@@ -113,7 +138,11 @@ def _register_forward(prefix, normalized):
     def hessians(xyz, l_max):
         return _forward(xyz, l_max, normalized, 2)
 
-    for name, fn in ((prefix, value), (f"{prefix}_with_gradients", gradients), (f"{prefix}_with_hessians", hessians)):
+    def vjp(xyz, sph_grad, l_max):
+        return _vjp(xyz, sph_grad, l_max, normalized)
+
+    for name, fn in ((prefix, value), (f"{prefix}_with_gradients", gradients),
+                     (f"{prefix}_with_hessians", hessians), (f"{prefix}_vjp", vjp)):
         _lib.impl(name, fn, "CUDA")
         _lib.impl(name, _no_cpu, "CPU")
 
@@ -189,8 +218,35 @@ torch.library.register_autograd(
 
 # ---- autograd of the six operators (register.py:82-175) ----------------------
 
+def _register_vjp(prefix):
+    """Shapes and derivatives of the fused product xyz_grad[i, a] = sum_k dsph[i, a, k] w[i, k]."""
+    hessians = getattr(_ops, f"{prefix}_with_hessians")
+
+    @torch.library.register_fake(f"{NAMESPACE}::{prefix}_vjp")
+    def fake(xyz, sph_grad, l_max):
+        return xyz.new_empty((xyz.shape[0], 3))
+
+    def setup_context(ctx, inputs, output):
+        xyz, sph_grad, ctx.l_max = inputs
+        ctx.save_for_backward(xyz, sph_grad)
+
+    def backward(ctx, grad):
+        xyz, sph_grad = ctx.saved_tensors
+        _, dsph, ddsph = hessians(xyz, ctx.l_max)
+        d_xyz = d_sph_grad = None
+        if ctx.needs_input_grad[0]:
+            # d/d xyz[i, b]: sum_{a, k} grad[i, a] w[i, k] ddsph[i, a, b, k]
+            d_xyz = _ops.contract_hessians(ddsph, grad.unsqueeze(2) * sph_grad.unsqueeze(1))
+        if ctx.needs_input_grad[1]:
+            d_sph_grad = torch.sum(grad.unsqueeze(2) * dsph, dim=1)
+        return d_xyz, d_sph_grad, None
+
+    torch.library.register_autograd(f"{NAMESPACE}::{prefix}_vjp", backward, setup_context=setup_context)
+
+
 def _register_value_autograd(prefix):
     gradients = getattr(_ops, f"{prefix}_with_gradients")
+    vjp = getattr(_ops, f"{prefix}_vjp")
 
     def setup_context(ctx, inputs, output):
         xyz, ctx.l_max = inputs
@@ -201,6 +257,8 @@ def _register_value_autograd(prefix):
         if not ctx.needs_input_grad[0] or grad_sph is None:
             return None, None
         (xyz,) = ctx.saved_tensors
+        if ctx.l_max <= FUSED_VJP_LMAX:
+            return vjp(xyz, grad_sph, ctx.l_max), None
         dsph = gradients(xyz, ctx.l_max)[1]
         return _ops.contract_gradients(dsph, grad_sph), None
 
@@ -281,6 +339,7 @@ for _prefix in ("spherical_harmonics", "solid_harmonics"):
     _register_fake(_prefix, 1)
     _register_fake(f"{_prefix}_with_gradients", 2)
     _register_fake(f"{_prefix}_with_hessians", 3)
+    _register_vjp(_prefix)
     _register_value_autograd(_prefix)
     _register_gradients_autograd(_prefix)
     _register_hessians_autograd(_prefix)

@@ -86,6 +86,38 @@ def test_contractions_equal_checker(oracle, dtype, tol, n_total):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("normalized", [True, False])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_fused_vjp_equals_checker_number_for_number(library, oracle, normalized, dtype):
+    """sphx_vjp_* sums over k in index order with one rounding per operation, as the checker's
+    contraction of the checker's gradients does: the results are identical, not merely close."""
+    rng = np.random.default_rng(11)
+    fn = library.sphx_vjp_f32 if dtype == np.float32 else library.sphx_vjp_f64
+    stream = torch.cuda.current_stream().cuda_stream
+    for l_max in range(7):
+        for n in (1, 63, 64, 65, 1000, 4099):
+            announce("fused vjp", normalized, np.dtype(dtype).name, l_max, n)
+            xyz = _points(n, dtype, seed=l_max * 10 + n)
+            weights = rng.standard_normal((n, (l_max + 1) ** 2)).astype(dtype)
+            _, dsph, _ = oracle.compute(xyz, l_max, normalized, "gradients")
+            want = oracle.backward(dsph, weights)
+            d_xyz, d_w = torch.from_numpy(xyz).cuda(), torch.from_numpy(weights).cuda()
+            out = torch.full((n, 3), float("nan"), dtype=d_xyz.dtype, device="cuda")
+            status = fn(d_xyz.data_ptr(), d_w.data_ptr(), n, l_max, int(normalized), out.data_ptr(), 0, stream)
+            assert status == 0, library.sphx_last_error()
+            np.testing.assert_array_equal(out.cpu().numpy(), want)
+            # accumulate: adds to what is there
+            start = rng.standard_normal((n, 3)).astype(dtype)
+            out = torch.from_numpy(start).cuda()
+            assert fn(d_xyz.data_ptr(), d_w.data_ptr(), n, l_max, int(normalized), out.data_ptr(), 1, stream) == 0
+            np.testing.assert_array_equal(out.cpu().numpy(), want + start)
+    # beyond the closed forms the entry point says so instead of computing
+    assert fn(d_xyz.data_ptr(), d_w.data_ptr(), 10, 7, 1, out.data_ptr(), 0, stream) == 2
+    assert b"l_max <= 6" in library.sphx_last_error()
+    assert fn(d_xyz.data_ptr(), d_w.data_ptr(), 0, 3, 1, None, 0, None) == 0
+
+
+@pytest.mark.gpu
 def test_contraction_accumulates_on_request(library, oracle):
     announce("contraction accumulate flag")
     rng = np.random.default_rng(5)
