@@ -34,6 +34,7 @@
 #include <mutex>
 #include <string>
 #include <type_traits>
+#include <vector>
 
 #include "../../include/sphx_launch.h"
 #include "sphx_device.hpp"
@@ -968,14 +969,62 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     return SPHX_OK;
 }
 
+// What a launch needs to know about a kernel on a device, asked from the runtime once per
+// (device, kernel, LDS size) instead of on every call: the calls take microseconds each, which
+// is the whole budget of a small evaluation.
+struct KernelFacts {
+    int device;
+    const void* kernel;
+    unsigned lds_bytes;
+    unsigned resident_workgroups; // on the whole device, a multiple of 8; 0 = unknown
+};
+static std::mutex g_facts_mutex;
+static std::vector<KernelFacts> g_facts;
+
+// Raises the kernel's dynamic LDS limit if needed and returns how many workgroups of `threads`
+// threads are resident on the device at once (0 if the runtime would not tell).
+static hipError_t kernel_facts(const void* kernel, unsigned threads, unsigned lds_bytes,
+                               unsigned* resident_workgroups) {
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return e;
+    {
+        std::lock_guard<std::mutex> lock(g_facts_mutex);
+        for (const KernelFacts& f : g_facts) {
+            if (f.device == device && f.kernel == kernel && f.lds_bytes == lds_bytes) {
+                *resident_workgroups = f.resident_workgroups;
+                return hipSuccess;
+            }
+        }
+    }
+    if (lds_bytes > 64u * 1024u) {
+        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(lds_bytes));
+        if (e != hipSuccess) return e;
+    }
+    KernelFacts fresh{device, kernel, lds_bytes, 0u};
+    int per_cu = 0;
+    const int cus = device >= 0 && device < kMaxDevices ? g_compute_units[device] : 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, static_cast<int>(threads),
+                                                     lds_bytes) == hipSuccess &&
+        per_cu > 0 && cus > 0) {
+        fresh.resident_workgroups = (static_cast<unsigned>(per_cu) * static_cast<unsigned>(cus)) & ~7u;
+    } else {
+        (void)hipGetLastError();
+    }
+    std::lock_guard<std::mutex> lock(g_facts_mutex);
+    g_facts.push_back(fresh);
+    *resident_workgroups = fresh.resident_workgroups;
+    return hipSuccess;
+}
+
 template <typename T, int MODE, bool NORM, int H, bool PREFIX>
 static hipError_t launch_closed(const Launch& l, const T* xyz, T* sph, T* dsph, T* ddsph,
                                 hipStream_t stream) {
     auto kernel = closed_form_kernel<T, MODE, NORM, H, PREFIX>;
     if (l.lds_bytes > 64u * 1024u) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(l.lds_bytes));
+        unsigned unused = 0;
+        hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &unused);
         if (e != hipSuccess) return e;
     }
     hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz,
@@ -987,25 +1036,13 @@ template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT>
 static hipError_t launch_recursion(const Launch& l, const T* xyz, T* sph, T* dsph, T* ddsph,
                                    hipStream_t stream) {
     auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT>;
-    if (l.lds_bytes > 64u * 1024u) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(l.lds_bytes));
-        if (e != hipSuccess) return e;
-    }
     // The workgroups are persistent: launch exactly as many as are resident at once (registers
     // may allow fewer per CU than LDS does), or the last ones would run alone after the rest.
     unsigned workgroups = l.workgroups;
-    int resident = 0, device = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kernel, static_cast<int>(l.threads),
-                                                     l.lds_bytes) == hipSuccess &&
-        resident > 0 && hipGetDevice(&device) == hipSuccess &&
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess) {
-        const unsigned cap = (static_cast<unsigned>(resident) * static_cast<unsigned>(cus)) & ~7u;
-        if (cap >= 8 && cap < workgroups) workgroups = cap;
-    } else {
-        (void)hipGetLastError();
-    }
+    unsigned cap = 0;
+    hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &cap);
+    if (e != hipSuccess) return e;
+    if (cap >= 8 && cap < workgroups) workgroups = cap;
     hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz,
                        sph, dsph, ddsph);
     return hipGetLastError();
