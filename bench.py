@@ -70,6 +70,14 @@ def parse():
         "(sphx_backward_*) on the gradients of the workload instead of the forward pass; "
         "vjp: the same product fused with the evaluation of the gradients (sphx_vjp_*, l_max <= 6)",
     )
+    p.add_argument(
+        "--rotate-mb",
+        type=int,
+        default=0,
+        help="forward pass only: write to a rotating set of output buffers of at least this many MB "
+        "in total, so that a workload whose outputs fit into the 256 MB Infinity Cache (cfg1, cfg2) "
+        "is also measured with every launch going to memory that is not cached",
+    )
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument(
         "--calibrate-copy",
@@ -212,6 +220,24 @@ def main():
             raise RuntimeError(lib.sphx_last_error().decode())
 
     bytes_per_launch = w.bytes_per_point * n
+    if args.rotate_mb > 0 and args.op == "forward":
+        copies = max(2, -(-args.rotate_mb * 1_000_000 // bytes_per_launch))
+        rotating = []
+        for _ in range(copies):
+            o = (torch.empty((n, ny), **opts),
+                 torch.empty((n, 3, ny), **opts) if mode >= 1 else None,
+                 torch.empty((n, 3, 3, ny), **opts) if mode >= 2 else None)
+            rotating.append((o, (xyz.data_ptr(), n, w.l_max, int(w.normalized), mode, o[0].data_ptr(),
+                                 o[1].data_ptr() if o[1] is not None else None,
+                                 o[2].data_ptr() if o[2] is not None else None, stream.cuda_stream)))
+        turn = [0]
+
+        def step():  # noqa: F811
+            status = forward(*rotating[turn[0] % copies][1])
+            turn[0] += 1
+            if status != 0:
+                raise RuntimeError(lib.sphx_last_error().decode())
+
     if args.op == "backward":
         if mode < 1:
             print("--op backward needs a workload with gradients", file=sys.stderr)
@@ -310,6 +336,7 @@ def main():
         "config": {
             "workload": f"{w.name}: {w.description}",
             "op": args.op,
+            "rotate_mb": args.rotate_mb,
             "settle_seconds": args.settle_seconds,
             "l_max": w.l_max,
             "n_samples": n,
