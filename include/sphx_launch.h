@@ -99,9 +99,10 @@ SPHX_EXPORT int sphx_backward_second_f64(const double* ddsph, const double* dsph
  *   xyz_grad[i][a] (+)= sum_k (d sph[i][k] / d xyz[i][a]) * sph_grad[i][k]
  *
  * without dsph ever reaching memory: reads xyz and sph_grad, writes xyz_grad.
- * Covers l_max <= 6 (the closed forms); beyond that returns SPHX_ERR_UNSUPPORTED
- * and the caller combines sphx_forward_* with sphx_backward_*. The numbers are
- * those of that combination summed over k in index order.
+ * For l_max <= 6 the sum runs over k in index order, one rounding per
+ * operation: the numbers are those of sphx_forward_* followed by a sequential
+ * contraction. Beyond that the terms are added in another order (lanes, then a
+ * butterfly), so the result agrees with that combination to rounding only.
  * No counterpart in the reference, whose torch binding recomputes dsph in
  * memory for its backward pass
  * (sphericart-torch/python/sphericart/torch/register.py:96-103). */

@@ -69,6 +69,7 @@ struct Tiling {
                              // limit, or (l, m, side) triples when the sides are split
     unsigned sequence_waves; // waves that run the bare recursions (1 or 2)
     unsigned points_per_pass; // points whose entry jobs fit side by side in the wide waves (>= 1)
+    unsigned vjp_accumulate; // fused product: add to xyz_grad instead of overwriting it
     unsigned chunk_shift;   // a workgroup takes 2^chunk_shift consecutive tiles at a time
     unsigned row_buffers;   // 2: tile n is flushed while tile n+1 is computed; 1: one after the other
     unsigned flush_waves;   // waves that do nothing but flush (row_buffers == 2)
@@ -227,6 +228,10 @@ __global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __re
 // with one rounding per operation: the result is what contracting the
 // gradients of the forward pass in that order gives, bit for bit.
 // ---------------------------------------------------------------------------
+//
+// g.ny is the length of a row of sph_grad: (H+1)^2 when l_max = H; longer when this kernel
+// takes only the first (H+1)^2 entries of every row and the recursion kernel adds the rest
+// (recursion_kernel with VJP).
 template <typename T, bool NORM, int H>
 __global__ __launch_bounds__(64) void closed_form_vjp_kernel(Tiling g, const T* __restrict__ xyz,
                                                             const T* __restrict__ sph_grad,
@@ -241,12 +246,19 @@ __global__ __launch_bounds__(64) void closed_form_vjp_kernel(Tiling g, const T* 
     const unsigned long long left = g.n_samples - first;
     const unsigned valid = left < 64ull ? static_cast<unsigned>(left) : 64u;
 
-    // the tile's rows of sph_grad are one contiguous run: consecutive lanes, consecutive addresses
-    const T* run = sph_grad + first * NY;
+    // l_max = H: the tile's rows of sph_grad are one contiguous run: consecutive lanes,
+    // consecutive addresses
+    const unsigned row_stride = static_cast<unsigned>(g.ny);
+    const T* run = sph_grad + first * row_stride;
     using V = typename Pack<T>::type;
     constexpr unsigned W = Pack<T>::width;
     const unsigned total = valid * NY;
-    if ((reinterpret_cast<uintptr_t>(run) & 15u) == 0 && total % W == 0) {
+    if (row_stride != NY) {
+        for (unsigned i = tid; i < total; i += 64) {
+            const unsigned s = i / NY;
+            weights[i + (STRIDE - NY) * s] = run[static_cast<unsigned long long>(s) * row_stride + (i - s * NY)];
+        }
+    } else if ((reinterpret_cast<uintptr_t>(run) & 15u) == 0 && total % W == 0) {
         const V* in = reinterpret_cast<const V*>(run);
         for (unsigned v = tid; v < total / W; v += 64) {
             const V four = in[v];
@@ -323,11 +335,12 @@ __global__ __launch_bounds__(64) void closed_form_vjp_kernel(Tiling g, const T* 
 // ---------------------------------------------------------------------------
 constexpr unsigned kRecursionThreads = 512;
 
-template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT>
+template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false>
 __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, const T* __restrict__ xyz,
                                                                      T* __restrict__ sph,
                                                                      T* __restrict__ dsph,
                                                                      T* __restrict__ ddsph) {
+    static_assert(!VJP || (MODE == 1 && !SPLIT), "the fused product is built on the gradient kernel");
     constexpr int H = MODE == 2 ? 1 : 6;
     constexpr unsigned NYH = (H + 1) * (H + 1);
     constexpr unsigned ARRAYS = MODE + 1; // iterate arrays per point: A, B, C
@@ -491,9 +504,10 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         // WHOLE: element 0 of a staging region stands for the start of the 128-byte line in
         // which the tile's run begins in HBM, so the run itself starts `phase` elements in
         const unsigned long long first_point = static_cast<unsigned long long>(tile_of(n)) * S;
-        const unsigned phase_sph = WHOLE ? phase_of(sph, first_point * ny) : 0u;
-        const unsigned phase_dsph = WHOLE && MODE >= 1 ? phase_of(dsph, first_point * 3 * ny) : 0u;
-        const unsigned phase_ddsph = WHOLE && MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
+        // (VJP: the rows never leave LDS, no position to match)
+        const unsigned phase_sph = WHOLE && !VJP ? phase_of(sph, first_point * ny) : 0u;
+        const unsigned phase_dsph = WHOLE && !VJP && MODE >= 1 ? phase_of(dsph, first_point * 3 * ny) : 0u;
+        const unsigned phase_ddsph = WHOLE && !VJP && MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
         if constexpr (WHOLE) {
             if (t < valid) {
                 const T* rec = point_data(n % 3u, t);
@@ -645,6 +659,40 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         }
     };
 
+    // VJP: in place of the flush. `sph` holds the upstream gradient sph_grad[N][ny] (read
+    // only), `dsph` is xyz_grad[N][3]. Wave 1 + r takes gradient row r of the tile (point r / 3,
+    // component r % 3): its lanes multiply the staged entries with the point's row of sph_grad
+    // and a butterfly adds the lanes' sums up. With WHOLE == false the staged rows begin at
+    // l = H + 1 and closed_form_vjp_kernel has already stored the sum over l <= H, so the
+    // result is added to what xyz_grad holds. Wave 0 stays out: it has loads in flight.
+    auto contract_stage = [&](unsigned n, unsigned buffer) {
+        if constexpr (VJP) {
+            const unsigned valid = valid_in(n);
+            const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
+            const T* staged = lds + buffer * g.rows_elems + g.off_dsph;
+            const T* upstream = sph;
+            T* xyz_grad = dsph;
+            if (wave == 0) return;
+            for (unsigned r = wave - 1; r < valid * 3; r += NT / 64 - 1) {
+                const unsigned s = r / 3;
+                const T* row = staged + r * nrow - skip; // indexed with the entry's index in the full row
+                const T* weight = upstream + (first + s) * ny;
+                T partial = 0;
+#pragma unroll 4
+                for (unsigned k = skip + lane; k < ny; k += 64) {
+                    partial += row[k] * weight[k];
+                }
+                for (unsigned offset = 32; offset > 0; offset >>= 1) {
+                    partial += __shfl_xor(partial, static_cast<int>(offset));
+                }
+                if (lane == 0) {
+                    T* out = xyz_grad + first * 3 + r;
+                    *out = (!WHOLE || g.vjp_accumulate) ? *out + partial : partial;
+                }
+            }
+        }
+    };
+
     // fill the pipeline: tables of tiles 0 and 1, iterates of tile 0
     T rx = 0, ry = 0, rz = 0;
     if (wave == 0) {
@@ -695,7 +743,11 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
                 entry_stage(n, 0);
             }
             __syncthreads(); // rows of tile n complete
-            flush_stage(n, 0, tid, NT, std::false_type{});
+            if constexpr (VJP) {
+                contract_stage(n, 0);
+            } else {
+                flush_stage(n, 0, tid, NT, std::false_type{});
+            }
         }
     }
 }
@@ -1032,10 +1084,10 @@ static hipError_t launch_closed(const Launch& l, const T* xyz, T* sph, T* dsph, 
     return hipGetLastError();
 }
 
-template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT>
+template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false>
 static hipError_t launch_recursion(const Launch& l, const T* xyz, T* sph, T* dsph, T* ddsph,
                                    hipStream_t stream) {
-    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT>;
+    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT, VJP>;
     // The workgroups are persistent: launch exactly as many as are resident at once (registers
     // may allow fewer per CU than LDS does), or the last ones would run alone after the rest.
     unsigned workgroups = l.workgroups;
@@ -1149,6 +1201,13 @@ static int forward(const T* xyz, size_t n_samples, int l_max, int normalized, in
     return status;
 }
 
+// l_max > 6: the gradient kernels with the contraction in place of the flush; the closed forms
+// either inside the recursion kernel or, when its tiles are small, in a launch of their own that
+// stores the sum over l <= 6, to which the recursion kernel then adds the rest.
+template <typename T, bool NORM>
+static hipError_t launch_vjp_recursion(const Plan& plan, const T* xyz, const T* sph_grad, T* xyz_grad,
+                                       int accumulate, hipStream_t stream);
+
 template <typename T, bool NORM, int H>
 static hipError_t launch_vjp(const Launch& l, const T* xyz, const T* sph_grad, T* xyz_grad,
                              int accumulate, hipStream_t stream) {
@@ -1174,17 +1233,27 @@ static hipError_t dispatch_vjp(const Launch& l, int l_max, const T* xyz, const T
     }
 }
 
+template <typename T, bool NORM>
+static hipError_t launch_vjp_recursion(const Plan& plan, const T* xyz, const T* sph_grad, T* xyz_grad,
+                                       int accumulate, hipStream_t stream) {
+    Launch rec = plan.rec;
+    rec.g.vjp_accumulate = accumulate != 0;
+    // the kernel reads its `sph` argument and writes three numbers per point through `dsph`
+    T* upstream = const_cast<T*>(sph_grad);
+    if (plan.whole) {
+        return launch_recursion<T, 1, NORM, true, false, true>(rec, xyz, upstream, xyz_grad, nullptr, stream);
+    }
+    hipError_t e = launch_vjp<T, NORM, 6>(plan.closed, xyz, sph_grad, xyz_grad, accumulate, stream);
+    if (e != hipSuccess) return e;
+    return launch_recursion<T, 1, NORM, false, false, true>(rec, xyz, upstream, xyz_grad, nullptr, stream);
+}
+
 template <typename T>
 static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int normalized,
                T* xyz_grad, int accumulate, void* stream) {
     t_error.clear();
     if (n_samples == 0) return SPHX_OK;
     if (l_max < 0) return fail(SPHX_ERR_ARGUMENT, "l_max must be non-negative");
-    if (l_max > 6) {
-        return fail(SPHX_ERR_UNSUPPORTED,
-                    "the fused vector-Jacobian product covers l_max <= 6; beyond that evaluate the "
-                    "gradients (sphx_forward_*) and contract them (sphx_backward_*)");
-    }
     if (xyz == nullptr || sph_grad == nullptr || xyz_grad == nullptr) {
         return fail(SPHX_ERR_ARGUMENT, "null pointer passed to the vector-Jacobian product");
     }
@@ -1200,13 +1269,21 @@ static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int
         SPHX_HIP(hipSetDevice(device));
     }
     int status = ensure_device_ready(device);
+    Plan plan;
     if (status == SPHX_OK) {
-        Launch l;
-        plan_closed(n_samples, l_max, l_max, 1, sizeof(T), &l);
+        status = make_plan(n_samples, l_max, 1, sizeof(T), g_lds_limit[device], g_compute_units[device],
+                           &plan);
+    }
+    if (status == SPHX_OK) {
         hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-        const hipError_t e = normalized
-                                 ? dispatch_vjp<T, true>(l, l_max, xyz, sph_grad, xyz_grad, accumulate, s)
-                                 : dispatch_vjp<T, false>(l, l_max, xyz, sph_grad, xyz_grad, accumulate, s);
+        hipError_t e;
+        if (plan.closed_only) {
+            e = normalized ? dispatch_vjp<T, true>(plan.closed, l_max, xyz, sph_grad, xyz_grad, accumulate, s)
+                           : dispatch_vjp<T, false>(plan.closed, l_max, xyz, sph_grad, xyz_grad, accumulate, s);
+        } else {
+            e = normalized ? launch_vjp_recursion<T, true>(plan, xyz, sph_grad, xyz_grad, accumulate, s)
+                           : launch_vjp_recursion<T, false>(plan, xyz, sph_grad, xyz_grad, accumulate, s);
+        }
         if (e != hipSuccess) {
             status = fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
         }

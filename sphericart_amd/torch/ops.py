@@ -11,13 +11,11 @@ The backward formulas are the reference's (register.py:82-175). Where it writes
 the vector-Jacobian products as ``torch.sum(grad.unsqueeze(1) * dsph, dim=2)``,
 two more operators, ``contract_gradients`` and ``contract_hessians``, do the
 same sums in one pass over ``dsph`` / ``ddsph`` (``sphx_backward_*``) without
-the product array. For ``l_max <= 6`` the backward pass of the value operators
-does not build ``dsph`` at all: ``*_vjp`` (``sphx_vjp_*``) evaluates the
-gradients in registers and contracts them on the fly. All of these are
-differentiable themselves, so double backward works as it does in the reference.
+the product array. The backward pass of the value operators does not build
+``dsph`` at all: ``*_vjp`` (``sphx_vjp_*``) evaluates the gradients on the chip
+and contracts them on the fly. All of these are differentiable themselves, so
+double backward works as it does in the reference.
 """
-
-FUSED_VJP_LMAX = 6  # what sphx_vjp_* covers
 
 import ctypes
 
@@ -245,7 +243,6 @@ def _register_vjp(prefix):
 
 
 def _register_value_autograd(prefix):
-    gradients = getattr(_ops, f"{prefix}_with_gradients")
     vjp = getattr(_ops, f"{prefix}_vjp")
 
     def setup_context(ctx, inputs, output):
@@ -257,10 +254,7 @@ def _register_value_autograd(prefix):
         if not ctx.needs_input_grad[0] or grad_sph is None:
             return None, None
         (xyz,) = ctx.saved_tensors
-        if ctx.l_max <= FUSED_VJP_LMAX:
-            return vjp(xyz, grad_sph, ctx.l_max), None
-        dsph = gradients(xyz, ctx.l_max)[1]
-        return _ops.contract_gradients(dsph, grad_sph), None
+        return vjp(xyz, grad_sph, ctx.l_max), None
 
     torch.library.register_autograd(f"{NAMESPACE}::{prefix}", backward, setup_context=setup_context)
 

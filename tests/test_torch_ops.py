@@ -111,10 +111,35 @@ def test_fused_vjp_equals_checker_number_for_number(library, oracle, normalized,
             out = torch.from_numpy(start).cuda()
             assert fn(d_xyz.data_ptr(), d_w.data_ptr(), n, l_max, int(normalized), out.data_ptr(), 1, stream) == 0
             np.testing.assert_array_equal(out.cpu().numpy(), want + start)
-    # beyond the closed forms the entry point says so instead of computing
-    assert fn(d_xyz.data_ptr(), d_w.data_ptr(), 10, 7, 1, out.data_ptr(), 0, stream) == 2
-    assert b"l_max <= 6" in library.sphx_last_error()
     assert fn(d_xyz.data_ptr(), d_w.data_ptr(), 0, 3, 1, None, 0, None) == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("normalized", [True, False])
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-5), (np.float64, 1e-12)])
+def test_fused_vjp_beyond_the_closed_forms(library, oracle, normalized, dtype, tol):
+    """l_max > 6: the recursion kernel contracts its staged rows; the terms are added in another
+    order than the checker's loop, so the comparison is relative to the sum of absolute terms."""
+    rng = np.random.default_rng(12)
+    fn = library.sphx_vjp_f32 if dtype == np.float32 else library.sphx_vjp_f64
+    stream = torch.cuda.current_stream().cuda_stream
+    for l_max in (7, 8, 11, 16, 24):
+        for n in (1, 17, 1000, 5003):
+            announce("fused vjp, recursion", normalized, np.dtype(dtype).name, l_max, n)
+            xyz = _points(n, dtype, seed=l_max * 10 + n)
+            weights = rng.standard_normal((n, (l_max + 1) ** 2)).astype(dtype)
+            _, dsph, _ = oracle.compute(xyz, l_max, normalized, "gradients")
+            want = oracle.backward(dsph, weights)
+            scale = np.einsum("iak,ik->ia", np.abs(dsph), np.abs(weights)) + 1
+            d_xyz, d_w = torch.from_numpy(xyz).cuda(), torch.from_numpy(weights).cuda()
+            for accumulate in (0, 1):
+                start = rng.standard_normal((n, 3)).astype(dtype)
+                out = torch.from_numpy(start).cuda()
+                status = fn(d_xyz.data_ptr(), d_w.data_ptr(), n, l_max, int(normalized), out.data_ptr(),
+                            accumulate, stream)
+                assert status == 0, library.sphx_last_error()
+                expect = want + start if accumulate else want
+                assert np.max(np.abs(out.cpu().numpy() - expect) / scale) <= tol, (l_max, n, accumulate)
 
 
 @pytest.mark.gpu
