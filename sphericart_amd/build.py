@@ -32,6 +32,10 @@ FLAGS = [
 ]
 
 
+EXAMPLE_SOURCE = os.path.join(os.path.dirname(HERE), "examples", "device_example.cpp")
+EXAMPLE = os.path.join(HERE, "device_example")
+
+
 def hipcc():
     found = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(found):
@@ -50,7 +54,22 @@ def build(verbose=False, extra_flags=()):
     if verbose and done.stderr:
         # hipcc's host pass does not know the packed-fp32 feature and says so
         print(done.stderr, file=sys.stderr)
+    build_example(verbose)
     return LIBRARY
+
+
+def build_example(verbose=False):
+    """The C++ consumer of the device classes that the GPU tests run (host code only)."""
+    command = [
+        hipcc(), "-O2", "-std=c++17", "-I" + os.path.join(os.path.dirname(HERE), "include"),
+        EXAMPLE_SOURCE, "-L" + HERE, "-lsphericart_amd", "-Wl,-rpath,$ORIGIN", "-o", EXAMPLE,
+    ]
+    if verbose:
+        print(" ".join(command), flush=True)
+    done = subprocess.run(command, capture_output=True, text=True)
+    if done.returncode != 0:
+        raise RuntimeError(f"hipcc failed on the example ({done.returncode}):\n{done.stdout}\n{done.stderr}")
+    return EXAMPLE
 
 
 if __name__ == "__main__":

@@ -42,6 +42,13 @@ def test_cxx_classes_are_exported(library):
         assert f"sphericart::cuda::SphericalHarmonics<double>::{method}(" in out
 
 
+def test_cxx_example_is_built_and_linked_against_the_library():
+    example = os.path.join(ROOT, "sphericart_amd", "device_example")
+    assert os.path.exists(example), "python -m sphericart_amd.build builds it next to the library"
+    needed = subprocess.run(["ldd", example], capture_output=True, text=True, check=True).stdout
+    assert "libsphericart_amd.so" in needed
+
+
 def test_header_compiles_as_c_and_cxx(tmp_path):
     """include/sphericart.h is a C header and a C++ header; sphx_launch.h is plain C."""
     c_file = tmp_path / "probe.c"
