@@ -615,6 +615,22 @@ __device__ __forceinline__ void copy_out(const T* __restrict__ staged, T* __rest
         for (; g < nvec; g += nthreads) {
             emit<T, STREAMING>(in[g], aligned + g);
         }
+    } else if (!PADDED && (reinterpret_cast<uintptr_t>(staged + head) & 15u) == 0) {
+        // staged data and destination at the same position within 16 bytes: vectors on both sides
+        const V* in = reinterpret_cast<const V*>(staged + head);
+        unsigned g = tid;
+        if constexpr (UNROLL > 1) {
+            for (; g + (UNROLL - 1) * nthreads < nvec; g += UNROLL * nthreads) {
+                V v[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) v[u] = in[g + u * nthreads];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) emit<T, STREAMING>(v[u], out - tid + g + u * nthreads);
+            }
+        }
+        for (; g < nvec; g += nthreads) {
+            emit<T, STREAMING>(in[g], out - tid + g);
+        }
     } else if (!PADDED) {
         // staged data and destination differ in their position within 16 bytes: the LDS side
         // is read element by element

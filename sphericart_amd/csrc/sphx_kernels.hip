@@ -354,6 +354,12 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
     const unsigned ny = g.ny;
     const unsigned nrow = WHOLE ? ny : ny - NYH; // staged elements per component row
     const unsigned skip = WHOLE ? 0u : NYH;      // first staged entry of a row
+    // Distance between staged rows. WHOLE == false: the rows are ny apart in HBM but only nrow
+    // long; a stride that equals ny modulo 16 bytes, with the first row placed like its HBM
+    // address modulo 16 bytes, puts every staged row at the same position within 16 bytes as
+    // its destination, so that the copy is 16-byte loads and stores on both sides.
+    constexpr unsigned W16 = 16u / static_cast<unsigned>(sizeof(T));
+    const unsigned row_stride = nrow + skip % W16;
     const unsigned tri_all = (L + 1) * (L + 2) / 2;
 
     T* F = lds + g.off_F;
@@ -504,9 +510,11 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         // WHOLE: element 0 of a staging region stands for the start of the 128-byte line in
         // which the tile's run begins in HBM, so the run itself starts `phase` elements in
         const unsigned long long first_point = static_cast<unsigned long long>(tile_of(n)) * S;
-        // (VJP: the rows never leave LDS, no position to match)
-        const unsigned phase_sph = WHOLE && !VJP ? phase_of(sph, first_point * ny) : 0u;
-        const unsigned phase_dsph = WHOLE && !VJP && MODE >= 1 ? phase_of(dsph, first_point * 3 * ny) : 0u;
+        // (WHOLE == false: position within 16 bytes of the first staged row, see row_stride;
+        // VJP: the rows never leave LDS, no position to match)
+        const unsigned phase_sph = VJP ? 0u : phase_of(sph, first_point * ny + skip) % (WHOLE ? LINE : W16);
+        const unsigned phase_dsph =
+            VJP || MODE < 1 ? 0u : phase_of(dsph, first_point * 3 * ny + skip) % (WHOLE ? LINE : W16);
         const unsigned phase_ddsph = WHOLE && !VJP && MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
         if constexpr (WHOLE) {
             if (t < valid) {
@@ -555,10 +563,10 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
             // rows are addressed with the entry's index in the full row; shift the bases when
             // the staged rows start at l = H + 1
             Rows<T> rows;
-            rows.ny = static_cast<int>(nrow);
-            rows.sph = staged + phase_sph + s * nrow - skip;
-            rows.dsph = staged + g.off_dsph + phase_dsph + s * 3 * nrow - skip;
-            rows.ddsph = staged + g.off_ddsph + phase_ddsph + s * 9 * nrow - skip;
+            rows.ny = static_cast<int>(row_stride);
+            rows.sph = staged + phase_sph + s * row_stride - skip;
+            rows.dsph = staged + g.off_dsph + phase_dsph + s * 3 * row_stride - skip;
+            rows.ddsph = staged + g.off_ddsph + phase_ddsph + s * 9 * row_stride - skip;
             for (unsigned e = e_first; e < g.jobs_per_point; e += wide_lanes) {
                 const unsigned packed = job_table[e];
                 const int m = static_cast<int>(packed & 0x7fu);
@@ -646,14 +654,14 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
             for (unsigned r = ft >> 6; r < valid * components_of(MODE); r += waves) {
                 // rows [0, valid) are values, the next 3 * valid are gradients
                 if (r < valid) {
-                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL>(staged + r * nrow,
-                                                              sph + (first + r) * ny + skip, nrow, nrow,
-                                                              0, 0, ft & 63u, 64);
+                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL>(
+                        staged + phase_of(sph, first * ny + skip) % W16 + r * row_stride,
+                        sph + (first + r) * ny + skip, nrow, nrow, 0, 0, ft & 63u, 64);
                 } else {
                     const unsigned q = r - valid;
-                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL>(staged + g.off_dsph + q * nrow,
-                                                              dsph + (first * 3 + q) * ny + skip, nrow,
-                                                              nrow, 0, 0, ft & 63u, 64);
+                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL>(
+                        staged + g.off_dsph + phase_of(dsph, first * 3 * ny + skip) % W16 + q * row_stride,
+                        dsph + (first * 3 + q) * ny + skip, nrow, nrow, 0, 0, ft & 63u, 64);
                 }
             }
         }
@@ -675,7 +683,7 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
             if (wave == 0) return;
             for (unsigned r = wave - 1; r < valid * 3; r += NT / 64 - 1) {
                 const unsigned s = r / 3;
-                const T* row = staged + r * nrow - skip; // indexed with the entry's index in the full row
+                const T* row = staged + r * row_stride - skip; // indexed with the entry's index in the full row
                 const T* weight = upstream + (first + s) * ny;
                 T partial = 0;
 #pragma unroll 4
@@ -870,7 +878,10 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     bool may_split = mode == 2 && env_int("SPHX_SPLIT_SIDES", 1) != 0;
     auto table_elems_for = [&](bool split) { return ((split ? jobs_split : jobs) * 4 + esize - 1) / esize; };
     // per point: the rows in every row buffer, point tables three times, iterates twice
-    const unsigned rows_per_point = components_of(mode) * nrow;
+    // staged rows are `row_stride` apart (recursion_kernel): nrow, or a little more when the rows
+    // are cut so that they keep their position within 16 bytes
+    const unsigned row_stride = nrow + (whole ? 0u : nyh % (16u / esize));
+    const unsigned rows_per_point = components_of(mode) * row_stride;
     const unsigned rest_per_point = 3 * (8 + 3 * (l_max + 1)) + 2 * arrays * tri_all;
     unsigned fixed = 0;
     auto bytes_for = [&](unsigned S, unsigned buffers) {
@@ -932,12 +943,12 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
 
     // in front of every staging region, room for the part of a 128-byte line that precedes the
     // tile's run (recursion_kernel, flush_run)
-    const unsigned line = whole ? 128u / esize : 0u;
-    unsigned at = align4(S * nrow + line);
+    const unsigned line = whole ? 128u / esize : 16u / esize;
+    unsigned at = align4(S * row_stride + line);
     g.off_dsph = at;
-    if (mode >= 1) at = align4(at + S * 3 * nrow + line);
+    if (mode >= 1) at = align4(at + S * 3 * row_stride + line);
     g.off_ddsph = at;
-    if (mode == 2) at = align4(at + S * 9 * nrow + line);
+    if (mode == 2) at = align4(at + S * 9 * row_stride + line);
     g.rows_elems = at;
     at *= buffers;
     g.off_F = at;
