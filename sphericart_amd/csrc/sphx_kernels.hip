@@ -70,6 +70,7 @@ struct Tiling {
     unsigned sequence_waves; // waves that run the bare recursions (1 or 2)
     unsigned points_per_pass; // points whose entry jobs fit side by side in the wide waves (>= 1)
     unsigned vjp_accumulate; // fused product: add to xyz_grad instead of overwriting it
+    unsigned az_shift;      // the point tables are made for 2^az_shift tiles at a time
     unsigned chunk_shift;   // a workgroup takes 2^chunk_shift consecutive tiles at a time
     unsigned row_buffers;   // 2: tile n is flushed while tile n+1 is computed; 1: one after the other
     unsigned flush_waves;   // waves that do nothing but flush (row_buffers == 2)
@@ -398,8 +399,16 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
 
     // per point: 8 numbers (x, y, z, x^2, y^2, z^2, 1/r, x^2 + y^2), then c, s, 2(m+1)z
     const unsigned point_stride = 8 + 3 * (L + 1);
-    auto point_data = [&](unsigned buffer, unsigned s) -> T* {
-        return lds + g.off_pts + (buffer * S + s) * point_stride;
+    // The tables are made for 2^az_shift tiles at a time (a batch), one lane per point, so that
+    // the recurrences, a chain of dependent operations that few lanes share, run once per batch
+    // instead of once per tile. Single tiles are made two rounds ahead and kept in three
+    // buffers; batches are made one batch ahead and kept in two.
+    const unsigned batch_tiles = 1u << g.az_shift;
+    const unsigned batch_lead = batch_tiles == 1 ? 2u : 1u;
+    const unsigned batch_buffers = batch_tiles == 1 ? 3u : 2u;
+    auto point_data = [&](unsigned n, unsigned s) -> T* { // point s of this workgroup's n-th tile
+        const unsigned slot = (((n >> g.az_shift) % batch_buffers) << g.az_shift) | (n & (batch_tiles - 1u));
+        return lds + g.off_pts + (slot * S + s) * point_stride;
     };
     auto iterates = [&](unsigned buffer, unsigned s, unsigned which, int l) -> T* {
         return lds + g.off_iter + ((buffer * S + s) * ARRAYS + which) * tri_all + l * (l + 1) / 2;
@@ -431,19 +440,24 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         const unsigned long long left = g.n_samples - first;
         return left < S ? static_cast<unsigned>(left) : S;
     };
-    auto fetch = [&](unsigned n, T& rx, T& ry, T& rz) {
+    // lane j of wave 0 takes point j % S of tile j / S of a batch (batch_tiles * S <= 64)
+    auto fetch = [&](unsigned batch, T& rx, T& ry, T& rz) {
         rx = ry = rz = 0;
-        if (lane < valid_in(n)) {
-            const T* src = xyz + (static_cast<unsigned long long>(tile_of(n)) * S + lane) * 3;
+        const unsigned n = (batch << g.az_shift) + lane / S;
+        const unsigned s = lane % S;
+        if (lane < batch_tiles * S && s < valid_in(n)) {
+            const T* src = xyz + (static_cast<unsigned long long>(tile_of(n)) * S + s) * 3;
             rx = src[0];
             ry = src[1];
             rz = src[2];
         }
     };
-    // stage one of tile n (wave 0; lane == tid there)
-    auto azimuth_stage = [&](unsigned n, T rx, T ry, T rz) {
-        if (lane < valid_in(n)) {
-            T* rec = point_data(n % 3u, lane);
+    // stage one of a batch of tiles (wave 0; lane == tid there)
+    auto azimuth_stage = [&](unsigned batch, T rx, T ry, T rz) {
+        const unsigned n = (batch << g.az_shift) + lane / S;
+        const unsigned s = lane % S;
+        if (lane < batch_tiles * S && s < valid_in(n)) {
+            T* rec = point_data(n, s);
             Point<T> p;
             p.x = rx;
             p.y = ry;
@@ -483,7 +497,7 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
             const int l = L - static_cast<int>(step); // longest recursions first
             const unsigned s = rest / ARRAYS;
             const unsigned which = rest - s * ARRAYS;
-            const T* rec = point_data(n % 3u, s);
+            const T* rec = point_data(n, s);
             sequence_job<T>(l, static_cast<int>(which), rec[2], rec[7], Q, rec + 8 + 2 * (L + 1),
                             iterates(n & 1u, s, which, l));
         }
@@ -518,7 +532,7 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         const unsigned phase_ddsph = WHOLE && !VJP && MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
         if constexpr (WHOLE) {
             if (t < valid) {
-                const T* rec = point_data(n % 3u, t);
+                const T* rec = point_data(n, t);
                 Point<T> p;
                 p.x = rec[0];
                 p.y = rec[1];
@@ -546,7 +560,7 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         for (unsigned s0 = 0; s0 < valid; s0 += g.points_per_pass) {
             const unsigned s = s0 + local;
             if (s >= valid || local >= g.points_per_pass) continue;
-            const T* rec = point_data(n % 3u, s);
+            const T* rec = point_data(n, s);
             Point<T> p;
             p.x = rec[0];
             p.y = rec[1];
@@ -708,10 +722,12 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         azimuth_stage(0, rx, ry, rz);
         fetch(1, rx, ry, rz);
     }
-    __syncthreads(); // prefactor tables, job table, tables of tile 0
+    __syncthreads(); // prefactor tables, job table, tables of batch 0
     if (wave == 0) {
-        azimuth_stage(1, rx, ry, rz);
-        fetch(2, rx, ry, rz);
+        if (batch_lead == 2) {
+            azimuth_stage(1, rx, ry, rz);
+            fetch(2, rx, ry, rz);
+        }
     } else if (wave < entry_first_wave) {
         recursion_stage(0);
     }
@@ -726,8 +742,10 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
             const unsigned before = n > 0 ? valid_in(n - 1) : 0u;
             if (valid == 0 && before == 0) break;
             if (wave == 0) {
-                azimuth_stage(n + 2, rx, ry, rz);
-                fetch(n + 3, rx, ry, rz); // needed one round from now
+                if ((n & (batch_tiles - 1u)) == 0) {
+                    azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
+                    fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz); // for the next batch
+                }
             } else if (wave < entry_first_wave) {
                 recursion_stage(n + 1);
             } else if (wave < entry_end_wave) {
@@ -743,8 +761,10 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
         for (unsigned n = 0; valid_in(n) != 0; ++n) {
             __syncthreads(); // tables of tile n+1, iterates of tile n in place; rows of tile n-1 flushed
             if (wave == 0) {
-                azimuth_stage(n + 2, rx, ry, rz);
-                fetch(n + 3, rx, ry, rz);
+                if ((n & (batch_tiles - 1u)) == 0) {
+                    azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
+                    fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz);
+                }
             } else if (wave < entry_first_wave) {
                 recursion_stage(n + 1);
             } else {
@@ -920,10 +940,31 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         S = static_cast<unsigned>(forced);
     }
 
+    // Point tables for several tiles at a time (recursion_kernel, az_shift): as many tiles as
+    // wave 0 has lanes for, eight at most, as long as the larger table area keeps the workgroup
+    // within the budget (or within what it needs anyway).
+    const unsigned point_record = 8 + 3 * static_cast<unsigned>(l_max + 1);
+    unsigned az_shift = 0;
+    {
+        const unsigned allowed = bytes_for(S, buffers) > budget ? bytes_for(S, buffers) : budget;
+        const int cap = env_int("SPHX_AZ_SHIFT", 3);
+        for (unsigned shift = cap < 0 ? 0u : (cap > 6 ? 6u : static_cast<unsigned>(cap)); shift >= 1; --shift) {
+            const unsigned tiles = 1u << shift;
+            if (tiles * S > 64) continue;
+            const unsigned extra = (2 * tiles - 3) * S * point_record * esize;
+            if (bytes_for(S, buffers) + extra <= allowed || bytes_for(S, buffers) + extra <= budget) {
+                az_shift = shift;
+                break;
+            }
+        }
+    }
+    const unsigned table_slots = az_shift == 0 ? 3u : 2u << az_shift;
+
     g.n_samples = n_samples;
     g.l_max = l_max;
     g.ny = static_cast<int>(ny);
     g.tile = static_cast<int>(S);
+    g.az_shift = az_shift;
     g.row_buffers = buffers;
     g.flush_waves = buffers == 2 ? static_cast<unsigned>(env_int("SPHX_FLUSH_WAVES", 1)) : 0u;
     if (g.flush_waves > 2) g.flush_waves = 2;
@@ -956,7 +997,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.off_Q = at;
     at += tri_all;
     g.off_pts = at;
-    at += 3 * S * (8 + 3 * (l_max + 1));
+    at += table_slots * S * point_record;
     g.off_iter = at;
     at += 2 * S * arrays * tri_all;
     g.off_jobs = at;
