@@ -164,7 +164,11 @@ __device__ __forceinline__ void stage(const Rows<T>& out, int k, const Point<T>&
 // All (H+1)^2 values and, if asked, their gradients stay in VGPRs until they
 // are staged. Second derivatives of l <= 1 vanish identically
 // (macros.hpp:56-131), which is the only case MODE == 2 reaches here.
-template <typename T, int MODE, bool NORM, int H>
+// KLO, KHI: only the entries KLO <= k < KHI are staged. The closed forms of one l use values of
+// lower l but hardly any gradients of lower l, so what a slice does not stage the compiler
+// drops: several waves can share the entries of a point, each evaluating little more than its
+// own slice.
+template <typename T, int MODE, bool NORM, int H, int KLO = 0, int KHI = (H + 1) * (H + 1)>
 __device__ __forceinline__ void closed_form_job(const Point<T>& p, const Rows<T>& out) {
     static_assert(MODE < 2 || H <= 1, "second derivatives in closed form stop at l = 1");
     constexpr int NH = (H + 1) * (H + 1);
@@ -172,14 +176,14 @@ __device__ __forceinline__ void closed_form_job(const Point<T>& p, const Rows<T>
     low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
     if constexpr (MODE == 0) {
 #pragma unroll
-        for (int k = 0; k < NH; ++k) {
+        for (int k = KLO; k < KHI; ++k) {
             out.sph[k] = Y[k];
         }
     } else {
         T DX[NH], DY[NH], DZ[NH];
         low_gradients<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y, DX, DY, DZ);
 #pragma unroll
-        for (int k = 0; k < NH; ++k) {
+        for (int k = KLO; k < KHI; ++k) {
             Entry<T> e;
             e.v = Y[k];
             e.gx = DX[k];

@@ -531,8 +531,12 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
             VJP || MODE < 1 ? 0u : phase_of(dsph, first_point * 3 * ny + skip) % (WHOLE ? LINE : W16);
         const unsigned phase_ddsph = WHOLE && !VJP && MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
         if constexpr (WHOLE) {
-            if (t < valid) {
-                const T* rec = point_data(n, t);
+            // closed forms: one lane per point; the entries of a point in slices (by l) that the
+            // entry waves share, so that no single wave carries all of the chain rule and staging
+            const unsigned entry_wave = t >> 6;
+            const unsigned entry_waves = wide_lanes >> 6;
+            if (lane < valid) {
+                const T* rec = point_data(n, lane);
                 Point<T> p;
                 p.x = rec[0];
                 p.y = rec[1];
@@ -543,10 +547,17 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
                 p.ir = rec[6];
                 Rows<T> rows;
                 rows.ny = static_cast<int>(ny);
-                rows.sph = staged + phase_sph + t * ny;
-                rows.dsph = staged + g.off_dsph + phase_dsph + t * 3 * ny;
-                rows.ddsph = staged + g.off_ddsph + phase_ddsph + t * 9 * ny;
-                closed_form_job<T, MODE, NORM, H>(p, rows);
+                rows.sph = staged + phase_sph + lane * ny;
+                rows.dsph = staged + g.off_dsph + phase_dsph + lane * 3 * ny;
+                rows.ddsph = staged + g.off_ddsph + phase_ddsph + lane * 9 * ny;
+                if constexpr (H == 6) {
+                    if (0 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 0, 16>(p, rows);
+                    if (1 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows);
+                    if (2 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 25, 36>(p, rows);
+                    if (3 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 36, 49>(p, rows);
+                } else {
+                    if (entry_wave == 0) closed_form_job<T, MODE, NORM, H>(p, rows);
+                }
             }
         }
         // One pass takes the jobs of as many points as fit side by side in the wide lanes
@@ -1047,7 +1058,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
         plan_closed(n_samples, l_max, l_max, mode, elem, &plan->closed);
         return SPHX_OK;
     }
-    const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", 76 * 1024));
+    const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", 80 * 1024));
     bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
                                &plan->split_sides);
     // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of
