@@ -336,8 +336,13 @@ __global__ __launch_bounds__(64) void closed_form_vjp_kernel(Tiling g, const T* 
 // ---------------------------------------------------------------------------
 constexpr unsigned kRecursionThreads = 512;
 
+// Values and gradients: at most 128 registers, so that two workgroups share a CU (four waves
+// per SIMD) wherever their LDS allows. Only the float64 closed forms exceed that on their own
+// and spill a few registers; with 170 registers and one workgroup per CU, l_max = 12 float64
+// gradients took 800 us instead of 513 us. The second-derivative kernels keep what they need
+// (forced to 128 they spill in the entry jobs: 918 us against 558 us at l_max = 10, float64).
 template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false>
-__global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, const T* __restrict__ xyz,
+__global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling g, const T* __restrict__ xyz,
                                                                      T* __restrict__ sph,
                                                                      T* __restrict__ dsph,
                                                                      T* __restrict__ ddsph) {
@@ -551,10 +556,14 @@ __global__ __launch_bounds__(kRecursionThreads) void recursion_kernel(Tiling g, 
                 rows.dsph = staged + g.off_dsph + phase_dsph + lane * 3 * ny;
                 rows.ddsph = staged + g.off_ddsph + phase_ddsph + lane * 9 * ny;
                 if constexpr (H == 6) {
-                    if (0 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 0, 16>(p, rows);
-                    if (1 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows);
-                    if (2 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 25, 36>(p, rows);
-                    if (3 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 36, 49>(p, rows);
+                    if (0 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows);
+                    if (1 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows);
+                    if (2 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows);
+                    if (3 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows);
+                    if (4 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows);
+                    if (5 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows);
+                    if (6 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows);
+                    if (7 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows);
                 } else {
                     if (entry_wave == 0) closed_form_job<T, MODE, NORM, H>(p, rows);
                 }
@@ -1061,10 +1070,14 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", 80 * 1024));
     bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
                                &plan->split_sides);
-    // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of
-    // a wave idle for a thousand instructions per tile: hand them to the closed-form kernel,
-    // which runs them 64 points at a time, and let the recursion kernel stage l >= 7 only.
-    const int split_below = env_int("SPHX_SPLIT_BELOW", 16);
+    // With very few points per tile the one-lane-per-point closed forms of l <= 6 would leave
+    // most of the lanes idle for some two thousand instructions per tile: hand them to the
+    // closed-form kernel, which runs them 64 points at a time, and let the recursion kernel stage
+    // l >= 7 only. The price is rows cut in two, each part a run of its own in HBM, so the
+    // threshold is low (measured, 1M/500k/200k points, gradients: float32 l_max = 16, 8 points
+    // per tile, 812 us whole against 1110 us cut; l_max = 24, 4 points, 593 against 729;
+    // float64 l_max = 12, 8 points, 513 against 655; l_max = 20, 2 points, 1801 against 1018).
+    const int split_below = env_int("SPHX_SPLIT_BELOW", elem == 4 ? 4 : 8);
     if (mode < 2 && (!fits || plan->rec.g.tile < split_below)) {
         Launch upper;
         if (plan_recursion(n_samples, l_max, mode, false, elem, budget, lds_limit, cus, &upper,
