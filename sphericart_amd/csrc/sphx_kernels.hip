@@ -556,14 +556,31 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
                 rows.dsph = staged + g.off_dsph + phase_dsph + lane * 3 * ny;
                 rows.ddsph = staged + g.off_ddsph + phase_ddsph + lane * 9 * ny;
                 if constexpr (H == 6) {
-                    if (0 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows);
-                    if (1 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows);
-                    if (2 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows);
-                    if (3 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows);
-                    if (4 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows);
-                    if (5 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows);
-                    if (6 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows);
-                    if (7 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows);
+                    // float32 rows a multiple of 32 words long (l_max = 7, 15, 23, ...): the
+                    // stores of all lanes would fall on one LDS bank; stored in rotated fours
+                    // instead (closed_form_job; l_max = 7, 500k points, gradients: 343 -> 216 us).
+                    // Not for float64 and not for values alone, where the selects cost registers
+                    // that the kernel does not have to spare (values: 68 -> 89, and l_max = 9 lost
+                    // its third workgroup per CU, 80 -> 106 us).
+                    constexpr bool MAY_ROTATE = sizeof(T) == 4 && MODE == 1;
+                    if (MAY_ROTATE && (ny & 31u) == 0) {
+                        const unsigned turn = lane & 3u;
+                        if (0 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 0, 8, true>(p, rows, turn);
+                        if (1 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 8, 16, true>(p, rows, turn);
+                        if (2 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 16, 24, true>(p, rows, turn);
+                        if (3 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 24, 32, true>(p, rows, turn);
+                        if (4 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 32, 40, true>(p, rows, turn);
+                        if (5 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 40, 49, true>(p, rows, turn);
+                    } else {
+                        if (0 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows);
+                        if (1 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows);
+                        if (2 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows);
+                        if (3 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows);
+                        if (4 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows);
+                        if (5 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows);
+                        if (6 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows);
+                        if (7 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows);
+                    }
                 } else {
                     if (entry_wave == 0) closed_form_job<T, MODE, NORM, H>(p, rows);
                 }
