@@ -111,6 +111,32 @@ SPHX_EXPORT int sphx_vjp_f32(const float* xyz, const float* sph_grad, size_t n_s
 SPHX_EXPORT int sphx_vjp_f64(const double* xyz, const double* sph_grad, size_t n_samples, int l_max,
                              int normalized, double* xyz_grad, int accumulate, void* stream);
 
+/* float32 arrays, evaluated in float64 and rounded once: what sphx_forward_f64
+ * returns for the same points, converted to float (round to nearest even).
+ * For callers that need float32 storage beyond the range of float32
+ * arithmetic: evaluated in float, the prefactors and Q_l^l = (2l-1)!! of
+ * sphericart/include/templates.hpp:54-97 overflow from l = 29 (the outputs of
+ * the reference and of sphx_forward_f32 hold NaN and inf there) and underflow
+ * to exact zeros at high |m| from l of about 20. No counterpart in the
+ * reference; never chosen implicitly, since parity with the reference is
+ * defined on sphx_forward_f32.
+ *
+ *   workspace        device memory, 16-byte aligned, of workspace_bytes bytes;
+ *                    the points are processed in chunks of as many as it holds
+ *                    (8 * (3 + (l_max+1)^2 * {1, 4, 13}) bytes each), enqueued
+ *                    one after the other on `stream`. NULL: the call allocates
+ *                    a workspace of its own (at most 256 MiB), waits for the
+ *                    stream and frees it, i.e. it is then synchronous.
+ *
+ * sphx_forward_f32_via_f64_workspace returns the size with which n_samples
+ * points are one chunk (0 for invalid arguments). Costs the float64 evaluation
+ * plus one pass over the float64 rows. */
+SPHX_EXPORT int sphx_forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max,
+                                         int normalized, int derivatives, float* sph, float* dsph,
+                                         float* ddsph, void* workspace, size_t workspace_bytes,
+                                         void* stream);
+SPHX_EXPORT size_t sphx_forward_f32_via_f64_workspace(size_t n_samples, int l_max, int derivatives);
+
 /* Host copy of the prefactor table the kernels use for this l_max: the F_l^m
  * block followed by the Q_l^m-recursion block, (l_max+1)(l_max+2) numbers.
  * Replaces compute_sph_prefactors<T> (sphericart/include/templates.hpp:54-97)

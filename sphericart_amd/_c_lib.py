@@ -30,6 +30,8 @@ LAUNCH_SYMBOLS = [
     "sphx_backward_second_f64",
     "sphx_vjp_f32",
     "sphx_vjp_f64",
+    "sphx_forward_f32_via_f64",
+    "sphx_forward_f32_via_f64_workspace",
     "sphx_prefactors_f32",
     "sphx_prefactors_f64",
     "sphx_device_count",
@@ -72,6 +74,11 @@ def _declare(lib):
         fn = getattr(lib, f"sphx_prefactors_{suffix}")
         fn.restype = c_int
         fn.argtypes = [c_int, c_void_p]
+    lib.sphx_forward_f32_via_f64.restype = c_int
+    lib.sphx_forward_f32_via_f64.argtypes = [
+        c_void_p, c_size_t, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]
+    lib.sphx_forward_f32_via_f64_workspace.restype = c_size_t
+    lib.sphx_forward_f32_via_f64_workspace.argtypes = [c_size_t, c_int, c_int]
     lib.sphx_device_count.restype = c_int
     lib.sphx_device_count.argtypes = []
     lib.sphx_last_error.restype = ctypes.c_char_p

@@ -1390,6 +1390,145 @@ static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int
     return status;
 }
 
+// ---------------------------------------------------------------------------
+// float32 arrays evaluated in float64. In float32 the reference's prefactors
+// and Q_l^l = (2l-1)!! leave the range of the type from l = 29 (NaN and inf in
+// the outputs) and high-|m| entries come out as exact zeros from l of about 20
+// (sphericart/include/templates.hpp:54-97 evaluated in float). This path, which
+// a caller must ask for, widens xyz, runs the float64 kernels into a workspace
+// and rounds every result once.
+// ---------------------------------------------------------------------------
+constexpr unsigned kConvertThreads = 256;
+
+__global__ __launch_bounds__(kConvertThreads) void widen_kernel(const float* __restrict__ in,
+                                                               double* __restrict__ out,
+                                                               unsigned long long count) {
+    const unsigned long long stride = static_cast<unsigned long long>(gridDim.x) * kConvertThreads;
+    for (unsigned long long i = static_cast<unsigned long long>(blockIdx.x) * kConvertThreads + threadIdx.x;
+         i < count; i += stride) {
+        out[i] = static_cast<double>(in[i]);
+    }
+}
+
+__global__ __launch_bounds__(kConvertThreads) void narrow_kernel(const double* __restrict__ in,
+                                                                float* __restrict__ out,
+                                                                unsigned long long count) {
+    const unsigned long long stride = static_cast<unsigned long long>(gridDim.x) * kConvertThreads;
+    for (unsigned long long i = static_cast<unsigned long long>(blockIdx.x) * kConvertThreads + threadIdx.x;
+         i < count; i += stride) {
+        out[i] = static_cast<float>(in[i]); // round to nearest even, overflow to infinity
+    }
+}
+
+static unsigned convert_blocks(unsigned long long count) {
+    const unsigned long long want = (count + kConvertThreads - 1) / kConvertThreads;
+    return static_cast<unsigned>(want < 16384ull ? (want ? want : 1ull) : 16384ull);
+}
+
+// float64 bytes one point needs in the workspace: its coordinates and its rows
+static size_t via_f64_bytes_per_point(int l_max, int mode) {
+    const size_t ny = static_cast<size_t>(l_max + 1) * (l_max + 1);
+    return sizeof(double) * (3 + ny * components_of(mode));
+}
+
+static int forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, int normalized, int mode,
+                               float* sph, float* dsph, float* ddsph, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+    t_error.clear();
+    if (n_samples == 0) return SPHX_OK;
+    if (l_max < 0) return fail(SPHX_ERR_ARGUMENT, "l_max must be non-negative");
+    if (mode < 0 || mode > 2) return fail(SPHX_ERR_ARGUMENT, "unknown derivative selector");
+    if (l_max > SPHX_TABLE_LMAX) {
+        return fail(SPHX_ERR_UNSUPPORTED, "l_max = " + std::to_string(l_max) +
+                                              " exceeds the device prefactor tables (" +
+                                              std::to_string(SPHX_TABLE_LMAX) + ")");
+    }
+    if (xyz == nullptr) return fail(SPHX_ERR_ARGUMENT, "xyz is a null pointer");
+    if (sph == nullptr) return fail(SPHX_ERR_ARGUMENT, "sph is a null pointer");
+    if (mode >= 1 && dsph == nullptr) return fail(SPHX_ERR_ARGUMENT, "dsph is a null pointer");
+    if (mode >= 2 && ddsph == nullptr) return fail(SPHX_ERR_ARGUMENT, "ddsph is a null pointer");
+
+    hipPointerAttribute_t attr;
+    SPHX_HIP(hipPointerGetAttributes(&attr, xyz));
+    int current = 0;
+    SPHX_HIP(hipGetDevice(&current));
+    const int device = attr.device;
+    if (device != current) SPHX_HIP(hipSetDevice(device));
+
+    const size_t per_point = via_f64_bytes_per_point(l_max, mode);
+    const size_t ny = static_cast<size_t>(l_max + 1) * (l_max + 1);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    int status = SPHX_OK;
+    void* owned = nullptr;
+    if (workspace == nullptr) {
+        // no workspace given: one of our own for at most 256 MiB worth of points at a time
+        size_t points = (size_t(256) << 20) / per_point;
+        if (points < 64) points = 64;
+        if (points > n_samples) points = n_samples;
+        workspace_bytes = points * per_point;
+        hipError_t e = hipMalloc(&owned, workspace_bytes);
+        if (e != hipSuccess) {
+            status = fail(SPHX_ERR_HIP, std::string("hipMalloc of the float64 workspace: ") + hipGetErrorString(e));
+        }
+        workspace = owned;
+    }
+    size_t chunk = workspace_bytes / per_point;
+    if (status == SPHX_OK && chunk == 0) {
+        status = fail(SPHX_ERR_ARGUMENT, "the workspace holds no point: " + std::to_string(per_point) +
+                                             " bytes are needed per point");
+    }
+    if (status == SPHX_OK && (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
+        status = fail(SPHX_ERR_ARGUMENT, "the workspace must be aligned to 16 bytes");
+    }
+    if (chunk > n_samples) chunk = n_samples;
+    if (chunk >= 64) chunk &= ~size_t(63); // whole tiles of the closed-form kernels
+    // workspace layout for a chunk of c points: sph[c][ny], dsph[c][3][ny], ddsph[c][9][ny], xyz[c][3]
+    double* w_sph = static_cast<double*>(workspace);
+    double* w_dsph = w_sph + chunk * ny;
+    double* w_ddsph = w_dsph + (mode >= 1 ? chunk * 3 * ny : 0);
+    double* w_xyz = w_ddsph + (mode >= 2 ? chunk * 9 * ny : 0);
+    for (size_t first = 0; status == SPHX_OK && first < n_samples; first += chunk) {
+        const size_t count = n_samples - first < chunk ? n_samples - first : chunk;
+        hipLaunchKernelGGL(widen_kernel, dim3(convert_blocks(count * 3)), dim3(kConvertThreads), 0, s,
+                           xyz + first * 3, w_xyz, static_cast<unsigned long long>(count * 3));
+        status = forward<double>(w_xyz, count, l_max, normalized, mode, w_sph, mode >= 1 ? w_dsph : nullptr,
+                                 mode >= 2 ? w_ddsph : nullptr, stream);
+        if (status != SPHX_OK) break;
+        hipLaunchKernelGGL(narrow_kernel, dim3(convert_blocks(count * ny)), dim3(kConvertThreads), 0, s,
+                           w_sph, sph + first * ny, static_cast<unsigned long long>(count * ny));
+        if (mode >= 1) {
+            hipLaunchKernelGGL(narrow_kernel, dim3(convert_blocks(count * 3 * ny)), dim3(kConvertThreads), 0,
+                               s, w_dsph, dsph + first * 3 * ny, static_cast<unsigned long long>(count * 3 * ny));
+        }
+        if (mode >= 2) {
+            hipLaunchKernelGGL(narrow_kernel, dim3(convert_blocks(count * 9 * ny)), dim3(kConvertThreads), 0,
+                               s, w_ddsph, ddsph + first * 9 * ny, static_cast<unsigned long long>(count * 9 * ny));
+        }
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            status = fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
+        }
+    }
+    if (owned != nullptr) {
+        // our own workspace: wait for the work that uses it, then give it back
+        hipError_t e = hipStreamSynchronize(s);
+        if (e != hipSuccess && status == SPHX_OK) {
+            status = fail(SPHX_ERR_HIP, std::string("hipStreamSynchronize: ") + hipGetErrorString(e));
+        }
+        e = hipFree(owned);
+        if (e != hipSuccess && status == SPHX_OK) {
+            status = fail(SPHX_ERR_HIP, std::string("hipFree: ") + hipGetErrorString(e));
+        }
+    }
+    if (device != current) {
+        hipError_t e = hipSetDevice(current);
+        if (e != hipSuccess && status == SPHX_OK) {
+            status = fail(SPHX_ERR_HIP, std::string("hipSetDevice: ") + hipGetErrorString(e));
+        }
+    }
+    return status;
+}
+
 } // namespace sphx
 
 extern "C" {
@@ -1404,6 +1543,18 @@ int sphx_forward_f64(const double* xyz, size_t n_samples, int l_max, int normali
                      int derivatives, double* sph, double* dsph, double* ddsph, void* stream) {
     return sphx::forward<double>(xyz, n_samples, l_max, normalized, derivatives, sph, dsph, ddsph,
                                  stream);
+}
+
+int sphx_forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, int normalized,
+                             int derivatives, float* sph, float* dsph, float* ddsph, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+    return sphx::forward_f32_via_f64(xyz, n_samples, l_max, normalized, derivatives, sph, dsph, ddsph,
+                                     workspace, workspace_bytes, stream);
+}
+
+size_t sphx_forward_f32_via_f64_workspace(size_t n_samples, int l_max, int derivatives) {
+    if (l_max < 0 || derivatives < 0 || derivatives > 2) return 0;
+    return n_samples * sphx::via_f64_bytes_per_point(l_max, derivatives);
 }
 
 int sphx_vjp_f32(const float* xyz, const float* sph_grad, size_t n_samples, int l_max, int normalized,

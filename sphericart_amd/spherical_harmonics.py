@@ -10,11 +10,16 @@ from ._c_lib import get_library
 class _BaseHarmonics:
     # reference: python/src/sphericart/spherical_harmonics.py:9-202
     _cuda_prefix = ""
+    _normalized = 0
 
-    def __init__(self, l_max: int):
+    def __init__(self, l_max: int, float32_via_float64: bool = False):
+        """``float32_via_float64`` (not in the reference, off by default): float32 arrays are
+        evaluated in float64 and rounded once (``sphx_forward_f32_via_f64``), which keeps
+        l_max >= 29 finite where float32 arithmetic, the reference's included, overflows."""
         if int(l_max) != l_max or l_max < 0:
             raise ValueError("l_max must be a non-negative integer")
         self._l_max = int(l_max)
+        self._float32_via_float64 = bool(float32_via_float64)
         self._lib = get_library()
         self._calculator_cuda = None
         self._calculator_cuda_f = None
@@ -67,6 +72,10 @@ class _BaseHarmonics:
         dsph = torch.empty((n_samples, 3, lmtotal), **options) if gradients else None
         ddsph = torch.empty((n_samples, 3, 3, lmtotal), **options) if hessians else None
 
+        if self._float32_via_float64 and xyz.dtype == torch.float32 and n_samples > 0:
+            self._compute_via_float64(xyz, sph, dsph, ddsph)
+            return (sph, dsph, ddsph) if hessians else (sph, dsph) if gradients else sph
+
         with torch.cuda.device(xyz.device):
             stream = torch.cuda.current_stream().cuda_stream
             suffix = "" if xyz.dtype == torch.float64 else "_f"
@@ -90,6 +99,27 @@ class _BaseHarmonics:
             return sph, dsph
         return sph
 
+    def _compute_via_float64(self, xyz, sph, dsph, ddsph):
+        derivatives = 2 if ddsph is not None else (1 if dsph is not None else 0)
+        n_samples = xyz.shape[0]
+        # a workspace from torch's allocator keeps the call asynchronous; at most 256 MiB, the
+        # library walks over the points in chunks of what it holds
+        wanted = self._lib.sphx_forward_f32_via_f64_workspace(n_samples, self._l_max, derivatives)
+        floor = self._lib.sphx_forward_f32_via_f64_workspace(min(n_samples, 64), self._l_max, derivatives)
+        size = max(min(wanted, 256 << 20), floor)
+        workspace = torch.empty(size, dtype=torch.uint8, device=xyz.device)
+        with torch.cuda.device(xyz.device):
+            stream = torch.cuda.current_stream()
+            status = self._lib.sphx_forward_f32_via_f64(
+                xyz.data_ptr(), n_samples, self._l_max, self._normalized, derivatives,
+                sph.data_ptr(), dsph.data_ptr() if dsph is not None else None,
+                ddsph.data_ptr() if ddsph is not None else None,
+                workspace.data_ptr(), size, stream.cuda_stream,
+            )
+            workspace.record_stream(stream)
+        if status != 0:
+            raise RuntimeError(self._lib.sphx_last_error().decode())
+
     def compute(self, xyz):
         """Values, ``(n_samples, (l_max+1)**2)``."""
         return self._compute_impl(xyz)
@@ -107,6 +137,7 @@ class SphericalHarmonics(_BaseHarmonics):
     """Real spherical harmonics :math:`Y^m_l` up to ``l_max`` of points given in Cartesian coordinates."""
 
     _cuda_prefix = "sphericart_cuda_spherical_harmonics"
+    _normalized = 1
 
 
 class SolidHarmonics(_BaseHarmonics):
