@@ -385,20 +385,23 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
             return (static_cast<unsigned>(l * (l + 1) / 2) << 16) | (static_cast<unsigned>(l) << 8) |
                    (static_cast<unsigned>(side) << 7) | static_cast<unsigned>(m);
         };
-        if (tid == 0) {
-            unsigned n = 0;
-            for (int side = 0; side < (SPLIT ? 2 : 1); ++side) {
-                for (int l = L; l > H; --l) {
-                    for (int m = l - 2; m >= 1; --m) job_table[n++] = pack(l, m, side);
-                }
+        // one thread per l fills that l's places (a single thread writing all of them took
+        // 10 us at l_max = 32, a third of the time of a small evaluation)
+        if (static_cast<int>(tid) < L - H) {
+            constexpr unsigned SIDES = SPLIT ? 2u : 1u;
+            const int l = L - static_cast<int>(tid);
+            const unsigned levels = static_cast<unsigned>(L - H);
+            auto bulk_above = [&](int from) { // sum of (l' - 2) over from < l' <= L
+                return static_cast<unsigned>(L * (L + 1) / 2 - from * (from + 1) / 2 - 2 * (L - from));
+            };
+            const unsigned bulk_all = bulk_above(H);
+            for (unsigned side = 0; side < SIDES; ++side) {
+                unsigned at = side * bulk_all + bulk_above(l);
+                for (int m = l - 2; m >= 1; --m) job_table[at++] = pack(l, m, static_cast<int>(side));
+                job_table[SIDES * bulk_all + side * levels + tid] = pack(l, l, static_cast<int>(side));
+                job_table[SIDES * (bulk_all + levels) + side * levels + tid] = pack(l, l - 1, static_cast<int>(side));
             }
-            for (int side = 0; side < (SPLIT ? 2 : 1); ++side) {
-                for (int l = L; l > H; --l) job_table[n++] = pack(l, l, side);
-            }
-            for (int side = 0; side < (SPLIT ? 2 : 1); ++side) {
-                for (int l = L; l > H; --l) job_table[n++] = pack(l, l - 1, side);
-            }
-            for (int l = L; l > H; --l) job_table[n++] = pack(l, 0, 0);
+            job_table[SIDES * (bulk_all + 2 * levels) + tid] = pack(l, 0, 0);
         }
     }
 
@@ -1052,11 +1055,16 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         const int want = env_int("SPHX_CHUNK_SHIFT", 3);
         g.chunk_shift = want < 0 ? 0u : (want > 10 ? 10u : static_cast<unsigned>(want));
     }
-    const unsigned chunks_per_xcd = (g.tiles_per_xcd + (1u << g.chunk_shift) - 1u) >> g.chunk_shift;
     unsigned per_cu = limit / out->lds_bytes;
     if (per_cu < 1) per_cu = 1;
     if (per_cu > 4) per_cu = 4; // 512 threads each: 2048 lanes per CU
     unsigned want = (static_cast<unsigned>(cus) * per_cu + 7u) & ~7u;
+    // Few points: shorter chunks, down to single tiles, until every resident workgroup has one
+    // (10 000 points at l_max = 8 are 625 tiles of 16: in chunks of 8 they kept 80 workgroups
+    // busy for 41 us, as single tiles they take 512 and a third of the time).
+    auto chunks_in_xcd = [&]() { return (g.tiles_per_xcd + (1u << g.chunk_shift) - 1u) >> g.chunk_shift; };
+    while (g.chunk_shift > 0 && chunks_in_xcd() * 8u < want) --g.chunk_shift;
+    const unsigned chunks_per_xcd = chunks_in_xcd();
     unsigned need = chunks_per_xcd * 8u;
     out->workgroups = want < need ? want : need;
     if (out->workgroups < 8) out->workgroups = 8;

@@ -18,7 +18,7 @@ from sphericart_amd.workloads import WORKLOADS
 
 pytestmark = pytest.mark.gpu
 
-L_MAX_SWEEP = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 16, 20, 25, 32]
+L_MAX_SWEEP = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 15, 16, 20, 23, 24, 25, 32]
 
 
 def check(got, want, what):
