@@ -524,26 +524,31 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
         return static_cast<unsigned>((reinterpret_cast<uintptr_t>(array) / sizeof(T) + element) % LINE);
     };
 
-    // stage three of tile n, into row buffer `buffer` (the entry waves)
-    auto entry_stage = [&](unsigned n, unsigned buffer) {
-        const unsigned valid = valid_in(n);
-        T* staged = lds + buffer * g.rows_elems;
-        const unsigned t = tid - wide_first;
-        // WHOLE: element 0 of a staging region stands for the start of the 128-byte line in
-        // which the tile's run begins in HBM, so the run itself starts `phase` elements in
+    // Where the rows of tile n start within their staging regions. WHOLE: element 0 of a region
+    // stands for the start of the 128-byte line in which the tile's run begins in HBM, so the run
+    // itself starts `phase` elements in. WHOLE == false: position within 16 bytes of the first
+    // staged row, see row_stride. VJP: the rows never leave LDS, no position to match.
+    struct Phases {
+        unsigned sph, dsph, ddsph;
+    };
+    auto phases_of = [&](unsigned n) -> Phases {
         const unsigned long long first_point = static_cast<unsigned long long>(tile_of(n)) * S;
-        // (WHOLE == false: position within 16 bytes of the first staged row, see row_stride;
-        // VJP: the rows never leave LDS, no position to match)
-        const unsigned phase_sph = VJP ? 0u : phase_of(sph, first_point * ny + skip) % (WHOLE ? LINE : W16);
-        const unsigned phase_dsph =
-            VJP || MODE < 1 ? 0u : phase_of(dsph, first_point * 3 * ny + skip) % (WHOLE ? LINE : W16);
-        const unsigned phase_ddsph = WHOLE && !VJP && MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
+        Phases ph;
+        ph.sph = VJP ? 0u : phase_of(sph, first_point * ny + skip) % (WHOLE ? LINE : W16);
+        ph.dsph = VJP || MODE < 1 ? 0u : phase_of(dsph, first_point * 3 * ny + skip) % (WHOLE ? LINE : W16);
+        ph.ddsph = WHOLE && !VJP && MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
+        return ph;
+    };
+
+    // WHOLE: the closed forms of tile n, one lane per point, into row buffer `buffer`. The
+    // entries of a point are cut in slices (by l), dealt to `among` waves of which this is number
+    // `who`, so that no single wave carries all of the chain rule and staging.
+    auto closed_stage = [&](unsigned n, unsigned buffer, unsigned who, unsigned among) {
         if constexpr (WHOLE) {
-            // closed forms: one lane per point; the entries of a point in slices (by l) that the
-            // entry waves share, so that no single wave carries all of the chain rule and staging
-            const unsigned entry_wave = t >> 6;
-            const unsigned entry_waves = wide_lanes >> 6;
+            const unsigned valid = valid_in(n);
             if (lane < valid) {
+                T* staged = lds + buffer * g.rows_elems;
+                const Phases ph = phases_of(n);
                 const T* rec = point_data(n, lane);
                 Point<T> p;
                 p.x = rec[0];
@@ -555,9 +560,9 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
                 p.ir = rec[6];
                 Rows<T> rows;
                 rows.ny = static_cast<int>(ny);
-                rows.sph = staged + phase_sph + lane * ny;
-                rows.dsph = staged + g.off_dsph + phase_dsph + lane * 3 * ny;
-                rows.ddsph = staged + g.off_ddsph + phase_ddsph + lane * 9 * ny;
+                rows.sph = staged + ph.sph + lane * ny;
+                rows.dsph = staged + g.off_dsph + ph.dsph + lane * 3 * ny;
+                rows.ddsph = staged + g.off_ddsph + ph.ddsph + lane * 9 * ny;
                 if constexpr (H == 6) {
                     // float32 rows a multiple of 32 words long (l_max = 7, 15, 23, ...): the
                     // stores of all lanes would fall on one LDS bank; stored in rotated fours
@@ -568,27 +573,36 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
                     constexpr bool MAY_ROTATE = sizeof(T) == 4 && MODE == 1;
                     if (MAY_ROTATE && (ny & 31u) == 0) {
                         const unsigned turn = lane & 3u;
-                        if (0 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 0, 8, true>(p, rows, turn);
-                        if (1 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 8, 16, true>(p, rows, turn);
-                        if (2 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 16, 24, true>(p, rows, turn);
-                        if (3 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 24, 32, true>(p, rows, turn);
-                        if (4 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 32, 40, true>(p, rows, turn);
-                        if (5 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 40, 49, true>(p, rows, turn);
+                        if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 8, true>(p, rows, turn);
+                        if (1 % among == who) closed_form_job<T, MODE, NORM, H, 8, 16, true>(p, rows, turn);
+                        if (2 % among == who) closed_form_job<T, MODE, NORM, H, 16, 24, true>(p, rows, turn);
+                        if (3 % among == who) closed_form_job<T, MODE, NORM, H, 24, 32, true>(p, rows, turn);
+                        if (4 % among == who) closed_form_job<T, MODE, NORM, H, 32, 40, true>(p, rows, turn);
+                        if (5 % among == who) closed_form_job<T, MODE, NORM, H, 40, 49, true>(p, rows, turn);
                     } else {
-                        if (0 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows);
-                        if (1 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows);
-                        if (2 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows);
-                        if (3 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows);
-                        if (4 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows);
-                        if (5 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows);
-                        if (6 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows);
-                        if (7 % entry_waves == entry_wave) closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows);
+                        if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows);
+                        if (1 % among == who) closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows);
+                        if (2 % among == who) closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows);
+                        if (3 % among == who) closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows);
+                        if (4 % among == who) closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows);
+                        if (5 % among == who) closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows);
+                        if (6 % among == who) closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows);
+                        if (7 % among == who) closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows);
                     }
                 } else {
-                    if (entry_wave == 0) closed_form_job<T, MODE, NORM, H>(p, rows);
+                    if (who == 0) closed_form_job<T, MODE, NORM, H>(p, rows);
                 }
             }
         }
+    };
+
+    // stage three of tile n, into row buffer `buffer` (the entry waves)
+    auto entry_stage = [&](unsigned n, unsigned buffer) {
+        const unsigned valid = valid_in(n);
+        T* staged = lds + buffer * g.rows_elems;
+        const unsigned t = tid - wide_first;
+        const Phases ph = phases_of(n);
+        const unsigned phase_sph = ph.sph, phase_dsph = ph.dsph, phase_ddsph = ph.ddsph;
         // One pass takes the jobs of as many points as fit side by side in the wide lanes
         // (of one point, in several rounds, when it has more jobs than there are lanes);
         // what depends on the point only is read once per pass.
@@ -789,7 +803,10 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
             } else if (wave < entry_first_wave) {
                 recursion_stage(n + 1);
             } else if (wave < entry_end_wave) {
-                if (valid != 0) entry_stage(n, n & 1u);
+                if (valid != 0) {
+                    closed_stage(n, n & 1u, wave - entry_first_wave, entry_end_wave - entry_first_wave);
+                    entry_stage(n, n & 1u);
+                }
             } else if (before != 0) {
                 flush_stage(n - 1, (n - 1) & 1u, tid - 64 * entry_end_wave, 64 * g.flush_waves,
                             std::true_type{});
@@ -800,6 +817,9 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
         // flush, after a second barrier.
         for (unsigned n = 0; valid_in(n) != 0; ++n) {
             __syncthreads(); // tables of tile n+1, iterates of tile n in place; rows of tile n-1 flushed
+            // the closed-form slices go round all waves: those that make tables and iterates
+            // have time to spare
+            closed_stage(n, 0, wave, NT / 64);
             if (wave == 0) {
                 if ((n & (batch_tiles - 1u)) == 0) {
                     azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
