@@ -215,6 +215,153 @@ __global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __re
 }
 
 // ---------------------------------------------------------------------------
+// Values only, l_max > 6, rows short enough that those of 64 points fit in LDS:
+// 64 points per workgroup, one point per lane, one to eight waves that share
+// the l channels of the same 64 points.
+//
+// Without derivatives an entry is three multiplications, so what counts is what
+// surrounds them. With one point per lane l and m are the same for the whole
+// wave: the prefactors come from constant memory through the scalar unit, no
+// job has to be decoded and no iterate passes through LDS, about 15
+// instructions per (l, +-m) pair of entries in all, a tenth of what the
+// recursion kernel spends on them. (With derivatives the entries themselves
+// dominate and rows are four and thirteen times as long, so that far fewer
+// than 64 points fit: there the recursion kernel stays.)
+//
+// The rows of 64 points take most of a CU's LDS from l_max of about 12 on, and
+// one wave would leave three of the four SIMDs idle: the l channels are dealt
+// to the waves of the workgroup (in snake order, long and short ones mixed),
+// each wave evaluating its channels for all 64 points (l_max = 15 float32,
+// 500k points: 245 us with one wave, 113 with four, 106 with six). When not
+// even 64 rows fit, 32 points per workgroup and half the lanes idle.
+//
+// Same operations in the same order as the reference: c_m, s_m, 2(m+1)z as in
+// templates.hpp:451-466, l <= 6 in closed form, then per l the recursion of
+// templates_core.hpp:122-123,155,202-204,393 downward in m, every iterate
+// multiplied by its prefactor and by c_m and s_m (:127-128,160-162,214-218,395).
+//
+// LDS: the rows of the tile in HBM layout, so that the waves stream them out
+// with 16-byte stores, and per point its table of (c_m, s_m, 2(m+1)z). A row
+// length that is a multiple of 8 words would put the same entry of all points
+// on few banks: such rows are kept one 16-byte vector apart.
+// g.rows_elems: row stride, g.off_pts: start of the tables, g.off_iter: table stride.
+// ---------------------------------------------------------------------------
+constexpr unsigned kValuesMaxThreads = 512;
+
+template <typename T, bool NORM>
+__global__ __launch_bounds__(kValuesMaxThreads) void values_kernel(Tiling g, const T* __restrict__ xyz,
+                                                                  T* __restrict__ sph) {
+    constexpr int H = 6;
+    constexpr unsigned NYH = (H + 1) * (H + 1);
+    using V = typename Pack<T>::type;
+    constexpr unsigned W = Pack<T>::width;
+    T* lds = reinterpret_cast<T*>(lds_raw);
+    const unsigned tid = threadIdx.x;
+    const unsigned lane = tid & 63u;
+    const unsigned wave = tid >> 6;
+    const unsigned waves = blockDim.x >> 6;
+    const int L = g.l_max;
+    const unsigned ny = g.ny;
+    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
+    if (group >= g.n_tiles) return;
+    const unsigned tile = static_cast<unsigned>(g.tile); // 64, or fewer when 64 rows do not fit
+    const unsigned long long first = static_cast<unsigned long long>(group) * tile;
+    const unsigned long long left = g.n_samples - first;
+    const unsigned valid = left < tile ? static_cast<unsigned>(left) : tile;
+
+    Point<T> p;
+    p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
+    T* row = lds + lane * g.rows_elems;
+    T* tab = lds + g.off_pts + lane * g.off_iter; // [m][3]: c_m, s_m, 2(m+1)z
+    if (lane < valid) {
+        p = load_point<T, NORM>(xyz + (first + lane) * 3);
+        if (wave == 0) {
+            const T twoz = p.z + p.z;
+            T cm = 1.0, sm = 0.0, tz = twoz;
+            tab[0] = cm;
+            tab[1] = sm;
+            tab[2] = tz;
+            for (int m = 1; m <= L; ++m) {
+                const T cn = cm * p.x - sm * p.y;
+                const T sn = cm * p.y + sm * p.x;
+                tz = tz + twoz;
+                cm = cn;
+                sm = sn;
+                tab[3 * m] = cm;
+                tab[3 * m + 1] = sm;
+                tab[3 * m + 2] = tz;
+            }
+        }
+        if (wave == waves - 1) { // the last wave gets the fewest channels below
+            T Y[NYH];
+            low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
+#pragma unroll
+            for (unsigned k = 0; k < NYH; ++k) row[k] = Y[k];
+        }
+    }
+    __syncthreads(); // the tables
+    if (lane < valid) {
+        const T rxy = p.x2 + p.y2;
+        const T* cF = table_F<T>();
+        const T* cQ = table_Q<T>();
+        // channel number i = L - l goes to wave i % waves in even rounds, backwards in odd ones
+        for (unsigned i = 0; static_cast<int>(i) < L - H; ++i) {
+            const unsigned pos = i % waves;
+            if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
+            const int l = L - static_cast<int>(i);
+            const int tri = l * (l + 1) / 2;
+            const T* pk = cF + tri;
+            const T* qk = cQ + tri;
+            T* mid = row + l * l + l;
+            T v2 = qk[l];
+            T v1 = -p.z * v2;
+            {
+                const T pq = v2 * pk[l];
+                mid[l] = pq * tab[3 * l];
+                mid[-l] = pq * tab[3 * l + 1];
+            }
+            {
+                const T pq = v1 * pk[l - 1];
+                mid[l - 1] = pq * tab[3 * (l - 1)];
+                mid[-(l - 1)] = pq * tab[3 * (l - 1) + 1];
+            }
+            for (int m = l - 2; m >= 1; --m) {
+                const T v0 = qk[m] * (tab[3 * m + 2] * v1 + rxy * v2);
+                const T pq = v0 * pk[m];
+                mid[m] = pq * tab[3 * m];
+                mid[-m] = pq * tab[3 * m + 1];
+                v2 = v1;
+                v1 = v0;
+            }
+            const T v0 = qk[0] * (tab[2] * v1 + rxy * v2);
+            mid[0] = v0 * pk[0];
+        }
+    }
+    __syncthreads(); // the rows
+    T* dst = sph + first * ny;
+    const unsigned len = valid * ny;
+    const unsigned threads = blockDim.x;
+    if (g.rows_elems == ny) {
+        copy_out<T, SPHX_STREAMING_STORES, false, 1>(lds, dst, len, ny, 0, 0, tid, threads);
+    } else if ((reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+        // rows one vector apart (their length is a whole number of vectors)
+        const unsigned per_row = ny / W;
+        const unsigned magic = magic_of(per_row);
+        const V* in = reinterpret_cast<const V*>(lds);
+        V* out = reinterpret_cast<V*>(dst);
+        const unsigned nvec = len / W;
+        for (unsigned v = tid; v < nvec; v += threads) {
+            emit<T, SPHX_STREAMING_STORES>(in[v + __umulhi(v, magic)], out + v);
+        }
+    } else {
+        for (unsigned e = tid; e < len; e += threads) {
+            const unsigned r = e / ny;
+            dst[e] = lds[e + r * (g.rows_elems - ny)];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Vector-Jacobian product without the Jacobian in memory, l_max <= 6:
 //
 //   xyz_grad[i][a] (+)= sum_k d sph[i][k] / d xyz[i][a] * sph_grad[i][k]
@@ -903,6 +1050,7 @@ struct Launch {
 };
 
 struct Plan {
+    bool lanes;       // values only, short rows: one launch of values_kernel (uses `closed`)
     bool closed_only; // l_max within the closed forms: one launch of closed_form_kernel
     bool whole;       // recursion_kernel evaluates the closed forms too: one launch
                       // otherwise closed_form_kernel<PREFIX> + recursion_kernel: two launches
@@ -937,6 +1085,50 @@ static void plan_closed(size_t n_samples, int l_max, int hard, int mode, size_t 
     if (mode >= 1) at = align4(at + per * (3 * nyh + pad));
     if (mode == 2) at = align4(at + per * (9 * nyh + pad));
     out->lds_bytes = at * static_cast<unsigned>(elem);
+}
+
+// values_kernel: 64 (or 32) points per workgroup, their rows and tables in LDS. Returns false
+// when that does not fit, and the recursion kernel takes over.
+static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit, Launch* out) {
+    Tiling& g = out->g;
+    std::memset(&g, 0, sizeof(g));
+    const unsigned esize = static_cast<unsigned>(elem);
+    const unsigned ny = static_cast<unsigned>(l_max + 1) * (l_max + 1);
+    const unsigned vec = 16u / esize;
+    // rows a multiple of 8 words long: one vector between them (values_kernel)
+    const unsigned row_stride = (ny * (esize / 4u)) % 8u == 0 ? ny + vec : ny;
+    const unsigned table_stride = (3u * static_cast<unsigned>(l_max + 1)) | 1u;
+    unsigned allowed = static_cast<unsigned>(env_int("SPHX_VALUES_LDS", 160 * 1024));
+    if (allowed > static_cast<unsigned>(lds_limit)) allowed = static_cast<unsigned>(lds_limit);
+    // Fewer than 64 points per workgroup leave lanes idle: with 32 the kernel still beats the
+    // recursion kernel (l_max = 32 float32, 500k points: 781 against 1 077 us; l_max = 20
+    // float64: 470 against 710), with 16 it does not (l_max = 28 float64: 1 404 against 1 089).
+    const unsigned smallest = static_cast<unsigned>(env_int("SPHX_VALUES_MIN_TILE", 32));
+    unsigned tile = 64, rows = 0, bytes = 0;
+    for (;; tile /= 2) {
+        if (tile < smallest || tile < 8) return false;
+        rows = (tile * row_stride + vec - 1u) / vec * vec;
+        bytes = (rows + tile * table_stride) * esize;
+        if (bytes <= allowed) break;
+    }
+    g.n_samples = n_samples;
+    g.l_max = l_max;
+    g.ny = static_cast<int>(ny);
+    g.tile = static_cast<int>(tile);
+    if ((n_samples + tile - 1) / tile > 0x7fffffffull) return false;
+    g.n_tiles = static_cast<unsigned>((n_samples + tile - 1) / tile);
+    g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
+    g.rows_elems = row_stride;
+    g.off_pts = rows;
+    g.off_iter = table_stride;
+    out->workgroups = g.tiles_per_xcd * 8u;
+    // one wave per l channel above the closed forms, eight at most
+    int waves = env_int("SPHX_VALUES_WAVES", 8);
+    waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
+    const int channels = l_max - 6;
+    out->threads = 64u * static_cast<unsigned>(channels < waves ? channels : waves);
+    out->lds_bytes = bytes;
+    return true;
 }
 
 // Tile size and LDS layout of the recursion kernel. Returns false when not even one point fits.
@@ -1105,11 +1297,16 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
         return fail(SPHX_ERR_UNSUPPORTED, "too many samples for one launch");
     }
     const int hard = mode == 2 ? 1 : 6;
+    plan->lanes = false;
     plan->closed_only = l_max <= hard;
     plan->whole = true;
     plan->split_sides = false;
     if (plan->closed_only) {
         plan_closed(n_samples, l_max, l_max, mode, elem, &plan->closed);
+        return SPHX_OK;
+    }
+    if (mode == 0 && plan_values(n_samples, l_max, elem, lds_limit, &plan->closed)) {
+        plan->lanes = true;
         return SPHX_OK;
     }
     const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", 80 * 1024));
@@ -1224,6 +1421,20 @@ static hipError_t launch_recursion(const Launch& l, const T* xyz, T* sph, T* dsp
 template <typename T, int MODE, bool NORM>
 static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* ddsph,
                            hipStream_t stream) {
+    if (plan.lanes) {
+        if constexpr (MODE == 0) {
+            const Launch& l = plan.closed;
+            auto kernel = values_kernel<T, NORM>;
+            if (l.lds_bytes > 64u * 1024u) {
+                unsigned unused = 0;
+                hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &unused);
+                if (e != hipSuccess) return e;
+            }
+            hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz, sph);
+            return hipGetLastError();
+        }
+        return hipErrorInvalidValue;
+    }
     if (!plan.closed_only) {
         if constexpr (MODE == 2) {
             if (plan.split_sides) {
@@ -1622,7 +1833,7 @@ int sphx_plan(size_t n_samples, int l_max, int derivatives, int is_f64, int* til
     int status = sphx::make_plan(n_samples ? n_samples : 1, l_max, derivatives,
                                  is_f64 ? sizeof(double) : sizeof(float), lds, cus, &plan);
     if (status != SPHX_OK) return status;
-    const sphx::Launch& main = plan.closed_only ? plan.closed : plan.rec;
+    const sphx::Launch& main = plan.closed_only || plan.lanes ? plan.closed : plan.rec;
     if (tile_samples) *tile_samples = main.g.tile;
     if (threads) *threads = static_cast<int>(main.threads);
     if (lds_bytes) *lds_bytes = static_cast<int>(main.lds_bytes);

@@ -17,7 +17,8 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-@pytest.mark.parametrize("l_max,mode", [(3, "values"), (6, "gradients"), (1, "hessians"), (9, "gradients"), (5, "hessians")])
+@pytest.mark.parametrize("l_max,mode", [(3, "values"), (6, "gradients"), (1, "hessians"), (9, "gradients"), (5, "hessians"),
+                                        (7, "values"), (12, "values"), (24, "values")])
 def test_ragged_sizes(oracle, l_max, mode):
     """Point counts around the tile sizes, including a single point (tail tiles are partial)."""
     rng = np.random.default_rng(0)
@@ -55,7 +56,8 @@ def test_unaligned_outputs_take_the_narrow_store_path(oracle, library):
     """Output pointers that are not 16-byte aligned still give the same numbers."""
     rng = np.random.default_rng(1)
     for dtype, tdtype in ((np.float32, torch.float32), (np.float64, torch.float64)):
-        for l_max, mode in ((6, "gradients"), (7, "gradients"), (3, "hessians"), (3, "values")):
+        for l_max, mode in ((6, "gradients"), (7, "gradients"), (3, "hessians"), (3, "values"), (7, "values"),
+                            (8, "values"), (11, "values"), (24, "values")):
             announce("unaligned", np.dtype(dtype).name, l_max, mode)
             n, ny = 333, (l_max + 1) ** 2
             xyz = special_points(dtype, rng, n)
