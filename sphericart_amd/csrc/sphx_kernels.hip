@@ -1104,13 +1104,18 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // recursion kernel (l_max = 32 float32, 500k points: 781 against 1 077 us; l_max = 20
     // float64: 470 against 710), with 16 it does not (l_max = 28 float64: 1 404 against 1 089).
     const unsigned smallest = static_cast<unsigned>(env_int("SPHX_VALUES_MIN_TILE", 32));
-    unsigned tile = 64, rows = 0, bytes = 0;
-    for (;; tile /= 2) {
-        if (tile < smallest || tile < 8) return false;
-        rows = (tile * row_stride + vec - 1u) / vec * vec;
-        bytes = (rows + tile * table_stride) * esize;
-        if (bytes <= allowed) break;
+    // Two workgroups per CU (80 KB each) overlap one's tables and flush with the other's
+    // arithmetic: preferred, also at half the lanes, over one workgroup with all of LDS
+    // (l_max = 16 float32, 500k points: 142 against 164 us; l_max = 12 float64: 115 against 146).
+    unsigned tile = 0, rows = 0, bytes = 0;
+    for (unsigned limit : {allowed < 80u * 1024u ? allowed : 80u * 1024u, allowed}) {
+        for (unsigned t = 64; t >= smallest && t >= 8 && tile == 0; t /= 2) {
+            rows = (t * row_stride + vec - 1u) / vec * vec;
+            bytes = (rows + t * table_stride) * esize;
+            if (bytes <= limit) tile = t;
+        }
     }
+    if (tile == 0) return false;
     g.n_samples = n_samples;
     g.l_max = l_max;
     g.ny = static_cast<int>(ny);
