@@ -448,6 +448,232 @@ __global__ __launch_bounds__(64) void closed_form_vjp_kernel(Tiling g, const T* 
 }
 
 // ---------------------------------------------------------------------------
+// Vector-Jacobian product, l_max > 6, one point per lane (the construction of
+// values_kernel): what passes through LDS is the tile's rows of sph_grad, read
+// from HBM with consecutive lanes at consecutive addresses, and the per-point
+// tables; the gradient entries never leave the registers. A lane runs the two
+// recursions a gradient needs (Q_l^m and Q_{l-1}^m, templates_core.hpp:202-212),
+// forms the entries (l, +-m) of the three gradient rows as the reference does
+// (:129-133, :163-170, :219-227, :396-399), multiplies them with the two
+// weights and adds to three sums. The chain rule of the normalised harmonics is
+// linear in the gradient (templates.hpp:608-612), so it is applied once, to the
+// sums. The l channels are dealt to the waves as in values_kernel; the last
+// wave also takes l <= 6 in closed form; the waves' sums meet in LDS and wave 0
+// adds them in a fixed order. The terms are added in another order than a
+// sequential loop over k would, so the result agrees with the contraction of
+// the forward gradients to rounding, not bit for bit.
+// g.rows_elems: row stride of the staged weights, g.off_pts: tables,
+// g.off_iter: table stride, g.off_jobs: the waves' sums.
+// ---------------------------------------------------------------------------
+template <typename T, bool NORM>
+__global__ __launch_bounds__(kValuesMaxThreads) void vjp_lanes_kernel(Tiling g, const T* __restrict__ xyz,
+                                                                     const T* __restrict__ sph_grad,
+                                                                     T* __restrict__ xyz_grad,
+                                                                     int accumulate) {
+    constexpr int H = 6;
+    constexpr unsigned NYH = (H + 1) * (H + 1);
+    using V = typename Pack<T>::type;
+    constexpr unsigned W = Pack<T>::width;
+    T* lds = reinterpret_cast<T*>(lds_raw);
+    const unsigned tid = threadIdx.x;
+    const unsigned lane = tid & 63u;
+    const unsigned wave = tid >> 6;
+    const unsigned threads = blockDim.x;
+    const unsigned waves = threads >> 6;
+    const int L = g.l_max;
+    const unsigned ny = g.ny;
+    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
+    if (group >= g.n_tiles) return;
+    const unsigned tile = static_cast<unsigned>(g.tile);
+    const unsigned long long first = static_cast<unsigned long long>(group) * tile;
+    const unsigned long long left = g.n_samples - first;
+    const unsigned valid = left < tile ? static_cast<unsigned>(left) : tile;
+
+    // the tile's rows of sph_grad, one contiguous run, into LDS (rows `rows_elems` apart)
+    {
+        const T* run = sph_grad + first * ny;
+        const unsigned len = valid * ny;
+        const unsigned gap = g.rows_elems - ny;
+        if ((reinterpret_cast<uintptr_t>(run) & 15u) == 0 && (gap == 0 || ny % W == 0)) {
+            const V* in = reinterpret_cast<const V*>(run);
+            V* staged = reinterpret_cast<V*>(lds);
+            const unsigned nvec = len / W;
+            const unsigned magic = magic_of(ny / W ? ny / W : 1u);
+            for (unsigned v = tid; v < nvec; v += threads) {
+                staged[gap == 0 ? v : v + __umulhi(v, magic) * (gap / W)] = in[v];
+            }
+            for (unsigned e = nvec * W + tid; e < len; e += threads) lds[e] = run[e]; // gap == 0 only
+        } else {
+            for (unsigned e = tid; e < len; e += threads) {
+                lds[e + (e / ny) * gap] = run[e];
+            }
+        }
+    }
+
+    Point<T> p;
+    p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
+    const T* weight = lds + lane * g.rows_elems;
+    T* tab = lds + g.off_pts + lane * g.off_iter; // [m][3]: c_m, s_m, 2(m+1)z
+    if (lane < valid) {
+        p = load_point<T, NORM>(xyz + (first + lane) * 3);
+        if (wave == 0) {
+            const T twoz = p.z + p.z;
+            T cm = 1.0, sm = 0.0, tz = twoz;
+            tab[0] = cm;
+            tab[1] = sm;
+            tab[2] = tz;
+            for (int m = 1; m <= L; ++m) {
+                const T cn = cm * p.x - sm * p.y;
+                const T sn = cm * p.y + sm * p.x;
+                tz = tz + twoz;
+                cm = cn;
+                sm = sn;
+                tab[3 * m] = cm;
+                tab[3 * m + 1] = sm;
+                tab[3 * m + 2] = tz;
+            }
+        }
+    }
+    __syncthreads(); // weights and tables
+
+    T sum_x = 0, sum_y = 0, sum_z = 0;
+    if (lane < valid) {
+        const T x = p.x, y = p.y;
+        const T rxy = p.x2 + p.y2;
+        const T* cF = table_F<T>();
+        const T* cQ = table_Q<T>();
+        for (unsigned i = 0; static_cast<int>(i) < L - H; ++i) {
+            const unsigned pos = i % waves;
+            if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
+            const int l = L - static_cast<int>(i);
+            const int tri = l * (l + 1) / 2;
+            const T* pk = cF + tri;
+            const T* qk = cQ + tri;
+            const T* kb = qk - l; // constants of the Q_{l-1} recursion
+            const T* wmid = weight + l * l + l;
+            // the entries (l, +m) and (l, -m) of the gradient rows times their weights
+            auto add = [&](int m, T gx_pos, T gy_pos, T gz_pos, T gx_neg, T gy_neg, T gz_neg) {
+                const T wp = wmid[m], wn = wmid[-m];
+                sum_x += gx_pos * wp;
+                sum_y += gy_pos * wp;
+                sum_z += gz_pos * wp;
+                sum_x += gx_neg * wn;
+                sum_y += gy_neg * wn;
+                sum_z += gz_neg * wn;
+            };
+            T a2 = qk[l];       // Q_l^l
+            T a1 = -p.z * a2;   // Q_l^{l-1}
+            T b2 = 0;           // the Q_{l-1} sequence: 0 at m = l,
+            T b1 = qk[-1];      // Q_{l-1}^{l-1} at m = l - 1
+            T c1 = tab[3 * (l - 1)], s1 = tab[3 * (l - 1) + 1]; // c, s at m - 1 of the step at hand
+            {
+                // m = l
+                T pq = a2 * pk[l];
+                pq *= l;
+                add(l, pq * c1, pq * -s1, T(0), pq * s1, pq * c1, T(0));
+            }
+            T c0 = c1, s0 = s1; // c, s at m
+            c1 = tab[3 * (l - 2)];
+            s1 = tab[3 * (l - 2) + 1];
+            {
+                // m = l - 1
+                const T pkm = pk[l - 1];
+                T pq = a1 * pkm;
+                pq *= (l - 1);
+                const T pdq = pkm * (l + l - 1) * b1;
+                add(l - 1, pq * c1, pq * -s1, pdq * c0, pq * s1, pq * c1, pdq * s0);
+            }
+            for (int m = l - 2; m >= 1; --m) {
+                c0 = c1;
+                s0 = s1;
+                c1 = tab[3 * (m - 1)];
+                s1 = tab[3 * (m - 1) + 1];
+                const T tz = tab[3 * m + 2];
+                const T a0 = qk[m] * (tz * a1 + rxy * a2);
+                const T b0 = kb[m] * (tz * b1 + rxy * b2);
+                const T pkm = pk[m];
+                T pq = a0 * pkm;
+                pq *= m;
+                const T pdq = pkm * b1;
+                const T pdqx = pdq * x;
+                const T pdqy = pdq * y;
+                const T pdz = pkm * (l + m) * b0;
+                add(m, pdqx * c0 + pq * c1, pdqy * c0 + pq * -s1, pdz * c0,
+                    pdqx * s0 + pq * s1, pdqy * s0 + pq * c1, pdz * s0);
+                a2 = a1;
+                a1 = a0;
+                b2 = b1;
+                b1 = b0;
+            }
+            {
+                // m = 0
+                const T b0 = kb[0] * (tab[2] * b1 + rxy * b2);
+                const T w0 = wmid[0];
+                sum_x += pk[0] * x * b1 * w0;
+                sum_y += pk[0] * y * b1 * w0;
+                sum_z += pk[0] * l * b0 * w0;
+            }
+        }
+        // l <= 6 in closed form, in slices of entries that go to the waves from the last one
+        // backwards (those have the fewest channels above); a slice evaluates little more than
+        // its own entries, see closed_form_job
+        auto closed_slice = [&](auto lo, auto hi) {
+            constexpr int KLO = decltype(lo)::value, KHI = decltype(hi)::value;
+            T Y[NYH], DX[NYH], DY[NYH], DZ[NYH];
+            low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
+            low_gradients<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y, DX, DY, DZ);
+#pragma unroll
+            for (int k = KLO; k < KHI; ++k) {
+                const T wk = weight[k];
+                sum_x += DX[k] * wk;
+                sum_y += DY[k] * wk;
+                sum_z += DZ[k] * wk;
+            }
+        };
+        const unsigned from_last = waves - 1u - wave;
+        using std::integral_constant;
+        if (0 % waves == from_last) closed_slice(integral_constant<int, 0>{}, integral_constant<int, 9>{});
+        if (1 % waves == from_last) closed_slice(integral_constant<int, 9>{}, integral_constant<int, 16>{});
+        if (2 % waves == from_last) closed_slice(integral_constant<int, 16>{}, integral_constant<int, 25>{});
+        if (3 % waves == from_last) closed_slice(integral_constant<int, 25>{}, integral_constant<int, 31>{});
+        if (4 % waves == from_last) closed_slice(integral_constant<int, 31>{}, integral_constant<int, 36>{});
+        if (5 % waves == from_last) closed_slice(integral_constant<int, 36>{}, integral_constant<int, 41>{});
+        if (6 % waves == from_last) closed_slice(integral_constant<int, 41>{}, integral_constant<int, 45>{});
+        if (7 % waves == from_last) closed_slice(integral_constant<int, 45>{}, integral_constant<int, 49>{});
+    }
+    // the waves' sums: [wave][component][point]
+    T* partial = lds + g.off_jobs;
+    if (wave != 0 && lane < valid) {
+        partial[(wave * 3 + 0) * tile + lane] = sum_x;
+        partial[(wave * 3 + 1) * tile + lane] = sum_y;
+        partial[(wave * 3 + 2) * tile + lane] = sum_z;
+    }
+    __syncthreads();
+    if (wave == 0 && lane < valid) {
+        for (unsigned w = 1; w < waves; ++w) {
+            sum_x += partial[(w * 3 + 0) * tile + lane];
+            sum_y += partial[(w * 3 + 1) * tile + lane];
+            sum_z += partial[(w * 3 + 2) * tile + lane];
+        }
+        if constexpr (NORM) {
+            const T tmp = sum_x * p.x + sum_y * p.y + sum_z * p.z;
+            sum_x = (sum_x - p.x * tmp) * p.ir;
+            sum_y = (sum_y - p.y * tmp) * p.ir;
+            sum_z = (sum_z - p.z * tmp) * p.ir;
+        }
+        T* out = xyz_grad + (first + lane) * 3;
+        if (accumulate) {
+            sum_x += out[0];
+            sum_y += out[1];
+            sum_z += out[2];
+        }
+        out[0] = sum_x;
+        out[1] = sum_y;
+        out[2] = sum_z;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // l > H through the recursion. 512 threads, persistent workgroups that walk
 // over tiles of `tile` consecutive points, four tiles in flight per workgroup,
 // every wave with a role of its own and one barrier per tile:
@@ -1089,7 +1315,8 @@ static void plan_closed(size_t n_samples, int l_max, int hard, int mode, size_t 
 
 // values_kernel: 64 (or 32) points per workgroup, their rows and tables in LDS. Returns false
 // when that does not fit, and the recursion kernel takes over.
-static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit, Launch* out) {
+static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit, Launch* out,
+                        bool with_sums = false) {
     Tiling& g = out->g;
     std::memset(&g, 0, sizeof(g));
     const unsigned esize = static_cast<unsigned>(elem);
@@ -1100,10 +1327,14 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     const unsigned table_stride = (3u * static_cast<unsigned>(l_max + 1)) | 1u;
     unsigned allowed = static_cast<unsigned>(env_int("SPHX_VALUES_LDS", 160 * 1024));
     if (allowed > static_cast<unsigned>(lds_limit)) allowed = static_cast<unsigned>(lds_limit);
-    // Fewer than 64 points per workgroup leave lanes idle: with 32 the kernel still beats the
-    // recursion kernel (l_max = 32 float32, 500k points: 781 against 1 077 us; l_max = 20
+    // Fewer than 64 points per workgroup leave lanes idle: with 32 the values kernel still beats
+    // the recursion kernel (l_max = 32 float32, 500k points: 781 against 1 077 us; l_max = 20
     // float64: 470 against 710), with 16 it does not (l_max = 28 float64: 1 404 against 1 089).
-    const unsigned smallest = static_cast<unsigned>(env_int("SPHX_VALUES_MIN_TILE", 32));
+    // The product keeps no rows for HBM in LDS and has far more arithmetic per point to win:
+    // it goes down to 8 points (l_max = 24 float64, 200k points: 830 us with 16 points per
+    // workgroup against 1 456 us through the recursion kernel).
+    const unsigned smallest = static_cast<unsigned>(
+        with_sums ? env_int("SPHX_VJP_MIN_TILE", 8) : env_int("SPHX_VALUES_MIN_TILE", 32));
     // Two workgroups per CU (80 KB each) overlap one's tables and flush with the other's
     // arithmetic: preferred, also at half the lanes, over one workgroup with all of LDS
     // (l_max = 16 float32, 500k points: 142 against 164 us; l_max = 12 float64: 115 against 146).
@@ -1111,7 +1342,7 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     for (unsigned limit : {allowed < 80u * 1024u ? allowed : 80u * 1024u, allowed}) {
         for (unsigned t = 64; t >= smallest && t >= 8 && tile == 0; t /= 2) {
             rows = (t * row_stride + vec - 1u) / vec * vec;
-            bytes = (rows + t * table_stride) * esize;
+            bytes = (rows + t * table_stride + (with_sums ? 8u * 3u * t : 0u)) * esize;
             if (bytes <= limit) tile = t;
         }
     }
@@ -1126,12 +1357,15 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     g.rows_elems = row_stride;
     g.off_pts = rows;
     g.off_iter = table_stride;
+    g.off_jobs = rows + tile * table_stride; // vjp_lanes_kernel: the waves' sums
     out->workgroups = g.tiles_per_xcd * 8u;
     // one wave per l channel above the closed forms, eight at most
     int waves = env_int("SPHX_VALUES_WAVES", 8);
     waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
-    const int channels = l_max - 6;
-    out->threads = 64u * static_cast<unsigned>(channels < waves ? channels : waves);
+    // (the product's closed-form slices want at least four)
+    int want = l_max - 6;
+    if (with_sums && want < 4) want = 4;
+    out->threads = 64u * static_cast<unsigned>(want < waves ? want : waves);
     out->lds_bytes = bytes;
     return true;
 }
@@ -1607,14 +1841,38 @@ static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int
     }
     int status = ensure_device_ready(device);
     Plan plan;
+    Launch lanes;
+    bool use_lanes = false;
     if (status == SPHX_OK) {
+        if (l_max > SPHX_TABLE_LMAX) {
+            status = fail(SPHX_ERR_UNSUPPORTED, "l_max = " + std::to_string(l_max) +
+                                                    " exceeds the device prefactor tables (" +
+                                                    std::to_string(SPHX_TABLE_LMAX) + ")");
+        } else if (l_max > 6 && env_int("SPHX_VJP_LANES", 1) != 0) {
+            use_lanes = plan_values(n_samples, l_max, sizeof(T), g_lds_limit[device], &lanes, true);
+        }
+    }
+    if (status == SPHX_OK && !use_lanes) {
         status = make_plan(n_samples, l_max, 1, sizeof(T), g_lds_limit[device], g_compute_units[device],
                            &plan);
     }
     if (status == SPHX_OK) {
         hipStream_t s = reinterpret_cast<hipStream_t>(stream);
         hipError_t e;
-        if (plan.closed_only) {
+        if (use_lanes) {
+            auto launch = [&](auto kernel) -> hipError_t {
+                if (lanes.lds_bytes > 64u * 1024u) {
+                    unsigned unused = 0;
+                    hipError_t err = kernel_facts(reinterpret_cast<const void*>(kernel), lanes.threads,
+                                                  lanes.lds_bytes, &unused);
+                    if (err != hipSuccess) return err;
+                }
+                hipLaunchKernelGGL(kernel, dim3(lanes.workgroups), dim3(lanes.threads), lanes.lds_bytes, s,
+                                   lanes.g, xyz, sph_grad, xyz_grad, accumulate);
+                return hipGetLastError();
+            };
+            e = normalized ? launch(vjp_lanes_kernel<T, true>) : launch(vjp_lanes_kernel<T, false>);
+        } else if (plan.closed_only) {
             e = normalized ? dispatch_vjp<T, true>(plan.closed, l_max, xyz, sph_grad, xyz_grad, accumulate, s)
                            : dispatch_vjp<T, false>(plan.closed, l_max, xyz, sph_grad, xyz_grad, accumulate, s);
         } else {
