@@ -1362,9 +1362,11 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // one wave per l channel above the closed forms, eight at most
     int waves = env_int("SPHX_VALUES_WAVES", 8);
     waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
-    // (the product's closed-form slices want at least four)
+    // (the product's closed-form slices want at least four; values: one for the tables, one for
+    // the closed forms)
     int want = l_max - 6;
     if (with_sums && want < 4) want = 4;
+    if (!with_sums && want < 2) want = env_int("SPHX_VALUES_MIN_WAVES", 2);
     out->threads = 64u * static_cast<unsigned>(want < waves ? want : waves);
     out->lds_bytes = bytes;
     return true;
