@@ -42,8 +42,8 @@ PEAK_HBM_GBPS = 8000.0
 # call added up.
 MEASURED_TRAFFIC_BYTES = {
     "cfg3": int((5930.6 * 2.0 + 765861.1) * 1024),
-    "cfg4": int((1337.0 * 2.0 + 2935187.4) * 1024),
-    "cfg5": int(((1233.3 + 1322.8) * 2.0 + 184039.4 + 3380394.2) * 1024),
+    "cfg4": int((1330.1 * 2.0 + 2935182.4) * 1024),
+    "cfg5": int(((1239.8 + 1316.8) * 2.0 + 184256.0 + 3380900.0) * 1024),
     "cfg3:backward": int((394551.2 * 2.0 + 11719.3) * 1024),
 }
 
