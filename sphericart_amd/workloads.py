@@ -115,7 +115,7 @@ def _cfg5(seed, n, first):
     return _on_axis(xyz, radius, 200, first)
 
 
-_GENERATORS = {"cfg1": _cfg1, "cfg2": _cfg2, "cfg3": _cfg3, "cfg4": _cfg4, "cfg5": _cfg5}
+_GENERATORS = {"cfg1": _cfg1, "cfg2": _cfg2, "cfg3": _cfg3, "cfg4": _cfg4, "cfg5": _cfg5, "val10": _cfg2}
 
 WORKLOADS = {
     "cfg1": Workload(
@@ -141,5 +141,11 @@ WORKLOADS = {
         "spherical, l_max=32, f32, values+gradients, 200k points, uniform directions, "
         "r log-uniform in [1e-2,1e2), 0.5% of the points on the +-z axis",
         32, "f32", True, "gradients", 200_000, 1005,
+    ),
+    # not one of the reference's configurations: values alone beyond the closed forms, the shape
+    # the values kernel is profiled on
+    "val10": Workload(
+        "val10", "spherical, l_max=10, f32, values, 1M points, uniform directions, r ~ U[0.5,5)",
+        10, "f32", True, "values", 1_000_000, 1010,
     ),
 }
