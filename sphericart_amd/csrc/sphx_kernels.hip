@@ -1609,8 +1609,11 @@ static hipError_t kernel_facts(const void* kernel, unsigned threads, unsigned ld
         }
     }
     if (lds_bytes > 64u * 1024u) {
-        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                static_cast<int>(lds_bytes));
+        // the limit of the device, not of this launch: the attribute belongs to the kernel, and
+        // a later launch with less must not lower it for one with more that is already cached
+        int limit = device >= 0 && device < kMaxDevices ? g_lds_limit[device] : 0;
+        if (limit < static_cast<int>(lds_bytes)) limit = static_cast<int>(lds_bytes);
+        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, limit);
         if (e != hipSuccess) return e;
     }
     KernelFacts fresh{device, kernel, lds_bytes, 0u};

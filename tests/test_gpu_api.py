@@ -104,6 +104,19 @@ def test_many_tiles_per_workgroup_with_shifted_outputs(oracle, library, shift):
                 assert torch.isnan(raw[i][:shift]).all() and torch.isnan(raw[i][shift + sizes[i]:]).all()
 
 
+def test_lds_size_alternates_between_launches(oracle):
+    """One kernel, launches that need more, then less, then more LDS again (all above 64 KB)."""
+    rng = np.random.default_rng(21)
+    xyz = special_points(np.float32, rng, 2000)
+    for l_max in (8, 10, 8, 12, 9, 8):
+        announce("alternating LDS", l_max)
+        want = oracle.compute(xyz, l_max, True, "gradients")
+        got = run_calculator(xyz, l_max, True, "gradients")
+        for g, w in zip(got, want):
+            if w is not None:
+                assert same_numbers(g, w).all(), l_max
+
+
 def test_non_contiguous_input(oracle):
     """Reference: sphericart-torch/python/tests/test_autograd.py:88-124 (inputs are made contiguous)."""
     rng = np.random.default_rng(2)
