@@ -678,8 +678,8 @@ __global__ __launch_bounds__(kValuesMaxThreads) void vjp_lanes_kernel(Tiling g, 
 // over tiles of `tile` consecutive points, four tiles in flight per workgroup,
 // every wave with a role of its own and one barrier per tile:
 //
-//   wave 0       tile i+2, one lane per point: normalised coordinates, c_m,
-//                s_m, 2(m+1)z into LDS (azimuth_job);
+//   wave 0       one batch of up to eight tiles ahead, one lane per point:
+//                normalised coordinates, c_m, s_m, 2(m+1)z into LDS (azimuth_job);
 //   wave 1 (, 2) tile i+1, one lane per (point, l, sequence): the bare Q recursions,
 //                every iterate into LDS (sequence_job);
 //   entry waves  tile i, one job per (point, l, m >= 0): the entries (l, +-m) of
@@ -703,7 +703,8 @@ __global__ __launch_bounds__(kValuesMaxThreads) void vjp_lanes_kernel(Tiling g, 
 // jobs.
 //
 // WHOLE == true: the closed forms of l <= H are evaluated here too (one lane
-// per point) and the tile's rows are complete, one contiguous run per array.
+// per point, the entries in slices that go round all waves) and the tile's
+// rows are complete, one contiguous run per array.
 // WHOLE == false: the rows start at l = H + 1 (closed_form_kernel<PREFIX>
 // writes the part below); every (point, component) row is its own run.
 // ---------------------------------------------------------------------------
