@@ -49,4 +49,6 @@ class SolidHarmonics(SphericalHarmonics):
     _prefix = "solid_harmonics"
 
 
-__all__ = ["SphericalHarmonics", "SolidHarmonics"]
+from .e3nn import e3nn_spherical_harmonics, patch_e3nn, unpatch_e3nn  # noqa: E402
+
+__all__ = ["SphericalHarmonics", "SolidHarmonics", "e3nn_spherical_harmonics", "patch_e3nn", "unpatch_e3nn"]
