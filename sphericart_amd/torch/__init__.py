@@ -17,9 +17,10 @@ from . import ops  # noqa: F401  (registers the operators)
 
 
 class SphericalHarmonics(torch.nn.Module):
-    """Real spherical harmonics of the directions of ``xyz`` up to ``l_max``, differentiable."""
+    """Real spherical harmonics of the directions of ``xyz`` up to ``l_max``, differentiable.
 
-    _prefix = "spherical_harmonics"
+    The operator names are written out (no lookup by string), so that ``torch.jit.script`` and
+    ``torch.compile(fullgraph=True)`` see through the module."""
 
     def __init__(self, l_max: int):
         super().__init__()
@@ -28,25 +29,44 @@ class SphericalHarmonics(torch.nn.Module):
         self._l_max = int(l_max)
 
     def forward(self, xyz: Tensor) -> Tensor:
-        return getattr(torch.ops.sphericart_amd, self._prefix)(xyz, self._l_max)
+        return torch.ops.sphericart_amd.spherical_harmonics(xyz, self._l_max)
 
     def compute(self, xyz: Tensor) -> Tensor:
         return self.forward(xyz)
 
     def compute_with_gradients(self, xyz: Tensor) -> Tuple[Tensor, Tensor]:
-        return getattr(torch.ops.sphericart_amd, f"{self._prefix}_with_gradients")(xyz, self._l_max)
+        return torch.ops.sphericart_amd.spherical_harmonics_with_gradients(xyz, self._l_max)
 
     def compute_with_hessians(self, xyz: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
-        return getattr(torch.ops.sphericart_amd, f"{self._prefix}_with_hessians")(xyz, self._l_max)
+        return torch.ops.sphericart_amd.spherical_harmonics_with_hessians(xyz, self._l_max)
 
     def l_max(self) -> int:
         return self._l_max
 
 
-class SolidHarmonics(SphericalHarmonics):
+class SolidHarmonics(torch.nn.Module):
     """Solid harmonics ``r^l Y_l^m`` of ``xyz`` up to ``l_max``, differentiable."""
 
-    _prefix = "solid_harmonics"
+    def __init__(self, l_max: int):
+        super().__init__()
+        if l_max < 0:
+            raise ValueError("l_max must be non-negative")
+        self._l_max = int(l_max)
+
+    def forward(self, xyz: Tensor) -> Tensor:
+        return torch.ops.sphericart_amd.solid_harmonics(xyz, self._l_max)
+
+    def compute(self, xyz: Tensor) -> Tensor:
+        return self.forward(xyz)
+
+    def compute_with_gradients(self, xyz: Tensor) -> Tuple[Tensor, Tensor]:
+        return torch.ops.sphericart_amd.solid_harmonics_with_gradients(xyz, self._l_max)
+
+    def compute_with_hessians(self, xyz: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+        return torch.ops.sphericart_amd.solid_harmonics_with_hessians(xyz, self._l_max)
+
+    def l_max(self) -> int:
+        return self._l_max
 
 
 from .e3nn import e3nn_spherical_harmonics, patch_e3nn, unpatch_e3nn  # noqa: E402
