@@ -381,7 +381,7 @@ __global__ __launch_bounds__(kValuesMaxThreads) void values_kernel(Tiling g, con
 // takes only the first (H+1)^2 entries of every row and the recursion kernel adds the rest
 // (recursion_kernel with VJP).
 template <typename T, bool NORM, int H>
-__global__ __launch_bounds__(64) void closed_form_vjp_kernel(Tiling g, const T* __restrict__ xyz,
+__global__ __launch_bounds__(64, 3) void closed_form_vjp_kernel(Tiling g, const T* __restrict__ xyz,
                                                             const T* __restrict__ sph_grad,
                                                             T* __restrict__ xyz_grad, int accumulate) {
     constexpr unsigned NY = (H + 1) * (H + 1);
@@ -424,17 +424,42 @@ __global__ __launch_bounds__(64) void closed_form_vjp_kernel(Tiling g, const T* 
     __syncthreads();
     if (tid >= valid) return;
 
-    Entry<T> E[NY];
     const Point<T> p = load_point<T, NORM>(xyz + (first + tid) * 3);
-    closed_form_entries<T, 1, NORM, H>(p, E);
     const T* mine = weights + tid * STRIDE;
     T sum_x = 0, sum_y = 0, sum_z = 0;
+    // The entries in slices, one after the other in index order: a slice evaluates little more
+    // than its own entries (see closed_form_job), so that far fewer numbers are alive at a time
+    // than with all 3 x 49 gradient entries of a point in registers (float64: 340 registers and
+    // one wave per SIMD before). Same entries, same order of the additions.
+    auto slice = [&](auto lo, auto hi) {
+        constexpr int KLO = decltype(lo)::value, KHI = decltype(hi)::value;
+        T Y[NY], DX[NY], DY[NY], DZ[NY];
+        low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
+        low_gradients<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y, DX, DY, DZ);
 #pragma unroll
-    for (unsigned k = 0; k < NY; ++k) {
-        const T wk = mine[k];
-        sum_x += E[k].gx * wk;
-        sum_y += E[k].gy * wk;
-        sum_z += E[k].gz * wk;
+        for (int k = KLO; k < KHI; ++k) {
+            Entry<T> e;
+            e.v = Y[k];
+            e.gx = DX[k];
+            e.gy = DY[k];
+            e.gz = DZ[k];
+            e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = static_cast<T>(0.0);
+            e = finish<T, 1, NORM>(p, e);
+            const T wk = mine[k];
+            sum_x += e.gx * wk;
+            sum_y += e.gy * wk;
+            sum_z += e.gz * wk;
+        }
+    };
+    using std::integral_constant;
+    if constexpr (H == 6) {
+        slice(integral_constant<int, 0>{}, integral_constant<int, 16>{});
+        slice(integral_constant<int, 16>{}, integral_constant<int, 25>{});
+        slice(integral_constant<int, 25>{}, integral_constant<int, 36>{});
+        slice(integral_constant<int, 36>{}, integral_constant<int, 42>{});
+        slice(integral_constant<int, 42>{}, integral_constant<int, 49>{});
+    } else {
+        slice(integral_constant<int, 0>{}, integral_constant<int, static_cast<int>(NY)>{});
     }
     T* out = xyz_grad + (first + tid) * 3;
     if (accumulate) {
