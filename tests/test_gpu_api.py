@@ -117,6 +117,49 @@ def test_lds_size_alternates_between_launches(oracle):
                 assert same_numbers(g, w).all(), l_max
 
 
+def test_calls_from_several_host_threads(oracle, library):
+    """Four host threads, each on a stream of its own, shapes that need different kernels and
+    LDS sizes, started together on a fresh set of shapes (the per-kernel facts are cached under a
+    lock, the last error is per thread)."""
+    import threading
+
+    rng = np.random.default_rng(33)
+    shapes = [(13, "values", np.float32), (9, "gradients", np.float64), (4, "hessians", np.float32),
+              (14, "gradients", np.float32)]
+    clouds = [special_points(dtype, rng, 1500) for _, _, dtype in shapes]
+    wanted = [oracle.compute(xyz, l_max, True, mode) for xyz, (l_max, mode, _) in zip(clouds, shapes)]
+    results, errors = [None] * len(shapes), []
+    gate = threading.Barrier(len(shapes))
+
+    def work(i):
+        try:
+            l_max, mode, _ = shapes[i]
+            stream = torch.cuda.Stream()
+            d_xyz = torch.from_numpy(clouds[i]).cuda()
+            torch.cuda.synchronize()
+            gate.wait()
+            for _ in range(20):
+                status, out = run_launch_layer(library, d_xyz, l_max, True, mode, stream=stream.cuda_stream)
+                if status != 0:
+                    raise RuntimeError(library.sphx_last_error())
+            stream.synchronize()
+            results[i] = [o.cpu().numpy() if o is not None else None for o in out]
+        except Exception as exc:  # reported by the main thread
+            errors.append((i, repr(exc)))
+
+    announce("host threads", shapes)
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(shapes))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for got, want in zip(results, wanted):
+        for g, w in zip(got, want):
+            if w is not None:
+                assert same_numbers(g, w).all()
+
+
 def test_non_contiguous_input(oracle):
     """Reference: sphericart-torch/python/tests/test_autograd.py:88-124 (inputs are made contiguous)."""
     rng = np.random.default_rng(2)
