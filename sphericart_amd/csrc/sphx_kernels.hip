@@ -524,7 +524,21 @@ __global__ __launch_bounds__(kValuesMaxThreads) void vjp_lanes_kernel(Tiling g, 
             V* staged = reinterpret_cast<V*>(lds);
             const unsigned nvec = len / W;
             const unsigned magic = magic_of(ny / W ? ny / W : 1u);
-            for (unsigned v = tid; v < nvec; v += threads) {
+            // many loads in flight per lane: the tile is read once, and with one load at a
+            // time the latency of HBM, several times over, was most of a large tile's time
+            constexpr unsigned DEPTH = 8;
+            unsigned v = tid;
+            for (; v + (DEPTH - 1) * threads < nvec; v += DEPTH * threads) {
+                V hold[DEPTH];
+#pragma unroll
+                for (unsigned u = 0; u < DEPTH; ++u) hold[u] = in[v + u * threads];
+#pragma unroll
+                for (unsigned u = 0; u < DEPTH; ++u) {
+                    const unsigned at = v + u * threads;
+                    staged[gap == 0 ? at : at + __umulhi(at, magic) * (gap / W)] = hold[u];
+                }
+            }
+            for (; v < nvec; v += threads) {
                 staged[gap == 0 ? v : v + __umulhi(v, magic) * (gap / W)] = in[v];
             }
             for (unsigned e = nvec * W + tid; e < len; e += threads) lds[e] = run[e]; // gap == 0 only
@@ -695,6 +709,263 @@ __global__ __launch_bounds__(kValuesMaxThreads) void vjp_lanes_kernel(Tiling g, 
         out[0] = sum_x;
         out[1] = sum_y;
         out[2] = sum_z;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// vjp_lanes_kernel for tiles of fewer than 64 points (the rows of sph_grad of 64
+// points no longer fit in LDS): a wave's lanes are 64 / tile groups of `tile`
+// lanes, every group with the same points and an l channel of its own, so that
+// no lane idles. l then differs within the wave: the prefactors come from
+// copies of the tables in LDS (one address per group) instead of the scalar
+// unit, and the groups of a wave, which take consecutive l, run one loop over m
+// from the largest l down, each lane joining at its own m = l.
+// g.off_F, g.off_Q: the tables; the waves' sums at g.off_jobs are
+// [wave][group][component][point].
+// ---------------------------------------------------------------------------
+template <typename T, bool NORM>
+__global__ __launch_bounds__(kValuesMaxThreads) void vjp_groups_kernel(Tiling g, const T* __restrict__ xyz,
+                                                                      const T* __restrict__ sph_grad,
+                                                                      T* __restrict__ xyz_grad,
+                                                                      int accumulate) {
+    constexpr int H = 6;
+    constexpr unsigned NYH = (H + 1) * (H + 1);
+    using V = typename Pack<T>::type;
+    constexpr unsigned W = Pack<T>::width;
+    T* lds = reinterpret_cast<T*>(lds_raw);
+    const unsigned tid = threadIdx.x;
+    const unsigned lane = tid & 63u;
+    const unsigned wave = tid >> 6;
+    const unsigned threads = blockDim.x;
+    const unsigned waves = threads >> 6;
+    const int L = g.l_max;
+    const unsigned ny = g.ny;
+    const unsigned group_of_tiles = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
+    if (group_of_tiles >= g.n_tiles) return;
+    const unsigned tile = static_cast<unsigned>(g.tile);
+    const unsigned groups = 64u / tile;           // lane groups per wave
+    const unsigned point = lane % tile;           // this lane's point within the tile
+    const unsigned group = lane / tile;           // this lane's group within the wave
+    const unsigned long long first = static_cast<unsigned long long>(group_of_tiles) * tile;
+    const unsigned long long left = g.n_samples - first;
+    const unsigned valid = left < tile ? static_cast<unsigned>(left) : tile;
+
+    {
+        const T* run = sph_grad + first * ny;
+        const unsigned len = valid * ny;
+        const unsigned gap = g.rows_elems - ny;
+        if ((reinterpret_cast<uintptr_t>(run) & 15u) == 0 && (gap == 0 || ny % W == 0)) {
+            const V* in = reinterpret_cast<const V*>(run);
+            V* staged = reinterpret_cast<V*>(lds);
+            const unsigned nvec = len / W;
+            const unsigned magic = magic_of(ny / W ? ny / W : 1u);
+            // many loads in flight per lane: the tile is read once, and with one load at a
+            // time the latency of HBM, several times over, was most of a large tile's time
+            constexpr unsigned DEPTH = 8;
+            unsigned v = tid;
+            for (; v + (DEPTH - 1) * threads < nvec; v += DEPTH * threads) {
+                V hold[DEPTH];
+#pragma unroll
+                for (unsigned u = 0; u < DEPTH; ++u) hold[u] = in[v + u * threads];
+#pragma unroll
+                for (unsigned u = 0; u < DEPTH; ++u) {
+                    const unsigned at = v + u * threads;
+                    staged[gap == 0 ? at : at + __umulhi(at, magic) * (gap / W)] = hold[u];
+                }
+            }
+            for (; v < nvec; v += threads) {
+                staged[gap == 0 ? v : v + __umulhi(v, magic) * (gap / W)] = in[v];
+            }
+            for (unsigned e = nvec * W + tid; e < len; e += threads) lds[e] = run[e];
+        } else {
+            for (unsigned e = tid; e < len; e += threads) {
+                lds[e + (e / ny) * gap] = run[e];
+            }
+        }
+        const unsigned tri_all = static_cast<unsigned>((L + 1) * (L + 2) / 2);
+        const T* cF = table_F<T>();
+        const T* cQ = table_Q<T>();
+        for (unsigned i = tid; i < tri_all; i += threads) {
+            lds[g.off_F + i] = cF[i];
+            lds[g.off_Q + i] = cQ[i];
+        }
+    }
+
+    Point<T> p;
+    p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
+    const T* weight = lds + point * g.rows_elems;
+    T* tab = lds + g.off_pts + point * g.off_iter; // [m][3]: c_m, s_m, 2(m+1)z
+    const bool has_point = point < valid;
+    if (has_point) {
+        p = load_point<T, NORM>(xyz + (first + point) * 3);
+        if (wave == 0 && group == 0) {
+            const T twoz = p.z + p.z;
+            T cm = 1.0, sm = 0.0, tz = twoz;
+            tab[0] = cm;
+            tab[1] = sm;
+            tab[2] = tz;
+            for (int m = 1; m <= L; ++m) {
+                const T cn = cm * p.x - sm * p.y;
+                const T sn = cm * p.y + sm * p.x;
+                tz = tz + twoz;
+                cm = cn;
+                sm = sn;
+                tab[3 * m] = cm;
+                tab[3 * m + 1] = sm;
+                tab[3 * m + 2] = tz;
+            }
+        }
+    }
+    __syncthreads(); // weights, tables
+
+    T sum_x = 0, sum_y = 0, sum_z = 0;
+    const T x = p.x, y = p.y;
+    const T rxy = p.x2 + p.y2;
+    const unsigned channels = static_cast<unsigned>(L - H);
+    const unsigned slots = (channels + groups - 1u) / groups; // a slot: `groups` consecutive channels
+    for (unsigned j = 0; j < slots; ++j) {
+        const unsigned pos = j % waves;
+        if ((((j / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue; // snake over the waves
+        const unsigned i = j * groups + group;      // channel number: l = L - i
+        const bool active = has_point && i < channels;
+        const int l = L - static_cast<int>(i);
+        const int l_top = L - static_cast<int>(j * groups); // the largest l of the slot
+        const int tri = active ? l * (l + 1) / 2 : 0;
+        const T* pk = lds + g.off_F + tri;
+        const T* qk = lds + g.off_Q + tri;
+        const T* kb = qk - l;
+        const T* wmid = weight + (active ? l * l + l : 0);
+        auto add = [&](int m, T gx_pos, T gy_pos, T gz_pos, T gx_neg, T gy_neg, T gz_neg) {
+            const T wp = wmid[m], wn = wmid[-m];
+            sum_x += gx_pos * wp;
+            sum_y += gy_pos * wp;
+            sum_z += gz_pos * wp;
+            sum_x += gx_neg * wn;
+            sum_y += gy_neg * wn;
+            sum_z += gz_neg * wn;
+        };
+        T a2 = 0, a1 = 0, b2 = 0, b1 = 0; // Q_l and Q_{l-1} at m + 2, m + 1
+        T c_hi = 0, s_hi = 0;             // c_m, s_m, carried from the step before
+        auto general = [&](int m) {
+            const T c_lo = tab[3 * (m - 1)], s_lo = tab[3 * (m - 1) + 1];
+            const T tz = tab[3 * m + 2];
+            const T a0 = qk[m] * (tz * a1 + rxy * a2);
+            const T b0 = kb[m] * (tz * b1 + rxy * b2);
+            const T pkm = pk[m];
+            T pq = a0 * pkm;
+            pq *= m;
+            const T pdq = pkm * b1;
+            const T pdqx = pdq * x;
+            const T pdqy = pdq * y;
+            const T pdz = pkm * (l + m) * b0;
+            add(m, pdqx * c_hi + pq * c_lo, pdqy * c_hi + pq * -s_lo, pdz * c_hi,
+                pdqx * s_hi + pq * s_lo, pdqy * s_hi + pq * c_lo, pdz * s_hi);
+            a2 = a1;
+            a1 = a0;
+            b2 = b1;
+            b1 = b0;
+            c_hi = c_lo;
+            s_hi = s_lo;
+        };
+        // the first steps, in which the groups join one after the other (m = l, then m = l - 1)
+        int m = l_top;
+        const int joined = l_top - static_cast<int>(groups); // from here down every lane is in the bulk
+        for (; m >= joined && m >= 1; --m) {
+            if (!active || m > l) continue;
+            if (m == l) {
+                const T c_lo = tab[3 * (m - 1)], s_lo = tab[3 * (m - 1) + 1];
+                a2 = qk[l];
+                a1 = -p.z * a2;
+                b2 = 0;
+                b1 = qk[-1];
+                T pq = a2 * pk[l];
+                pq *= l;
+                add(l, pq * c_lo, pq * -s_lo, T(0), pq * s_lo, pq * c_lo, T(0));
+                c_hi = c_lo;
+                s_hi = s_lo;
+            } else if (m == l - 1) {
+                const T c_lo = tab[3 * (m - 1)], s_lo = tab[3 * (m - 1) + 1];
+                const T pkm = pk[m];
+                T pq = a1 * pkm;
+                pq *= m;
+                const T pdq = pkm * (l + l - 1) * b1;
+                add(m, pq * c_lo, pq * -s_lo, pdq * c_hi, pq * s_lo, pq * c_lo, pdq * s_hi);
+                c_hi = c_lo;
+                s_hi = s_lo;
+            } else {
+                general(m);
+            }
+        }
+        // the bulk: the same straight-line step for every lane
+        if (active) {
+#pragma unroll 2
+            for (; m >= 1; --m) general(m);
+        }
+        if (active) {
+            // m = 0
+            const T b0 = kb[0] * (tab[2] * b1 + rxy * b2);
+            const T w0 = wmid[0];
+            sum_x += pk[0] * x * b1 * w0;
+            sum_y += pk[0] * y * b1 * w0;
+            sum_z += pk[0] * l * b0 * w0;
+        }
+    }
+    if (has_point && group == 0) {
+        // l <= 6 in closed form, slices dealt to the waves from the last one backwards
+        auto closed_slice = [&](auto lo, auto hi) {
+            constexpr int KLO = decltype(lo)::value, KHI = decltype(hi)::value;
+            T Y[NYH], DX[NYH], DY[NYH], DZ[NYH];
+            low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
+            low_gradients<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y, DX, DY, DZ);
+#pragma unroll
+            for (int k = KLO; k < KHI; ++k) {
+                const T wk = weight[k];
+                sum_x += DX[k] * wk;
+                sum_y += DY[k] * wk;
+                sum_z += DZ[k] * wk;
+            }
+        };
+        const unsigned from_last = waves - 1u - wave;
+        using std::integral_constant;
+        if (0 % waves == from_last) closed_slice(integral_constant<int, 0>{}, integral_constant<int, 9>{});
+        if (1 % waves == from_last) closed_slice(integral_constant<int, 9>{}, integral_constant<int, 16>{});
+        if (2 % waves == from_last) closed_slice(integral_constant<int, 16>{}, integral_constant<int, 25>{});
+        if (3 % waves == from_last) closed_slice(integral_constant<int, 25>{}, integral_constant<int, 31>{});
+        if (4 % waves == from_last) closed_slice(integral_constant<int, 31>{}, integral_constant<int, 36>{});
+        if (5 % waves == from_last) closed_slice(integral_constant<int, 36>{}, integral_constant<int, 41>{});
+        if (6 % waves == from_last) closed_slice(integral_constant<int, 41>{}, integral_constant<int, 45>{});
+        if (7 % waves == from_last) closed_slice(integral_constant<int, 45>{}, integral_constant<int, 49>{});
+    }
+    // every lane's sums: [wave][component][lane]; lane `point` of wave 0 adds those of its point
+    T* partial = lds + g.off_jobs;
+    partial[(wave * 3 + 0) * 64 + lane] = sum_x;
+    partial[(wave * 3 + 1) * 64 + lane] = sum_y;
+    partial[(wave * 3 + 2) * 64 + lane] = sum_z;
+    __syncthreads();
+    if (wave == 0 && group == 0 && has_point) {
+        T total_x = 0, total_y = 0, total_z = 0;
+        for (unsigned w = 0; w < waves; ++w) {
+            for (unsigned q = 0; q < groups; ++q) {
+                total_x += partial[(w * 3 + 0) * 64 + q * tile + point];
+                total_y += partial[(w * 3 + 1) * 64 + q * tile + point];
+                total_z += partial[(w * 3 + 2) * 64 + q * tile + point];
+            }
+        }
+        if constexpr (NORM) {
+            const T tmp = total_x * p.x + total_y * p.y + total_z * p.z;
+            total_x = (total_x - p.x * tmp) * p.ir;
+            total_y = (total_y - p.y * tmp) * p.ir;
+            total_z = (total_z - p.z * tmp) * p.ir;
+        }
+        T* out = xyz_grad + (first + point) * 3;
+        if (accumulate) {
+            total_x += out[0];
+            total_y += out[1];
+            total_z += out[2];
+        }
+        out[0] = total_x;
+        out[1] = total_y;
+        out[2] = total_z;
     }
 }
 
@@ -1351,6 +1622,7 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // rows a multiple of 8 words long: one vector between them (values_kernel)
     const unsigned row_stride = (ny * (esize / 4u)) % 8u == 0 ? ny + vec : ny;
     const unsigned table_stride = (3u * static_cast<unsigned>(l_max + 1)) | 1u;
+    const unsigned tri_all = static_cast<unsigned>(l_max + 1) * (l_max + 2) / 2;
     unsigned allowed = static_cast<unsigned>(env_int("SPHX_VALUES_LDS", 160 * 1024));
     if (allowed > static_cast<unsigned>(lds_limit)) allowed = static_cast<unsigned>(lds_limit);
     // Fewer than 64 points per workgroup leave lanes idle: with 32 the values kernel still beats
@@ -1368,7 +1640,10 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     for (unsigned limit : {allowed < 80u * 1024u ? allowed : 80u * 1024u, allowed}) {
         for (unsigned t = 64; t >= smallest && t >= 8 && tile == 0; t /= 2) {
             rows = (t * row_stride + vec - 1u) / vec * vec;
-            bytes = (rows + t * table_stride + (with_sums ? 8u * 3u * t : 0u)) * esize;
+            // the product: the waves' sums; with fewer than 64 points also copies of the
+            // prefactor tables (vjp_groups_kernel)
+            const unsigned extra = !with_sums ? 0u : (t == 64 ? 8u * 3u * 64u : 8u * 3u * 64u + 2u * tri_all);
+            bytes = (rows + t * table_stride + extra) * esize;
             if (bytes <= limit) tile = t;
         }
     }
@@ -1383,7 +1658,9 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     g.rows_elems = row_stride;
     g.off_pts = rows;
     g.off_iter = table_stride;
-    g.off_jobs = rows + tile * table_stride; // vjp_lanes_kernel: the waves' sums
+    g.off_jobs = rows + tile * table_stride; // the product: the waves' sums,
+    g.off_F = g.off_jobs + 8u * 3u * 64u;    // and (fewer than 64 points) the prefactor tables
+    g.off_Q = g.off_F + tri_all;
     out->workgroups = g.tiles_per_xcd * 8u;
     // one wave per l channel above the closed forms, eight at most
     int waves = env_int("SPHX_VALUES_WAVES", 8);
@@ -1902,7 +2179,15 @@ static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int
                                    lanes.g, xyz, sph_grad, xyz_grad, accumulate);
                 return hipGetLastError();
             };
-            e = normalized ? launch(vjp_lanes_kernel<T, true>) : launch(vjp_lanes_kernel<T, false>);
+            // groups of lanes with channels of their own pay off from tiles of 16 points down
+            // (200k points, float32 l_max = 24: 225 against 279 us; float64 l_max = 24: 665
+            // against 866; with tiles of 32 the scalar-unit kernel is ahead, float64 l_max = 12:
+            // 329 against 397)
+            if (lanes.g.tile > env_int("SPHX_VJP_GROUPS_BELOW", 16)) {
+                e = normalized ? launch(vjp_lanes_kernel<T, true>) : launch(vjp_lanes_kernel<T, false>);
+            } else {
+                e = normalized ? launch(vjp_groups_kernel<T, true>) : launch(vjp_groups_kernel<T, false>);
+            }
         } else if (plan.closed_only) {
             e = normalized ? dispatch_vjp<T, true>(plan.closed, l_max, xyz, sph_grad, xyz_grad, accumulate, s)
                            : dispatch_vjp<T, false>(plan.closed, l_max, xyz, sph_grad, xyz_grad, accumulate, s);
