@@ -46,7 +46,7 @@ MEASURED_TRAFFIC_BYTES = {
     "cfg5": int(((1239.8 + 1316.8) * 2.0 + 184256.0 + 3380900.0) * 1024),
     "cfg3:backward": int((394551.2 * 2.0 + 11719.3) * 1024),
     "cfg3:vjp": int((101629.1 * 2.0 + 11718.8) * 1024),
-    "cfg5:vjp": int((426697.3 * 2.0 + 2352.4) * 1024),
+    "cfg5:vjp": int((426681.8 * 2.0 + 2344.1) * 1024),
     "val10": int((5912.5 * 2.0 + 472881.4) * 1024),
 }
 
