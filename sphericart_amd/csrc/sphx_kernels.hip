@@ -362,6 +362,190 @@ __global__ __launch_bounds__(kValuesMaxThreads) void values_kernel(Tiling g, con
 }
 
 // ---------------------------------------------------------------------------
+// Values and gradients, l_max just above 6, where the four rows of 32 or 64 points
+// still fit in LDS: the construction of values_kernel with the gradient entries
+// added. One point per lane; wave 0 makes the (c_m, s_m, 2(m+1)z) tables; the
+// closed forms of l <= 6 go in slices to the waves from the last one backwards,
+// the l channels above to the waves in snake order; a lane runs the recursions
+// of Q_l^m and Q_{l-1}^m in registers and stages the entries (l, +-m) of its point
+// with the same functions as the recursion kernel (Entry, finish, put): same
+// operations, same order, same numbers. All waves then stream out the two runs.
+// g.rows_elems / g.off_dsph / g.off_ddsph: stride of a point's values row, start of
+// the gradient rows, stride of a point's three gradient rows; g.off_pts, g.off_iter:
+// the tables and their stride.
+// ---------------------------------------------------------------------------
+template <typename T, bool NORM>
+__global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tiling g, const T* __restrict__ xyz,
+                                                                           T* __restrict__ sph,
+                                                                           T* __restrict__ dsph) {
+    constexpr int H = 6;
+    using V = typename Pack<T>::type;
+    constexpr unsigned W = Pack<T>::width;
+    T* lds = reinterpret_cast<T*>(lds_raw);
+    const unsigned tid = threadIdx.x;
+    const unsigned lane = tid & 63u;
+    const unsigned wave = tid >> 6;
+    const unsigned threads = blockDim.x;
+    const unsigned waves = threads >> 6;
+    const int L = g.l_max;
+    const unsigned ny = g.ny;
+    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
+    if (group >= g.n_tiles) return;
+    const unsigned tile = static_cast<unsigned>(g.tile);
+    const unsigned long long first = static_cast<unsigned long long>(group) * tile;
+    const unsigned long long left = g.n_samples - first;
+    const unsigned valid = left < tile ? static_cast<unsigned>(left) : tile;
+
+    Point<T> p;
+    p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
+    Rows<T> rows;
+    rows.ny = static_cast<int>(ny);
+    rows.sph = lds + lane * g.rows_elems;
+    rows.dsph = lds + g.off_dsph + lane * g.off_ddsph;
+    rows.ddsph = nullptr;
+    T* tab = lds + g.off_pts + lane * g.off_iter; // [m][3]: c_m, s_m, 2(m+1)z
+    if (lane < valid) {
+        p = load_point<T, NORM>(xyz + (first + lane) * 3);
+        if (wave == 0) {
+            const T twoz = p.z + p.z;
+            T cm = 1.0, sm = 0.0, tz = twoz;
+            tab[0] = cm;
+            tab[1] = sm;
+            tab[2] = tz;
+            for (int m = 1; m <= L; ++m) {
+                const T cn = cm * p.x - sm * p.y;
+                const T sn = cm * p.y + sm * p.x;
+                tz = tz + twoz;
+                cm = cn;
+                sm = sn;
+                tab[3 * m] = cm;
+                tab[3 * m + 1] = sm;
+                tab[3 * m + 2] = tz;
+            }
+        }
+        const unsigned from_last = waves - 1u - wave;
+        if (0 % waves == from_last) closed_form_job<T, 1, NORM, H, 0, 9>(p, rows);
+        if (1 % waves == from_last) closed_form_job<T, 1, NORM, H, 9, 16>(p, rows);
+        if (2 % waves == from_last) closed_form_job<T, 1, NORM, H, 16, 25>(p, rows);
+        if (3 % waves == from_last) closed_form_job<T, 1, NORM, H, 25, 31>(p, rows);
+        if (4 % waves == from_last) closed_form_job<T, 1, NORM, H, 31, 36>(p, rows);
+        if (5 % waves == from_last) closed_form_job<T, 1, NORM, H, 36, 41>(p, rows);
+        if (6 % waves == from_last) closed_form_job<T, 1, NORM, H, 41, 45>(p, rows);
+        if (7 % waves == from_last) closed_form_job<T, 1, NORM, H, 45, 49>(p, rows);
+    }
+    __syncthreads(); // the tables
+    if (lane < valid) {
+        const T x = p.x, y = p.y;
+        const T rxy = p.x2 + p.y2;
+        const T zero = static_cast<T>(0.0);
+        const T* cF = table_F<T>();
+        const T* cQ = table_Q<T>();
+        auto entry = [&](T v, T gx, T gy, T gz) {
+            Entry<T> e;
+            e.v = v;
+            e.gx = gx;
+            e.gy = gy;
+            e.gz = gz;
+            e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = zero;
+            return e;
+        };
+        for (unsigned i = 0; static_cast<int>(i) < L - H; ++i) {
+            const unsigned pos = i % waves;
+            if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
+            const int l = L - static_cast<int>(i);
+            const int tri = l * (l + 1) / 2;
+            const int mid = 2 * tri;
+            const T* pk = cF + tri;
+            const T* qk = cQ + tri;
+            const T* kb = qk - l; // constants of the Q_{l-1} recursion
+            T a2 = qk[l];         // Q_l^l
+            T a1 = -p.z * a2;     // Q_l^{l-1}
+            T b2 = 0;             // the Q_{l-1} sequence: 0 at m = l,
+            T b1 = qk[-1];        // Q_{l-1}^{l-1} at m = l - 1
+            T c1 = tab[3 * (l - 1)], s1 = tab[3 * (l - 1) + 1];
+            T c0 = tab[3 * l], s0 = tab[3 * l + 1];
+            {
+                // m = l (templates_core.hpp:122-152)
+                auto pq = a2 * pk[l];
+                const T vp = pq * c0, vn = pq * s0;
+                pq *= l;
+                stage<T, 1, NORM>(rows, mid + l, p, entry(vp, pq * c1, pq * -s1, zero));
+                stage<T, 1, NORM>(rows, mid - l, p, entry(vn, pq * s1, pq * c1, zero));
+            }
+            c0 = c1;
+            s0 = s1;
+            c1 = tab[3 * (l - 2)];
+            s1 = tab[3 * (l - 2) + 1];
+            {
+                // m = l - 1 (:154-198)
+                const T pkm = pk[l - 1];
+                auto pq = a1 * pkm;
+                const T vp = pq * c0, vn = pq * s0;
+                pq *= (l - 1);
+                auto pdq = pkm * (l + l - 1) * b1;
+                stage<T, 1, NORM>(rows, mid + l - 1, p, entry(vp, pq * c1, pq * -s1, pdq * c0));
+                stage<T, 1, NORM>(rows, mid - (l - 1), p, entry(vn, pq * s1, pq * c1, pdq * s0));
+            }
+            for (int m = l - 2; m >= 1; --m) {
+                // :201-390
+                c0 = c1;
+                s0 = s1;
+                c1 = tab[3 * (m - 1)];
+                s1 = tab[3 * (m - 1) + 1];
+                const T tz = tab[3 * m + 2];
+                const T a0 = qk[m] * (tz * a1 + rxy * a2);
+                const T b0 = kb[m] * (tz * b1 + rxy * b2);
+                const T pkm = pk[m];
+                auto pq = a0 * pkm;
+                const T vp = pq * c0, vn = pq * s0;
+                pq *= m;
+                auto pdq = pkm * b1;
+                auto pdqx = pdq * x;
+                auto pdqy = pdq * y;
+                auto pdz = pkm * (l + m) * b0;
+                stage<T, 1, NORM>(rows, mid + m, p,
+                                  entry(vp, (pdqx * c0 + pq * c1), (pdqy * c0 + pq * -s1), pdz * c0));
+                stage<T, 1, NORM>(rows, mid - m, p,
+                                  entry(vn, (pdqx * s0 + pq * s1), (pdqy * s0 + pq * c1), pdz * s0));
+                a2 = a1;
+                a1 = a0;
+                b2 = b1;
+                b1 = b0;
+            }
+            {
+                // m = 0 (:392-426)
+                const T tz = tab[2];
+                const T a0 = qk[0] * (tz * a1 + rxy * a2);
+                const T b0 = kb[0] * (tz * b1 + rxy * b2);
+                stage<T, 1, NORM>(rows, mid, p,
+                                  entry(a0 * pk[0], pk[0] * x * b1, pk[0] * y * b1, pk[0] * l * b0));
+            }
+        }
+    }
+    __syncthreads(); // the rows
+    // one run of valid * row elements per array; the points' blocks `stride` apart in LDS
+    auto flush = [&](const T* staged, unsigned stride, unsigned row, T* dst) {
+        const unsigned len = valid * row;
+        if (stride == row) {
+            copy_out<T, SPHX_STREAMING_STORES, false, 1>(staged, dst, len, row, 0, 0, tid, threads);
+        } else if ((reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+            const unsigned per_row = row / W;
+            const unsigned magic = magic_of(per_row);
+            const V* in = reinterpret_cast<const V*>(staged);
+            V* out = reinterpret_cast<V*>(dst);
+            const unsigned nvec = len / W;
+            for (unsigned v = tid; v < nvec; v += threads) {
+                emit<T, SPHX_STREAMING_STORES>(in[v + __umulhi(v, magic)], out + v);
+            }
+        } else {
+            for (unsigned e = tid; e < len; e += threads) dst[e] = staged[e + (e / row) * (stride - row)];
+        }
+    };
+    flush(lds, g.rows_elems, ny, sph + first * ny);
+    flush(lds + g.off_dsph, g.off_ddsph, 3 * ny, dsph + first * 3 * ny);
+}
+
+// ---------------------------------------------------------------------------
 // Vector-Jacobian product without the Jacobian in memory, l_max <= 6:
 //
 //   xyz_grad[i][a] (+)= sum_k d sph[i][k] / d xyz[i][a] * sph_grad[i][k]
@@ -1675,6 +1859,64 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     return true;
 }
 
+// gradients_lanes_kernel: 64, 32 or 16 points per workgroup with their four rows and tables in
+// LDS. Returns false when too few points would be resident on a CU for it to pay.
+static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int lds_limit, Launch* out) {
+    Tiling& g = out->g;
+    std::memset(&g, 0, sizeof(g));
+    const unsigned esize = static_cast<unsigned>(elem);
+    const unsigned ny = static_cast<unsigned>(l_max + 1) * (l_max + 1);
+    const unsigned vec = 16u / esize;
+    auto stride_of = [&](unsigned block) { return (block * (esize / 4u)) % 8u == 0 ? block + vec : block; };
+    const unsigned s_stride = stride_of(ny), d_stride = stride_of(3u * ny);
+    const unsigned table_stride = (3u * static_cast<unsigned>(l_max + 1)) | 1u;
+    const unsigned limit = static_cast<unsigned>(lds_limit);
+    // Which tile: the one that keeps most points resident on a CU (tile times the workgroups
+    // that fit), a tile of 16 counted at three quarters because it leaves three lanes in four
+    // idle; between equals the larger tile, unless its workgroup would be alone on the CU (two
+    // overlap one another's phases). Measured, 500k points, float32: l_max = 7 105 us with
+    // 2 x 64 points against 119 with 4 x 32; l_max = 9 173 us with 2 x 32 against 186 with 64;
+    // l_max = 13 357 us with 3 x 16 against 433 with 32; l_max = 15 579 us with 32 against 651
+    // with 2 x 16. Below 32 resident points (or 3 x 16) the recursion kernel is the faster one
+    // (l_max = 18: 1 038 us against 1 236).
+    unsigned tile = 0, off_d = 0, off_t = 0, bytes = 0, best = 0, best_groups = 0;
+    for (unsigned t = 64; t >= 16; t /= 2) {
+        const unsigned od = (t * s_stride + vec - 1u) / vec * vec;
+        const unsigned ot = od + (t * d_stride + vec - 1u) / vec * vec;
+        const unsigned b = (ot + t * table_stride) * esize;
+        if (b > limit) continue;
+        unsigned score = (limit / b) * t * (t >= 32 ? 4u : 3u);
+        if (static_cast<unsigned>(env_int("SPHX_GRADIENT_LANES_TILE", 0)) == t) score = 1u << 30;
+        if (score > best || (score == best && best_groups < 2)) {
+            best = score;
+            best_groups = limit / b;
+            tile = t;
+            off_d = od;
+            off_t = ot;
+            bytes = b;
+        }
+    }
+    if (best < 32u * 4u) tile = 0;
+    if (tile == 0 || (n_samples + tile - 1) / tile > 0x7fffffffull) return false;
+    g.n_samples = n_samples;
+    g.l_max = l_max;
+    g.ny = static_cast<int>(ny);
+    g.tile = static_cast<int>(tile);
+    g.n_tiles = static_cast<unsigned>((n_samples + tile - 1) / tile);
+    g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
+    g.rows_elems = s_stride;
+    g.off_dsph = off_d;
+    g.off_ddsph = d_stride;
+    g.off_pts = off_t;
+    g.off_iter = table_stride;
+    out->workgroups = g.tiles_per_xcd * 8u;
+    int waves = env_int("SPHX_GRADIENT_LANES_WAVES", 8);
+    waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
+    out->threads = 64u * static_cast<unsigned>(waves);
+    out->lds_bytes = bytes;
+    return true;
+}
+
 // Tile size and LDS layout of the recursion kernel. Returns false when not even one point fits.
 static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, size_t elem,
                            unsigned budget, int lds_limit, int cus, Launch* out, bool* split_sides) {
@@ -1829,7 +2071,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
 
 // Choose kernels, tile sizes and LDS layouts. `lds_limit` / `cus` describe the device.
 static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit, int cus,
-                     Plan* plan) {
+                     Plan* plan, bool lane_kernels = true) {
     if (l_max < 0) return fail(SPHX_ERR_ARGUMENT, "l_max must be non-negative");
     if (mode < 0 || mode > 2) return fail(SPHX_ERR_ARGUMENT, "unknown derivative selector");
     if (l_max > SPHX_TABLE_LMAX) {
@@ -1849,7 +2091,12 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
         plan_closed(n_samples, l_max, l_max, mode, elem, &plan->closed);
         return SPHX_OK;
     }
-    if (mode == 0 && plan_values(n_samples, l_max, elem, lds_limit, &plan->closed)) {
+    if (lane_kernels && mode == 0 && plan_values(n_samples, l_max, elem, lds_limit, &plan->closed)) {
+        plan->lanes = true;
+        return SPHX_OK;
+    }
+    if (lane_kernels && mode == 1 && env_int("SPHX_GRADIENT_LANES", 1) != 0 &&
+        plan_gradient_lanes(n_samples, l_max, elem, lds_limit, &plan->closed)) {
         plan->lanes = true;
         return SPHX_OK;
     }
@@ -1978,6 +2225,18 @@ static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* d
                 if (e != hipSuccess) return e;
             }
             hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz, sph);
+            return hipGetLastError();
+        }
+        if constexpr (MODE == 1) {
+            const Launch& l = plan.closed;
+            auto kernel = gradients_lanes_kernel<T, NORM>;
+            if (l.lds_bytes > 64u * 1024u) {
+                unsigned unused = 0;
+                hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &unused);
+                if (e != hipSuccess) return e;
+            }
+            hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz, sph,
+                               dsph);
             return hipGetLastError();
         }
         return hipErrorInvalidValue;
@@ -2161,8 +2420,9 @@ static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int
         }
     }
     if (status == SPHX_OK && !use_lanes) {
+        // the closed-form or the recursion kernels with the contraction in place of the flush
         status = make_plan(n_samples, l_max, 1, sizeof(T), g_lds_limit[device], g_compute_units[device],
-                           &plan);
+                           &plan, false);
     }
     if (status == SPHX_OK) {
         hipStream_t s = reinterpret_cast<hipStream_t>(stream);
