@@ -115,7 +115,7 @@ def _cfg5(seed, n, first):
     return _on_axis(xyz, radius, 200, first)
 
 
-_GENERATORS = {"cfg1": _cfg1, "cfg2": _cfg2, "cfg3": _cfg3, "cfg4": _cfg4, "cfg5": _cfg5, "val10": _cfg2}
+_GENERATORS = {"cfg1": _cfg1, "cfg2": _cfg2, "cfg3": _cfg3, "cfg4": _cfg4, "cfg5": _cfg5, "val10": _cfg2, "grad10": _cfg3}
 
 WORKLOADS = {
     "cfg1": Workload(
@@ -147,5 +147,12 @@ WORKLOADS = {
     "val10": Workload(
         "val10", "spherical, l_max=10, f32, values, 1M points, uniform directions, r ~ U[0.5,5)",
         10, "f32", True, "values", 1_000_000, 1010,
+    ),
+    # likewise for the gradients kernel of l_max just above the closed forms
+    "grad10": Workload(
+        "grad10",
+        "spherical, l_max=10, f32, values+gradients, 1M points, uniform directions, r ~ U[0.5,5), "
+        "1% of the points exactly on the +-z axis",
+        10, "f32", True, "gradients", 1_000_000, 1011,
     ),
 }
