@@ -226,7 +226,8 @@ __global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __re
 // instructions per (l, +-m) pair of entries in all, a tenth of what the
 // recursion kernel spends on them. (With derivatives the entries themselves
 // dominate and rows are four and thirteen times as long, so that far fewer
-// than 64 points fit: there the recursion kernel stays.)
+// than 64 points fit: gradients_lanes_kernel takes l_max up to about 16, the
+// recursion kernel the rest.)
 //
 // The rows of 64 points take most of a CU's LDS from l_max of about 12 on, and
 // one wave would leave three of the four SIMDs idle: the l channels are dealt
