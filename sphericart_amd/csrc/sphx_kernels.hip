@@ -547,6 +547,106 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
 }
 
 // ---------------------------------------------------------------------------
+// Values, gradients and second derivatives for small l_max, where the thirteen
+// rows of 32 or 64 points fit in LDS: one point per lane again, built from the
+// recursion kernel's own jobs. A lane of wave 0 makes its point's c_m, s_m,
+// 2(m+1)z (azimuth_job) while the last wave stages l <= 1 in closed form. The l
+// channels are dealt to the waves in snake order; for a channel a lane runs the
+// three bare recursions into a scratch of its own in LDS (sequence_job) and
+// then turns every m into entries (entry_job), with no barrier in between. l
+// and m are the same for all lanes of a wave, so the branches of entry_job are
+// uniform and the prefactors come through the scalar unit; staging is free of
+// bank conflicts as every lane writes the same entry of its own point. The
+// arithmetic is the recursion kernel's, hence the reference's.
+// g.rows_elems, g.off_dsph, g.off_ddsph strides, g.off_F, g.off_Q starts of the gradient and
+// second-derivative rows; g.off_pts, g.off_iter: tables [c | s | 2(m+1)z] and their stride;
+// g.off_jobs, g.jobs_per_point: the waves' scratch [A | B | C] and a lane's share of it.
+// ---------------------------------------------------------------------------
+constexpr unsigned kHessianLaneThreads = 256; // float64 entries need more than 128 registers
+
+template <typename T, bool NORM>
+__global__ __launch_bounds__(kHessianLaneThreads) void hessians_lanes_kernel(Tiling g, const T* __restrict__ xyz,
+                                                                            T* __restrict__ sph,
+                                                                            T* __restrict__ dsph,
+                                                                            T* __restrict__ ddsph) {
+    constexpr int H = 1;
+    using V = typename Pack<T>::type;
+    constexpr unsigned W = Pack<T>::width;
+    T* lds = reinterpret_cast<T*>(lds_raw);
+    const unsigned tid = threadIdx.x;
+    const unsigned lane = tid & 63u;
+    const unsigned wave = tid >> 6;
+    const unsigned threads = blockDim.x;
+    const unsigned waves = threads >> 6;
+    const int L = g.l_max;
+    const unsigned ny = g.ny;
+    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
+    if (group >= g.n_tiles) return;
+    const unsigned tile = static_cast<unsigned>(g.tile);
+    const unsigned long long first = static_cast<unsigned long long>(group) * tile;
+    const unsigned long long left = g.n_samples - first;
+    const unsigned valid = left < tile ? static_cast<unsigned>(left) : tile;
+
+    Point<T> p;
+    p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
+    Rows<T> rows;
+    rows.ny = static_cast<int>(ny);
+    rows.sph = lds + lane * g.rows_elems;
+    rows.dsph = lds + g.off_F + lane * g.off_dsph;
+    rows.ddsph = lds + g.off_Q + lane * g.off_ddsph;
+    T* c = lds + g.off_pts + lane * g.off_iter;
+    T* sn = c + (L + 1);
+    T* tmz = sn + (L + 1);
+    if (lane < valid) {
+        p = load_point<T, NORM>(xyz + (first + lane) * 3);
+        if (wave == 0) azimuth_job<T>(p, L, c, sn, tmz);
+        if (wave == waves - 1) closed_form_job<T, 2, NORM, H>(p, rows);
+    }
+    __syncthreads(); // the tables
+    if (lane < valid) {
+        const T rxy = p.x2 + p.y2;
+        const T* cF = table_F<T>();
+        const T* cQ = table_Q<T>();
+        T* A = lds + g.off_jobs + (wave * tile + lane) * g.jobs_per_point;
+        T* B = A + (L + 1);
+        T* C = B + (L + 1);
+        for (unsigned i = 0; static_cast<int>(i) < L - H; ++i) {
+            const unsigned pos = i % waves;
+            if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
+            const int l = L - static_cast<int>(i);
+            const int tri = l * (l + 1) / 2;
+            sequence_job<T>(l, 0, p.z, rxy, cQ, tmz, A);
+            sequence_job<T>(l, 1, p.z, rxy, cQ, tmz, B);
+            sequence_job<T>(l, 2, p.z, rxy, cQ, tmz, C);
+            for (int m = l; m >= 0; --m) {
+                entry_job<T, 2, NORM, false>(l, m, tri, 0, p, cF + tri, c, sn, A, B, C, rows);
+            }
+        }
+    }
+    __syncthreads(); // the rows
+    auto flush = [&](const T* staged, unsigned stride, unsigned row, T* dst) {
+        const unsigned len = valid * row;
+        if (stride == row) {
+            copy_out<T, SPHX_STREAMING_STORES, false, 1>(staged, dst, len, row, 0, 0, tid, threads);
+        } else if ((reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+            const unsigned per_row = row / W;
+            const unsigned magic = magic_of(per_row);
+            const V* in = reinterpret_cast<const V*>(staged);
+            V* out = reinterpret_cast<V*>(dst);
+            const unsigned nvec = len / W;
+            for (unsigned v = tid; v < nvec; v += threads) {
+                emit<T, SPHX_STREAMING_STORES>(in[v + __umulhi(v, magic)], out + v);
+            }
+        } else {
+            for (unsigned e = tid; e < len; e += threads) dst[e] = staged[e + (e / row) * (stride - row)];
+        }
+    };
+    flush(lds, g.rows_elems, ny, sph + first * ny);
+    flush(lds + g.off_F, g.off_dsph, 3 * ny, dsph + first * 3 * ny);
+    flush(lds + g.off_Q, g.off_ddsph, 9 * ny, ddsph + first * 9 * ny);
+}
+
+// ---------------------------------------------------------------------------
 // Vector-Jacobian product without the Jacobian in memory, l_max <= 6:
 //
 //   xyz_grad[i][a] (+)= sum_k d sph[i][k] / d xyz[i][a] * sph_grad[i][k]
@@ -1918,6 +2018,63 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     return true;
 }
 
+// hessians_lanes_kernel: 64 or 32 points per workgroup with their thirteen rows, tables and
+// iterates in LDS. Returns false when 32 points do not fit.
+static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds_limit, Launch* out) {
+    Tiling& g = out->g;
+    std::memset(&g, 0, sizeof(g));
+    const unsigned esize = static_cast<unsigned>(elem);
+    const unsigned ny = static_cast<unsigned>(l_max + 1) * (l_max + 1);
+    const unsigned vec = 16u / esize;
+    auto stride_of = [&](unsigned block) { return (block * (esize / 4u)) % 8u == 0 ? block + vec : block; };
+    const unsigned s_stride = stride_of(ny), d_stride = stride_of(3u * ny), dd_stride = stride_of(9u * ny);
+    const unsigned table_stride = (3u * static_cast<unsigned>(l_max + 1)) | 1u;
+    const unsigned channels = static_cast<unsigned>(l_max - 1);
+    const unsigned most = kHessianLaneThreads / 64u;
+    const unsigned waves = channels < most ? channels : most;
+    const unsigned limit = static_cast<unsigned>(lds_limit);
+    unsigned tile = 0, off_d = 0, off_dd = 0, off_t = 0, off_s = 0, bytes = 0, best = 0, best_groups = 0;
+    for (unsigned t = 64; t >= 32; t /= 2) {
+        const unsigned od = (t * s_stride + vec - 1u) / vec * vec;
+        const unsigned odd = od + (t * d_stride + vec - 1u) / vec * vec;
+        const unsigned ot = odd + (t * dd_stride + vec - 1u) / vec * vec;
+        const unsigned os = ot + t * table_stride;
+        const unsigned b = (os + waves * t * table_stride) * esize;
+        if (b > limit) continue;
+        const unsigned score = (limit / b) * t;
+        if (score > best || (score == best && best_groups < 2)) {
+            best = score;
+            best_groups = limit / b;
+            tile = t;
+            off_d = od;
+            off_dd = odd;
+            off_t = ot;
+            off_s = os;
+            bytes = b;
+        }
+    }
+    if (tile == 0 || (n_samples + tile - 1) / tile > 0x7fffffffull) return false;
+    g.n_samples = n_samples;
+    g.l_max = l_max;
+    g.ny = static_cast<int>(ny);
+    g.tile = static_cast<int>(tile);
+    g.n_tiles = static_cast<unsigned>((n_samples + tile - 1) / tile);
+    g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
+    g.rows_elems = s_stride;
+    g.off_dsph = d_stride;
+    g.off_ddsph = dd_stride;
+    g.off_F = off_d;
+    g.off_Q = off_dd;
+    g.off_pts = off_t;
+    g.off_iter = table_stride;
+    g.off_jobs = off_s;
+    g.jobs_per_point = table_stride;
+    out->workgroups = g.tiles_per_xcd * 8u;
+    out->threads = 64u * waves;
+    out->lds_bytes = bytes;
+    return true;
+}
+
 // Tile size and LDS layout of the recursion kernel. Returns false when not even one point fits.
 static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, size_t elem,
                            unsigned budget, int lds_limit, int cus, Launch* out, bool* split_sides) {
@@ -2096,6 +2253,15 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
         plan->lanes = true;
         return SPHX_OK;
     }
+    // Second derivatives at small l_max: one point per lane where that was measured to be faster
+    // than the recursion kernel (SPHX_HESSIAN_LANES: 0 never, 2 wherever the rows fit).
+    const int hessian_lanes = env_int("SPHX_HESSIAN_LANES", 1);
+    const bool hessian_lanes_pay = elem == 4 ? (l_max <= 5 || l_max == 7) : l_max <= 5;
+    if (lane_kernels && mode == 2 && (hessian_lanes == 2 || (hessian_lanes == 1 && hessian_lanes_pay)) &&
+        plan_hessian_lanes(n_samples, l_max, elem, lds_limit, &plan->closed)) {
+        plan->lanes = true;
+        return SPHX_OK;
+    }
     if (lane_kernels && mode == 1 && env_int("SPHX_GRADIENT_LANES", 1) != 0 &&
         plan_gradient_lanes(n_samples, l_max, elem, lds_limit, &plan->closed)) {
         plan->lanes = true;
@@ -2238,6 +2404,18 @@ static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* d
             }
             hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz, sph,
                                dsph);
+            return hipGetLastError();
+        }
+        if constexpr (MODE == 2) {
+            const Launch& l = plan.closed;
+            auto kernel = hessians_lanes_kernel<T, NORM>;
+            if (l.lds_bytes > 64u * 1024u) {
+                unsigned unused = 0;
+                hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &unused);
+                if (e != hipSuccess) return e;
+            }
+            hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz, sph,
+                               dsph, ddsph);
             return hipGetLastError();
         }
         return hipErrorInvalidValue;

@@ -104,6 +104,34 @@ def test_many_tiles_per_workgroup_with_shifted_outputs(oracle, library, shift):
                 assert torch.isnan(raw[i][:shift]).all() and torch.isnan(raw[i][shift + sizes[i]:]).all()
 
 
+@pytest.mark.parametrize("route", ["lanes", "recursion"])
+@pytest.mark.parametrize("dtype,tdtype", [(np.float32, torch.float32), (np.float64, torch.float64)])
+def test_second_derivatives_at_small_l_max_by_both_kernels(oracle, library, route, dtype, tdtype, monkeypatch):
+    """l_max 2 ... 8 with Hessians through the one-point-per-lane kernel wherever its rows fit and
+    through the recursion kernel (the library picks per l_max by itself; the switch is read at
+    every call), sizes around a tile, shifted outputs with guard elements."""
+    monkeypatch.setenv("SPHX_HESSIAN_LANES", "2" if route == "lanes" else "0")
+    rng = np.random.default_rng(17)
+    for l_max in range(2, 9):
+        for n, shift in ((1, 0), (31, 1), (64, 0), (65, 2), (2049, 0), (4133, 3)):
+            normalized = bool((l_max + n) & 1)
+            announce("small l_max hessians", route, np.dtype(dtype).name, l_max, n, shift, normalized)
+            ny = (l_max + 1) ** 2
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, normalized, "hessians")
+            sizes = (n * ny, 3 * n * ny, 9 * n * ny)
+            shapes = ((n, ny), (n, 3, ny), (n, 3, 3, ny))
+            raw = [torch.full((s + 16,), float("nan"), dtype=tdtype, device="cuda") for s in sizes]
+            out = tuple(raw[i][shift:shift + sizes[i]].view(shapes[i]) for i in range(3))
+            status, _ = run_launch_layer(library, torch.from_numpy(xyz).cuda(), l_max, normalized, "hessians",
+                                         out=out)
+            assert status == 0, library.sphx_last_error()
+            torch.cuda.synchronize()
+            for i, (o, w) in enumerate(zip(out, want)):
+                assert same_numbers(o.cpu().numpy(), w).all(), (l_max, n, i)
+                assert torch.isnan(raw[i][:shift]).all() and torch.isnan(raw[i][shift + sizes[i]:]).all()
+
+
 def test_lds_size_alternates_between_launches(oracle):
     """One kernel, launches that need more, then less, then more LDS again (all above 64 KB)."""
     rng = np.random.default_rng(21)
