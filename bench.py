@@ -49,6 +49,7 @@ MEASURED_TRAFFIC_BYTES = {
     "cfg5:vjp": int((426681.8 * 2.0 + 2344.1) * 1024),
     "val10": int((5912.5 * 2.0 + 472881.4) * 1024),
     "grad10": int((5987.7 * 2.0 + 1890801.8) * 1024),
+    "hess5": int((3075.4 * 2.0 + 914180.9) * 1024),
 }
 
 

@@ -115,7 +115,8 @@ def _cfg5(seed, n, first):
     return _on_axis(xyz, radius, 200, first)
 
 
-_GENERATORS = {"cfg1": _cfg1, "cfg2": _cfg2, "cfg3": _cfg3, "cfg4": _cfg4, "cfg5": _cfg5, "val10": _cfg2, "grad10": _cfg3}
+_GENERATORS = {"cfg1": _cfg1, "cfg2": _cfg2, "cfg3": _cfg3, "cfg4": _cfg4, "cfg5": _cfg5, "val10": _cfg2, "grad10": _cfg3,
+               "hess5": _cfg3}
 
 WORKLOADS = {
     "cfg1": Workload(
@@ -154,5 +155,12 @@ WORKLOADS = {
         "spherical, l_max=10, f32, values+gradients, 1M points, uniform directions, r ~ U[0.5,5), "
         "1% of the points exactly on the +-z axis",
         10, "f32", True, "gradients", 1_000_000, 1011,
+    ),
+    # and for the kernel of second derivatives at small l_max
+    "hess5": Workload(
+        "hess5",
+        "spherical, l_max=5, f32, values+gradients+Hessians, 500k points, uniform directions, r ~ U[0.5,5), "
+        "1% of the points exactly on the +-z axis",
+        5, "f32", True, "hessians", 500_000, 1012,
     ),
 }

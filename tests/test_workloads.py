@@ -40,6 +40,6 @@ def test_distributions():
 
 
 def test_bytes_per_point():
-    want = {"cfg1": 2616, "cfg2": 76, "cfg3": 796, "cfg4": 30080, "cfg5": 17436, "val10": 496, "grad10": 1948}
+    want = {"cfg1": 2616, "cfg2": 76, "cfg3": 796, "cfg4": 30080, "cfg5": 17436, "val10": 496, "grad10": 1948, "hess5": 1884}
     for name, w in WORKLOADS.items():
         assert w.bytes_per_point == want[name]
