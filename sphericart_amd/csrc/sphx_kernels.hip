@@ -1,5 +1,6 @@
-// HIP kernels (gfx950) and the C-ABI launch layer declared in
-// include/sphx_launch.h.
+// The C-ABI launch layer declared in include/sphx_launch.h: plans, dispatch and
+// entry points. The kernels (gfx950) are in sphx_closed_form_kernel.hpp,
+// sphx_lane_kernels.hpp, sphx_vjp_kernels.hpp and sphx_recursion_kernel.hpp.
 //
 // Work decomposition. The outputs of consecutive points are consecutive in
 // every output array, so a workgroup takes a *tile* of S consecutive points,
@@ -40,1760 +41,13 @@
 #include "sphx_device.hpp"
 #include "sphx_tables.hpp"
 
+#include "sphx_tiling.hpp"
+#include "sphx_closed_form_kernel.hpp"
+#include "sphx_lane_kernels.hpp"
+#include "sphx_vjp_kernels.hpp"
+#include "sphx_recursion_kernel.hpp"
+
 namespace sphx {
-
-constexpr int kTableEntries = (SPHX_TABLE_LMAX + 1) * (SPHX_TABLE_LMAX + 2) / 2;
-
-__constant__ float kF32[kTableEntries];
-__constant__ float kQ32[kTableEntries];
-__constant__ double kF64[kTableEntries];
-__constant__ double kQ64[kTableEntries];
-
-template <typename T> __device__ __forceinline__ const T* table_F();
-template <typename T> __device__ __forceinline__ const T* table_Q();
-template <> __device__ __forceinline__ const float* table_F<float>() { return kF32; }
-template <> __device__ __forceinline__ const float* table_Q<float>() { return kQ32; }
-template <> __device__ __forceinline__ const double* table_F<double>() { return kF64; }
-template <> __device__ __forceinline__ const double* table_Q<double>() { return kQ64; }
-
-// Everything a kernel needs to know about the tiling; filled in on the host.
-struct Tiling {
-    unsigned long long n_samples;
-    unsigned n_tiles;       // tiles of `tile` points (recursion) or groups of 64 points (closed form)
-    unsigned tiles_per_xcd; // workgroups of one XCD walk one contiguous stretch of tiles
-    int l_max;
-    int ny;                 // (l_max + 1)^2: length of one component row in HBM
-    int tile;               // points whose rows are staged in LDS at a time
-    unsigned magic_jobs;    // ceil(2^32 / jobs_per_point)
-    unsigned jobs_per_point; // entry jobs per point: (l, m >= 0) pairs above the closed-form
-                             // limit, or (l, m, side) triples when the sides are split
-    unsigned sequence_waves; // waves that run the bare recursions (1 or 2)
-    unsigned points_per_pass; // points whose entry jobs fit side by side in the wide waves (>= 1)
-    unsigned vjp_accumulate; // fused product: add to xyz_grad instead of overwriting it
-    unsigned az_shift;      // the point tables are made for 2^az_shift tiles at a time
-    unsigned chunk_shift;   // a workgroup takes 2^chunk_shift consecutive tiles at a time
-    unsigned row_buffers;   // 2: tile n is flushed while tile n+1 is computed; 1: one after the other
-    unsigned flush_waves;   // waves that do nothing but flush (row_buffers == 2)
-    // LDS carve-up, in elements of T: the row buffers come first, rows_elems each, with the
-    // gradient and second-derivative rows at off_dsph and off_ddsph inside a buffer; the other
-    // offsets count from the start of dynamic LDS
-    unsigned rows_elems, off_dsph, off_ddsph, off_F, off_Q, off_pts, off_iter, off_jobs;
-};
-
-extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-
-// Output lines are written once and never read back by the kernel: store them with the
-// non-temporal hint (measured 10-20 % faster than plain stores here).
-#ifndef SPHX_STREAMING_STORES
-#define SPHX_STREAMING_STORES true
-#endif
-
-// LDS loads a flushing wave of the recursion kernel keeps in flight
-#ifndef SPHX_FLUSH_UNROLL
-#define SPHX_FLUSH_UNROLL 4
-#endif
-
-__host__ __device__ constexpr unsigned magic_of(unsigned long long divisor) {
-    return static_cast<unsigned>(((1ull << 32) + divisor - 1) / divisor);
-}
-
-// ---------------------------------------------------------------------------
-// l <= H in closed form. One wave per workgroup, one point per lane, 64 points
-// per workgroup.
-//
-// The finished numbers of a point stay in the lane's VGPRs; LDS is only the
-// transposition buffer between "one point per lane" and "consecutive addresses
-// per lane". The 64 points go through the buffer in PHASES passes of
-// 64 / PHASES points each when all of them do not fit.
-//
-// PREFIX == false: l_max == H. The slice of every output array that a pass
-// covers is one contiguous run, streamed out with 16-byte stores.
-// PREFIX == true: l_max > H; only the first (H+1)^2 entries of every component
-// row are produced here (the recursion kernel fills in the rest), so the runs
-// are (H+1)^2 long and ny apart.
-// ---------------------------------------------------------------------------
-// Bytes of LDS one pass may use: 52 KB lets three workgroups share a CU. Measured on MI355X,
-// l_max = 6 float32 with gradients runs fastest with a single pass (50 KB).
-#ifndef SPHX_PHASE_LDS_BUDGET
-#define SPHX_PHASE_LDS_BUDGET (52 * 1024)
-#endif
-
-__host__ __device__ constexpr unsigned components_of(int mode) {
-    return mode == 0 ? 1u : (mode == 1 ? 4u : 13u);
-}
-
-// LDS elements per point in the closed-form kernel: the rows of all arrays, each array padded
-// by one element when (H+1)^2 is even so that the per-point stride is odd (lanes staging the
-// same entry of different points then hit different banks).
-__host__ __device__ constexpr unsigned closed_form_pad(int H) {
-    return ((H + 1) * (H + 1)) % 2 == 0 ? 1u : 0u;
-}
-
-__host__ __device__ constexpr unsigned closed_form_phases(unsigned elem, int mode, int H) {
-    const unsigned ny = (H + 1) * (H + 1);
-    const unsigned per_point = (components_of(mode) * ny + (mode + 1) * closed_form_pad(H)) * elem;
-    unsigned phases = 1;
-    while (phases < 16 && (64 / phases) * per_point > SPHX_PHASE_LDS_BUDGET) {
-        phases *= 2;
-    }
-    return phases;
-}
-
-template <typename T, int MODE, bool NORM, int H, bool PREFIX>
-__global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __restrict__ xyz,
-                                                        T* __restrict__ sph, T* __restrict__ dsph,
-                                                        T* __restrict__ ddsph) {
-    constexpr unsigned PHASES = closed_form_phases(sizeof(T), MODE, H);
-    constexpr unsigned PER = 64 / PHASES;
-    constexpr unsigned NY = (H + 1) * (H + 1);
-    constexpr unsigned PAD = closed_form_pad(H);
-    // LDS: [PER][NY + PAD] values, then [PER][3 NY + PAD] gradients, then [PER][9 NY + PAD]
-    constexpr unsigned OFF_D = (PER * (NY + PAD) + 3u) & ~3u;
-    constexpr unsigned OFF_DD = (OFF_D + PER * (3 * NY + PAD) + 3u) & ~3u;
-    T* lds = reinterpret_cast<T*>(lds_raw);
-    const unsigned tid = threadIdx.x;
-    // Workgroups are handed to the 8 XCDs round-robin; give each XCD one contiguous stretch of
-    // points, so that what one XCD writes at any moment is a compact window of each array
-    // (measured: 6 % faster than the identity mapping).
-    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
-    if (group >= g.n_tiles) return;
-    const unsigned long long first = static_cast<unsigned long long>(group) * 64;
-    const unsigned long long left = g.n_samples - first;
-    const unsigned valid = left < 64ull ? static_cast<unsigned>(left) : 64u;
-
-    Entry<T> E[NY];
-    if (tid < valid) {
-        const Point<T> p = load_point<T, NORM>(xyz + (first + tid) * 3);
-        closed_form_entries<T, MODE, NORM, H>(p, E);
-    }
-#pragma unroll
-    for (unsigned phase = 0; phase < PHASES; ++phase) {
-        const unsigned base = phase * PER;
-        if (base >= valid) break; // uniform across the wave
-        if (phase > 0) __syncthreads();
-        if (tid >= base && tid < base + PER && tid < valid) {
-            const unsigned s = tid - base;
-            Rows<T> rows;
-            rows.ny = NY;
-            rows.sph = lds + s * (NY + PAD);
-            rows.dsph = lds + OFF_D + s * (3 * NY + PAD);
-            rows.ddsph = lds + OFF_DD + s * (9 * NY + PAD);
-#pragma unroll
-            for (unsigned k = 0; k < NY; ++k) {
-                put<T, MODE>(rows, k, E[k]);
-            }
-        }
-        __syncthreads();
-        const unsigned count = valid - base < PER ? valid - base : PER;
-        const unsigned long long at = first + base;
-        if constexpr (!PREFIX) {
-            copy_out<T, SPHX_STREAMING_STORES, PAD != 0>(lds, sph + at * NY, count * NY, NY, PAD,
-                                                         magic_of(NY), tid, 64);
-            if constexpr (MODE >= 1) {
-                copy_out<T, SPHX_STREAMING_STORES, PAD != 0>(lds + OFF_D, dsph + at * 3 * NY,
-                                                             count * 3 * NY, 3 * NY, PAD,
-                                                             magic_of(3 * NY), tid, 64);
-            }
-            if constexpr (MODE == 2) {
-                copy_out<T, SPHX_STREAMING_STORES, PAD != 0>(lds + OFF_DD, ddsph + at * 9 * NY,
-                                                             count * 9 * NY, 9 * NY, PAD,
-                                                             magic_of(9 * NY), tid, 64);
-            }
-        } else {
-            const unsigned ny = g.ny;
-            copy_prefixes<T, SPHX_STREAMING_STORES, NY, 1>(lds, sph + at * ny, count, ny, PAD, tid, 64);
-            if constexpr (MODE >= 1) {
-                copy_prefixes<T, SPHX_STREAMING_STORES, NY, 3>(lds + OFF_D, dsph + at * 3 * ny, count,
-                                                              ny, PAD, tid, 64);
-            }
-            if constexpr (MODE == 2) {
-                copy_prefixes<T, SPHX_STREAMING_STORES, NY, 9>(lds + OFF_DD, ddsph + at * 9 * ny,
-                                                              count, ny, PAD, tid, 64);
-            }
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// Values only, l_max > 6, rows short enough that those of 64 points fit in LDS:
-// 64 points per workgroup, one point per lane, one to eight waves that share
-// the l channels of the same 64 points.
-//
-// Without derivatives an entry is three multiplications, so what counts is what
-// surrounds them. With one point per lane l and m are the same for the whole
-// wave: the prefactors come from constant memory through the scalar unit, no
-// job has to be decoded and no iterate passes through LDS, about 15
-// instructions per (l, +-m) pair of entries in all, a tenth of what the
-// recursion kernel spends on them. (With derivatives the entries themselves
-// dominate and rows are four and thirteen times as long, so that far fewer
-// than 64 points fit: gradients_lanes_kernel takes l_max up to about 16, the
-// recursion kernel the rest.)
-//
-// The rows of 64 points take most of a CU's LDS from l_max of about 12 on, and
-// one wave would leave three of the four SIMDs idle: the l channels are dealt
-// to the waves of the workgroup (in snake order, long and short ones mixed),
-// each wave evaluating its channels for all 64 points (l_max = 15 float32,
-// 500k points: 245 us with one wave, 113 with four, 106 with six). When not
-// even 64 rows fit, 32 points per workgroup and half the lanes idle.
-//
-// Same operations in the same order as the reference: c_m, s_m, 2(m+1)z as in
-// templates.hpp:451-466, l <= 6 in closed form, then per l the recursion of
-// templates_core.hpp:122-123,155,202-204,393 downward in m, every iterate
-// multiplied by its prefactor and by c_m and s_m (:127-128,160-162,214-218,395).
-//
-// LDS: the rows of the tile in HBM layout, so that the waves stream them out
-// with 16-byte stores, and per point its table of (c_m, s_m, 2(m+1)z). A row
-// length that is a multiple of 8 words would put the same entry of all points
-// on few banks: such rows are kept one 16-byte vector apart.
-// g.rows_elems: row stride, g.off_pts: start of the tables, g.off_iter: table stride.
-// ---------------------------------------------------------------------------
-constexpr unsigned kValuesMaxThreads = 512;
-
-template <typename T, bool NORM>
-__global__ __launch_bounds__(kValuesMaxThreads) void values_kernel(Tiling g, const T* __restrict__ xyz,
-                                                                  T* __restrict__ sph) {
-    constexpr int H = 6;
-    constexpr unsigned NYH = (H + 1) * (H + 1);
-    using V = typename Pack<T>::type;
-    constexpr unsigned W = Pack<T>::width;
-    T* lds = reinterpret_cast<T*>(lds_raw);
-    const unsigned tid = threadIdx.x;
-    const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
-    const unsigned waves = blockDim.x >> 6;
-    const int L = g.l_max;
-    const unsigned ny = g.ny;
-    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
-    if (group >= g.n_tiles) return;
-    const unsigned tile = static_cast<unsigned>(g.tile); // 64, or fewer when 64 rows do not fit
-    const unsigned long long first = static_cast<unsigned long long>(group) * tile;
-    const unsigned long long left = g.n_samples - first;
-    const unsigned valid = left < tile ? static_cast<unsigned>(left) : tile;
-
-    Point<T> p;
-    p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
-    T* row = lds + lane * g.rows_elems;
-    T* tab = lds + g.off_pts + lane * g.off_iter; // [m][3]: c_m, s_m, 2(m+1)z
-    if (lane < valid) {
-        p = load_point<T, NORM>(xyz + (first + lane) * 3);
-        if (wave == 0) {
-            const T twoz = p.z + p.z;
-            T cm = 1.0, sm = 0.0, tz = twoz;
-            tab[0] = cm;
-            tab[1] = sm;
-            tab[2] = tz;
-            for (int m = 1; m <= L; ++m) {
-                const T cn = cm * p.x - sm * p.y;
-                const T sn = cm * p.y + sm * p.x;
-                tz = tz + twoz;
-                cm = cn;
-                sm = sn;
-                tab[3 * m] = cm;
-                tab[3 * m + 1] = sm;
-                tab[3 * m + 2] = tz;
-            }
-        }
-        if (wave == waves - 1) { // the last wave gets the fewest channels below
-            T Y[NYH];
-            low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
-#pragma unroll
-            for (unsigned k = 0; k < NYH; ++k) row[k] = Y[k];
-        }
-    }
-    __syncthreads(); // the tables
-    if (lane < valid) {
-        const T rxy = p.x2 + p.y2;
-        const T* cF = table_F<T>();
-        const T* cQ = table_Q<T>();
-        // channel number i = L - l goes to wave i % waves in even rounds, backwards in odd ones
-        for (unsigned i = 0; static_cast<int>(i) < L - H; ++i) {
-            const unsigned pos = i % waves;
-            if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
-            const int l = L - static_cast<int>(i);
-            const int tri = l * (l + 1) / 2;
-            const T* pk = cF + tri;
-            const T* qk = cQ + tri;
-            T* mid = row + l * l + l;
-            T v2 = qk[l];
-            T v1 = -p.z * v2;
-            {
-                const T pq = v2 * pk[l];
-                mid[l] = pq * tab[3 * l];
-                mid[-l] = pq * tab[3 * l + 1];
-            }
-            {
-                const T pq = v1 * pk[l - 1];
-                mid[l - 1] = pq * tab[3 * (l - 1)];
-                mid[-(l - 1)] = pq * tab[3 * (l - 1) + 1];
-            }
-            for (int m = l - 2; m >= 1; --m) {
-                const T v0 = qk[m] * (tab[3 * m + 2] * v1 + rxy * v2);
-                const T pq = v0 * pk[m];
-                mid[m] = pq * tab[3 * m];
-                mid[-m] = pq * tab[3 * m + 1];
-                v2 = v1;
-                v1 = v0;
-            }
-            const T v0 = qk[0] * (tab[2] * v1 + rxy * v2);
-            mid[0] = v0 * pk[0];
-        }
-    }
-    __syncthreads(); // the rows
-    T* dst = sph + first * ny;
-    const unsigned len = valid * ny;
-    const unsigned threads = blockDim.x;
-    if (g.rows_elems == ny) {
-        copy_out<T, SPHX_STREAMING_STORES, false, 1>(lds, dst, len, ny, 0, 0, tid, threads);
-    } else if ((reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
-        // rows one vector apart (their length is a whole number of vectors)
-        const unsigned per_row = ny / W;
-        const unsigned magic = magic_of(per_row);
-        const V* in = reinterpret_cast<const V*>(lds);
-        V* out = reinterpret_cast<V*>(dst);
-        const unsigned nvec = len / W;
-        for (unsigned v = tid; v < nvec; v += threads) {
-            emit<T, SPHX_STREAMING_STORES>(in[v + __umulhi(v, magic)], out + v);
-        }
-    } else {
-        for (unsigned e = tid; e < len; e += threads) {
-            const unsigned r = e / ny;
-            dst[e] = lds[e + r * (g.rows_elems - ny)];
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// Values and gradients, l_max just above 6, where the four rows of 32 or 64 points
-// still fit in LDS: the construction of values_kernel with the gradient entries
-// added. One point per lane; wave 0 makes the (c_m, s_m, 2(m+1)z) tables; the
-// closed forms of l <= 6 go in slices to the waves from the last one backwards,
-// the l channels above to the waves in snake order; a lane runs the recursions
-// of Q_l^m and Q_{l-1}^m in registers and stages the entries (l, +-m) of its point
-// with the same functions as the recursion kernel (Entry, finish, put): same
-// operations, same order, same numbers. All waves then stream out the two runs.
-// g.rows_elems / g.off_dsph / g.off_ddsph: stride of a point's values row, start of
-// the gradient rows, stride of a point's three gradient rows; g.off_pts, g.off_iter:
-// the tables and their stride.
-// ---------------------------------------------------------------------------
-template <typename T, bool NORM>
-__global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tiling g, const T* __restrict__ xyz,
-                                                                           T* __restrict__ sph,
-                                                                           T* __restrict__ dsph) {
-    constexpr int H = 6;
-    using V = typename Pack<T>::type;
-    constexpr unsigned W = Pack<T>::width;
-    T* lds = reinterpret_cast<T*>(lds_raw);
-    const unsigned tid = threadIdx.x;
-    const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
-    const unsigned threads = blockDim.x;
-    const unsigned waves = threads >> 6;
-    const int L = g.l_max;
-    const unsigned ny = g.ny;
-    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
-    if (group >= g.n_tiles) return;
-    const unsigned tile = static_cast<unsigned>(g.tile);
-    const unsigned long long first = static_cast<unsigned long long>(group) * tile;
-    const unsigned long long left = g.n_samples - first;
-    const unsigned valid = left < tile ? static_cast<unsigned>(left) : tile;
-
-    Point<T> p;
-    p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
-    Rows<T> rows;
-    rows.ny = static_cast<int>(ny);
-    rows.sph = lds + lane * g.rows_elems;
-    rows.dsph = lds + g.off_dsph + lane * g.off_ddsph;
-    rows.ddsph = nullptr;
-    T* tab = lds + g.off_pts + lane * g.off_iter; // [m][3]: c_m, s_m, 2(m+1)z
-    if (lane < valid) {
-        p = load_point<T, NORM>(xyz + (first + lane) * 3);
-        if (wave == 0) {
-            const T twoz = p.z + p.z;
-            T cm = 1.0, sm = 0.0, tz = twoz;
-            tab[0] = cm;
-            tab[1] = sm;
-            tab[2] = tz;
-            for (int m = 1; m <= L; ++m) {
-                const T cn = cm * p.x - sm * p.y;
-                const T sn = cm * p.y + sm * p.x;
-                tz = tz + twoz;
-                cm = cn;
-                sm = sn;
-                tab[3 * m] = cm;
-                tab[3 * m + 1] = sm;
-                tab[3 * m + 2] = tz;
-            }
-        }
-        const unsigned from_last = waves - 1u - wave;
-        if (0 % waves == from_last) closed_form_job<T, 1, NORM, H, 0, 9>(p, rows);
-        if (1 % waves == from_last) closed_form_job<T, 1, NORM, H, 9, 16>(p, rows);
-        if (2 % waves == from_last) closed_form_job<T, 1, NORM, H, 16, 25>(p, rows);
-        if (3 % waves == from_last) closed_form_job<T, 1, NORM, H, 25, 31>(p, rows);
-        if (4 % waves == from_last) closed_form_job<T, 1, NORM, H, 31, 36>(p, rows);
-        if (5 % waves == from_last) closed_form_job<T, 1, NORM, H, 36, 41>(p, rows);
-        if (6 % waves == from_last) closed_form_job<T, 1, NORM, H, 41, 45>(p, rows);
-        if (7 % waves == from_last) closed_form_job<T, 1, NORM, H, 45, 49>(p, rows);
-    }
-    __syncthreads(); // the tables
-    if (lane < valid) {
-        const T x = p.x, y = p.y;
-        const T rxy = p.x2 + p.y2;
-        const T zero = static_cast<T>(0.0);
-        const T* cF = table_F<T>();
-        const T* cQ = table_Q<T>();
-        auto entry = [&](T v, T gx, T gy, T gz) {
-            Entry<T> e;
-            e.v = v;
-            e.gx = gx;
-            e.gy = gy;
-            e.gz = gz;
-            e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = zero;
-            return e;
-        };
-        for (unsigned i = 0; static_cast<int>(i) < L - H; ++i) {
-            const unsigned pos = i % waves;
-            if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
-            const int l = L - static_cast<int>(i);
-            const int tri = l * (l + 1) / 2;
-            const int mid = 2 * tri;
-            const T* pk = cF + tri;
-            const T* qk = cQ + tri;
-            const T* kb = qk - l; // constants of the Q_{l-1} recursion
-            T a2 = qk[l];         // Q_l^l
-            T a1 = -p.z * a2;     // Q_l^{l-1}
-            T b2 = 0;             // the Q_{l-1} sequence: 0 at m = l,
-            T b1 = qk[-1];        // Q_{l-1}^{l-1} at m = l - 1
-            T c1 = tab[3 * (l - 1)], s1 = tab[3 * (l - 1) + 1];
-            T c0 = tab[3 * l], s0 = tab[3 * l + 1];
-            {
-                // m = l (templates_core.hpp:122-152)
-                auto pq = a2 * pk[l];
-                const T vp = pq * c0, vn = pq * s0;
-                pq *= l;
-                stage<T, 1, NORM>(rows, mid + l, p, entry(vp, pq * c1, pq * -s1, zero));
-                stage<T, 1, NORM>(rows, mid - l, p, entry(vn, pq * s1, pq * c1, zero));
-            }
-            c0 = c1;
-            s0 = s1;
-            c1 = tab[3 * (l - 2)];
-            s1 = tab[3 * (l - 2) + 1];
-            {
-                // m = l - 1 (:154-198)
-                const T pkm = pk[l - 1];
-                auto pq = a1 * pkm;
-                const T vp = pq * c0, vn = pq * s0;
-                pq *= (l - 1);
-                auto pdq = pkm * (l + l - 1) * b1;
-                stage<T, 1, NORM>(rows, mid + l - 1, p, entry(vp, pq * c1, pq * -s1, pdq * c0));
-                stage<T, 1, NORM>(rows, mid - (l - 1), p, entry(vn, pq * s1, pq * c1, pdq * s0));
-            }
-            for (int m = l - 2; m >= 1; --m) {
-                // :201-390
-                c0 = c1;
-                s0 = s1;
-                c1 = tab[3 * (m - 1)];
-                s1 = tab[3 * (m - 1) + 1];
-                const T tz = tab[3 * m + 2];
-                const T a0 = qk[m] * (tz * a1 + rxy * a2);
-                const T b0 = kb[m] * (tz * b1 + rxy * b2);
-                const T pkm = pk[m];
-                auto pq = a0 * pkm;
-                const T vp = pq * c0, vn = pq * s0;
-                pq *= m;
-                auto pdq = pkm * b1;
-                auto pdqx = pdq * x;
-                auto pdqy = pdq * y;
-                auto pdz = pkm * (l + m) * b0;
-                stage<T, 1, NORM>(rows, mid + m, p,
-                                  entry(vp, (pdqx * c0 + pq * c1), (pdqy * c0 + pq * -s1), pdz * c0));
-                stage<T, 1, NORM>(rows, mid - m, p,
-                                  entry(vn, (pdqx * s0 + pq * s1), (pdqy * s0 + pq * c1), pdz * s0));
-                a2 = a1;
-                a1 = a0;
-                b2 = b1;
-                b1 = b0;
-            }
-            {
-                // m = 0 (:392-426)
-                const T tz = tab[2];
-                const T a0 = qk[0] * (tz * a1 + rxy * a2);
-                const T b0 = kb[0] * (tz * b1 + rxy * b2);
-                stage<T, 1, NORM>(rows, mid, p,
-                                  entry(a0 * pk[0], pk[0] * x * b1, pk[0] * y * b1, pk[0] * l * b0));
-            }
-        }
-    }
-    __syncthreads(); // the rows
-    // one run of valid * row elements per array; the points' blocks `stride` apart in LDS
-    auto flush = [&](const T* staged, unsigned stride, unsigned row, T* dst) {
-        const unsigned len = valid * row;
-        if (stride == row) {
-            copy_out<T, SPHX_STREAMING_STORES, false, 1>(staged, dst, len, row, 0, 0, tid, threads);
-        } else if ((reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
-            const unsigned per_row = row / W;
-            const unsigned magic = magic_of(per_row);
-            const V* in = reinterpret_cast<const V*>(staged);
-            V* out = reinterpret_cast<V*>(dst);
-            const unsigned nvec = len / W;
-            for (unsigned v = tid; v < nvec; v += threads) {
-                emit<T, SPHX_STREAMING_STORES>(in[v + __umulhi(v, magic)], out + v);
-            }
-        } else {
-            for (unsigned e = tid; e < len; e += threads) dst[e] = staged[e + (e / row) * (stride - row)];
-        }
-    };
-    flush(lds, g.rows_elems, ny, sph + first * ny);
-    flush(lds + g.off_dsph, g.off_ddsph, 3 * ny, dsph + first * 3 * ny);
-}
-
-// ---------------------------------------------------------------------------
-// Values, gradients and second derivatives for small l_max, where the thirteen
-// rows of 32 or 64 points fit in LDS: one point per lane again, built from the
-// recursion kernel's own jobs. A lane of wave 0 makes its point's c_m, s_m,
-// 2(m+1)z (azimuth_job) while the last wave stages l <= 1 in closed form. The l
-// channels are dealt to the waves in snake order; for a channel a lane runs the
-// three bare recursions into a scratch of its own in LDS (sequence_job) and
-// then turns every m into entries (entry_job), with no barrier in between. l
-// and m are the same for all lanes of a wave, so the branches of entry_job are
-// uniform and the prefactors come through the scalar unit; staging is free of
-// bank conflicts as every lane writes the same entry of its own point. The
-// arithmetic is the recursion kernel's, hence the reference's.
-// g.rows_elems, g.off_dsph, g.off_ddsph strides, g.off_F, g.off_Q starts of the gradient and
-// second-derivative rows; g.off_pts, g.off_iter: tables [c | s | 2(m+1)z] and their stride;
-// g.off_jobs, g.jobs_per_point: the waves' scratch [A | B | C] and a lane's share of it.
-// ---------------------------------------------------------------------------
-constexpr unsigned kHessianLaneThreads = 256; // float64 entries need more than 128 registers
-
-template <typename T, bool NORM>
-__global__ __launch_bounds__(kHessianLaneThreads) void hessians_lanes_kernel(Tiling g, const T* __restrict__ xyz,
-                                                                            T* __restrict__ sph,
-                                                                            T* __restrict__ dsph,
-                                                                            T* __restrict__ ddsph) {
-    constexpr int H = 1;
-    using V = typename Pack<T>::type;
-    constexpr unsigned W = Pack<T>::width;
-    T* lds = reinterpret_cast<T*>(lds_raw);
-    const unsigned tid = threadIdx.x;
-    const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
-    const unsigned threads = blockDim.x;
-    const unsigned waves = threads >> 6;
-    const int L = g.l_max;
-    const unsigned ny = g.ny;
-    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
-    if (group >= g.n_tiles) return;
-    const unsigned tile = static_cast<unsigned>(g.tile);
-    const unsigned long long first = static_cast<unsigned long long>(group) * tile;
-    const unsigned long long left = g.n_samples - first;
-    const unsigned valid = left < tile ? static_cast<unsigned>(left) : tile;
-
-    Point<T> p;
-    p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
-    Rows<T> rows;
-    rows.ny = static_cast<int>(ny);
-    rows.sph = lds + lane * g.rows_elems;
-    rows.dsph = lds + g.off_F + lane * g.off_dsph;
-    rows.ddsph = lds + g.off_Q + lane * g.off_ddsph;
-    T* c = lds + g.off_pts + lane * g.off_iter;
-    T* sn = c + (L + 1);
-    T* tmz = sn + (L + 1);
-    if (lane < valid) {
-        p = load_point<T, NORM>(xyz + (first + lane) * 3);
-        if (wave == 0) azimuth_job<T>(p, L, c, sn, tmz);
-        if (wave == waves - 1) closed_form_job<T, 2, NORM, H>(p, rows);
-    }
-    __syncthreads(); // the tables
-    if (lane < valid) {
-        const T rxy = p.x2 + p.y2;
-        const T* cF = table_F<T>();
-        const T* cQ = table_Q<T>();
-        T* A = lds + g.off_jobs + (wave * tile + lane) * g.jobs_per_point;
-        T* B = A + (L + 1);
-        T* C = B + (L + 1);
-        for (unsigned i = 0; static_cast<int>(i) < L - H; ++i) {
-            const unsigned pos = i % waves;
-            if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
-            const int l = L - static_cast<int>(i);
-            const int tri = l * (l + 1) / 2;
-            sequence_job<T>(l, 0, p.z, rxy, cQ, tmz, A);
-            sequence_job<T>(l, 1, p.z, rxy, cQ, tmz, B);
-            sequence_job<T>(l, 2, p.z, rxy, cQ, tmz, C);
-            for (int m = l; m >= 0; --m) {
-                entry_job<T, 2, NORM, false>(l, m, tri, 0, p, cF + tri, c, sn, A, B, C, rows);
-            }
-        }
-    }
-    __syncthreads(); // the rows
-    auto flush = [&](const T* staged, unsigned stride, unsigned row, T* dst) {
-        const unsigned len = valid * row;
-        if (stride == row) {
-            copy_out<T, SPHX_STREAMING_STORES, false, 1>(staged, dst, len, row, 0, 0, tid, threads);
-        } else if ((reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
-            const unsigned per_row = row / W;
-            const unsigned magic = magic_of(per_row);
-            const V* in = reinterpret_cast<const V*>(staged);
-            V* out = reinterpret_cast<V*>(dst);
-            const unsigned nvec = len / W;
-            for (unsigned v = tid; v < nvec; v += threads) {
-                emit<T, SPHX_STREAMING_STORES>(in[v + __umulhi(v, magic)], out + v);
-            }
-        } else {
-            for (unsigned e = tid; e < len; e += threads) dst[e] = staged[e + (e / row) * (stride - row)];
-        }
-    };
-    flush(lds, g.rows_elems, ny, sph + first * ny);
-    flush(lds + g.off_F, g.off_dsph, 3 * ny, dsph + first * 3 * ny);
-    flush(lds + g.off_Q, g.off_ddsph, 9 * ny, ddsph + first * 9 * ny);
-}
-
-// ---------------------------------------------------------------------------
-// Vector-Jacobian product without the Jacobian in memory, l_max <= 6:
-//
-//   xyz_grad[i][a] (+)= sum_k d sph[i][k] / d xyz[i][a] * sph_grad[i][k]
-//
-// Same evaluation as closed_form_kernel with gradients (one point per lane, the
-// finished entries in VGPRs), but instead of staging 4 (l_max+1)^2 numbers per
-// point for HBM the lane multiplies its gradient entries with the point's row of
-// sph_grad and keeps three sums: (l_max+1)^2 + 3 numbers read and 3 written per
-// point instead of 4 (l_max+1)^2 written and read again. LDS only turns the
-// coalesced load of the tile's sph_grad rows into one row per lane (row stride
-// odd, so the lanes hit different banks). The sums run over k in index order
-// with one rounding per operation: the result is what contracting the
-// gradients of the forward pass in that order gives, bit for bit.
-// ---------------------------------------------------------------------------
-//
-// g.ny is the length of a row of sph_grad: (H+1)^2 when l_max = H; longer when this kernel
-// takes only the first (H+1)^2 entries of every row and the recursion kernel adds the rest
-// (recursion_kernel with VJP).
-template <typename T, bool NORM, int H>
-__global__ __launch_bounds__(64, 3) void closed_form_vjp_kernel(Tiling g, const T* __restrict__ xyz,
-                                                            const T* __restrict__ sph_grad,
-                                                            T* __restrict__ xyz_grad, int accumulate) {
-    constexpr unsigned NY = (H + 1) * (H + 1);
-    constexpr unsigned STRIDE = NY + closed_form_pad(H);
-    T* weights = reinterpret_cast<T*>(lds_raw);
-    const unsigned tid = threadIdx.x;
-    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
-    if (group >= g.n_tiles) return;
-    const unsigned long long first = static_cast<unsigned long long>(group) * 64;
-    const unsigned long long left = g.n_samples - first;
-    const unsigned valid = left < 64ull ? static_cast<unsigned>(left) : 64u;
-
-    // l_max = H: the tile's rows of sph_grad are one contiguous run: consecutive lanes,
-    // consecutive addresses
-    const unsigned row_stride = static_cast<unsigned>(g.ny);
-    const T* run = sph_grad + first * row_stride;
-    using V = typename Pack<T>::type;
-    constexpr unsigned W = Pack<T>::width;
-    const unsigned total = valid * NY;
-    if (row_stride != NY) {
-        for (unsigned i = tid; i < total; i += 64) {
-            const unsigned s = i / NY;
-            weights[i + (STRIDE - NY) * s] = run[static_cast<unsigned long long>(s) * row_stride + (i - s * NY)];
-        }
-    } else if ((reinterpret_cast<uintptr_t>(run) & 15u) == 0 && total % W == 0) {
-        const V* in = reinterpret_cast<const V*>(run);
-        for (unsigned v = tid; v < total / W; v += 64) {
-            const V four = in[v];
-#pragma unroll
-            for (unsigned e = 0; e < W; ++e) {
-                const unsigned i = v * W + e;
-                weights[i + (STRIDE - NY) * (i / NY)] = four[e];
-            }
-        }
-    } else {
-        for (unsigned i = tid; i < total; i += 64) {
-            weights[i + (STRIDE - NY) * (i / NY)] = run[i];
-        }
-    }
-    __syncthreads();
-    if (tid >= valid) return;
-
-    const Point<T> p = load_point<T, NORM>(xyz + (first + tid) * 3);
-    const T* mine = weights + tid * STRIDE;
-    T sum_x = 0, sum_y = 0, sum_z = 0;
-    // The entries in slices, one after the other in index order: a slice evaluates little more
-    // than its own entries (see closed_form_job), so that far fewer numbers are alive at a time
-    // than with all 3 x 49 gradient entries of a point in registers (float64: 340 registers and
-    // one wave per SIMD before). Same entries, same order of the additions.
-    auto slice = [&](auto lo, auto hi) {
-        constexpr int KLO = decltype(lo)::value, KHI = decltype(hi)::value;
-        T Y[NY], DX[NY], DY[NY], DZ[NY];
-        low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
-        low_gradients<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y, DX, DY, DZ);
-#pragma unroll
-        for (int k = KLO; k < KHI; ++k) {
-            Entry<T> e;
-            e.v = Y[k];
-            e.gx = DX[k];
-            e.gy = DY[k];
-            e.gz = DZ[k];
-            e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = static_cast<T>(0.0);
-            e = finish<T, 1, NORM>(p, e);
-            const T wk = mine[k];
-            sum_x += e.gx * wk;
-            sum_y += e.gy * wk;
-            sum_z += e.gz * wk;
-        }
-    };
-    using std::integral_constant;
-    if constexpr (H == 6) {
-        slice(integral_constant<int, 0>{}, integral_constant<int, 16>{});
-        slice(integral_constant<int, 16>{}, integral_constant<int, 25>{});
-        slice(integral_constant<int, 25>{}, integral_constant<int, 36>{});
-        slice(integral_constant<int, 36>{}, integral_constant<int, 42>{});
-        slice(integral_constant<int, 42>{}, integral_constant<int, 49>{});
-    } else {
-        slice(integral_constant<int, 0>{}, integral_constant<int, static_cast<int>(NY)>{});
-    }
-    T* out = xyz_grad + (first + tid) * 3;
-    if (accumulate) {
-        sum_x += out[0];
-        sum_y += out[1];
-        sum_z += out[2];
-    }
-    out[0] = sum_x;
-    out[1] = sum_y;
-    out[2] = sum_z;
-}
-
-// ---------------------------------------------------------------------------
-// Vector-Jacobian product, l_max > 6, one point per lane (the construction of
-// values_kernel): what passes through LDS is the tile's rows of sph_grad, read
-// from HBM with consecutive lanes at consecutive addresses, and the per-point
-// tables; the gradient entries never leave the registers. A lane runs the two
-// recursions a gradient needs (Q_l^m and Q_{l-1}^m, templates_core.hpp:202-212),
-// forms the entries (l, +-m) of the three gradient rows as the reference does
-// (:129-133, :163-170, :219-227, :396-399), multiplies them with the two
-// weights and adds to three sums. The chain rule of the normalised harmonics is
-// linear in the gradient (templates.hpp:608-612), so it is applied once, to the
-// sums. The l channels are dealt to the waves as in values_kernel; the last
-// wave also takes l <= 6 in closed form; the waves' sums meet in LDS and wave 0
-// adds them in a fixed order. The terms are added in another order than a
-// sequential loop over k would, so the result agrees with the contraction of
-// the forward gradients to rounding, not bit for bit.
-// g.rows_elems: row stride of the staged weights, g.off_pts: tables,
-// g.off_iter: table stride, g.off_jobs: the waves' sums.
-// ---------------------------------------------------------------------------
-template <typename T, bool NORM>
-__global__ __launch_bounds__(kValuesMaxThreads) void vjp_lanes_kernel(Tiling g, const T* __restrict__ xyz,
-                                                                     const T* __restrict__ sph_grad,
-                                                                     T* __restrict__ xyz_grad,
-                                                                     int accumulate) {
-    constexpr int H = 6;
-    constexpr unsigned NYH = (H + 1) * (H + 1);
-    using V = typename Pack<T>::type;
-    constexpr unsigned W = Pack<T>::width;
-    T* lds = reinterpret_cast<T*>(lds_raw);
-    const unsigned tid = threadIdx.x;
-    const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
-    const unsigned threads = blockDim.x;
-    const unsigned waves = threads >> 6;
-    const int L = g.l_max;
-    const unsigned ny = g.ny;
-    const unsigned group = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
-    if (group >= g.n_tiles) return;
-    const unsigned tile = static_cast<unsigned>(g.tile);
-    const unsigned long long first = static_cast<unsigned long long>(group) * tile;
-    const unsigned long long left = g.n_samples - first;
-    const unsigned valid = left < tile ? static_cast<unsigned>(left) : tile;
-
-    // the tile's rows of sph_grad, one contiguous run, into LDS (rows `rows_elems` apart)
-    {
-        const T* run = sph_grad + first * ny;
-        const unsigned len = valid * ny;
-        const unsigned gap = g.rows_elems - ny;
-        if ((reinterpret_cast<uintptr_t>(run) & 15u) == 0 && (gap == 0 || ny % W == 0)) {
-            const V* in = reinterpret_cast<const V*>(run);
-            V* staged = reinterpret_cast<V*>(lds);
-            const unsigned nvec = len / W;
-            const unsigned magic = magic_of(ny / W ? ny / W : 1u);
-            // many loads in flight per lane: the tile is read once, and with one load at a
-            // time the latency of HBM, several times over, was most of a large tile's time
-            constexpr unsigned DEPTH = 8;
-            unsigned v = tid;
-            for (; v + (DEPTH - 1) * threads < nvec; v += DEPTH * threads) {
-                V hold[DEPTH];
-#pragma unroll
-                for (unsigned u = 0; u < DEPTH; ++u) hold[u] = in[v + u * threads];
-#pragma unroll
-                for (unsigned u = 0; u < DEPTH; ++u) {
-                    const unsigned at = v + u * threads;
-                    staged[gap == 0 ? at : at + __umulhi(at, magic) * (gap / W)] = hold[u];
-                }
-            }
-            for (; v < nvec; v += threads) {
-                staged[gap == 0 ? v : v + __umulhi(v, magic) * (gap / W)] = in[v];
-            }
-            for (unsigned e = nvec * W + tid; e < len; e += threads) lds[e] = run[e]; // gap == 0 only
-        } else {
-            for (unsigned e = tid; e < len; e += threads) {
-                lds[e + (e / ny) * gap] = run[e];
-            }
-        }
-    }
-
-    Point<T> p;
-    p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
-    const T* weight = lds + lane * g.rows_elems;
-    T* tab = lds + g.off_pts + lane * g.off_iter; // [m][3]: c_m, s_m, 2(m+1)z
-    if (lane < valid) {
-        p = load_point<T, NORM>(xyz + (first + lane) * 3);
-        if (wave == 0) {
-            const T twoz = p.z + p.z;
-            T cm = 1.0, sm = 0.0, tz = twoz;
-            tab[0] = cm;
-            tab[1] = sm;
-            tab[2] = tz;
-            for (int m = 1; m <= L; ++m) {
-                const T cn = cm * p.x - sm * p.y;
-                const T sn = cm * p.y + sm * p.x;
-                tz = tz + twoz;
-                cm = cn;
-                sm = sn;
-                tab[3 * m] = cm;
-                tab[3 * m + 1] = sm;
-                tab[3 * m + 2] = tz;
-            }
-        }
-    }
-    __syncthreads(); // weights and tables
-
-    T sum_x = 0, sum_y = 0, sum_z = 0;
-    if (lane < valid) {
-        const T x = p.x, y = p.y;
-        const T rxy = p.x2 + p.y2;
-        const T* cF = table_F<T>();
-        const T* cQ = table_Q<T>();
-        for (unsigned i = 0; static_cast<int>(i) < L - H; ++i) {
-            const unsigned pos = i % waves;
-            if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
-            const int l = L - static_cast<int>(i);
-            const int tri = l * (l + 1) / 2;
-            const T* pk = cF + tri;
-            const T* qk = cQ + tri;
-            const T* kb = qk - l; // constants of the Q_{l-1} recursion
-            const T* wmid = weight + l * l + l;
-            // the entries (l, +m) and (l, -m) of the gradient rows times their weights
-            auto add = [&](int m, T gx_pos, T gy_pos, T gz_pos, T gx_neg, T gy_neg, T gz_neg) {
-                const T wp = wmid[m], wn = wmid[-m];
-                sum_x += gx_pos * wp;
-                sum_y += gy_pos * wp;
-                sum_z += gz_pos * wp;
-                sum_x += gx_neg * wn;
-                sum_y += gy_neg * wn;
-                sum_z += gz_neg * wn;
-            };
-            T a2 = qk[l];       // Q_l^l
-            T a1 = -p.z * a2;   // Q_l^{l-1}
-            T b2 = 0;           // the Q_{l-1} sequence: 0 at m = l,
-            T b1 = qk[-1];      // Q_{l-1}^{l-1} at m = l - 1
-            T c1 = tab[3 * (l - 1)], s1 = tab[3 * (l - 1) + 1]; // c, s at m - 1 of the step at hand
-            {
-                // m = l
-                T pq = a2 * pk[l];
-                pq *= l;
-                add(l, pq * c1, pq * -s1, T(0), pq * s1, pq * c1, T(0));
-            }
-            T c0 = c1, s0 = s1; // c, s at m
-            c1 = tab[3 * (l - 2)];
-            s1 = tab[3 * (l - 2) + 1];
-            {
-                // m = l - 1
-                const T pkm = pk[l - 1];
-                T pq = a1 * pkm;
-                pq *= (l - 1);
-                const T pdq = pkm * (l + l - 1) * b1;
-                add(l - 1, pq * c1, pq * -s1, pdq * c0, pq * s1, pq * c1, pdq * s0);
-            }
-            for (int m = l - 2; m >= 1; --m) {
-                c0 = c1;
-                s0 = s1;
-                c1 = tab[3 * (m - 1)];
-                s1 = tab[3 * (m - 1) + 1];
-                const T tz = tab[3 * m + 2];
-                const T a0 = qk[m] * (tz * a1 + rxy * a2);
-                const T b0 = kb[m] * (tz * b1 + rxy * b2);
-                const T pkm = pk[m];
-                T pq = a0 * pkm;
-                pq *= m;
-                const T pdq = pkm * b1;
-                const T pdqx = pdq * x;
-                const T pdqy = pdq * y;
-                const T pdz = pkm * (l + m) * b0;
-                add(m, pdqx * c0 + pq * c1, pdqy * c0 + pq * -s1, pdz * c0,
-                    pdqx * s0 + pq * s1, pdqy * s0 + pq * c1, pdz * s0);
-                a2 = a1;
-                a1 = a0;
-                b2 = b1;
-                b1 = b0;
-            }
-            {
-                // m = 0
-                const T b0 = kb[0] * (tab[2] * b1 + rxy * b2);
-                const T w0 = wmid[0];
-                sum_x += pk[0] * x * b1 * w0;
-                sum_y += pk[0] * y * b1 * w0;
-                sum_z += pk[0] * l * b0 * w0;
-            }
-        }
-        // l <= 6 in closed form, in slices of entries that go to the waves from the last one
-        // backwards (those have the fewest channels above); a slice evaluates little more than
-        // its own entries, see closed_form_job
-        auto closed_slice = [&](auto lo, auto hi) {
-            constexpr int KLO = decltype(lo)::value, KHI = decltype(hi)::value;
-            T Y[NYH], DX[NYH], DY[NYH], DZ[NYH];
-            low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
-            low_gradients<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y, DX, DY, DZ);
-#pragma unroll
-            for (int k = KLO; k < KHI; ++k) {
-                const T wk = weight[k];
-                sum_x += DX[k] * wk;
-                sum_y += DY[k] * wk;
-                sum_z += DZ[k] * wk;
-            }
-        };
-        const unsigned from_last = waves - 1u - wave;
-        using std::integral_constant;
-        if (0 % waves == from_last) closed_slice(integral_constant<int, 0>{}, integral_constant<int, 9>{});
-        if (1 % waves == from_last) closed_slice(integral_constant<int, 9>{}, integral_constant<int, 16>{});
-        if (2 % waves == from_last) closed_slice(integral_constant<int, 16>{}, integral_constant<int, 25>{});
-        if (3 % waves == from_last) closed_slice(integral_constant<int, 25>{}, integral_constant<int, 31>{});
-        if (4 % waves == from_last) closed_slice(integral_constant<int, 31>{}, integral_constant<int, 36>{});
-        if (5 % waves == from_last) closed_slice(integral_constant<int, 36>{}, integral_constant<int, 41>{});
-        if (6 % waves == from_last) closed_slice(integral_constant<int, 41>{}, integral_constant<int, 45>{});
-        if (7 % waves == from_last) closed_slice(integral_constant<int, 45>{}, integral_constant<int, 49>{});
-    }
-    // the waves' sums: [wave][component][point]
-    T* partial = lds + g.off_jobs;
-    if (wave != 0 && lane < valid) {
-        partial[(wave * 3 + 0) * tile + lane] = sum_x;
-        partial[(wave * 3 + 1) * tile + lane] = sum_y;
-        partial[(wave * 3 + 2) * tile + lane] = sum_z;
-    }
-    __syncthreads();
-    if (wave == 0 && lane < valid) {
-        for (unsigned w = 1; w < waves; ++w) {
-            sum_x += partial[(w * 3 + 0) * tile + lane];
-            sum_y += partial[(w * 3 + 1) * tile + lane];
-            sum_z += partial[(w * 3 + 2) * tile + lane];
-        }
-        if constexpr (NORM) {
-            const T tmp = sum_x * p.x + sum_y * p.y + sum_z * p.z;
-            sum_x = (sum_x - p.x * tmp) * p.ir;
-            sum_y = (sum_y - p.y * tmp) * p.ir;
-            sum_z = (sum_z - p.z * tmp) * p.ir;
-        }
-        T* out = xyz_grad + (first + lane) * 3;
-        if (accumulate) {
-            sum_x += out[0];
-            sum_y += out[1];
-            sum_z += out[2];
-        }
-        out[0] = sum_x;
-        out[1] = sum_y;
-        out[2] = sum_z;
-    }
-}
-
-// ---------------------------------------------------------------------------
-// vjp_lanes_kernel for tiles of fewer than 64 points (the rows of sph_grad of 64
-// points no longer fit in LDS): a wave's lanes are 64 / tile groups of `tile`
-// lanes, every group with the same points and an l channel of its own, so that
-// no lane idles. l then differs within the wave: the prefactors come from
-// copies of the tables in LDS (one address per group) instead of the scalar
-// unit, and the groups of a wave, which take consecutive l, run one loop over m
-// from the largest l down, each lane joining at its own m = l.
-// g.off_F, g.off_Q: the tables; the waves' sums at g.off_jobs are
-// [wave][group][component][point].
-// ---------------------------------------------------------------------------
-template <typename T, bool NORM>
-__global__ __launch_bounds__(kValuesMaxThreads) void vjp_groups_kernel(Tiling g, const T* __restrict__ xyz,
-                                                                      const T* __restrict__ sph_grad,
-                                                                      T* __restrict__ xyz_grad,
-                                                                      int accumulate) {
-    constexpr int H = 6;
-    constexpr unsigned NYH = (H + 1) * (H + 1);
-    using V = typename Pack<T>::type;
-    constexpr unsigned W = Pack<T>::width;
-    T* lds = reinterpret_cast<T*>(lds_raw);
-    const unsigned tid = threadIdx.x;
-    const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
-    const unsigned threads = blockDim.x;
-    const unsigned waves = threads >> 6;
-    const int L = g.l_max;
-    const unsigned ny = g.ny;
-    const unsigned group_of_tiles = (blockIdx.x & 7u) * g.tiles_per_xcd + (blockIdx.x >> 3);
-    if (group_of_tiles >= g.n_tiles) return;
-    const unsigned tile = static_cast<unsigned>(g.tile);
-    const unsigned groups = 64u / tile;           // lane groups per wave
-    const unsigned point = lane % tile;           // this lane's point within the tile
-    const unsigned group = lane / tile;           // this lane's group within the wave
-    const unsigned long long first = static_cast<unsigned long long>(group_of_tiles) * tile;
-    const unsigned long long left = g.n_samples - first;
-    const unsigned valid = left < tile ? static_cast<unsigned>(left) : tile;
-
-    {
-        const T* run = sph_grad + first * ny;
-        const unsigned len = valid * ny;
-        const unsigned gap = g.rows_elems - ny;
-        if ((reinterpret_cast<uintptr_t>(run) & 15u) == 0 && (gap == 0 || ny % W == 0)) {
-            const V* in = reinterpret_cast<const V*>(run);
-            V* staged = reinterpret_cast<V*>(lds);
-            const unsigned nvec = len / W;
-            const unsigned magic = magic_of(ny / W ? ny / W : 1u);
-            // many loads in flight per lane: the tile is read once, and with one load at a
-            // time the latency of HBM, several times over, was most of a large tile's time
-            constexpr unsigned DEPTH = 8;
-            unsigned v = tid;
-            for (; v + (DEPTH - 1) * threads < nvec; v += DEPTH * threads) {
-                V hold[DEPTH];
-#pragma unroll
-                for (unsigned u = 0; u < DEPTH; ++u) hold[u] = in[v + u * threads];
-#pragma unroll
-                for (unsigned u = 0; u < DEPTH; ++u) {
-                    const unsigned at = v + u * threads;
-                    staged[gap == 0 ? at : at + __umulhi(at, magic) * (gap / W)] = hold[u];
-                }
-            }
-            for (; v < nvec; v += threads) {
-                staged[gap == 0 ? v : v + __umulhi(v, magic) * (gap / W)] = in[v];
-            }
-            for (unsigned e = nvec * W + tid; e < len; e += threads) lds[e] = run[e];
-        } else {
-            for (unsigned e = tid; e < len; e += threads) {
-                lds[e + (e / ny) * gap] = run[e];
-            }
-        }
-        const unsigned tri_all = static_cast<unsigned>((L + 1) * (L + 2) / 2);
-        const T* cF = table_F<T>();
-        const T* cQ = table_Q<T>();
-        for (unsigned i = tid; i < tri_all; i += threads) {
-            lds[g.off_F + i] = cF[i];
-            lds[g.off_Q + i] = cQ[i];
-        }
-    }
-
-    Point<T> p;
-    p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
-    const T* weight = lds + point * g.rows_elems;
-    T* tab = lds + g.off_pts + point * g.off_iter; // [m][3]: c_m, s_m, 2(m+1)z
-    const bool has_point = point < valid;
-    if (has_point) {
-        p = load_point<T, NORM>(xyz + (first + point) * 3);
-        if (wave == 0 && group == 0) {
-            const T twoz = p.z + p.z;
-            T cm = 1.0, sm = 0.0, tz = twoz;
-            tab[0] = cm;
-            tab[1] = sm;
-            tab[2] = tz;
-            for (int m = 1; m <= L; ++m) {
-                const T cn = cm * p.x - sm * p.y;
-                const T sn = cm * p.y + sm * p.x;
-                tz = tz + twoz;
-                cm = cn;
-                sm = sn;
-                tab[3 * m] = cm;
-                tab[3 * m + 1] = sm;
-                tab[3 * m + 2] = tz;
-            }
-        }
-    }
-    __syncthreads(); // weights, tables
-
-    T sum_x = 0, sum_y = 0, sum_z = 0;
-    const T x = p.x, y = p.y;
-    const T rxy = p.x2 + p.y2;
-    const unsigned channels = static_cast<unsigned>(L - H);
-    const unsigned slots = (channels + groups - 1u) / groups; // a slot: `groups` consecutive channels
-    for (unsigned j = 0; j < slots; ++j) {
-        const unsigned pos = j % waves;
-        if ((((j / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue; // snake over the waves
-        const unsigned i = j * groups + group;      // channel number: l = L - i
-        const bool active = has_point && i < channels;
-        const int l = L - static_cast<int>(i);
-        const int l_top = L - static_cast<int>(j * groups); // the largest l of the slot
-        const int tri = active ? l * (l + 1) / 2 : 0;
-        const T* pk = lds + g.off_F + tri;
-        const T* qk = lds + g.off_Q + tri;
-        const T* kb = qk - l;
-        const T* wmid = weight + (active ? l * l + l : 0);
-        auto add = [&](int m, T gx_pos, T gy_pos, T gz_pos, T gx_neg, T gy_neg, T gz_neg) {
-            const T wp = wmid[m], wn = wmid[-m];
-            sum_x += gx_pos * wp;
-            sum_y += gy_pos * wp;
-            sum_z += gz_pos * wp;
-            sum_x += gx_neg * wn;
-            sum_y += gy_neg * wn;
-            sum_z += gz_neg * wn;
-        };
-        T a2 = 0, a1 = 0, b2 = 0, b1 = 0; // Q_l and Q_{l-1} at m + 2, m + 1
-        T c_hi = 0, s_hi = 0;             // c_m, s_m, carried from the step before
-        auto general = [&](int m) {
-            const T c_lo = tab[3 * (m - 1)], s_lo = tab[3 * (m - 1) + 1];
-            const T tz = tab[3 * m + 2];
-            const T a0 = qk[m] * (tz * a1 + rxy * a2);
-            const T b0 = kb[m] * (tz * b1 + rxy * b2);
-            const T pkm = pk[m];
-            T pq = a0 * pkm;
-            pq *= m;
-            const T pdq = pkm * b1;
-            const T pdqx = pdq * x;
-            const T pdqy = pdq * y;
-            const T pdz = pkm * (l + m) * b0;
-            add(m, pdqx * c_hi + pq * c_lo, pdqy * c_hi + pq * -s_lo, pdz * c_hi,
-                pdqx * s_hi + pq * s_lo, pdqy * s_hi + pq * c_lo, pdz * s_hi);
-            a2 = a1;
-            a1 = a0;
-            b2 = b1;
-            b1 = b0;
-            c_hi = c_lo;
-            s_hi = s_lo;
-        };
-        // the first steps, in which the groups join one after the other (m = l, then m = l - 1)
-        int m = l_top;
-        const int joined = l_top - static_cast<int>(groups); // from here down every lane is in the bulk
-        for (; m >= joined && m >= 1; --m) {
-            if (!active || m > l) continue;
-            if (m == l) {
-                const T c_lo = tab[3 * (m - 1)], s_lo = tab[3 * (m - 1) + 1];
-                a2 = qk[l];
-                a1 = -p.z * a2;
-                b2 = 0;
-                b1 = qk[-1];
-                T pq = a2 * pk[l];
-                pq *= l;
-                add(l, pq * c_lo, pq * -s_lo, T(0), pq * s_lo, pq * c_lo, T(0));
-                c_hi = c_lo;
-                s_hi = s_lo;
-            } else if (m == l - 1) {
-                const T c_lo = tab[3 * (m - 1)], s_lo = tab[3 * (m - 1) + 1];
-                const T pkm = pk[m];
-                T pq = a1 * pkm;
-                pq *= m;
-                const T pdq = pkm * (l + l - 1) * b1;
-                add(m, pq * c_lo, pq * -s_lo, pdq * c_hi, pq * s_lo, pq * c_lo, pdq * s_hi);
-                c_hi = c_lo;
-                s_hi = s_lo;
-            } else {
-                general(m);
-            }
-        }
-        // the bulk: the same straight-line step for every lane
-        if (active) {
-#pragma unroll 2
-            for (; m >= 1; --m) general(m);
-        }
-        if (active) {
-            // m = 0
-            const T b0 = kb[0] * (tab[2] * b1 + rxy * b2);
-            const T w0 = wmid[0];
-            sum_x += pk[0] * x * b1 * w0;
-            sum_y += pk[0] * y * b1 * w0;
-            sum_z += pk[0] * l * b0 * w0;
-        }
-    }
-    if (has_point && group == 0) {
-        // l <= 6 in closed form, slices dealt to the waves from the last one backwards
-        auto closed_slice = [&](auto lo, auto hi) {
-            constexpr int KLO = decltype(lo)::value, KHI = decltype(hi)::value;
-            T Y[NYH], DX[NYH], DY[NYH], DZ[NYH];
-            low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
-            low_gradients<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y, DX, DY, DZ);
-#pragma unroll
-            for (int k = KLO; k < KHI; ++k) {
-                const T wk = weight[k];
-                sum_x += DX[k] * wk;
-                sum_y += DY[k] * wk;
-                sum_z += DZ[k] * wk;
-            }
-        };
-        const unsigned from_last = waves - 1u - wave;
-        using std::integral_constant;
-        if (0 % waves == from_last) closed_slice(integral_constant<int, 0>{}, integral_constant<int, 9>{});
-        if (1 % waves == from_last) closed_slice(integral_constant<int, 9>{}, integral_constant<int, 16>{});
-        if (2 % waves == from_last) closed_slice(integral_constant<int, 16>{}, integral_constant<int, 25>{});
-        if (3 % waves == from_last) closed_slice(integral_constant<int, 25>{}, integral_constant<int, 31>{});
-        if (4 % waves == from_last) closed_slice(integral_constant<int, 31>{}, integral_constant<int, 36>{});
-        if (5 % waves == from_last) closed_slice(integral_constant<int, 36>{}, integral_constant<int, 41>{});
-        if (6 % waves == from_last) closed_slice(integral_constant<int, 41>{}, integral_constant<int, 45>{});
-        if (7 % waves == from_last) closed_slice(integral_constant<int, 45>{}, integral_constant<int, 49>{});
-    }
-    // every lane's sums: [wave][component][lane]; lane `point` of wave 0 adds those of its point
-    T* partial = lds + g.off_jobs;
-    partial[(wave * 3 + 0) * 64 + lane] = sum_x;
-    partial[(wave * 3 + 1) * 64 + lane] = sum_y;
-    partial[(wave * 3 + 2) * 64 + lane] = sum_z;
-    __syncthreads();
-    if (wave == 0 && group == 0 && has_point) {
-        T total_x = 0, total_y = 0, total_z = 0;
-        for (unsigned w = 0; w < waves; ++w) {
-            for (unsigned q = 0; q < groups; ++q) {
-                total_x += partial[(w * 3 + 0) * 64 + q * tile + point];
-                total_y += partial[(w * 3 + 1) * 64 + q * tile + point];
-                total_z += partial[(w * 3 + 2) * 64 + q * tile + point];
-            }
-        }
-        if constexpr (NORM) {
-            const T tmp = total_x * p.x + total_y * p.y + total_z * p.z;
-            total_x = (total_x - p.x * tmp) * p.ir;
-            total_y = (total_y - p.y * tmp) * p.ir;
-            total_z = (total_z - p.z * tmp) * p.ir;
-        }
-        T* out = xyz_grad + (first + point) * 3;
-        if (accumulate) {
-            total_x += out[0];
-            total_y += out[1];
-            total_z += out[2];
-        }
-        out[0] = total_x;
-        out[1] = total_y;
-        out[2] = total_z;
-    }
-}
-
-// ---------------------------------------------------------------------------
-// l > H through the recursion. 512 threads, persistent workgroups that walk
-// over tiles of `tile` consecutive points, four tiles in flight per workgroup,
-// every wave with a role of its own and one barrier per tile:
-//
-//   wave 0       one batch of up to eight tiles ahead, one lane per point:
-//                normalised coordinates, c_m, s_m, 2(m+1)z into LDS (azimuth_job);
-//   wave 1 (, 2) tile i+1, one lane per (point, l, sequence): the bare Q recursions,
-//                every iterate into LDS (sequence_job);
-//   entry waves  tile i, one job per (point, l, m >= 0): the entries (l, +-m) of
-//                every requested array, chain rule included, staged in LDS in
-//                HBM layout (entry_job). Neighbouring lanes take neighbouring m
-//                of one (point, l), so their LDS traffic falls on neighbouring
-//                banks;
-//   flush waves  tile i-1: stream its staged rows to HBM with 16-byte stores.
-//
-// The first two stages are short chains of dependent operations that only a
-// few lanes can share; running them one and two tiles ahead of the wide stage
-// takes them off the critical path. The last stage is bound by HBM, the entry
-// stage by the vector ALUs: side by side, neither waits for the other. The
-// point tables are kept in three buffers, the iterates and the staged rows in
-// two. When the rows of a single point are too long for two row buffers there
-// is one, no wave is set aside for flushing, and all waves flush tile i after
-// a second barrier.
-//
-// SPLIT == true (second derivatives, so few points per tile that the (l, m)
-// pairs of a tile leave lanes idle): the entries (l, +m) and (l, -m) are two
-// jobs.
-//
-// WHOLE == true: the closed forms of l <= H are evaluated here too (one lane
-// per point, the entries in slices that go round all waves) and the tile's
-// rows are complete, one contiguous run per array.
-// WHOLE == false: the rows start at l = H + 1 (closed_form_kernel<PREFIX>
-// writes the part below); every (point, component) row is its own run.
-// ---------------------------------------------------------------------------
-constexpr unsigned kRecursionThreads = 512;
-
-// Values and gradients: at most 128 registers, so that two workgroups share a CU (four waves
-// per SIMD) wherever their LDS allows. Only the float64 closed forms exceed that on their own
-// and spill a few registers; with 170 registers and one workgroup per CU, l_max = 12 float64
-// gradients took 800 us instead of 513 us. The second-derivative kernels keep what they need
-// (forced to 128 they spill in the entry jobs: 918 us against 558 us at l_max = 10, float64).
-template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false>
-__global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling g, const T* __restrict__ xyz,
-                                                                     T* __restrict__ sph,
-                                                                     T* __restrict__ dsph,
-                                                                     T* __restrict__ ddsph) {
-    static_assert(!VJP || (MODE == 1 && !SPLIT), "the fused product is built on the gradient kernel");
-    constexpr int H = MODE == 2 ? 1 : 6;
-    constexpr unsigned NYH = (H + 1) * (H + 1);
-    constexpr unsigned ARRAYS = MODE + 1; // iterate arrays per point: A, B, C
-    constexpr unsigned NT = kRecursionThreads;
-    T* lds = reinterpret_cast<T*>(lds_raw);
-    const unsigned tid = threadIdx.x;
-    const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
-    const int L = g.l_max;
-    const unsigned S = g.tile;
-    const unsigned ny = g.ny;
-    const unsigned nrow = WHOLE ? ny : ny - NYH; // staged elements per component row
-    const unsigned skip = WHOLE ? 0u : NYH;      // first staged entry of a row
-    // Distance between staged rows. WHOLE == false: the rows are ny apart in HBM but only nrow
-    // long; a stride that equals ny modulo 16 bytes, with the first row placed like its HBM
-    // address modulo 16 bytes, puts every staged row at the same position within 16 bytes as
-    // its destination, so that the copy is 16-byte loads and stores on both sides.
-    constexpr unsigned W16 = 16u / static_cast<unsigned>(sizeof(T));
-    const unsigned row_stride = nrow + skip % W16;
-    const unsigned tri_all = (L + 1) * (L + 2) / 2;
-
-    T* F = lds + g.off_F;
-    T* Q = lds + g.off_Q;
-    unsigned* job_table = reinterpret_cast<unsigned*>(lds + g.off_jobs);
-    {
-        const T* cF = table_F<T>();
-        const T* cQ = table_Q<T>();
-        for (unsigned i = tid; i < tri_all; i += NT) {
-            F[i] = cF[i];
-            Q[i] = cQ[i];
-        }
-        // (l, m) pairs: the bulk 1 <= m <= l - 2 first, then the special cases m = l, l - 1 and
-        // 0 each as one block, so that the lanes of a wave mostly share one branch of entry_job
-        // one word per job: m in bits 0-6, the side in bit 7, l in bits 8-15, l(l+1)/2 above
-        auto pack = [](int l, int m, int side) -> unsigned {
-            return (static_cast<unsigned>(l * (l + 1) / 2) << 16) | (static_cast<unsigned>(l) << 8) |
-                   (static_cast<unsigned>(side) << 7) | static_cast<unsigned>(m);
-        };
-        // one thread per l fills that l's places (a single thread writing all of them took
-        // 10 us at l_max = 32, a third of the time of a small evaluation)
-        if (static_cast<int>(tid) < L - H) {
-            constexpr unsigned SIDES = SPLIT ? 2u : 1u;
-            const int l = L - static_cast<int>(tid);
-            const unsigned levels = static_cast<unsigned>(L - H);
-            auto bulk_above = [&](int from) { // sum of (l' - 2) over from < l' <= L
-                return static_cast<unsigned>(L * (L + 1) / 2 - from * (from + 1) / 2 - 2 * (L - from));
-            };
-            const unsigned bulk_all = bulk_above(H);
-            for (unsigned side = 0; side < SIDES; ++side) {
-                unsigned at = side * bulk_all + bulk_above(l);
-                for (int m = l - 2; m >= 1; --m) job_table[at++] = pack(l, m, static_cast<int>(side));
-                job_table[SIDES * bulk_all + side * levels + tid] = pack(l, l, static_cast<int>(side));
-                job_table[SIDES * (bulk_all + levels) + side * levels + tid] = pack(l, l - 1, static_cast<int>(side));
-            }
-            job_table[SIDES * (bulk_all + 2 * levels) + tid] = pack(l, 0, 0);
-        }
-    }
-
-    // per point: 8 numbers (x, y, z, x^2, y^2, z^2, 1/r, x^2 + y^2), then c, s, 2(m+1)z
-    const unsigned point_stride = 8 + 3 * (L + 1);
-    // The tables are made for 2^az_shift tiles at a time (a batch), one lane per point, so that
-    // the recurrences, a chain of dependent operations that few lanes share, run once per batch
-    // instead of once per tile. Single tiles are made two rounds ahead and kept in three
-    // buffers; batches are made one batch ahead and kept in two.
-    const unsigned batch_tiles = 1u << g.az_shift;
-    const unsigned batch_lead = batch_tiles == 1 ? 2u : 1u;
-    const unsigned batch_buffers = batch_tiles == 1 ? 3u : 2u;
-    auto point_data = [&](unsigned n, unsigned s) -> T* { // point s of this workgroup's n-th tile
-        const unsigned slot = (((n >> g.az_shift) % batch_buffers) << g.az_shift) | (n & (batch_tiles - 1u));
-        return lds + g.off_pts + (slot * S + s) * point_stride;
-    };
-    auto iterates = [&](unsigned buffer, unsigned s, unsigned which, int l) -> T* {
-        return lds + g.off_iter + ((buffer * S + s) * ARRAYS + which) * tri_all + l * (l + 1) / 2;
-    };
-
-    // same XCD-contiguous walk as the closed-form kernel
-    const unsigned xcd = blockIdx.x & 7u;
-    const unsigned rank_in_xcd = blockIdx.x >> 3;
-    const unsigned groups_per_xcd = gridDim.x >> 3;
-    const unsigned xcd_first = xcd * g.tiles_per_xcd;
-    unsigned xcd_last = xcd_first + g.tiles_per_xcd;
-    if (xcd_last > g.n_tiles) xcd_last = g.n_tiles;
-    // A workgroup takes chunks of C consecutive tiles; the chunks of an XCD's workgroups lie
-    // side by side. Consecutive tiles in one workgroup share the 128-byte lines in which one
-    // ends and the next begins (see flush_run); C stays small so that what the XCD writes at any
-    // moment remains a compact window.
-    const unsigned chunk_mask = (1u << g.chunk_shift) - 1u;
-    if (xcd_first + (rank_in_xcd << g.chunk_shift) >= xcd_last) return; // whole workgroup
-
-    // the n-th tile of this workgroup, and how many points it has (0 past the end)
-    auto tile_of = [&](unsigned n) -> unsigned {
-        return xcd_first + ((((n >> g.chunk_shift) * groups_per_xcd + rank_in_xcd)) << g.chunk_shift) +
-               (n & chunk_mask);
-    };
-    auto valid_in = [&](unsigned n) -> unsigned {
-        const unsigned t = tile_of(n);
-        if (t >= xcd_last) return 0u;
-        const unsigned long long first = static_cast<unsigned long long>(t) * S;
-        const unsigned long long left = g.n_samples - first;
-        return left < S ? static_cast<unsigned>(left) : S;
-    };
-    // lane j of wave 0 takes point j % S of tile j / S of a batch (batch_tiles * S <= 64)
-    auto fetch = [&](unsigned batch, T& rx, T& ry, T& rz) {
-        rx = ry = rz = 0;
-        const unsigned n = (batch << g.az_shift) + lane / S;
-        const unsigned s = lane % S;
-        if (lane < batch_tiles * S && s < valid_in(n)) {
-            const T* src = xyz + (static_cast<unsigned long long>(tile_of(n)) * S + s) * 3;
-            rx = src[0];
-            ry = src[1];
-            rz = src[2];
-        }
-    };
-    // stage one of a batch of tiles (wave 0; lane == tid there)
-    auto azimuth_stage = [&](unsigned batch, T rx, T ry, T rz) {
-        const unsigned n = (batch << g.az_shift) + lane / S;
-        const unsigned s = lane % S;
-        if (lane < batch_tiles * S && s < valid_in(n)) {
-            T* rec = point_data(n, s);
-            Point<T> p;
-            p.x = rx;
-            p.y = ry;
-            p.z = rz;
-            p.x2 = p.x * p.x;
-            p.y2 = p.y * p.y;
-            p.z2 = p.z * p.z;
-            p.ir = 0.0;
-            if constexpr (NORM) {
-                p.ir = 1 / root(p.x2 + p.y2 + p.z2);
-                p.x *= p.ir;
-                p.y *= p.ir;
-                p.z *= p.ir;
-                p.x2 = p.x * p.x;
-                p.y2 = p.y * p.y;
-                p.z2 = p.z * p.z;
-            }
-            rec[0] = p.x;
-            rec[1] = p.y;
-            rec[2] = p.z;
-            rec[3] = p.x2;
-            rec[4] = p.y2;
-            rec[5] = p.z2;
-            rec[6] = p.ir;
-            rec[7] = p.x2 + p.y2;
-            azimuth_job<T>(p, L, rec + 8, rec + 8 + (L + 1), rec + 8 + 2 * (L + 1));
-        }
-    };
-    // stage two of tile n (waves 1 .. g.sequence_waves)
-    auto recursion_stage = [&](unsigned n) {
-        const unsigned count = valid_in(n);
-        const unsigned per_l = count * ARRAYS;
-        const unsigned jobs = per_l * static_cast<unsigned>(L - H);
-        for (unsigned j = tid - 64; j < jobs; j += 64 * g.sequence_waves) { // waves 1 .. sequence_waves
-            const unsigned step = j / per_l;
-            const unsigned rest = j - step * per_l;
-            const int l = L - static_cast<int>(step); // longest recursions first
-            const unsigned s = rest / ARRAYS;
-            const unsigned which = rest - s * ARRAYS;
-            const T* rec = point_data(n, s);
-            sequence_job<T>(l, static_cast<int>(which), rec[2], rec[7], Q, rec + 8 + 2 * (L + 1),
-                            iterates(n & 1u, s, which, l));
-        }
-    };
-
-    // The waves between the sequence waves and the flush waves compute entries.
-    const bool streaming = g.row_buffers == 2;
-    const unsigned entry_first_wave = 1 + g.sequence_waves;
-    const unsigned entry_end_wave = NT / 64 - (streaming ? g.flush_waves : 0u);
-    const unsigned wide_first = 64 * entry_first_wave;
-    const unsigned wide_lanes = 64 * (entry_end_wave - entry_first_wave);
-
-    constexpr unsigned LINE = 128u / static_cast<unsigned>(sizeof(T)); // elements per 128-byte line
-    // position within its 128-byte line of element `element` of an output array
-    auto phase_of = [](const T* array, unsigned long long element) -> unsigned {
-        return static_cast<unsigned>((reinterpret_cast<uintptr_t>(array) / sizeof(T) + element) % LINE);
-    };
-
-    // Where the rows of tile n start within their staging regions. WHOLE: element 0 of a region
-    // stands for the start of the 128-byte line in which the tile's run begins in HBM, so the run
-    // itself starts `phase` elements in. WHOLE == false: position within 16 bytes of the first
-    // staged row, see row_stride. VJP: the rows never leave LDS, no position to match.
-    struct Phases {
-        unsigned sph, dsph, ddsph;
-    };
-    auto phases_of = [&](unsigned n) -> Phases {
-        const unsigned long long first_point = static_cast<unsigned long long>(tile_of(n)) * S;
-        Phases ph;
-        ph.sph = VJP ? 0u : phase_of(sph, first_point * ny + skip) % (WHOLE ? LINE : W16);
-        ph.dsph = VJP || MODE < 1 ? 0u : phase_of(dsph, first_point * 3 * ny + skip) % (WHOLE ? LINE : W16);
-        ph.ddsph = WHOLE && !VJP && MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
-        return ph;
-    };
-
-    // WHOLE: the closed forms of tile n, one lane per point, into row buffer `buffer`. The
-    // entries of a point are cut in slices (by l), dealt to `among` waves of which this is number
-    // `who`, so that no single wave carries all of the chain rule and staging.
-    auto closed_stage = [&](unsigned n, unsigned buffer, unsigned who, unsigned among) {
-        if constexpr (WHOLE) {
-            const unsigned valid = valid_in(n);
-            if (lane < valid) {
-                T* staged = lds + buffer * g.rows_elems;
-                const Phases ph = phases_of(n);
-                const T* rec = point_data(n, lane);
-                Point<T> p;
-                p.x = rec[0];
-                p.y = rec[1];
-                p.z = rec[2];
-                p.x2 = rec[3];
-                p.y2 = rec[4];
-                p.z2 = rec[5];
-                p.ir = rec[6];
-                Rows<T> rows;
-                rows.ny = static_cast<int>(ny);
-                rows.sph = staged + ph.sph + lane * ny;
-                rows.dsph = staged + g.off_dsph + ph.dsph + lane * 3 * ny;
-                rows.ddsph = staged + g.off_ddsph + ph.ddsph + lane * 9 * ny;
-                if constexpr (H == 6) {
-                    // float32 rows a multiple of 32 words long (l_max = 7, 15, 23, ...): the
-                    // stores of all lanes would fall on one LDS bank; stored in rotated fours
-                    // instead (closed_form_job; l_max = 7, 500k points, gradients: 343 -> 216 us).
-                    // Not for float64 and not for values alone, where the selects cost registers
-                    // that the kernel does not have to spare (values: 68 -> 89, and l_max = 9 lost
-                    // its third workgroup per CU, 80 -> 106 us).
-                    constexpr bool MAY_ROTATE = sizeof(T) == 4 && MODE == 1;
-                    if (MAY_ROTATE && (ny & 31u) == 0) {
-                        const unsigned turn = lane & 3u;
-                        if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 8, true>(p, rows, turn);
-                        if (1 % among == who) closed_form_job<T, MODE, NORM, H, 8, 16, true>(p, rows, turn);
-                        if (2 % among == who) closed_form_job<T, MODE, NORM, H, 16, 24, true>(p, rows, turn);
-                        if (3 % among == who) closed_form_job<T, MODE, NORM, H, 24, 32, true>(p, rows, turn);
-                        if (4 % among == who) closed_form_job<T, MODE, NORM, H, 32, 40, true>(p, rows, turn);
-                        if (5 % among == who) closed_form_job<T, MODE, NORM, H, 40, 49, true>(p, rows, turn);
-                    } else {
-                        if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows);
-                        if (1 % among == who) closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows);
-                        if (2 % among == who) closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows);
-                        if (3 % among == who) closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows);
-                        if (4 % among == who) closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows);
-                        if (5 % among == who) closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows);
-                        if (6 % among == who) closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows);
-                        if (7 % among == who) closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows);
-                    }
-                } else {
-                    if (who == 0) closed_form_job<T, MODE, NORM, H>(p, rows);
-                }
-            }
-        }
-    };
-
-    // stage three of tile n, into row buffer `buffer` (the entry waves)
-    auto entry_stage = [&](unsigned n, unsigned buffer) {
-        const unsigned valid = valid_in(n);
-        T* staged = lds + buffer * g.rows_elems;
-        const unsigned t = tid - wide_first;
-        const Phases ph = phases_of(n);
-        const unsigned phase_sph = ph.sph, phase_dsph = ph.dsph, phase_ddsph = ph.ddsph;
-        // One pass takes the jobs of as many points as fit side by side in the wide lanes
-        // (of one point, in several rounds, when it has more jobs than there are lanes);
-        // what depends on the point only is read once per pass.
-        unsigned local = 0, e_first = t;
-        if (g.points_per_pass > 1) {
-            local = __umulhi(t, g.magic_jobs);
-            e_first = t - local * g.jobs_per_point;
-        }
-        for (unsigned s0 = 0; s0 < valid; s0 += g.points_per_pass) {
-            const unsigned s = s0 + local;
-            if (s >= valid || local >= g.points_per_pass) continue;
-            const T* rec = point_data(n, s);
-            Point<T> p;
-            p.x = rec[0];
-            p.y = rec[1];
-            p.z = rec[2];
-            p.x2 = rec[3];
-            p.y2 = rec[4];
-            p.z2 = rec[5];
-            p.ir = rec[6];
-            const T* c = rec + 8;
-            const T* sn = rec + 8 + (L + 1);
-            const T* itA = iterates(n & 1u, s, 0, 0);
-            const T* itB = iterates(n & 1u, s, MODE >= 1 ? 1 : 0, 0);
-            const T* itC = iterates(n & 1u, s, MODE == 2 ? 2 : 0, 0);
-            // rows are addressed with the entry's index in the full row; shift the bases when
-            // the staged rows start at l = H + 1
-            Rows<T> rows;
-            rows.ny = static_cast<int>(row_stride);
-            rows.sph = staged + phase_sph + s * row_stride - skip;
-            rows.dsph = staged + g.off_dsph + phase_dsph + s * 3 * row_stride - skip;
-            rows.ddsph = staged + g.off_ddsph + phase_ddsph + s * 9 * row_stride - skip;
-            for (unsigned e = e_first; e < g.jobs_per_point; e += wide_lanes) {
-                const unsigned packed = job_table[e];
-                const int m = static_cast<int>(packed & 0x7fu);
-                const int side = static_cast<int>((packed >> 7) & 1u);
-                const int l = static_cast<int>((packed >> 8) & 0xffu);
-                const int tri = static_cast<int>(packed >> 16);
-                entry_job<T, MODE, NORM, SPLIT>(l, m, tri, side, p, F + tri, c, sn, itA + tri,
-                                                itB + tri, itC + tri, rows);
-            }
-        }
-    };
-
-    // last stage of tile n: row buffer `buffer` to HBM, by `count` threads of which this is
-    // number `ft`. `lone` (a std::integral_constant): the copy of a run is the work of a single
-    // wave, which then keeps several LDS loads in flight; with all waves of the workgroup on one
-    // run, loads and stores alternating one by one measured faster.
-    auto flush_stage = [&](unsigned n, unsigned buffer, unsigned ft, unsigned count, auto lone) {
-        constexpr int WHOLE_UNROLL = decltype(lone)::value ? SPHX_FLUSH_UNROLL : 1;
-        const unsigned valid = valid_in(n);
-        const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
-        const T* staged = lds + buffer * g.rows_elems;
-        if constexpr (WHOLE) {
-            // The tile's run of `len` elements of one output array starts at element `at` of that
-            // array. Only whole 128-byte lines go out with vector stores. The line in which the
-            // run ends is completed by the next tile: when that tile is this workgroup's next one
-            // (same chunk), the unfinished part is carried over into the region the next tile is
-            // staged in; at the ends of a chunk the partial lines are stored element by element.
-            const bool starts = (n & chunk_mask) == 0;
-            const bool ends = (n & chunk_mask) == chunk_mask || valid_in(n + 1) == 0;
-            T* carry_to = lds + (streaming ? (buffer ^ 1u) : buffer) * g.rows_elems;
-            auto flush_run = [&](unsigned region_offset, T* array, unsigned long long at, unsigned len) {
-                using V = typename Pack<T>::type;
-                constexpr unsigned W = Pack<T>::width;
-                T* region = lds + buffer * g.rows_elems + region_offset;
-                const unsigned phase = phase_of(array, at);
-                T* line0 = array + (at - phase); // HBM address of region element 0
-                const unsigned lo = starts ? phase : 0u; // first element that holds data
-                const unsigned hi = phase + len;
-                const unsigned full_lo = (lo + LINE - 1u) / LINE * LINE;
-                const unsigned full_hi = hi / LINE * LINE;
-                unsigned tail_from; // what follows the head and the whole lines
-                if (full_hi > full_lo) {
-                    const unsigned nvec = (full_hi - full_lo) / W;
-                    const V* in = reinterpret_cast<const V*>(region + full_lo);
-                    V* out = reinterpret_cast<V*>(line0 + full_lo);
-                    unsigned v = ft;
-                    if constexpr (WHOLE_UNROLL > 1) {
-                        for (; v + (WHOLE_UNROLL - 1) * count < nvec; v += WHOLE_UNROLL * count) {
-                            V hold[WHOLE_UNROLL];
-#pragma unroll
-                            for (int u = 0; u < WHOLE_UNROLL; ++u) hold[u] = in[v + u * count];
-#pragma unroll
-                            for (int u = 0; u < WHOLE_UNROLL; ++u) {
-                                emit<T, SPHX_STREAMING_STORES>(hold[u], out + v + u * count);
-                            }
-                        }
-                    }
-                    for (; v < nvec; v += count) {
-                        emit<T, SPHX_STREAMING_STORES>(in[v], out + v);
-                    }
-                    tail_from = full_hi;
-                } else {
-                    tail_from = full_lo < hi ? full_lo : hi;
-                }
-                // head: the part of the first line that belongs to this chunk
-                const unsigned head_end = full_lo < hi ? full_lo : hi;
-                if (lo + ft < head_end) line0[lo + ft] = region[lo + ft];
-                // tail: stored if the chunk ends here, else handed to the next tile
-                const unsigned tail = hi - tail_from;
-                if (ft < tail) {
-                    const T value = region[tail_from + ft];
-                    if (ends) {
-                        line0[tail_from + ft] = value;
-                    } else if (carry_to + region_offset != region || tail_from != 0) {
-                        carry_to[region_offset + ft] = value;
-                    }
-                }
-            };
-            flush_run(0, sph, first * ny, valid * ny);
-            if constexpr (MODE >= 1) flush_run(g.off_dsph, dsph, first * 3 * ny, valid * 3 * ny);
-            if constexpr (MODE == 2) flush_run(g.off_ddsph, ddsph, first * 9 * ny, valid * 9 * ny);
-        } else {
-            // one run per (point, component) row, dealt to the waves in turn
-            const unsigned waves = count / 64;
-            for (unsigned r = ft >> 6; r < valid * components_of(MODE); r += waves) {
-                // rows [0, valid) are values, the next 3 * valid are gradients
-                if (r < valid) {
-                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL>(
-                        staged + phase_of(sph, first * ny + skip) % W16 + r * row_stride,
-                        sph + (first + r) * ny + skip, nrow, nrow, 0, 0, ft & 63u, 64);
-                } else {
-                    const unsigned q = r - valid;
-                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL>(
-                        staged + g.off_dsph + phase_of(dsph, first * 3 * ny + skip) % W16 + q * row_stride,
-                        dsph + (first * 3 + q) * ny + skip, nrow, nrow, 0, 0, ft & 63u, 64);
-                }
-            }
-        }
-    };
-
-    // VJP: in place of the flush. `sph` holds the upstream gradient sph_grad[N][ny] (read
-    // only), `dsph` is xyz_grad[N][3]. Wave 1 + r takes gradient row r of the tile (point r / 3,
-    // component r % 3): its lanes multiply the staged entries with the point's row of sph_grad
-    // and a butterfly adds the lanes' sums up. With WHOLE == false the staged rows begin at
-    // l = H + 1 and closed_form_vjp_kernel has already stored the sum over l <= H, so the
-    // result is added to what xyz_grad holds. Wave 0 stays out: it has loads in flight.
-    auto contract_stage = [&](unsigned n, unsigned buffer) {
-        if constexpr (VJP) {
-            const unsigned valid = valid_in(n);
-            const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
-            const T* staged = lds + buffer * g.rows_elems + g.off_dsph;
-            const T* upstream = sph;
-            T* xyz_grad = dsph;
-            if (wave == 0) return;
-            for (unsigned r = wave - 1; r < valid * 3; r += NT / 64 - 1) {
-                const unsigned s = r / 3;
-                const T* row = staged + r * row_stride - skip; // indexed with the entry's index in the full row
-                const T* weight = upstream + (first + s) * ny;
-                T partial = 0;
-#pragma unroll 4
-                for (unsigned k = skip + lane; k < ny; k += 64) {
-                    partial += row[k] * weight[k];
-                }
-                for (unsigned offset = 32; offset > 0; offset >>= 1) {
-                    partial += __shfl_xor(partial, static_cast<int>(offset));
-                }
-                if (lane == 0) {
-                    T* out = xyz_grad + first * 3 + r;
-                    *out = (!WHOLE || g.vjp_accumulate) ? *out + partial : partial;
-                }
-            }
-        }
-    };
-
-    // fill the pipeline: tables of tiles 0 and 1, iterates of tile 0
-    T rx = 0, ry = 0, rz = 0;
-    if (wave == 0) {
-        fetch(0, rx, ry, rz);
-        azimuth_stage(0, rx, ry, rz);
-        fetch(1, rx, ry, rz);
-    }
-    __syncthreads(); // prefactor tables, job table, tables of batch 0
-    if (wave == 0) {
-        if (batch_lead == 2) {
-            azimuth_stage(1, rx, ry, rz);
-            fetch(2, rx, ry, rz);
-        }
-    } else if (wave < entry_first_wave) {
-        recursion_stage(0);
-    }
-
-    if (streaming) {
-        // Two row buffers: while the entry waves fill one with tile n, the flush waves send the
-        // other, tile n - 1, to HBM; one barrier per tile, and the stores never pause for the
-        // arithmetic. One more round after the last tile flushes it.
-        for (unsigned n = 0;; ++n) {
-            __syncthreads(); // tables of tile n+1, iterates of tile n, rows of tile n-1 complete
-            const unsigned valid = valid_in(n);
-            const unsigned before = n > 0 ? valid_in(n - 1) : 0u;
-            if (valid == 0 && before == 0) break;
-            if (wave == 0) {
-                if ((n & (batch_tiles - 1u)) == 0) {
-                    azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
-                    fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz); // for the next batch
-                }
-            } else if (wave < entry_first_wave) {
-                recursion_stage(n + 1);
-            } else if (wave < entry_end_wave) {
-                if (valid != 0) {
-                    closed_stage(n, n & 1u, wave - entry_first_wave, entry_end_wave - entry_first_wave);
-                    entry_stage(n, n & 1u);
-                }
-            } else if (before != 0) {
-                flush_stage(n - 1, (n - 1) & 1u, tid - 64 * entry_end_wave, 64 * g.flush_waves,
-                            std::true_type{});
-            }
-        }
-    } else {
-        // One row buffer (the rows of one point fill most of LDS): every wave takes part in the
-        // flush, after a second barrier.
-        for (unsigned n = 0; valid_in(n) != 0; ++n) {
-            __syncthreads(); // tables of tile n+1, iterates of tile n in place; rows of tile n-1 flushed
-            // the closed-form slices go round all waves: those that make tables and iterates
-            // have time to spare
-            closed_stage(n, 0, wave, NT / 64);
-            if (wave == 0) {
-                if ((n & (batch_tiles - 1u)) == 0) {
-                    azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
-                    fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz);
-                }
-            } else if (wave < entry_first_wave) {
-                recursion_stage(n + 1);
-            } else {
-                entry_stage(n, 0);
-            }
-            __syncthreads(); // rows of tile n complete
-            if constexpr (VJP) {
-                contract_stage(n, 0);
-            } else {
-                flush_stage(n, 0, tid, NT, std::false_type{});
-            }
-        }
-    }
-}
 
 // ---------------------------------------------------------------------------
 // Host side of the launch layer

@@ -1,0 +1,558 @@
+// recursion_kernel: the general case, persistent workgroups whose waves have roles of their own.
+#ifndef SPHX_RECURSION_KERNEL_HPP
+#define SPHX_RECURSION_KERNEL_HPP
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <type_traits>
+
+#include "sphx_tiling.hpp"
+#include "sphx_closed_form_kernel.hpp"
+
+namespace sphx {
+
+// ---------------------------------------------------------------------------
+// l > H through the recursion. 512 threads, persistent workgroups that walk
+// over tiles of `tile` consecutive points, four tiles in flight per workgroup,
+// every wave with a role of its own and one barrier per tile:
+//
+//   wave 0       one batch of up to eight tiles ahead, one lane per point:
+//                normalised coordinates, c_m, s_m, 2(m+1)z into LDS (azimuth_job);
+//   wave 1 (, 2) tile i+1, one lane per (point, l, sequence): the bare Q recursions,
+//                every iterate into LDS (sequence_job);
+//   entry waves  tile i, one job per (point, l, m >= 0): the entries (l, +-m) of
+//                every requested array, chain rule included, staged in LDS in
+//                HBM layout (entry_job). Neighbouring lanes take neighbouring m
+//                of one (point, l), so their LDS traffic falls on neighbouring
+//                banks;
+//   flush waves  tile i-1: stream its staged rows to HBM with 16-byte stores.
+//
+// The first two stages are short chains of dependent operations that only a
+// few lanes can share; running them one and two tiles ahead of the wide stage
+// takes them off the critical path. The last stage is bound by HBM, the entry
+// stage by the vector ALUs: side by side, neither waits for the other. The
+// point tables are kept in three buffers, the iterates and the staged rows in
+// two. When the rows of a single point are too long for two row buffers there
+// is one, no wave is set aside for flushing, and all waves flush tile i after
+// a second barrier.
+//
+// SPLIT == true (second derivatives, so few points per tile that the (l, m)
+// pairs of a tile leave lanes idle): the entries (l, +m) and (l, -m) are two
+// jobs.
+//
+// WHOLE == true: the closed forms of l <= H are evaluated here too (one lane
+// per point, the entries in slices that go round all waves) and the tile's
+// rows are complete, one contiguous run per array.
+// WHOLE == false: the rows start at l = H + 1 (closed_form_kernel<PREFIX>
+// writes the part below); every (point, component) row is its own run.
+// ---------------------------------------------------------------------------
+constexpr unsigned kRecursionThreads = 512;
+
+// Values and gradients: at most 128 registers, so that two workgroups share a CU (four waves
+// per SIMD) wherever their LDS allows. Only the float64 closed forms exceed that on their own
+// and spill a few registers; with 170 registers and one workgroup per CU, l_max = 12 float64
+// gradients took 800 us instead of 513 us. The second-derivative kernels keep what they need
+// (forced to 128 they spill in the entry jobs: 918 us against 558 us at l_max = 10, float64).
+template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false>
+__global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling g, const T* __restrict__ xyz,
+                                                                     T* __restrict__ sph,
+                                                                     T* __restrict__ dsph,
+                                                                     T* __restrict__ ddsph) {
+    static_assert(!VJP || (MODE == 1 && !SPLIT), "the fused product is built on the gradient kernel");
+    constexpr int H = MODE == 2 ? 1 : 6;
+    constexpr unsigned NYH = (H + 1) * (H + 1);
+    constexpr unsigned ARRAYS = MODE + 1; // iterate arrays per point: A, B, C
+    constexpr unsigned NT = kRecursionThreads;
+    T* lds = reinterpret_cast<T*>(lds_raw);
+    const unsigned tid = threadIdx.x;
+    const unsigned lane = tid & 63u;
+    const unsigned wave = tid >> 6;
+    const int L = g.l_max;
+    const unsigned S = g.tile;
+    const unsigned ny = g.ny;
+    const unsigned nrow = WHOLE ? ny : ny - NYH; // staged elements per component row
+    const unsigned skip = WHOLE ? 0u : NYH;      // first staged entry of a row
+    // Distance between staged rows. WHOLE == false: the rows are ny apart in HBM but only nrow
+    // long; a stride that equals ny modulo 16 bytes, with the first row placed like its HBM
+    // address modulo 16 bytes, puts every staged row at the same position within 16 bytes as
+    // its destination, so that the copy is 16-byte loads and stores on both sides.
+    constexpr unsigned W16 = 16u / static_cast<unsigned>(sizeof(T));
+    const unsigned row_stride = nrow + skip % W16;
+    const unsigned tri_all = (L + 1) * (L + 2) / 2;
+
+    T* F = lds + g.off_F;
+    T* Q = lds + g.off_Q;
+    unsigned* job_table = reinterpret_cast<unsigned*>(lds + g.off_jobs);
+    {
+        const T* cF = table_F<T>();
+        const T* cQ = table_Q<T>();
+        for (unsigned i = tid; i < tri_all; i += NT) {
+            F[i] = cF[i];
+            Q[i] = cQ[i];
+        }
+        // (l, m) pairs: the bulk 1 <= m <= l - 2 first, then the special cases m = l, l - 1 and
+        // 0 each as one block, so that the lanes of a wave mostly share one branch of entry_job
+        // one word per job: m in bits 0-6, the side in bit 7, l in bits 8-15, l(l+1)/2 above
+        auto pack = [](int l, int m, int side) -> unsigned {
+            return (static_cast<unsigned>(l * (l + 1) / 2) << 16) | (static_cast<unsigned>(l) << 8) |
+                   (static_cast<unsigned>(side) << 7) | static_cast<unsigned>(m);
+        };
+        // one thread per l fills that l's places (a single thread writing all of them took
+        // 10 us at l_max = 32, a third of the time of a small evaluation)
+        if (static_cast<int>(tid) < L - H) {
+            constexpr unsigned SIDES = SPLIT ? 2u : 1u;
+            const int l = L - static_cast<int>(tid);
+            const unsigned levels = static_cast<unsigned>(L - H);
+            auto bulk_above = [&](int from) { // sum of (l' - 2) over from < l' <= L
+                return static_cast<unsigned>(L * (L + 1) / 2 - from * (from + 1) / 2 - 2 * (L - from));
+            };
+            const unsigned bulk_all = bulk_above(H);
+            for (unsigned side = 0; side < SIDES; ++side) {
+                unsigned at = side * bulk_all + bulk_above(l);
+                for (int m = l - 2; m >= 1; --m) job_table[at++] = pack(l, m, static_cast<int>(side));
+                job_table[SIDES * bulk_all + side * levels + tid] = pack(l, l, static_cast<int>(side));
+                job_table[SIDES * (bulk_all + levels) + side * levels + tid] = pack(l, l - 1, static_cast<int>(side));
+            }
+            job_table[SIDES * (bulk_all + 2 * levels) + tid] = pack(l, 0, 0);
+        }
+    }
+
+    // per point: 8 numbers (x, y, z, x^2, y^2, z^2, 1/r, x^2 + y^2), then c, s, 2(m+1)z
+    const unsigned point_stride = 8 + 3 * (L + 1);
+    // The tables are made for 2^az_shift tiles at a time (a batch), one lane per point, so that
+    // the recurrences, a chain of dependent operations that few lanes share, run once per batch
+    // instead of once per tile. Single tiles are made two rounds ahead and kept in three
+    // buffers; batches are made one batch ahead and kept in two.
+    const unsigned batch_tiles = 1u << g.az_shift;
+    const unsigned batch_lead = batch_tiles == 1 ? 2u : 1u;
+    const unsigned batch_buffers = batch_tiles == 1 ? 3u : 2u;
+    auto point_data = [&](unsigned n, unsigned s) -> T* { // point s of this workgroup's n-th tile
+        const unsigned slot = (((n >> g.az_shift) % batch_buffers) << g.az_shift) | (n & (batch_tiles - 1u));
+        return lds + g.off_pts + (slot * S + s) * point_stride;
+    };
+    auto iterates = [&](unsigned buffer, unsigned s, unsigned which, int l) -> T* {
+        return lds + g.off_iter + ((buffer * S + s) * ARRAYS + which) * tri_all + l * (l + 1) / 2;
+    };
+
+    // same XCD-contiguous walk as the closed-form kernel
+    const unsigned xcd = blockIdx.x & 7u;
+    const unsigned rank_in_xcd = blockIdx.x >> 3;
+    const unsigned groups_per_xcd = gridDim.x >> 3;
+    const unsigned xcd_first = xcd * g.tiles_per_xcd;
+    unsigned xcd_last = xcd_first + g.tiles_per_xcd;
+    if (xcd_last > g.n_tiles) xcd_last = g.n_tiles;
+    // A workgroup takes chunks of C consecutive tiles; the chunks of an XCD's workgroups lie
+    // side by side. Consecutive tiles in one workgroup share the 128-byte lines in which one
+    // ends and the next begins (see flush_run); C stays small so that what the XCD writes at any
+    // moment remains a compact window.
+    const unsigned chunk_mask = (1u << g.chunk_shift) - 1u;
+    if (xcd_first + (rank_in_xcd << g.chunk_shift) >= xcd_last) return; // whole workgroup
+
+    // the n-th tile of this workgroup, and how many points it has (0 past the end)
+    auto tile_of = [&](unsigned n) -> unsigned {
+        return xcd_first + ((((n >> g.chunk_shift) * groups_per_xcd + rank_in_xcd)) << g.chunk_shift) +
+               (n & chunk_mask);
+    };
+    auto valid_in = [&](unsigned n) -> unsigned {
+        const unsigned t = tile_of(n);
+        if (t >= xcd_last) return 0u;
+        const unsigned long long first = static_cast<unsigned long long>(t) * S;
+        const unsigned long long left = g.n_samples - first;
+        return left < S ? static_cast<unsigned>(left) : S;
+    };
+    // lane j of wave 0 takes point j % S of tile j / S of a batch (batch_tiles * S <= 64)
+    auto fetch = [&](unsigned batch, T& rx, T& ry, T& rz) {
+        rx = ry = rz = 0;
+        const unsigned n = (batch << g.az_shift) + lane / S;
+        const unsigned s = lane % S;
+        if (lane < batch_tiles * S && s < valid_in(n)) {
+            const T* src = xyz + (static_cast<unsigned long long>(tile_of(n)) * S + s) * 3;
+            rx = src[0];
+            ry = src[1];
+            rz = src[2];
+        }
+    };
+    // stage one of a batch of tiles (wave 0; lane == tid there)
+    auto azimuth_stage = [&](unsigned batch, T rx, T ry, T rz) {
+        const unsigned n = (batch << g.az_shift) + lane / S;
+        const unsigned s = lane % S;
+        if (lane < batch_tiles * S && s < valid_in(n)) {
+            T* rec = point_data(n, s);
+            Point<T> p;
+            p.x = rx;
+            p.y = ry;
+            p.z = rz;
+            p.x2 = p.x * p.x;
+            p.y2 = p.y * p.y;
+            p.z2 = p.z * p.z;
+            p.ir = 0.0;
+            if constexpr (NORM) {
+                p.ir = 1 / root(p.x2 + p.y2 + p.z2);
+                p.x *= p.ir;
+                p.y *= p.ir;
+                p.z *= p.ir;
+                p.x2 = p.x * p.x;
+                p.y2 = p.y * p.y;
+                p.z2 = p.z * p.z;
+            }
+            rec[0] = p.x;
+            rec[1] = p.y;
+            rec[2] = p.z;
+            rec[3] = p.x2;
+            rec[4] = p.y2;
+            rec[5] = p.z2;
+            rec[6] = p.ir;
+            rec[7] = p.x2 + p.y2;
+            azimuth_job<T>(p, L, rec + 8, rec + 8 + (L + 1), rec + 8 + 2 * (L + 1));
+        }
+    };
+    // stage two of tile n (waves 1 .. g.sequence_waves)
+    auto recursion_stage = [&](unsigned n) {
+        const unsigned count = valid_in(n);
+        const unsigned per_l = count * ARRAYS;
+        const unsigned jobs = per_l * static_cast<unsigned>(L - H);
+        for (unsigned j = tid - 64; j < jobs; j += 64 * g.sequence_waves) { // waves 1 .. sequence_waves
+            const unsigned step = j / per_l;
+            const unsigned rest = j - step * per_l;
+            const int l = L - static_cast<int>(step); // longest recursions first
+            const unsigned s = rest / ARRAYS;
+            const unsigned which = rest - s * ARRAYS;
+            const T* rec = point_data(n, s);
+            sequence_job<T>(l, static_cast<int>(which), rec[2], rec[7], Q, rec + 8 + 2 * (L + 1),
+                            iterates(n & 1u, s, which, l));
+        }
+    };
+
+    // The waves between the sequence waves and the flush waves compute entries.
+    const bool streaming = g.row_buffers == 2;
+    const unsigned entry_first_wave = 1 + g.sequence_waves;
+    const unsigned entry_end_wave = NT / 64 - (streaming ? g.flush_waves : 0u);
+    const unsigned wide_first = 64 * entry_first_wave;
+    const unsigned wide_lanes = 64 * (entry_end_wave - entry_first_wave);
+
+    constexpr unsigned LINE = 128u / static_cast<unsigned>(sizeof(T)); // elements per 128-byte line
+    // position within its 128-byte line of element `element` of an output array
+    auto phase_of = [](const T* array, unsigned long long element) -> unsigned {
+        return static_cast<unsigned>((reinterpret_cast<uintptr_t>(array) / sizeof(T) + element) % LINE);
+    };
+
+    // Where the rows of tile n start within their staging regions. WHOLE: element 0 of a region
+    // stands for the start of the 128-byte line in which the tile's run begins in HBM, so the run
+    // itself starts `phase` elements in. WHOLE == false: position within 16 bytes of the first
+    // staged row, see row_stride. VJP: the rows never leave LDS, no position to match.
+    struct Phases {
+        unsigned sph, dsph, ddsph;
+    };
+    auto phases_of = [&](unsigned n) -> Phases {
+        const unsigned long long first_point = static_cast<unsigned long long>(tile_of(n)) * S;
+        Phases ph;
+        ph.sph = VJP ? 0u : phase_of(sph, first_point * ny + skip) % (WHOLE ? LINE : W16);
+        ph.dsph = VJP || MODE < 1 ? 0u : phase_of(dsph, first_point * 3 * ny + skip) % (WHOLE ? LINE : W16);
+        ph.ddsph = WHOLE && !VJP && MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
+        return ph;
+    };
+
+    // WHOLE: the closed forms of tile n, one lane per point, into row buffer `buffer`. The
+    // entries of a point are cut in slices (by l), dealt to `among` waves of which this is number
+    // `who`, so that no single wave carries all of the chain rule and staging.
+    auto closed_stage = [&](unsigned n, unsigned buffer, unsigned who, unsigned among) {
+        if constexpr (WHOLE) {
+            const unsigned valid = valid_in(n);
+            if (lane < valid) {
+                T* staged = lds + buffer * g.rows_elems;
+                const Phases ph = phases_of(n);
+                const T* rec = point_data(n, lane);
+                Point<T> p;
+                p.x = rec[0];
+                p.y = rec[1];
+                p.z = rec[2];
+                p.x2 = rec[3];
+                p.y2 = rec[4];
+                p.z2 = rec[5];
+                p.ir = rec[6];
+                Rows<T> rows;
+                rows.ny = static_cast<int>(ny);
+                rows.sph = staged + ph.sph + lane * ny;
+                rows.dsph = staged + g.off_dsph + ph.dsph + lane * 3 * ny;
+                rows.ddsph = staged + g.off_ddsph + ph.ddsph + lane * 9 * ny;
+                if constexpr (H == 6) {
+                    // float32 rows a multiple of 32 words long (l_max = 7, 15, 23, ...): the
+                    // stores of all lanes would fall on one LDS bank; stored in rotated fours
+                    // instead (closed_form_job; l_max = 7, 500k points, gradients: 343 -> 216 us).
+                    // Not for float64 and not for values alone, where the selects cost registers
+                    // that the kernel does not have to spare (values: 68 -> 89, and l_max = 9 lost
+                    // its third workgroup per CU, 80 -> 106 us).
+                    constexpr bool MAY_ROTATE = sizeof(T) == 4 && MODE == 1;
+                    if (MAY_ROTATE && (ny & 31u) == 0) {
+                        const unsigned turn = lane & 3u;
+                        if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 8, true>(p, rows, turn);
+                        if (1 % among == who) closed_form_job<T, MODE, NORM, H, 8, 16, true>(p, rows, turn);
+                        if (2 % among == who) closed_form_job<T, MODE, NORM, H, 16, 24, true>(p, rows, turn);
+                        if (3 % among == who) closed_form_job<T, MODE, NORM, H, 24, 32, true>(p, rows, turn);
+                        if (4 % among == who) closed_form_job<T, MODE, NORM, H, 32, 40, true>(p, rows, turn);
+                        if (5 % among == who) closed_form_job<T, MODE, NORM, H, 40, 49, true>(p, rows, turn);
+                    } else {
+                        if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows);
+                        if (1 % among == who) closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows);
+                        if (2 % among == who) closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows);
+                        if (3 % among == who) closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows);
+                        if (4 % among == who) closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows);
+                        if (5 % among == who) closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows);
+                        if (6 % among == who) closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows);
+                        if (7 % among == who) closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows);
+                    }
+                } else {
+                    if (who == 0) closed_form_job<T, MODE, NORM, H>(p, rows);
+                }
+            }
+        }
+    };
+
+    // stage three of tile n, into row buffer `buffer` (the entry waves)
+    auto entry_stage = [&](unsigned n, unsigned buffer) {
+        const unsigned valid = valid_in(n);
+        T* staged = lds + buffer * g.rows_elems;
+        const unsigned t = tid - wide_first;
+        const Phases ph = phases_of(n);
+        const unsigned phase_sph = ph.sph, phase_dsph = ph.dsph, phase_ddsph = ph.ddsph;
+        // One pass takes the jobs of as many points as fit side by side in the wide lanes
+        // (of one point, in several rounds, when it has more jobs than there are lanes);
+        // what depends on the point only is read once per pass.
+        unsigned local = 0, e_first = t;
+        if (g.points_per_pass > 1) {
+            local = __umulhi(t, g.magic_jobs);
+            e_first = t - local * g.jobs_per_point;
+        }
+        for (unsigned s0 = 0; s0 < valid; s0 += g.points_per_pass) {
+            const unsigned s = s0 + local;
+            if (s >= valid || local >= g.points_per_pass) continue;
+            const T* rec = point_data(n, s);
+            Point<T> p;
+            p.x = rec[0];
+            p.y = rec[1];
+            p.z = rec[2];
+            p.x2 = rec[3];
+            p.y2 = rec[4];
+            p.z2 = rec[5];
+            p.ir = rec[6];
+            const T* c = rec + 8;
+            const T* sn = rec + 8 + (L + 1);
+            const T* itA = iterates(n & 1u, s, 0, 0);
+            const T* itB = iterates(n & 1u, s, MODE >= 1 ? 1 : 0, 0);
+            const T* itC = iterates(n & 1u, s, MODE == 2 ? 2 : 0, 0);
+            // rows are addressed with the entry's index in the full row; shift the bases when
+            // the staged rows start at l = H + 1
+            Rows<T> rows;
+            rows.ny = static_cast<int>(row_stride);
+            rows.sph = staged + phase_sph + s * row_stride - skip;
+            rows.dsph = staged + g.off_dsph + phase_dsph + s * 3 * row_stride - skip;
+            rows.ddsph = staged + g.off_ddsph + phase_ddsph + s * 9 * row_stride - skip;
+            for (unsigned e = e_first; e < g.jobs_per_point; e += wide_lanes) {
+                const unsigned packed = job_table[e];
+                const int m = static_cast<int>(packed & 0x7fu);
+                const int side = static_cast<int>((packed >> 7) & 1u);
+                const int l = static_cast<int>((packed >> 8) & 0xffu);
+                const int tri = static_cast<int>(packed >> 16);
+                entry_job<T, MODE, NORM, SPLIT>(l, m, tri, side, p, F + tri, c, sn, itA + tri,
+                                                itB + tri, itC + tri, rows);
+            }
+        }
+    };
+
+    // last stage of tile n: row buffer `buffer` to HBM, by `count` threads of which this is
+    // number `ft`. `lone` (a std::integral_constant): the copy of a run is the work of a single
+    // wave, which then keeps several LDS loads in flight; with all waves of the workgroup on one
+    // run, loads and stores alternating one by one measured faster.
+    auto flush_stage = [&](unsigned n, unsigned buffer, unsigned ft, unsigned count, auto lone) {
+        constexpr int WHOLE_UNROLL = decltype(lone)::value ? SPHX_FLUSH_UNROLL : 1;
+        const unsigned valid = valid_in(n);
+        const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
+        const T* staged = lds + buffer * g.rows_elems;
+        if constexpr (WHOLE) {
+            // The tile's run of `len` elements of one output array starts at element `at` of that
+            // array. Only whole 128-byte lines go out with vector stores. The line in which the
+            // run ends is completed by the next tile: when that tile is this workgroup's next one
+            // (same chunk), the unfinished part is carried over into the region the next tile is
+            // staged in; at the ends of a chunk the partial lines are stored element by element.
+            const bool starts = (n & chunk_mask) == 0;
+            const bool ends = (n & chunk_mask) == chunk_mask || valid_in(n + 1) == 0;
+            T* carry_to = lds + (streaming ? (buffer ^ 1u) : buffer) * g.rows_elems;
+            auto flush_run = [&](unsigned region_offset, T* array, unsigned long long at, unsigned len) {
+                using V = typename Pack<T>::type;
+                constexpr unsigned W = Pack<T>::width;
+                T* region = lds + buffer * g.rows_elems + region_offset;
+                const unsigned phase = phase_of(array, at);
+                T* line0 = array + (at - phase); // HBM address of region element 0
+                const unsigned lo = starts ? phase : 0u; // first element that holds data
+                const unsigned hi = phase + len;
+                const unsigned full_lo = (lo + LINE - 1u) / LINE * LINE;
+                const unsigned full_hi = hi / LINE * LINE;
+                unsigned tail_from; // what follows the head and the whole lines
+                if (full_hi > full_lo) {
+                    const unsigned nvec = (full_hi - full_lo) / W;
+                    const V* in = reinterpret_cast<const V*>(region + full_lo);
+                    V* out = reinterpret_cast<V*>(line0 + full_lo);
+                    unsigned v = ft;
+                    if constexpr (WHOLE_UNROLL > 1) {
+                        for (; v + (WHOLE_UNROLL - 1) * count < nvec; v += WHOLE_UNROLL * count) {
+                            V hold[WHOLE_UNROLL];
+#pragma unroll
+                            for (int u = 0; u < WHOLE_UNROLL; ++u) hold[u] = in[v + u * count];
+#pragma unroll
+                            for (int u = 0; u < WHOLE_UNROLL; ++u) {
+                                emit<T, SPHX_STREAMING_STORES>(hold[u], out + v + u * count);
+                            }
+                        }
+                    }
+                    for (; v < nvec; v += count) {
+                        emit<T, SPHX_STREAMING_STORES>(in[v], out + v);
+                    }
+                    tail_from = full_hi;
+                } else {
+                    tail_from = full_lo < hi ? full_lo : hi;
+                }
+                // head: the part of the first line that belongs to this chunk
+                const unsigned head_end = full_lo < hi ? full_lo : hi;
+                if (lo + ft < head_end) line0[lo + ft] = region[lo + ft];
+                // tail: stored if the chunk ends here, else handed to the next tile
+                const unsigned tail = hi - tail_from;
+                if (ft < tail) {
+                    const T value = region[tail_from + ft];
+                    if (ends) {
+                        line0[tail_from + ft] = value;
+                    } else if (carry_to + region_offset != region || tail_from != 0) {
+                        carry_to[region_offset + ft] = value;
+                    }
+                }
+            };
+            flush_run(0, sph, first * ny, valid * ny);
+            if constexpr (MODE >= 1) flush_run(g.off_dsph, dsph, first * 3 * ny, valid * 3 * ny);
+            if constexpr (MODE == 2) flush_run(g.off_ddsph, ddsph, first * 9 * ny, valid * 9 * ny);
+        } else {
+            // one run per (point, component) row, dealt to the waves in turn
+            const unsigned waves = count / 64;
+            for (unsigned r = ft >> 6; r < valid * components_of(MODE); r += waves) {
+                // rows [0, valid) are values, the next 3 * valid are gradients
+                if (r < valid) {
+                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL>(
+                        staged + phase_of(sph, first * ny + skip) % W16 + r * row_stride,
+                        sph + (first + r) * ny + skip, nrow, nrow, 0, 0, ft & 63u, 64);
+                } else {
+                    const unsigned q = r - valid;
+                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL>(
+                        staged + g.off_dsph + phase_of(dsph, first * 3 * ny + skip) % W16 + q * row_stride,
+                        dsph + (first * 3 + q) * ny + skip, nrow, nrow, 0, 0, ft & 63u, 64);
+                }
+            }
+        }
+    };
+
+    // VJP: in place of the flush. `sph` holds the upstream gradient sph_grad[N][ny] (read
+    // only), `dsph` is xyz_grad[N][3]. Wave 1 + r takes gradient row r of the tile (point r / 3,
+    // component r % 3): its lanes multiply the staged entries with the point's row of sph_grad
+    // and a butterfly adds the lanes' sums up. With WHOLE == false the staged rows begin at
+    // l = H + 1 and closed_form_vjp_kernel has already stored the sum over l <= H, so the
+    // result is added to what xyz_grad holds. Wave 0 stays out: it has loads in flight.
+    auto contract_stage = [&](unsigned n, unsigned buffer) {
+        if constexpr (VJP) {
+            const unsigned valid = valid_in(n);
+            const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
+            const T* staged = lds + buffer * g.rows_elems + g.off_dsph;
+            const T* upstream = sph;
+            T* xyz_grad = dsph;
+            if (wave == 0) return;
+            for (unsigned r = wave - 1; r < valid * 3; r += NT / 64 - 1) {
+                const unsigned s = r / 3;
+                const T* row = staged + r * row_stride - skip; // indexed with the entry's index in the full row
+                const T* weight = upstream + (first + s) * ny;
+                T partial = 0;
+#pragma unroll 4
+                for (unsigned k = skip + lane; k < ny; k += 64) {
+                    partial += row[k] * weight[k];
+                }
+                for (unsigned offset = 32; offset > 0; offset >>= 1) {
+                    partial += __shfl_xor(partial, static_cast<int>(offset));
+                }
+                if (lane == 0) {
+                    T* out = xyz_grad + first * 3 + r;
+                    *out = (!WHOLE || g.vjp_accumulate) ? *out + partial : partial;
+                }
+            }
+        }
+    };
+
+    // fill the pipeline: tables of tiles 0 and 1, iterates of tile 0
+    T rx = 0, ry = 0, rz = 0;
+    if (wave == 0) {
+        fetch(0, rx, ry, rz);
+        azimuth_stage(0, rx, ry, rz);
+        fetch(1, rx, ry, rz);
+    }
+    __syncthreads(); // prefactor tables, job table, tables of batch 0
+    if (wave == 0) {
+        if (batch_lead == 2) {
+            azimuth_stage(1, rx, ry, rz);
+            fetch(2, rx, ry, rz);
+        }
+    } else if (wave < entry_first_wave) {
+        recursion_stage(0);
+    }
+
+    if (streaming) {
+        // Two row buffers: while the entry waves fill one with tile n, the flush waves send the
+        // other, tile n - 1, to HBM; one barrier per tile, and the stores never pause for the
+        // arithmetic. One more round after the last tile flushes it.
+        for (unsigned n = 0;; ++n) {
+            __syncthreads(); // tables of tile n+1, iterates of tile n, rows of tile n-1 complete
+            const unsigned valid = valid_in(n);
+            const unsigned before = n > 0 ? valid_in(n - 1) : 0u;
+            if (valid == 0 && before == 0) break;
+            if (wave == 0) {
+                if ((n & (batch_tiles - 1u)) == 0) {
+                    azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
+                    fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz); // for the next batch
+                }
+            } else if (wave < entry_first_wave) {
+                recursion_stage(n + 1);
+            } else if (wave < entry_end_wave) {
+                if (valid != 0) {
+                    closed_stage(n, n & 1u, wave - entry_first_wave, entry_end_wave - entry_first_wave);
+                    entry_stage(n, n & 1u);
+                }
+            } else if (before != 0) {
+                flush_stage(n - 1, (n - 1) & 1u, tid - 64 * entry_end_wave, 64 * g.flush_waves,
+                            std::true_type{});
+            }
+        }
+    } else {
+        // One row buffer (the rows of one point fill most of LDS): every wave takes part in the
+        // flush, after a second barrier.
+        for (unsigned n = 0; valid_in(n) != 0; ++n) {
+            __syncthreads(); // tables of tile n+1, iterates of tile n in place; rows of tile n-1 flushed
+            // the closed-form slices go round all waves: those that make tables and iterates
+            // have time to spare
+            closed_stage(n, 0, wave, NT / 64);
+            if (wave == 0) {
+                if ((n & (batch_tiles - 1u)) == 0) {
+                    azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
+                    fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz);
+                }
+            } else if (wave < entry_first_wave) {
+                recursion_stage(n + 1);
+            } else {
+                entry_stage(n, 0);
+            }
+            __syncthreads(); // rows of tile n complete
+            if constexpr (VJP) {
+                contract_stage(n, 0);
+            } else {
+                flush_stage(n, 0, tid, NT, std::false_type{});
+            }
+        }
+    }
+}
+
+} // namespace sphx
+
+#endif

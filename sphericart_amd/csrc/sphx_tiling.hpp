@@ -1,0 +1,73 @@
+// What every kernel of the launch layer shares: the prefactor tables in constant memory, the
+// description of a launch's tiling that the host fills in, and the dynamic LDS array.
+#ifndef SPHX_TILING_HPP
+#define SPHX_TILING_HPP
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <type_traits>
+
+#include "sphx_device.hpp"
+#include "sphx_tables.hpp"
+
+namespace sphx {
+
+constexpr int kTableEntries = (SPHX_TABLE_LMAX + 1) * (SPHX_TABLE_LMAX + 2) / 2;
+
+__constant__ float kF32[kTableEntries];
+__constant__ float kQ32[kTableEntries];
+__constant__ double kF64[kTableEntries];
+__constant__ double kQ64[kTableEntries];
+
+template <typename T> __device__ __forceinline__ const T* table_F();
+template <typename T> __device__ __forceinline__ const T* table_Q();
+template <> __device__ __forceinline__ const float* table_F<float>() { return kF32; }
+template <> __device__ __forceinline__ const float* table_Q<float>() { return kQ32; }
+template <> __device__ __forceinline__ const double* table_F<double>() { return kF64; }
+template <> __device__ __forceinline__ const double* table_Q<double>() { return kQ64; }
+
+// Everything a kernel needs to know about the tiling; filled in on the host.
+struct Tiling {
+    unsigned long long n_samples;
+    unsigned n_tiles;       // tiles of `tile` points (recursion) or groups of 64 points (closed form)
+    unsigned tiles_per_xcd; // workgroups of one XCD walk one contiguous stretch of tiles
+    int l_max;
+    int ny;                 // (l_max + 1)^2: length of one component row in HBM
+    int tile;               // points whose rows are staged in LDS at a time
+    unsigned magic_jobs;    // ceil(2^32 / jobs_per_point)
+    unsigned jobs_per_point; // entry jobs per point: (l, m >= 0) pairs above the closed-form
+                             // limit, or (l, m, side) triples when the sides are split
+    unsigned sequence_waves; // waves that run the bare recursions (1 or 2)
+    unsigned points_per_pass; // points whose entry jobs fit side by side in the wide waves (>= 1)
+    unsigned vjp_accumulate; // fused product: add to xyz_grad instead of overwriting it
+    unsigned az_shift;      // the point tables are made for 2^az_shift tiles at a time
+    unsigned chunk_shift;   // a workgroup takes 2^chunk_shift consecutive tiles at a time
+    unsigned row_buffers;   // 2: tile n is flushed while tile n+1 is computed; 1: one after the other
+    unsigned flush_waves;   // waves that do nothing but flush (row_buffers == 2)
+    // LDS carve-up, in elements of T: the row buffers come first, rows_elems each, with the
+    // gradient and second-derivative rows at off_dsph and off_ddsph inside a buffer; the other
+    // offsets count from the start of dynamic LDS
+    unsigned rows_elems, off_dsph, off_ddsph, off_F, off_Q, off_pts, off_iter, off_jobs;
+};
+
+extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+
+// Output lines are written once and never read back by the kernel: store them with the
+// non-temporal hint (measured 10-20 % faster than plain stores here).
+#ifndef SPHX_STREAMING_STORES
+#define SPHX_STREAMING_STORES true
+#endif
+
+// LDS loads a flushing wave of the recursion kernel keeps in flight
+#ifndef SPHX_FLUSH_UNROLL
+#define SPHX_FLUSH_UNROLL 4
+#endif
+
+__host__ __device__ constexpr unsigned magic_of(unsigned long long divisor) {
+    return static_cast<unsigned>(((1ull << 32) + divisor - 1) / divisor);
+}
+
+} // namespace sphx
+
+#endif
