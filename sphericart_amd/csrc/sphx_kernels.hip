@@ -524,20 +524,23 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", 80 * 1024));
     bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
                                &plan->split_sides);
-    // With very few points per tile the one-lane-per-point closed forms of l <= 6 would leave
-    // most of the lanes idle for some two thousand instructions per tile: hand them to the
-    // closed-form kernel, which runs them 64 points at a time, and let the recursion kernel stage
-    // l >= 7 only. The price is rows cut in two, each part a run of its own in HBM, so the
-    // threshold is low (measured, 1M/500k/200k points, gradients: float32 l_max = 16, 8 points
-    // per tile, 812 us whole against 1110 us cut; l_max = 24, 4 points, 593 against 729;
-    // float64 l_max = 12, 8 points, 513 against 655; l_max = 20, 2 points, 1801 against 1018).
-    const int split_below = env_int("SPHX_SPLIT_BELOW", elem == 4 ? 4 : 8);
+    // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of
+    // the lanes idle for some two thousand instructions per tile: then the recursion kernel
+    // stages l >= 7 only and its wave 0, which mostly waits, writes l <= 6 straight from
+    // registers, 64 points at a time (prefix_inside). The price is rows cut in two, each part a
+    // run of its own in HBM. Measured, gradients, 200k float32 / 100k float64 points, whole
+    // against cut: float32 l_max = 17 (8 points per tile) 321 against 359 us, l_max = 19-23 (4)
+    // 548-623 against 497-587, l_max = 24-28 (4, 2) within 4 %, l_max = 32 (2) 1 050 against
+    // 885; float64 l_max = 12-13 (8) 179, 204 against 169, 194, l_max = 14-18 (4) 270-390 against
+    // 221-327, l_max = 20 (2) 559 against 460.
+    const int split_below = env_int("SPHX_SPLIT_BELOW", elem == 4 ? 8 : 16);
     if (mode < 2 && (!fits || plan->rec.g.tile < split_below)) {
         Launch upper;
         if (plan_recursion(n_samples, l_max, mode, false, elem, budget, lds_limit, cus, &upper,
                            &plan->split_sides)) {
             plan->whole = false;
             plan->rec = upper;
+            plan->rec.g.prefix_inside = lane_kernels && env_int("SPHX_PREFIX_INSIDE", 1) != 0 ? 1u : 0u;
             plan_closed(n_samples, l_max, hard, mode, elem, &plan->closed);
             fits = true;
         }
@@ -683,6 +686,9 @@ static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* d
         } else {
             if (plan.whole) {
                 return launch_recursion<T, MODE, NORM, true, false>(plan.rec, xyz, sph, dsph, ddsph, stream);
+            }
+            if (plan.rec.g.prefix_inside != 0) {
+                return launch_recursion<T, MODE, NORM, false, false>(plan.rec, xyz, sph, dsph, ddsph, stream);
             }
             // the two kernels write disjoint parts of every row
             hipError_t e = launch_closed<T, MODE, NORM, 6, true>(plan.closed, xyz, sph, dsph, ddsph, stream);

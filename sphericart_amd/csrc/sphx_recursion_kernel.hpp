@@ -147,7 +147,55 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
     // ends and the next begins (see flush_run); C stays small so that what the XCD writes at any
     // moment remains a compact window.
     const unsigned chunk_mask = (1u << g.chunk_shift) - 1u;
-    if (xcd_first + (rank_in_xcd << g.chunk_shift) >= xcd_last) return; // whole workgroup
+
+    // WHOLE == false with g.prefix_inside: l <= H of every row is written by this launch as well,
+    // by wave 0, which otherwise waits at the barriers most of the time. 64 points at a time, one
+    // per lane, the entries in eight slices straight from registers to HBM: the runs are 196 or
+    // 392 bytes long, one per component row, so staging them would not make the stores any
+    // better. The batches of 64 points are dealt to the workgroups of the launch and have
+    // nothing to do with the tiles a workgroup walks; one call takes one slice of one batch.
+    [[maybe_unused]] unsigned prefix_next = 0;
+    [[maybe_unused]] auto prefix_slice = [&]() -> bool {
+        if constexpr (!WHOLE && !VJP && H == 6) {
+            const unsigned long long first =
+                (static_cast<unsigned long long>(prefix_next >> 3) * gridDim.x + blockIdx.x) * 64u;
+            if (first >= g.n_samples) return false;
+            const unsigned slice = prefix_next & 7u;
+            ++prefix_next;
+            const unsigned long long i = first + lane;
+            if (i < g.n_samples) {
+                const Point<T> p = load_point<T, NORM>(xyz + i * 3);
+                Rows<T> rows;
+                rows.ny = static_cast<int>(ny);
+                rows.sph = sph + i * ny;
+                rows.dsph = MODE >= 1 ? dsph + i * 3 * ny : nullptr;
+                rows.ddsph = nullptr;
+                switch (slice) {
+                case 0: closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows); break;
+                case 1: closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows); break;
+                case 2: closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows); break;
+                case 3: closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows); break;
+                case 4: closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows); break;
+                case 5: closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows); break;
+                case 6: closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows); break;
+                default: closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows); break;
+                }
+            }
+            return true;
+        } else {
+            return false;
+        }
+    };
+    const bool prefix_wave = !WHOLE && !VJP && H == 6 && g.prefix_inside != 0 && wave == 0;
+
+    if (xcd_first + (rank_in_xcd << g.chunk_shift) >= xcd_last) {
+        // no tiles for this workgroup; its share of the batches remains
+        if (prefix_wave) {
+            while (prefix_slice()) {
+            }
+        }
+        return;
+    }
 
     // the n-th tile of this workgroup, and how many points it has (0 past the end)
     auto tile_of = [&](unsigned n) -> unsigned {
@@ -513,6 +561,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
                     azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
                     fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz); // for the next batch
                 }
+                if (prefix_wave) prefix_slice();
             } else if (wave < entry_first_wave) {
                 recursion_stage(n + 1);
             } else if (wave < entry_end_wave) {
@@ -538,6 +587,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
                     azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
                     fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz);
                 }
+                if (prefix_wave) prefix_slice();
             } else if (wave < entry_first_wave) {
                 recursion_stage(n + 1);
             } else {
@@ -549,6 +599,11 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
             } else {
                 flush_stage(n, 0, tid, NT, std::false_type{});
             }
+        }
+    }
+    // what is left of this workgroup's share of the batches (no barrier follows)
+    if (prefix_wave) {
+        while (prefix_slice()) {
         }
     }
 }

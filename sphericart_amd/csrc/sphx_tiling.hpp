@@ -45,6 +45,7 @@ struct Tiling {
     unsigned chunk_shift;   // a workgroup takes 2^chunk_shift consecutive tiles at a time
     unsigned row_buffers;   // 2: tile n is flushed while tile n+1 is computed; 1: one after the other
     unsigned flush_waves;   // waves that do nothing but flush (row_buffers == 2)
+    unsigned prefix_inside; // rows that start at l = 7: the recursion kernel writes l <= 6 too
     // LDS carve-up, in elements of T: the row buffers come first, rows_elems each, with the
     // gradient and second-derivative rows at off_dsph and off_ddsph inside a buffer; the other
     // offsets count from the start of dynamic LDS

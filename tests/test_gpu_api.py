@@ -132,6 +132,37 @@ def test_second_derivatives_at_small_l_max_by_both_kernels(oracle, library, rout
                 assert torch.isnan(raw[i][:shift]).all() and torch.isnan(raw[i][shift + sizes[i]:]).all()
 
 
+@pytest.mark.parametrize("launches", ["one", "two"])
+def test_rows_cut_at_l7_by_one_launch_and_by_two(oracle, library, launches, monkeypatch):
+    """Few points per tile: the recursion kernel stages l >= 7 and l <= 6 comes either from its
+    wave 0 (the default) or from a launch of the closed-form kernel before it (the switch is read
+    at every call). Sizes around the batches of 64 points, workgroups without tiles included."""
+    monkeypatch.setenv("SPHX_PREFIX_INSIDE", "1" if launches == "one" else "0")
+    rng = np.random.default_rng(23)
+    cases = ((np.float32, torch.float32, 20, "gradients"), (np.float32, torch.float32, 32, "gradients"),
+             (np.float64, torch.float64, 14, "gradients"), (np.float32, torch.float32, 36, "values"),
+             (np.float64, torch.float64, 26, "values"))
+    for dtype, tdtype, l_max, mode in cases:
+        for n, shift in ((1, 0), (63, 1), (65, 0), (1000, 3), (4133, 0)):
+            normalized = bool((l_max + n) & 1)
+            announce("rows cut", launches, np.dtype(dtype).name, l_max, mode, n, shift, normalized)
+            ny = (l_max + 1) ** 2
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, normalized, mode)
+            sizes = (n * ny, 3 * n * ny)
+            shapes = ((n, ny), (n, 3, ny))
+            raw = [torch.full((s + 16,), float("nan"), dtype=tdtype, device="cuda") for s in sizes]
+            out = tuple(raw[i][shift:shift + sizes[i]].view(shapes[i]) if want[i] is not None else None
+                        for i in range(2)) + (None,)
+            status, _ = run_launch_layer(library, torch.from_numpy(xyz).cuda(), l_max, normalized, mode, out=out)
+            assert status == 0, library.sphx_last_error()
+            torch.cuda.synchronize()
+            for i in range(2):
+                if want[i] is not None:
+                    assert same_numbers(out[i].cpu().numpy(), want[i]).all(), (l_max, n, i)
+                    assert torch.isnan(raw[i][:shift]).all() and torch.isnan(raw[i][shift + sizes[i]:]).all()
+
+
 def test_lds_size_alternates_between_launches(oracle):
     """One kernel, launches that need more, then less, then more LDS again (all above 64 KB)."""
     rng = np.random.default_rng(21)
