@@ -528,12 +528,15 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // the lanes idle for some two thousand instructions per tile: then the recursion kernel
     // stages l >= 7 only and its wave 0, which mostly waits, writes l <= 6 straight from
     // registers, 64 points at a time (prefix_inside). The price is rows cut in two, each part a
-    // run of its own in HBM. Measured, gradients, 200k float32 / 100k float64 points, whole
-    // against cut: float32 l_max = 17 (8 points per tile) 321 against 359 us, l_max = 19-23 (4)
-    // 548-623 against 497-587, l_max = 24-28 (4, 2) within 4 %, l_max = 32 (2) 1 050 against
-    // 885; float64 l_max = 12-13 (8) 179, 204 against 169, 194, l_max = 14-18 (4) 270-390 against
-    // 221-327, l_max = 20 (2) 559 against 460.
-    const int split_below = env_int("SPHX_SPLIT_BELOW", elem == 4 ? 8 : 16);
+    // run of its own in HBM, which costs the more the shorter the rows are. Measured with 2.5 GB
+    // of output (smaller outputs flatter the cut rows: the last-level cache merges the parts),
+    // gradients, whole against cut, us: float32 l_max = 17, 18 (8 points per tile) 765, 900
+    // against 845, 940; l_max = 19-26 (4) 1 197, 1 125, 922, 710, 685 against 991, 983, 819,
+    // 672, 653; l_max = 28-40 (2, 1) 884, 780, 787 against 751, 632, 591. float64 l_max = 12
+    // (8) 736 against 928; l_max = 13-18 (4) 1 032, 882, 922, 779, 813 against 760, 918, 776,
+    // 787, 699; l_max = 20-32 (2, 1) 999, 892, 706, 896, 735 against 779, 664, 537, 585, 498.
+    // Values alone: cut rows win on every shape that reaches this kernel (by 11-20 %).
+    const int split_below = env_int("SPHX_SPLIT_BELOW", 8);
     if (mode < 2 && (!fits || plan->rec.g.tile < split_below)) {
         Launch upper;
         if (plan_recursion(n_samples, l_max, mode, false, elem, budget, lds_limit, cus, &upper,
