@@ -529,14 +529,16 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // stages l >= 7 only and its wave 0, which mostly waits, writes l <= 6 straight from
     // registers, 64 points at a time (prefix_inside). The price is rows cut in two, each part a
     // run of its own in HBM, which costs the more the shorter the rows are. Measured with 2.5 GB
-    // of output (smaller outputs flatter the cut rows: the last-level cache merges the parts),
-    // gradients, whole against cut, us: float32 l_max = 17, 18 (8 points per tile) 765, 900
-    // against 845, 940; l_max = 19-26 (4) 1 197, 1 125, 922, 710, 685 against 991, 983, 819,
-    // 672, 653; l_max = 28-40 (2, 1) 884, 780, 787 against 751, 632, 591. float64 l_max = 12
-    // (8) 736 against 928; l_max = 13-18 (4) 1 032, 882, 922, 779, 813 against 760, 918, 776,
-    // 787, 699; l_max = 20-32 (2, 1) 999, 892, 706, 896, 735 against 779, 664, 537, 585, 498.
-    // Values alone: cut rows win on every shape that reaches this kernel (by 11-20 %).
-    const int split_below = env_int("SPHX_SPLIT_BELOW", 8);
+    // of output and 400 calls in a row (in bursts of 60 calls, or with a few hundred MB of
+    // output, the last-level cache merges the parts and the cut rows look 10-30 % better than
+    // they are), whole against cut, us. Gradients, float32: l_max = 17 (8 points per tile) 764
+    // against 1 014; l_max = 19, 20, 22 (4) 1 196, 1 121, 922 against 992, 988, 817; l_max = 24
+    // (4) 707 against 741; l_max = 28, 32 (2) 881, 781 against 883, 636. Gradients, float64:
+    // l_max = 12 (8) 737 against 1 084; l_max = 13, 14, 16, 18 (4) 1 029, 878, 775, 812 against
+    // 1 049, 1 059, 918, 848; l_max = 20, 24 (2) 995, 706 against 886, 626. Values: float32
+    // l_max = 36, 40 (4) 1 004, 977 against 885, 865; float64 l_max = 24, 28 (4) 924, 856
+    // against 741, 749.
+    const int split_below = env_int("SPHX_SPLIT_BELOW", mode == 0 || elem == 4 ? 8 : 4);
     if (mode < 2 && (!fits || plan->rec.g.tile < split_below)) {
         Launch upper;
         if (plan_recursion(n_samples, l_max, mode, false, elem, budget, lds_limit, cus, &upper,
