@@ -382,7 +382,13 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     if (bytes_for(1, buffers) > limit) return false;
     unsigned S = 1;
     if (bytes_for(1, buffers) <= budget) {
-        S = pow2_floor((budget / esize - fixed) / (buffers * rows_per_point + rest_per_point));
+        // as many points as the budget holds, a power of two or not: fewer barrier rounds per
+        // point (2 GB of output, gradients, float64 l_max = 13: 824 us with 4 points per tile,
+        // 611 with 7; l_max = 14: 705 with 4, 602 with 6; float32 l_max = 21: 639 with 4, 603
+        // with 6; second derivatives, float64 l_max = 12: 783 with 2, 547 with 3; never more
+        // than 4 % slower than the power of two below)
+        S = (budget / esize - fixed) / (buffers * rows_per_point + rest_per_point);
+        if (env_int("SPHX_TILE_POW2", 0) != 0) S = pow2_floor(S);
         if (S > 64) S = 64;
     }
     const int forced = env_int("SPHX_TILE", 0);
@@ -420,14 +426,19 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     if (g.flush_waves > 2) g.flush_waves = 2;
     if (buffers == 2 && g.flush_waves < 1) g.flush_waves = 1;
     g.sequence_waves = S * arrays * static_cast<unsigned>(l_max - hard) > 64 ? 2u : 1u;
-    // Split the sides when that lets the entries of a tile go through the entry waves in fewer
-    // rounds than it costs: a one-sided job is about 0.6 of a two-sided one.
+    // float64: split the sides when that lets the entries of a tile go through the entry waves
+    // in fewer rounds than it costs, a one-sided job being about 0.6 of a two-sided one.
+    // float32: always; the two-sided job measured slower at every l_max and tile size (1.5 GB of
+    // output, l_max = 5, 16 points per tile: 895 against 652 us; l_max = 10, 8 points: 826
+    // against 598; l_max = 12, 4 points: 1 005 against 642; l_max = 15, 4 points: 780 against
+    // 460), while float64 with the sides always split loses 10-20 % at most l_max.
     const unsigned wide = kRecursionThreads - 64 * (1 + g.sequence_waves + g.flush_waves);
     auto per_pass = [&](unsigned j) { return j >= wide ? 1u : wide / j; };
     auto rounds = [&](unsigned j) {
         return ((S + per_pass(j) - 1) / per_pass(j)) * ((j + wide - 1) / wide);
     };
-    *split_sides = may_split && 6 * rounds(jobs_split) < 10 * rounds(jobs);
+    const unsigned one_side_costs = static_cast<unsigned>(env_int("SPHX_SPLIT_RATIO", elem == 4 ? 1 : 6));
+    *split_sides = may_split && one_side_costs * rounds(jobs_split) < 10 * rounds(jobs);
     g.jobs_per_point = *split_sides ? jobs_split : jobs;
     g.magic_jobs = magic_of(g.jobs_per_point);
     g.points_per_pass = per_pass(g.jobs_per_point);
@@ -510,7 +521,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // Second derivatives at small l_max: one point per lane where that was measured to be faster
     // than the recursion kernel (SPHX_HESSIAN_LANES: 0 never, 2 wherever the rows fit).
     const int hessian_lanes = env_int("SPHX_HESSIAN_LANES", 1);
-    const bool hessian_lanes_pay = elem == 4 ? (l_max <= 5 || l_max == 7) : l_max <= 5;
+    const bool hessian_lanes_pay = elem == 4 ? l_max <= 5 : l_max <= 3;
     if (lane_kernels && mode == 2 && (hessian_lanes == 2 || (hessian_lanes == 1 && hessian_lanes_pay)) &&
         plan_hessian_lanes(n_samples, l_max, elem, lds_limit, &plan->closed)) {
         plan->lanes = true;

@@ -163,6 +163,31 @@ def test_rows_cut_at_l7_by_one_launch_and_by_two(oracle, library, launches, monk
                     assert torch.isnan(raw[i][:shift]).all() and torch.isnan(raw[i][shift + sizes[i]:]).all()
 
 
+@pytest.mark.parametrize("tile", [3, 5, 7])
+def test_recursion_kernel_with_tiles_that_are_no_power_of_two(oracle, library, tile, monkeypatch):
+    """The planner takes as many points per tile as fit; here sizes it would not pick are forced
+    (the switches are read at every call), with the lane kernels off so that the recursion kernel
+    runs at every l_max."""
+    monkeypatch.setenv("SPHX_TILE", str(tile))
+    monkeypatch.setenv("SPHX_GRADIENT_LANES", "0")
+    monkeypatch.setenv("SPHX_HESSIAN_LANES", "0")
+    monkeypatch.setenv("SPHX_VALUES_LDS", "1")
+    rng = np.random.default_rng(29 + tile)
+    cases = ((np.float32, 9, "hessians"), (np.float64, 8, "hessians"), (np.float32, 12, "gradients"),
+             (np.float64, 13, "gradients"), (np.float32, 20, "gradients"), (np.float64, 10, "values"))
+    for dtype, l_max, mode in cases:
+        for n in (1, tile, 8 * tile + 1, 3001):
+            announce("odd tiles", tile, np.dtype(dtype).name, l_max, mode, n)
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, True, mode)
+            status, out = run_launch_layer(library, torch.from_numpy(xyz).cuda(), l_max, True, mode)
+            assert status == 0, library.sphx_last_error()
+            torch.cuda.synchronize()
+            for o, w in zip(out, want):
+                if w is not None:
+                    assert same_numbers(o.cpu().numpy().reshape(w.shape), w).all(), (l_max, mode, n)
+
+
 def test_lds_size_alternates_between_launches(oracle):
     """One kernel, launches that need more, then less, then more LDS again (all above 64 KB)."""
     rng = np.random.default_rng(21)
