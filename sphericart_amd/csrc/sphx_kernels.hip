@@ -470,10 +470,14 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.n_tiles = static_cast<unsigned>((n_samples + S - 1) / S);
     g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
     // Chunks of consecutive tiles per workgroup: only where a tile is one run per array, and a
-    // run is at least a line long (so that a carried part never spans two tiles).
+    // run is at least a line long (so that a carried part never spans two tiles). About eight
+    // points per chunk: chunks of eight tiles whatever their size were as good for tiles of one
+    // or two points and worse for larger ones (second derivatives, float64, 1.5 GB of output:
+    // l_max = 16, 4 points per tile, 446 us in chunks of eight tiles, 394 in chunks of two;
+    // l_max = 8, 14 points, 632 against 561 for single tiles; cfg4 562 against 528).
     g.chunk_shift = 0;
     if (whole && S * nrow * esize >= 128u) {
-        const int want = env_int("SPHX_CHUNK_SHIFT", 3);
+        const int want = env_int("SPHX_CHUNK_SHIFT", S >= 5 ? 0 : (S >= 3 ? 1 : (S == 2 ? 2 : 3)));
         g.chunk_shift = want < 0 ? 0u : (want > 10 ? 10u : static_cast<unsigned>(want));
     }
     unsigned per_cu = limit / out->lds_bytes;
@@ -521,7 +525,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // Second derivatives at small l_max: one point per lane where that was measured to be faster
     // than the recursion kernel (SPHX_HESSIAN_LANES: 0 never, 2 wherever the rows fit).
     const int hessian_lanes = env_int("SPHX_HESSIAN_LANES", 1);
-    const bool hessian_lanes_pay = elem == 4 ? l_max <= 5 : l_max <= 3;
+    const bool hessian_lanes_pay = elem == 4 ? l_max <= 5 : (l_max == 3 || l_max == 5);
     if (lane_kernels && mode == 2 && (hessian_lanes == 2 || (hessian_lanes == 1 && hessian_lanes_pay)) &&
         plan_hessian_lanes(n_samples, l_max, elem, lds_limit, &plan->closed)) {
         plan->lanes = true;
@@ -532,7 +536,14 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
         plan->lanes = true;
         return SPHX_OK;
     }
-    const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", 80 * 1024));
+    // LDS a workgroup of the recursion kernel may take: half a CU's, so that two share the CU.
+    // With second derivatives in float64 the kernel needs more than 128 registers per lane,
+    // one workgroup of 512 threads is all a CU holds, and half of LDS would lie idle: there
+    // the tile takes all of it (1.5 GB of output, l_max = 6: 694 -> 473 us, l_max = 10: 582 ->
+    // 479, l_max = 12: 545 -> 468; solid harmonics l_max = 4-12: 10-20 % less, l_max = 16, 100k
+    // points: 580 -> 560).
+    const int whole_cu = mode == 2 && elem == 8 ? lds_limit : 80 * 1024;
+    const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", whole_cu));
     bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
                                &plan->split_sides);
     // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of
