@@ -42,7 +42,7 @@ PEAK_HBM_GBPS = 8000.0
 # call added up.
 MEASURED_TRAFFIC_BYTES = {
     "cfg3": int((5930.6 * 2.0 + 765861.1) * 1024),
-    "cfg4": int((1330.1 * 2.0 + 2935182.4) * 1024),
+    "cfg4": int((1323.1 * 2.0 + 2935253.2) * 1024),
     "cfg5": int((2914.8 * 2.0 + 3785830.1) * 1024),
     "cfg3:backward": int((394551.2 * 2.0 + 11719.3) * 1024),
     "cfg3:vjp": int((101629.1 * 2.0 + 11718.8) * 1024),
