@@ -561,7 +561,15 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // l_max = 36, 40 (4) 1 004, 977 against 885, 865; float64 l_max = 24, 28 (4) 924, 856
     // against 741, 749.
     const int split_below = env_int("SPHX_SPLIT_BELOW", mode == 0 || elem == 4 ? 8 : 4);
-    if (mode < 2 && (!fits || plan->rec.g.tile < split_below)) {
+    bool cut = plan->rec.g.tile < split_below;
+    // float32 gradients with three or four points per tile are the exception (1.5 GB of output,
+    // whole against cut: l_max = 28 450 against 530 us, l_max = 30 443 against 510, l_max = 24
+    // and 26 within 3 %), unless a switch says otherwise
+    if (mode == 1 && elem == 4 && (plan->rec.g.tile == 3 || plan->rec.g.tile == 4) &&
+        env_int("SPHX_SPLIT_BELOW", -1) < 0) {
+        cut = false;
+    }
+    if (mode < 2 && (!fits || cut)) {
         Launch upper;
         if (plan_recursion(n_samples, l_max, mode, false, elem, budget, lds_limit, cus, &upper,
                            &plan->split_sides)) {
