@@ -265,7 +265,11 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     g.off_pts = off_t;
     g.off_iter = table_stride;
     out->workgroups = g.tiles_per_xcd * 8u;
-    int waves = env_int("SPHX_GRADIENT_LANES_WAVES", 8);
+    // Eight waves share the closed-form slices and the channels; with one or two channels four
+    // are enough and leave room for more workgroups (1.5 GB of output: float64 l_max = 8 469 us
+    // with eight waves, 345 with four; float32 l_max = 7, 8 286, 274 against 273, 261; from three
+    // channels on eight waves are faster, l_max = 12: 357 against 411).
+    int waves = env_int("SPHX_GRADIENT_LANES_WAVES", l_max <= 8 ? 4 : 8);
     waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
     out->threads = 64u * static_cast<unsigned>(waves);
     out->lds_bytes = bytes;
