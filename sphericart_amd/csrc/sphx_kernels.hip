@@ -395,6 +395,23 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         if (env_int("SPHX_TILE_POW2", 0) != 0) S = pow2_floor(S);
         if (S > 64) S = 64;
     }
+    // Few points: with the largest tile there would be fewer tiles than workgroups that a launch
+    // keeps resident. Then the tile is just large enough to give every one of them a tile (for
+    // values and gradients four points at least: below that the closed forms of l <= 6 weigh
+    // too much). 500 points, us: second derivatives float64 l_max = 6 16.1 -> 10.2, l_max = 16
+    // 16.6 -> 12.6, float32 l_max = 12 17.5 -> 11.2; gradients float32 l_max = 20 23.9 -> 12.7.
+    if (S > 1 && env_int("SPHX_TILE_SMALL_N", 1) != 0) {
+        unsigned per_cu = limit / bytes_for(S, buffers);
+        per_cu = per_cu < 1 ? 1u : (per_cu > 2 ? 2u : per_cu);
+        if (mode == 2 && elem == 8) per_cu = 1; // more than 128 registers per lane
+        const unsigned long long resident = static_cast<unsigned long long>(cus > 0 ? cus : 1) * per_cu;
+        if ((n_samples + S - 1) / S <= resident) {
+            unsigned long long enough = (n_samples + resident - 1) / resident;
+            const unsigned least = mode < 2 ? 4u : 1u;
+            if (enough < least) enough = least;
+            if (enough < S) S = static_cast<unsigned>(enough);
+        }
+    }
     const int forced = env_int("SPHX_TILE", 0);
     if (forced > 0 && forced <= 64 && bytes_for(forced, buffers) <= limit) {
         S = static_cast<unsigned>(forced);
