@@ -207,7 +207,10 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // (the product's closed-form slices want at least four; values: one for the tables, one for
     // the closed forms)
     int want = l_max - 6;
-    if (with_sums && want < 4) want = 4;
+    // the product, 0.8 GB of sph_grad, us: l_max = 9, 10 (three and four channels) 266, 310 with
+    // four waves, 207, 282 with three (float64 279, 333 against 233, 304); l_max = 12 350 with six,
+    // 316 with four (float64 385 against 321); one or two channels are best with four
+    if (with_sums) want = want <= 2 ? 4 : (want <= 4 ? 3 : (want <= 6 ? 4 : want));
     if (!with_sums && want < 2) want = env_int("SPHX_VALUES_MIN_WAVES", 2);
     out->threads = 64u * static_cast<unsigned>(want < waves ? want : waves);
     out->lds_bytes = bytes;
