@@ -338,7 +338,8 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
 
 // Tile size and LDS layout of the recursion kernel. Returns false when not even one point fits.
 static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, size_t elem,
-                           unsigned budget, int lds_limit, int cus, Launch* out, bool* split_sides) {
+                           unsigned budget, int lds_limit, int cus, Launch* out, bool* split_sides,
+                           bool normalized = true) {
     Tiling& g = out->g;
     std::memset(&g, 0, sizeof(g));
     const int hard = mode == 2 ? 1 : 6;
@@ -450,18 +451,21 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     if (g.flush_waves > 2) g.flush_waves = 2;
     if (buffers == 2 && g.flush_waves < 1) g.flush_waves = 1;
     g.sequence_waves = S * arrays * static_cast<unsigned>(l_max - hard) > 64 ? 2u : 1u;
-    // float64: split the sides when that lets the entries of a tile go through the entry waves
-    // in fewer rounds than it costs, a one-sided job being about 0.6 of a two-sided one.
-    // float32: always; the two-sided job measured slower at every l_max and tile size (1.5 GB of
+    // Split the sides when that lets the entries of a tile go through the entry waves in fewer
+    // rounds than it costs, a one-sided job being about 0.6 of a two-sided one. Normalised
+    // float32 is the exception: always split, because the two-sided kernel needs 152 registers
+    // per lane, so that only one workgroup fits on a CU, and the one-sided 116 (1.5 GB of
     // output, l_max = 5, 16 points per tile: 895 against 652 us; l_max = 10, 8 points: 826
     // against 598; l_max = 12, 4 points: 1 005 against 642; l_max = 15, 4 points: 780 against
-    // 460), while float64 with the sides always split loses 10-20 % at most l_max.
+    // 460). For solid harmonics in float32 both fit twice (119 and 88 registers) and the rule
+    // holds (l_max = 10: 319 us by the rule, 404 always split; l_max = 12: 327 against 399);
+    // float64 with the sides always split loses 10-20 % at most l_max.
     const unsigned wide = kRecursionThreads - 64 * (1 + g.sequence_waves + g.flush_waves);
     auto per_pass = [&](unsigned j) { return j >= wide ? 1u : wide / j; };
     auto rounds = [&](unsigned j) {
         return ((S + per_pass(j) - 1) / per_pass(j)) * ((j + wide - 1) / wide);
     };
-    const unsigned one_side_costs = static_cast<unsigned>(env_int("SPHX_SPLIT_RATIO", elem == 4 ? 1 : 6));
+    const unsigned one_side_costs = static_cast<unsigned>(env_int("SPHX_SPLIT_RATIO", elem == 4 && normalized ? 1 : 6));
     *split_sides = may_split && one_side_costs * rounds(jobs_split) < 10 * rounds(jobs);
     g.jobs_per_point = *split_sides ? jobs_split : jobs;
     g.magic_jobs = magic_of(g.jobs_per_point);
@@ -522,7 +526,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
 
 // Choose kernels, tile sizes and LDS layouts. `lds_limit` / `cus` describe the device.
 static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit, int cus,
-                     Plan* plan, bool lane_kernels = true) {
+                     Plan* plan, bool lane_kernels = true, bool normalized = true) {
     if (l_max < 0) return fail(SPHX_ERR_ARGUMENT, "l_max must be non-negative");
     if (mode < 0 || mode > 2) return fail(SPHX_ERR_ARGUMENT, "unknown derivative selector");
     if (l_max > SPHX_TABLE_LMAX) {
@@ -549,7 +553,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // Second derivatives at small l_max: one point per lane where that was measured to be faster
     // than the recursion kernel (SPHX_HESSIAN_LANES: 0 never, 2 wherever the rows fit).
     const int hessian_lanes = env_int("SPHX_HESSIAN_LANES", 1);
-    const bool hessian_lanes_pay = elem == 4 ? l_max <= 5 : (l_max == 3 || l_max == 5);
+    const bool hessian_lanes_pay = elem == 4 ? l_max <= 5 : (l_max == 3 || (l_max == 5 && normalized));
     if (lane_kernels && mode == 2 && (hessian_lanes == 2 || (hessian_lanes == 1 && hessian_lanes_pay)) &&
         plan_hessian_lanes(n_samples, l_max, elem, lds_limit, &plan->closed)) {
         plan->lanes = true;
@@ -569,7 +573,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     const int whole_cu = mode == 2 && elem == 8 ? lds_limit : 80 * 1024;
     const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", whole_cu));
     bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
-                               &plan->split_sides);
+                               &plan->split_sides, normalized);
     // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of
     // the lanes idle for some two thousand instructions per tile: then the recursion kernel
     // stages l >= 7 only and its wave 0, which mostly waits, writes l <= 6 straight from
@@ -809,7 +813,7 @@ static int forward(const T* xyz, size_t n_samples, int l_max, int normalized, in
     Plan plan;
     if (status == SPHX_OK) {
         status = make_plan(n_samples, l_max, mode, sizeof(T), g_lds_limit[device],
-                           g_compute_units[device], &plan);
+                           g_compute_units[device], &plan, true, normalized != 0);
     }
     if (status == SPHX_OK) {
         hipStream_t s = reinterpret_cast<hipStream_t>(stream);
