@@ -460,13 +460,37 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // 460). For solid harmonics in float32 both fit twice (119 and 88 registers) and the rule
     // holds (l_max = 10: 319 us by the rule, 404 always split; l_max = 12: 327 against 399);
     // float64 with the sides always split loses 10-20 % at most l_max.
-    const unsigned wide = kRecursionThreads - 64 * (1 + g.sequence_waves + g.flush_waves);
+    const unsigned one_side_costs = static_cast<unsigned>(env_int("SPHX_SPLIT_RATIO", elem == 4 && normalized ? 1 : 6));
+    unsigned wide = 0;
     auto per_pass = [&](unsigned j) { return j >= wide ? 1u : wide / j; };
     auto rounds = [&](unsigned j) {
         return ((S + per_pass(j) - 1) / per_pass(j)) * ((j + wide - 1) / wide);
     };
-    const unsigned one_side_costs = static_cast<unsigned>(env_int("SPHX_SPLIT_RATIO", elem == 4 && normalized ? 1 : 6));
-    *split_sides = may_split && one_side_costs * rounds(jobs_split) < 10 * rounds(jobs);
+    // rounds of the entry waves per tile, in tenths of two-sided jobs, with `waves` sequence waves
+    auto entry_cost = [&](unsigned waves, bool* split) {
+        wide = kRecursionThreads - 64 * (1 + waves + g.flush_waves);
+        *split = may_split && one_side_costs * rounds(jobs_split) < 10 * rounds(jobs);
+        return *split ? one_side_costs * rounds(jobs_split) : 10 * rounds(jobs);
+    };
+    // A second sequence wave takes a wave from the entries. One is enough where it saves the
+    // entry waves a round per tile, and for values alone, whose recursions are a third of the
+    // work (1.5 GB of output, one against two: gradients float32 l_max = 18, 19 437, 449 against
+    // 545, 595 us; float64 l_max = 15, 16, 18 475, 423, 428 against 522, 460, 494; second
+    // derivatives float32 l_max = 10, 13 496, 490 against 637, 637; values float32 l_max = 40,
+    // 48 468, 428 against 527, 477; with equal rounds two are faster by 2-3 % with derivatives).
+    // Second derivatives in float64 follow no such rule (l_max = 6, 8, 10: 555, 437, 505 against
+    // 449, 558, 445) and keep two.
+    if (g.sequence_waves == 2 && !(mode == 2 && elem == 8)) {
+        bool split_one = false, split_two = false;
+        const unsigned with_one = entry_cost(1, &split_one);
+        const unsigned with_two = entry_cost(2, &split_two);
+        if (mode == 0 || with_one < with_two) g.sequence_waves = 1;
+    }
+    {
+        const int forced_seq = env_int("SPHX_SEQUENCE_WAVES", 0);
+        if (forced_seq >= 1 && forced_seq <= 4) g.sequence_waves = static_cast<unsigned>(forced_seq);
+    }
+    entry_cost(g.sequence_waves, split_sides); // leaves `wide` as it will be
     g.jobs_per_point = *split_sides ? jobs_split : jobs;
     g.magic_jobs = magic_of(g.jobs_per_point);
     g.points_per_pass = per_pass(g.jobs_per_point);
