@@ -463,8 +463,15 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     const unsigned one_side_costs = static_cast<unsigned>(env_int("SPHX_SPLIT_RATIO", elem == 4 && normalized ? 1 : 6));
     unsigned wide = 0;
     auto per_pass = [&](unsigned j) { return j >= wide ? 1u : wide / j; };
-    auto rounds = [&](unsigned j) {
+    // rounds of the entry lanes per tile: whole points side by side, or (fewer, where the
+    // points leave lanes idle) the jobs of all points as one list
+    auto rounds_by_point = [&](unsigned j) {
         return ((S + per_pass(j) - 1) / per_pass(j)) * ((j + wide - 1) / wide);
+    };
+    auto rounds = [&](unsigned j) {
+        const unsigned as_list = (S * j + wide - 1) / wide;
+        const unsigned by_point = rounds_by_point(j);
+        return S >= 3 && per_pass(j) <= 2 && as_list < by_point ? as_list : by_point;
     };
     // rounds of the entry waves per tile, in tenths of two-sided jobs, with `waves` sequence waves
     auto entry_cost = [&](unsigned waves, bool* split) {
@@ -494,6 +501,16 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.jobs_per_point = *split_sides ? jobs_split : jobs;
     g.magic_jobs = magic_of(g.jobs_per_point);
     g.points_per_pass = per_pass(g.jobs_per_point);
+    // The list costs a few instructions per job: only where it saves a round (1.5 GB of output,
+    // gradients float32 l_max = 17, 20, 30: 466, 563, 442 -> 379, 453, 371 us; second derivatives
+    // float64 l_max = 14: 580 -> 426; with equal rounds, l_max = 32: 390 -> 423). It did not pay
+    // with two points per tile (l_max = 32, three rounds instead of four: 387 -> 424 us) nor
+    // where four points go side by side anyway (second derivatives float32 l_max = 8: 580 -> 631).
+    const int want_list = env_int("SPHX_JOB_LIST", -1);
+    const bool saves_a_round = (S * g.jobs_per_point + wide - 1) / wide < rounds_by_point(g.jobs_per_point);
+    if (want_list != 0 && saves_a_round && (want_list > 0 || (S >= 3 && g.points_per_pass <= 2))) {
+        g.points_per_pass = 0;
+    }
 
     // in front of every staging region, room for the part of a 128-byte line that precedes the
     // tile's run (recursion_kernel, flush_run)
@@ -632,6 +649,12 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
             fits = true;
         }
     }
+    if (fits && !lane_kernels && plan->rec.g.points_per_pass == 0) {
+        // the fused product has no job-list variant of the kernel: whole points side by side
+        const Tiling& g = plan->rec.g;
+        const unsigned wide = kRecursionThreads - 64 * (1 + g.sequence_waves + g.flush_waves);
+        plan->rec.g.points_per_pass = g.jobs_per_point >= wide ? 1u : wide / g.jobs_per_point;
+    }
     if (!fits) {
         return fail(SPHX_ERR_UNSUPPORTED,
                     "l_max = " + std::to_string(l_max) +
@@ -707,10 +730,16 @@ static hipError_t launch_closed(const Launch& l, const T* xyz, T* sph, T* dsph, 
     return hipGetLastError();
 }
 
-template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false>
+template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false>
 static hipError_t launch_recursion(const Launch& l, const T* xyz, T* sph, T* dsph, T* ddsph,
                                    hipStream_t stream) {
-    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT, VJP>;
+    if constexpr (!VJP && !LIST) {
+        // the variant whose entry lanes take the jobs of a tile as one list
+        if (l.g.points_per_pass == 0) {
+            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, false, true>(l, xyz, sph, dsph, ddsph, stream);
+        }
+    }
+    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST>;
     // The workgroups are persistent: launch exactly as many as are resident at once (registers
     // may allow fewer per CU than LDS does), or the last ones would run alone after the rest.
     unsigned workgroups = l.workgroups;

@@ -54,7 +54,7 @@ constexpr unsigned kRecursionThreads = 512;
 // and spill a few registers; with 170 registers and one workgroup per CU, l_max = 12 float64
 // gradients took 800 us instead of 513 us. The second-derivative kernels keep what they need
 // (forced to 128 they spill in the entry jobs: 918 us against 558 us at l_max = 10, float64).
-template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false>
+template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false>
 __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling g, const T* __restrict__ xyz,
                                                                      T* __restrict__ sph,
                                                                      T* __restrict__ dsph,
@@ -364,19 +364,19 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
         const unsigned t = tid - wide_first;
         const Phases ph = phases_of(n);
         const unsigned phase_sph = ph.sph, phase_dsph = ph.dsph, phase_ddsph = ph.ddsph;
-        // One pass takes the jobs of as many points as fit side by side in the wide lanes
-        // (of one point, in several rounds, when it has more jobs than there are lanes);
-        // what depends on the point only is read once per pass.
-        unsigned local = 0, e_first = t;
-        if (g.points_per_pass > 1) {
-            local = __umulhi(t, g.magic_jobs);
-            e_first = t - local * g.jobs_per_point;
-        }
-        for (unsigned s0 = 0; s0 < valid; s0 += g.points_per_pass) {
-            const unsigned s = s0 + local;
-            if (s >= valid || local >= g.points_per_pass) continue;
+        // what depends on the point only
+        Point<T> p;
+        p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
+        const T* c = nullptr;
+        const T* sn = nullptr;
+        const T* itA = nullptr;
+        const T* itB = nullptr;
+        const T* itC = nullptr;
+        Rows<T> rows;
+        rows.ny = static_cast<int>(row_stride);
+        rows.sph = rows.dsph = rows.ddsph = nullptr;
+        auto take_point = [&](unsigned s) {
             const T* rec = point_data(n, s);
-            Point<T> p;
             p.x = rec[0];
             p.y = rec[1];
             p.z = rec[2];
@@ -384,26 +384,57 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
             p.y2 = rec[4];
             p.z2 = rec[5];
             p.ir = rec[6];
-            const T* c = rec + 8;
-            const T* sn = rec + 8 + (L + 1);
-            const T* itA = iterates(n & 1u, s, 0, 0);
-            const T* itB = iterates(n & 1u, s, MODE >= 1 ? 1 : 0, 0);
-            const T* itC = iterates(n & 1u, s, MODE == 2 ? 2 : 0, 0);
+            c = rec + 8;
+            sn = rec + 8 + (L + 1);
+            itA = iterates(n & 1u, s, 0, 0);
+            itB = iterates(n & 1u, s, MODE >= 1 ? 1 : 0, 0);
+            itC = iterates(n & 1u, s, MODE == 2 ? 2 : 0, 0);
             // rows are addressed with the entry's index in the full row; shift the bases when
             // the staged rows start at l = H + 1
-            Rows<T> rows;
-            rows.ny = static_cast<int>(row_stride);
             rows.sph = staged + phase_sph + s * row_stride - skip;
             rows.dsph = staged + g.off_dsph + phase_dsph + s * 3 * row_stride - skip;
             rows.ddsph = staged + g.off_ddsph + phase_ddsph + s * 9 * row_stride - skip;
-            for (unsigned e = e_first; e < g.jobs_per_point; e += wide_lanes) {
-                const unsigned packed = job_table[e];
-                const int m = static_cast<int>(packed & 0x7fu);
-                const int side = static_cast<int>((packed >> 7) & 1u);
-                const int l = static_cast<int>((packed >> 8) & 0xffu);
-                const int tri = static_cast<int>(packed >> 16);
-                entry_job<T, MODE, NORM, SPLIT>(l, m, tri, side, p, F + tri, c, sn, itA + tri,
-                                                itB + tri, itC + tri, rows);
+        };
+        auto take_job = [&](unsigned e) {
+            const unsigned packed = job_table[e];
+            const int m = static_cast<int>(packed & 0x7fu);
+            const int side = static_cast<int>((packed >> 7) & 1u);
+            const int l = static_cast<int>((packed >> 8) & 0xffu);
+            const int tri = static_cast<int>(packed >> 16);
+            entry_job<T, MODE, NORM, SPLIT>(l, m, tri, side, p, F + tri, c, sn, itA + tri, itB + tri,
+                                            itC + tri, rows);
+        };
+        const unsigned per_point = g.jobs_per_point;
+        if constexpr (LIST) {
+            // The jobs of the tile's points as one list, point after point, dealt to the wide
+            // lanes round after round: only the last round can leave lanes idle. The host
+            // launches this variant where it saves rounds (l_max = 20: 203 jobs per point on 320
+            // lanes, seven points in five rounds instead of seven); a lane looks at every job's
+            // point. (Both loops in one kernel made either slower by some 5 %.)
+            const unsigned total = valid * per_point;
+            unsigned current = ~0u;
+            for (unsigned q = t; q < total; q += wide_lanes) {
+                const unsigned s = __umulhi(q, g.magic_jobs); // exact: q * per_point < 2^32
+                if (s != current) {
+                    current = s;
+                    take_point(s);
+                }
+                take_job(q - s * per_point);
+            }
+        } else {
+            // One pass takes the jobs of as many points as fit side by side in the wide lanes
+            // (of one point, in several rounds, when it has more jobs than there are lanes);
+            // what depends on the point only is read once per pass.
+            unsigned local = 0, e_first = t;
+            if (g.points_per_pass > 1) {
+                local = __umulhi(t, g.magic_jobs);
+                e_first = t - local * per_point;
+            }
+            for (unsigned s0 = 0; s0 < valid; s0 += g.points_per_pass) {
+                const unsigned s = s0 + local;
+                if (s >= valid || local >= g.points_per_pass) continue;
+                take_point(s);
+                for (unsigned e = e_first; e < per_point; e += wide_lanes) take_job(e);
             }
         }
     };

@@ -39,7 +39,8 @@ struct Tiling {
     unsigned jobs_per_point; // entry jobs per point: (l, m >= 0) pairs above the closed-form
                              // limit, or (l, m, side) triples when the sides are split
     unsigned sequence_waves; // waves that run the bare recursions (1 or 2)
-    unsigned points_per_pass; // points whose entry jobs fit side by side in the wide waves (>= 1)
+    unsigned points_per_pass; // points whose entry jobs fit side by side in the wide waves;
+                              // 0: the jobs of all points of a tile as one list
     unsigned vjp_accumulate; // fused product: add to xyz_grad instead of overwriting it
     unsigned az_shift;      // the point tables are made for 2^az_shift tiles at a time
     unsigned chunk_shift;   // a workgroup takes 2^chunk_shift consecutive tiles at a time

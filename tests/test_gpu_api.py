@@ -188,6 +188,33 @@ def test_recursion_kernel_with_tiles_that_are_no_power_of_two(oracle, library, t
                     assert same_numbers(o.cpu().numpy().reshape(w.shape), w).all(), (l_max, mode, n)
 
 
+@pytest.mark.parametrize("order", ["list", "points"])
+def test_entry_jobs_as_one_list_and_point_by_point(oracle, library, order, monkeypatch):
+    """The two variants of the recursion kernel's entry stage (the jobs of a tile as one list
+    over the lanes, or whole points side by side; the planner picks per shape, the switch forces
+    one wherever the other would save nothing), with enough points for full tiles."""
+    monkeypatch.setenv("SPHX_JOB_LIST", "1" if order == "list" else "0")
+    monkeypatch.setenv("SPHX_GRADIENT_LANES", "0")
+    monkeypatch.setenv("SPHX_HESSIAN_LANES", "0")
+    monkeypatch.setenv("SPHX_VALUES_LDS", "1")
+    rng = np.random.default_rng(31)
+    cases = ((np.float32, 17, "gradients"), (np.float32, 20, "gradients"), (np.float64, 16, "gradients"),
+             (np.float32, 14, "hessians"), (np.float64, 14, "hessians"), (np.float32, 34, "values"),
+             (np.float64, 9, "gradients"), (np.float32, 8, "hessians"))
+    for dtype, l_max, mode in cases:
+        n = 6007
+        normalized = bool(l_max & 1)
+        announce("entry jobs", order, np.dtype(dtype).name, l_max, mode, normalized)
+        xyz = special_points(dtype, rng, n)
+        want = oracle.compute(xyz, l_max, normalized, mode)
+        status, out = run_launch_layer(library, torch.from_numpy(xyz).cuda(), l_max, normalized, mode)
+        assert status == 0, library.sphx_last_error()
+        torch.cuda.synchronize()
+        for o, w in zip(out, want):
+            if w is not None:
+                assert same_numbers(o.cpu().numpy().reshape(w.shape), w).all(), (l_max, mode)
+
+
 def test_lds_size_alternates_between_launches(oracle):
     """One kernel, launches that need more, then less, then more LDS again (all above 64 KB)."""
     rng = np.random.default_rng(21)
