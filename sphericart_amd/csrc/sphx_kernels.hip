@@ -629,15 +629,13 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // 1 049, 1 059, 918, 848; l_max = 20, 24 (2) 995, 706 against 886, 626. Values: float32
     // l_max = 36, 40 (4) 1 004, 977 against 885, 865; float64 l_max = 24, 28 (4) 924, 856
     // against 741, 749.
-    const int split_below = env_int("SPHX_SPLIT_BELOW", mode == 0 || elem == 4 ? 8 : 4);
-    bool cut = plan->rec.g.tile < split_below;
-    // float32 gradients with three or four points per tile are the exception (1.5 GB of output,
-    // whole against cut: l_max = 28 450 against 530 us, l_max = 30 443 against 510, l_max = 24
-    // and 26 within 3 %), unless a switch says otherwise
-    if (mode == 1 && elem == 4 && (plan->rec.g.tile == 3 || plan->rec.g.tile == 4) &&
-        env_int("SPHX_SPLIT_BELOW", -1) < 0) {
-        cut = false;
-    }
+    // (With the job-list variant of the kernel the whole rows gained more than the cut ones:
+    // float32 gradients, 1.5 GB of output, whole against cut: l_max = 19-22 (5-7 points per tile)
+    // 393, 407, 373, 399 us against 431, 451, 419, 424; l_max = 28, 30 (3) 396, 371 against 532,
+    // 510; l_max = 32 (2) 462 against 389. Float32 gradients are therefore cut below three
+    // points per tile only; values below eight, float64 gradients below four as before.)
+    const int split_below = env_int("SPHX_SPLIT_BELOW", mode == 0 ? 8 : (elem == 4 ? 3 : 4));
+    const bool cut = plan->rec.g.tile < split_below;
     if (mode < 2 && (!fits || cut)) {
         Launch upper;
         if (plan_recursion(n_samples, l_max, mode, false, elem, budget, lds_limit, cus, &upper,
