@@ -162,7 +162,13 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     const unsigned row_stride = (ny * (esize / 4u)) % 8u == 0 ? ny + vec : ny;
     const unsigned table_stride = (3u * static_cast<unsigned>(l_max + 1)) | 1u;
     const unsigned tri_all = static_cast<unsigned>(l_max + 1) * (l_max + 2) / 2;
-    unsigned allowed = static_cast<unsigned>(env_int("SPHX_VALUES_LDS", 160 * 1024));
+    // float32 values whose 32 rows need more than half a CU's LDS (l_max >= 23) are left to the
+    // recursion kernel, which with its job-list variant is faster there (1 GB of output, l_max =
+    // 24, 28, 32: 508, 505, 472 us against 574, 567, 543; l_max = 26 is the exception, 627
+    // against 546); in float64 the values kernel still wins with a whole CU's LDS (l_max = 18,
+    // 20, 22: 426, 401, 380 against 483, 436, 429).
+    unsigned allowed = static_cast<unsigned>(
+        env_int("SPHX_VALUES_LDS", with_sums || elem == 8 ? 160 * 1024 : 80 * 1024));
     if (allowed > static_cast<unsigned>(lds_limit)) allowed = static_cast<unsigned>(lds_limit);
     // Fewer than 64 points per workgroup leave lanes idle: with 32 the values kernel still beats
     // the recursion kernel (l_max = 32 float32, 500k points: 781 against 1 077 us; l_max = 20
