@@ -9,13 +9,24 @@ preallocated outputs. The default workload is the configuration the headline
 metric is quoted on: real spherical harmonics, l_max = 6, float32, values and
 gradients, 1,000,000 points.
 
+The K timed steps are enqueued back to back between one pair of events and
+one pair of host clock readings (`value`, `ms_per_step`); a second pass of K
+steps with an event pair around every launch gives the duration of the single
+launch that `roofline` is computed from.
+
 One JSON line is printed. Next to the contract fields it carries
 
   roofline      achieved HBM bandwidth of the kernel: algorithmic bytes per
                 launch (sizeof(T) * (3 + (l_max+1)^2 * components) per point)
                 divided by the average launch duration, measured with events
-                on the launch stream around every timed launch, against the
-                8 TB/s peak of MI355X;
+                on the launch stream around every launch of the second pass,
+                against the 8 TB/s peak of MI355X;
+  roofline_by_config
+                (default workload only) the same figure for the other four
+                configurations of the reference's benchmark set, each with the
+                kernel it launches, and for cfg1-cfg3 a second figure with the
+                outputs rotating through 1 GB of buffers, so that no launch
+                finds its lines in the 256 MB Infinity Cache;
   cpu_baseline  the reference CPU implementation (oracle/_ref, built from the
                 reference's own sources; the repository's restatement when that
                 is absent) timed on the host cores on a bounded number of
@@ -23,6 +34,7 @@ One JSON line is printed. Next to the contract fields it carries
 """
 
 import argparse
+import ctypes
 import json
 import os
 import statistics
@@ -84,6 +96,8 @@ def parse():
         "is also measured with every launch going to memory that is not cached",
     )
     p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--no-by-config", action="store_true",
+                   help="default workload only: leave out the measurements of the other four configurations")
     p.add_argument(
         "--calibrate-copy",
         action="store_true",
@@ -181,6 +195,156 @@ def cpu_vjp_baseline(workload, xyz, sph_grad):
     }
 
 
+class Prepared:
+    """A workload's points and preallocated outputs on the GPU and the call that evaluates them."""
+
+    def __init__(self, lib, w, rotate_mb=0):
+        import torch
+
+        self.lib, self.w = lib, w
+        self.xyz_host = w.points()
+        self.xyz = torch.from_numpy(self.xyz_host).cuda()
+        self.n, self.ny = w.n_samples, (w.l_max + 1) ** 2
+        self.opts = dict(dtype=self.xyz.dtype, device=self.xyz.device)
+        self.mode = {"values": 0, "gradients": 1, "hessians": 2}[w.derivatives]
+        self.forward = lib.sphx_forward_f32 if w.dtype == "f32" else lib.sphx_forward_f64
+        self.stream = torch.cuda.current_stream()
+        self.bytes_per_launch = w.bytes_per_point * self.n
+        copies = 1
+        if rotate_mb > 0:
+            copies = max(2, -(-rotate_mb * 1_000_000 // self.bytes_per_launch))
+        self.outputs = [self._allocate() for _ in range(copies)]
+        self.calls = [self._pointers(o) for o in self.outputs]
+        self.turn = 0
+
+    def _allocate(self):
+        import torch
+
+        n, ny, mode = self.n, self.ny, self.mode
+        return (torch.empty((n, ny), **self.opts),
+                torch.empty((n, 3, ny), **self.opts) if mode >= 1 else None,
+                torch.empty((n, 3, 3, ny), **self.opts) if mode >= 2 else None)
+
+    def _pointers(self, o):
+        return (self.xyz.data_ptr(), self.n, self.w.l_max, int(self.w.normalized), self.mode, o[0].data_ptr(),
+                o[1].data_ptr() if o[1] is not None else None,
+                o[2].data_ptr() if o[2] is not None else None, self.stream.cuda_stream)
+
+    def step(self):
+        status = self.forward(*self.calls[self.turn % len(self.calls)])
+        self.turn += 1
+        if status != 0:
+            raise RuntimeError(self.lib.sphx_last_error().decode())
+
+    def kernels(self):
+        text = ctypes.create_string_buffer(1024)
+        status = self.lib.sphx_describe_plan(self.n, self.w.l_max, self.mode, int(self.w.dtype == "f64"),
+                                             int(self.w.normalized), text, len(text))
+        return text.value.decode() if status == 0 else None
+
+
+def settle(step, seconds, warmup):
+    import torch
+
+    until = time.perf_counter() + seconds
+    while time.perf_counter() < until:
+        for _ in range(50):
+            step()
+        torch.cuda.synchronize()
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+
+
+def time_back_to_back(step, steps, stream):
+    """K steps enqueued one after the other: host seconds between two synchronisations, and
+    device milliseconds between one event before the first and one after the last launch."""
+    import torch
+
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    begin.record(stream)
+    for _ in range(steps):
+        step()
+    end.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, begin.elapsed_time(end)
+
+
+def time_each_launch(step, steps, stream):
+    """Milliseconds of every one of K launches, an event pair around each."""
+    import torch
+
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    for begin, end in events:
+        begin.record(stream)
+        step()
+        end.record(stream)
+    torch.cuda.synchronize()
+    return [b.elapsed_time(e) for b, e in events]
+
+
+def roofline_of(launch_ms, bytes_per_launch):
+    avg_s = sum(launch_ms) / len(launch_ms) / 1e3
+    achieved = bytes_per_launch / avg_s / 1e9
+    return {
+        "bound": "hbm",
+        "achieved": achieved,
+        "peak": PEAK_HBM_GBPS,
+        "unit": "GB/s",
+        "frac": achieved / PEAK_HBM_GBPS,
+        "algorithmic_bytes_per_launch": bytes_per_launch,
+        "avg_launch_us": avg_s * 1e6,
+        "median_launch_us": statistics.median(launch_ms) * 1e3,
+        "min_launch_us": min(launch_ms) * 1e3,
+    }
+
+
+def measure_config(lib, name, steps, settle_seconds, with_cold):
+    """One of the benchmark configurations next to the headline: per-launch event times with the
+    outputs in place and, for the small ones, rotating through 1 GB of output buffers."""
+    import torch
+
+    from sphericart_amd.workloads import WORKLOADS
+
+    w = WORKLOADS[name]
+    steps = max(steps, 50)
+    prepared = Prepared(lib, w)
+    settle(prepared.step, settle_seconds, 10)
+    wall, device_ms = time_back_to_back(prepared.step, steps, prepared.stream)
+    entry = roofline_of(time_each_launch(prepared.step, steps, prepared.stream), prepared.bytes_per_launch)
+    entry.update({
+        "workload": f"{w.name}: {w.description}",
+        "dtype": w.dtype,
+        "kernels": prepared.kernels(),
+        "launches_timed": steps,
+        "points_per_s": w.n_samples * steps / wall,
+        "back_to_back_us_per_launch": device_ms / steps * 1e3,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(name),
+    })
+    del prepared
+    torch.cuda.empty_cache()
+    if with_cold:
+        cold = Prepared(lib, w, rotate_mb=1024)
+        settle(cold.step, settle_seconds, 10)
+        launch_ms = time_each_launch(cold.step, steps, cold.stream)
+        r = roofline_of(launch_ms, cold.bytes_per_launch)
+        entry["cold"] = {
+            "rotate_mb": 1024,
+            "output_buffers": len(cold.outputs),
+            "avg_launch_us": r["avg_launch_us"],
+            "min_launch_us": r["min_launch_us"],
+            "achieved": r["achieved"],
+            "frac": r["frac"],
+        }
+        del cold
+        torch.cuda.empty_cache()
+    return entry
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -203,45 +367,12 @@ def main():
     lib = sphericart_amd.get_library()
     torch.cuda.set_device(0)
 
-    xyz_host = w.points()
-    xyz = torch.from_numpy(xyz_host).cuda()
-    n, ny = w.n_samples, (w.l_max + 1) ** 2
-    opts = dict(dtype=xyz.dtype, device=xyz.device)
-    mode = {"values": 0, "gradients": 1, "hessians": 2}[w.derivatives]
-    sph = torch.empty((n, ny), **opts)
-    dsph = torch.empty((n, 3, ny), **opts) if mode >= 1 else None
-    ddsph = torch.empty((n, 3, 3, ny), **opts) if mode >= 2 else None
-    forward = lib.sphx_forward_f32 if w.dtype == "f32" else lib.sphx_forward_f64
-    stream = torch.cuda.current_stream()
-    pointers = (
-        xyz.data_ptr(), n, w.l_max, int(w.normalized), mode, sph.data_ptr(),
-        dsph.data_ptr() if dsph is not None else None,
-        ddsph.data_ptr() if ddsph is not None else None, stream.cuda_stream,
-    )
-
-    def step():
-        status = forward(*pointers)
-        if status != 0:
-            raise RuntimeError(lib.sphx_last_error().decode())
-
-    bytes_per_launch = w.bytes_per_point * n
-    if args.rotate_mb > 0 and args.op == "forward":
-        copies = max(2, -(-args.rotate_mb * 1_000_000 // bytes_per_launch))
-        rotating = []
-        for _ in range(copies):
-            o = (torch.empty((n, ny), **opts),
-                 torch.empty((n, 3, ny), **opts) if mode >= 1 else None,
-                 torch.empty((n, 3, 3, ny), **opts) if mode >= 2 else None)
-            rotating.append((o, (xyz.data_ptr(), n, w.l_max, int(w.normalized), mode, o[0].data_ptr(),
-                                 o[1].data_ptr() if o[1] is not None else None,
-                                 o[2].data_ptr() if o[2] is not None else None, stream.cuda_stream)))
-        turn = [0]
-
-        def step():  # noqa: F811
-            status = forward(*rotating[turn[0] % copies][1])
-            turn[0] += 1
-            if status != 0:
-                raise RuntimeError(lib.sphx_last_error().decode())
+    prepared = Prepared(lib, w, args.rotate_mb if args.op == "forward" else 0)
+    xyz_host, xyz = prepared.xyz_host, prepared.xyz
+    n, ny, mode, opts, stream = prepared.n, prepared.ny, prepared.mode, prepared.opts, prepared.stream
+    sph, dsph, ddsph = prepared.outputs[0]
+    step = prepared.step
+    bytes_per_launch = prepared.bytes_per_launch
 
     if args.op == "backward":
         if mode < 1:
@@ -300,28 +431,15 @@ def main():
         }))
         return 0
 
-    settle_until = time.perf_counter() + args.settle_seconds
-    while time.perf_counter() < settle_until:
-        for _ in range(50):
-            step()
-        torch.cuda.synchronize()
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for begin, end in events:
-        begin.record(stream)
-        step()
-        end.record(stream)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-
-    launch_ms = [b.elapsed_time(e) for b, e in events]
-    avg_launch_s = sum(launch_ms) / len(launch_ms) / 1e3
-    achieved = bytes_per_launch / avg_launch_s / 1e9
+    settle(step, args.settle_seconds, args.warmup)
+    # the timed region: K steps back to back
+    wall, device_ms = time_back_to_back(step, args.steps, stream)
+    # the single launch: K more steps, an event pair around each
+    roofline = roofline_of(time_each_launch(step, args.steps, stream), bytes_per_launch)
+    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(
+        args.workload if args.op == "forward" else f"{args.workload}:{args.op}")
+    roofline["back_to_back_us_per_launch"] = device_ms / args.steps * 1e3
+    headline = args.workload == "cfg3" and args.op == "forward" and args.rotate_mb == 0
 
     result = {
         "metric": "points/sec + achieved HBM GB/s (% peak), l_max=6 fp32 w/ gradients, 1M pts"
@@ -348,19 +466,9 @@ def main():
             "derivatives": w.derivatives,
             "harmonics": "spherical" if w.normalized else "solid",
             "seed": w.seed,
+            "kernels": prepared.kernels() if args.op == "forward" else None,
         },
-        "roofline": {
-            "bound": "hbm",
-            "achieved": achieved,
-            "peak": PEAK_HBM_GBPS,
-            "unit": "GB/s",
-            "frac": achieved / PEAK_HBM_GBPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload if args.op == "forward" else f"{args.workload}:{args.op}"),
-            "algorithmic_bytes_per_launch": bytes_per_launch,
-            "avg_launch_us": avg_launch_s * 1e6,
-            "median_launch_us": statistics.median(launch_ms) * 1e3,
-            "min_launch_us": min(launch_ms) * 1e3,
-        },
+        "roofline": roofline,
     }
     if not args.no_cpu_baseline:
         if args.op == "forward":
@@ -369,6 +477,20 @@ def main():
             result["cpu_baseline"] = cpu_vjp_baseline(w, xyz_host, sph_grad.cpu().numpy())
         else:
             result["cpu_baseline"] = cpu_backward_baseline(dsph.cpu().numpy(), sph_grad.cpu().numpy())
+    if headline and not args.no_by_config:
+        cold = Prepared(lib, w, rotate_mb=1024)
+        settle(cold.step, args.settle_seconds, 10)
+        r = roofline_of(time_each_launch(cold.step, max(args.steps, 50), cold.stream), cold.bytes_per_launch)
+        result["roofline"]["cold"] = {
+            "rotate_mb": 1024, "output_buffers": len(cold.outputs), "avg_launch_us": r["avg_launch_us"],
+            "min_launch_us": r["min_launch_us"], "achieved": r["achieved"], "frac": r["frac"],
+        }
+        del cold, prepared, sph, dsph, ddsph
+        torch.cuda.empty_cache()
+        result["roofline_by_config"] = {
+            name: measure_config(lib, name, args.steps, args.settle_seconds, with_cold=name in ("cfg1", "cfg2"))
+            for name in ("cfg1", "cfg2", "cfg4", "cfg5")
+        }
     print(json.dumps(result))
     return 0
 

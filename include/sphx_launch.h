@@ -124,9 +124,10 @@ SPHX_EXPORT int sphx_vjp_f64(const double* xyz, const double* sph_grad, size_t n
  *   workspace        device memory, 16-byte aligned, of workspace_bytes bytes;
  *                    the points are processed in chunks of as many as it holds
  *                    (8 * (3 + (l_max+1)^2 * {1, 4, 13}) bytes each), enqueued
- *                    one after the other on `stream`. NULL: the call allocates
- *                    a workspace of its own (at most 256 MiB), waits for the
- *                    stream and frees it, i.e. it is then synchronous.
+ *                    one after the other on `stream`. NULL: the call takes a
+ *                    workspace of at most 256 MiB from the device's memory
+ *                    pool and returns it, both in stream order
+ *                    (hipMallocAsync / hipFreeAsync): it still only enqueues.
  *
  * sphx_forward_f32_via_f64_workspace returns the size with which n_samples
  * points are one chunk (0 for invalid arguments). Costs the float64 evaluation
@@ -161,6 +162,24 @@ SPHX_EXPORT const char* sphx_last_error(void);
  * (its geometry is fixed at 8 x 8 threads, sphericart/src/cuda_base.cpp:89-94). */
 SPHX_EXPORT int sphx_plan(size_t n_samples, int l_max, int derivatives, int is_f64,
                           int* tile_samples, int* threads, int* lds_bytes, int* workgroups);
+
+/* The same as text: the kernel or kernels a call of this shape launches, with
+ * their template arguments as a profiler prints them, and the geometry of each
+ * launch. At most `capacity` bytes are written, NUL included. For benchmark
+ * records; no counterpart in the reference. */
+SPHX_EXPORT int sphx_describe_plan(size_t n_samples, int l_max, int derivatives, int is_f64,
+                                   int normalized, char* out, size_t capacity);
+
+/* Override one decision of the launch planner, for measurements and for tests
+ * that want both sides of a choice exercised: `name` is one of the SPHX_*
+ * names listed in sphx_kernels.hip (SPHX_TILE, SPHX_JOB_LIST, ...), unknown
+ * names return SPHX_ERR_ARGUMENT. Process-wide; takes effect with the next
+ * call on any thread. sphx_reset_switches() drops all overrides. Without
+ * overrides a call is planned from its shape alone. The environment variables
+ * of the same names are read once, when the library is first used, and only if
+ * SPHX_DEBUG_SWITCHES is set. No counterpart in the reference. */
+SPHX_EXPORT int sphx_set_switch(const char* name, int value);
+SPHX_EXPORT void sphx_reset_switches(void);
 
 #ifdef __cplusplus
 }

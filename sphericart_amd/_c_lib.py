@@ -37,6 +37,9 @@ LAUNCH_SYMBOLS = [
     "sphx_device_count",
     "sphx_last_error",
     "sphx_plan",
+    "sphx_describe_plan",
+    "sphx_set_switch",
+    "sphx_reset_switches",
 ]
 
 
@@ -79,6 +82,12 @@ def _declare(lib):
         c_void_p, c_size_t, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]
     lib.sphx_forward_f32_via_f64_workspace.restype = c_size_t
     lib.sphx_forward_f32_via_f64_workspace.argtypes = [c_size_t, c_int, c_int]
+    lib.sphx_describe_plan.restype = c_int
+    lib.sphx_describe_plan.argtypes = [c_size_t, c_int, c_int, c_int, c_int, ctypes.c_char_p, c_size_t]
+    lib.sphx_set_switch.restype = c_int
+    lib.sphx_set_switch.argtypes = [ctypes.c_char_p, c_int]
+    lib.sphx_reset_switches.restype = None
+    lib.sphx_reset_switches.argtypes = []
     lib.sphx_device_count.restype = c_int
     lib.sphx_device_count.argtypes = []
     lib.sphx_last_error.restype = ctypes.c_char_p

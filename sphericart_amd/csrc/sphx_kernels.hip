@@ -31,6 +31,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <atomic>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -92,16 +93,70 @@ static int ensure_device_ready(int device) {
     int lds = 0, cus = 0;
     SPHX_HIP(hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device));
     SPHX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+    // The kernels deal their workgroups to eight XCDs (`blockIdx.x & 7`): on a device partitioned
+    // otherwise the results would still be right but every XCD would write all over the outputs.
+    // Said once, not enforced; a runtime that does not know the attribute is left alone.
+    int xcds = 0;
+    if (hipDeviceGetAttribute(&xcds, hipDeviceAttributeNumberOfXccs, device) != hipSuccess) {
+        (void)hipGetLastError();
+    } else if (xcds != 8 && xcds > 0) {
+        std::fprintf(stderr,
+                     "sphericart_amd: device %d reports %d XCDs; the kernels' workgroup order is laid out "
+                     "for the 8 XCDs of an MI355X in SPX mode and will be slower here\n",
+                     device, xcds);
+    }
     g_lds_limit[device] = lds;
     g_compute_units[device] = cus;
     g_tables_ready[device] = true;
     return SPHX_OK;
 }
 
-static int env_int(const char* name, int fallback) {
-    const char* v = std::getenv(name);
-    if (!v || !*v) return fallback;
-    return std::atoi(v);
+// Overrides of single planning decisions, for measurements and tests (sphx_set_switch). None is
+// set in normal use: a call is then planned from its shape alone and no environment variable is
+// looked at. The variables of the same names are read once, when the library is first used, and
+// only if SPHX_DEBUG_SWITCHES is set to something other than 0.
+enum Switch : int {
+    SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_FLUSH_WAVES, SW_GRADIENT_LANES, SW_GRADIENT_LANES_TILE,
+    SW_GRADIENT_LANES_WAVES, SW_HESSIAN_LANES, SW_JOB_LIST, SW_PREFIX_INSIDE, SW_ROW_BUFFERS,
+    SW_SEQUENCE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_TILE, SW_TILE_LDS_BUDGET,
+    SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
+    SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_COUNT
+};
+static const char* const kSwitchNames[SW_COUNT] = {
+    "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_FLUSH_WAVES", "SPHX_GRADIENT_LANES",
+    "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_HESSIAN_LANES", "SPHX_JOB_LIST",
+    "SPHX_PREFIX_INSIDE", "SPHX_ROW_BUFFERS", "SPHX_SEQUENCE_WAVES", "SPHX_SPLIT_BELOW",
+    "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
+    "SPHX_TILE_SMALL_N", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
+    "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE",
+};
+struct Switches {
+    bool set[SW_COUNT] = {};
+    int value[SW_COUNT] = {};
+};
+static std::mutex g_switch_mutex;
+static Switches g_switches;                       // guarded by g_switch_mutex
+static std::atomic<unsigned> g_switch_generation{1}; // bumped whenever g_switches changes
+static std::once_flag g_switch_env_once;
+
+static void read_switches_from_environment() {
+    const char* debug = std::getenv("SPHX_DEBUG_SWITCHES");
+    if (!debug || !*debug || std::strcmp(debug, "0") == 0) return;
+    std::lock_guard<std::mutex> lock(g_switch_mutex);
+    for (int i = 0; i < SW_COUNT; ++i) {
+        const char* v = std::getenv(kSwitchNames[i]);
+        if (v && *v) {
+            g_switches.set[i] = true;
+            g_switches.value[i] = std::atoi(v);
+        }
+    }
+    g_switch_generation.fetch_add(1);
+}
+
+// The overrides as a planning call sees them: a copy taken once per plan.
+static thread_local Switches t_switches;
+static int switch_or(Switch which, int fallback) {
+    return t_switches.set[which] ? t_switches.value[which] : fallback;
 }
 
 struct Launch {
@@ -168,7 +223,7 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // against 546); in float64 the values kernel still wins with a whole CU's LDS (l_max = 18,
     // 20, 22: 426, 401, 380 against 483, 436, 429).
     unsigned allowed = static_cast<unsigned>(
-        env_int("SPHX_VALUES_LDS", with_sums || elem == 8 ? 160 * 1024 : 80 * 1024));
+        switch_or(SW_VALUES_LDS, with_sums || elem == 8 ? 160 * 1024 : 80 * 1024));
     if (allowed > static_cast<unsigned>(lds_limit)) allowed = static_cast<unsigned>(lds_limit);
     // Fewer than 64 points per workgroup leave lanes idle: with 32 the values kernel still beats
     // the recursion kernel (l_max = 32 float32, 500k points: 781 against 1 077 us; l_max = 20
@@ -177,7 +232,7 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // it goes down to 8 points (l_max = 24 float64, 200k points: 830 us with 16 points per
     // workgroup against 1 456 us through the recursion kernel).
     const unsigned smallest = static_cast<unsigned>(
-        with_sums ? env_int("SPHX_VJP_MIN_TILE", 8) : env_int("SPHX_VALUES_MIN_TILE", 32));
+        with_sums ? switch_or(SW_VJP_MIN_TILE, 8) : switch_or(SW_VALUES_MIN_TILE, 32));
     // Two workgroups per CU (80 KB each) overlap one's tables and flush with the other's
     // arithmetic: preferred, also at half the lanes, over one workgroup with all of LDS
     // (l_max = 16 float32, 500k points: 142 against 164 us; l_max = 12 float64: 115 against 146).
@@ -208,7 +263,7 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     g.off_Q = g.off_F + tri_all;
     out->workgroups = g.tiles_per_xcd * 8u;
     // one wave per l channel above the closed forms, eight at most
-    int waves = env_int("SPHX_VALUES_WAVES", 8);
+    int waves = switch_or(SW_VALUES_WAVES, 8);
     waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
     // (the product's closed-form slices want at least four; values: one for the tables, one for
     // the closed forms)
@@ -217,7 +272,7 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // four waves, 207, 282 with three (float64 279, 333 against 233, 304); l_max = 12 350 with six,
     // 316 with four (float64 385 against 321); one or two channels are best with four
     if (with_sums) want = want <= 2 ? 4 : (want <= 4 ? 3 : (want <= 6 ? 4 : want));
-    if (!with_sums && want < 2) want = env_int("SPHX_VALUES_MIN_WAVES", 2);
+    if (!with_sums && want < 2) want = switch_or(SW_VALUES_MIN_WAVES, 2);
     out->threads = 64u * static_cast<unsigned>(want < waves ? want : waves);
     out->lds_bytes = bytes;
     return true;
@@ -250,7 +305,7 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
         const unsigned b = (ot + t * table_stride) * esize;
         if (b > limit) continue;
         unsigned score = (limit / b) * t * (t >= 32 ? 4u : 3u);
-        if (static_cast<unsigned>(env_int("SPHX_GRADIENT_LANES_TILE", 0)) == t) score = 1u << 30;
+        if (static_cast<unsigned>(switch_or(SW_GRADIENT_LANES_TILE, 0)) == t) score = 1u << 30;
         if (score > best || (score == best && best_groups < 2)) {
             best = score;
             best_groups = limit / b;
@@ -278,7 +333,7 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     // are enough and leave room for more workgroups (1.5 GB of output: float64 l_max = 8 469 us
     // with eight waves, 345 with four; float32 l_max = 7, 8 286, 274 against 273, 261; from three
     // channels on eight waves are faster, l_max = 12: 357 against 411).
-    int waves = env_int("SPHX_GRADIENT_LANES_WAVES", l_max <= 8 ? 4 : 8);
+    int waves = switch_or(SW_GRADIENT_LANES_WAVES, l_max <= 8 ? 4 : 8);
     waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
     out->threads = 64u * static_cast<unsigned>(waves);
     out->lds_bytes = bytes;
@@ -359,7 +414,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     for (int l = hard + 1; l <= l_max; ++l) jobs += l + 1;
     // with the sides split every (l, m > 0) pair is two jobs; the job table is sized for that
     const unsigned jobs_split = 2 * jobs - static_cast<unsigned>(l_max - hard);
-    bool may_split = mode == 2 && env_int("SPHX_SPLIT_SIDES", 1) != 0;
+    bool may_split = mode == 2 && switch_or(SW_SPLIT_SIDES, 1) != 0;
     auto table_elems_for = [&](bool split) { return ((split ? jobs_split : jobs) * 4 + esize - 1) / esize; };
     // per point: the rows in every row buffer, point tables three times, iterates twice
     // staged rows are `row_stride` apart (recursion_kernel): nrow, or a little more when the rows
@@ -384,7 +439,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // the flush of such a tile is long: measured with second derivatives (l_max = 16, float64:
     // 770 us against 810 us). With many points per tile, or with the rows cut in two kernels,
     // one buffer flushed by all waves measured faster.
-    int want_buffers = env_int("SPHX_ROW_BUFFERS", 0);
+    int want_buffers = switch_or(SW_ROW_BUFFERS, 0);
     if (want_buffers == 0) {
         const unsigned single = bytes_for(1, 1) <= budget
                                     ? (budget / esize - fixed) / (rows_per_point + rest_per_point)
@@ -402,7 +457,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         // with 6; second derivatives, float64 l_max = 12: 783 with 2, 547 with 3; never more
         // than 4 % slower than the power of two below)
         S = (budget / esize - fixed) / (buffers * rows_per_point + rest_per_point);
-        if (env_int("SPHX_TILE_POW2", 0) != 0) S = pow2_floor(S);
+        if (switch_or(SW_TILE_POW2, 0) != 0) S = pow2_floor(S);
         if (S > 64) S = 64;
     }
     // Few points: with the largest tile there would be fewer tiles than workgroups that a launch
@@ -410,7 +465,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // values and gradients four points at least: below that the closed forms of l <= 6 weigh
     // too much). 500 points, us: second derivatives float64 l_max = 6 16.1 -> 10.2, l_max = 16
     // 16.6 -> 12.6, float32 l_max = 12 17.5 -> 11.2; gradients float32 l_max = 20 23.9 -> 12.7.
-    if (S > 1 && env_int("SPHX_TILE_SMALL_N", 1) != 0) {
+    if (S > 1 && switch_or(SW_TILE_SMALL_N, 1) != 0) {
         unsigned per_cu = limit / bytes_for(S, buffers);
         per_cu = per_cu < 1 ? 1u : (per_cu > 2 ? 2u : per_cu);
         if (mode == 2 && elem == 8) per_cu = 1; // more than 128 registers per lane
@@ -422,7 +477,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
             if (enough < S) S = static_cast<unsigned>(enough);
         }
     }
-    const int forced = env_int("SPHX_TILE", 0);
+    const int forced = switch_or(SW_TILE, 0);
     if (forced > 0 && forced <= 64 && bytes_for(forced, buffers) <= limit) {
         S = static_cast<unsigned>(forced);
     }
@@ -434,7 +489,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     unsigned az_shift = 0;
     {
         const unsigned allowed = bytes_for(S, buffers) > budget ? bytes_for(S, buffers) : budget;
-        const int cap = env_int("SPHX_AZ_SHIFT", 3);
+        const int cap = switch_or(SW_AZ_SHIFT, 3);
         for (unsigned shift = cap < 0 ? 0u : (cap > 6 ? 6u : static_cast<unsigned>(cap)); shift >= 1; --shift) {
             const unsigned tiles = 1u << shift;
             if (tiles * S > 64) continue;
@@ -453,7 +508,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.tile = static_cast<int>(S);
     g.az_shift = az_shift;
     g.row_buffers = buffers;
-    g.flush_waves = buffers == 2 ? static_cast<unsigned>(env_int("SPHX_FLUSH_WAVES", 1)) : 0u;
+    g.flush_waves = buffers == 2 ? static_cast<unsigned>(switch_or(SW_FLUSH_WAVES, 1)) : 0u;
     if (g.flush_waves > 2) g.flush_waves = 2;
     if (buffers == 2 && g.flush_waves < 1) g.flush_waves = 1;
     g.sequence_waves = S * arrays * static_cast<unsigned>(l_max - hard) > 64 ? 2u : 1u;
@@ -466,7 +521,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // 460). For solid harmonics in float32 both fit twice (119 and 88 registers) and the rule
     // holds (l_max = 10: 319 us by the rule, 404 always split; l_max = 12: 327 against 399);
     // float64 with the sides always split loses 10-20 % at most l_max.
-    const unsigned one_side_costs = static_cast<unsigned>(env_int("SPHX_SPLIT_RATIO", elem == 4 && normalized ? 1 : 6));
+    const unsigned one_side_costs = static_cast<unsigned>(switch_or(SW_SPLIT_RATIO, elem == 4 && normalized ? 1 : 6));
     unsigned wide = 0;
     auto per_pass = [&](unsigned j) { return j >= wide ? 1u : wide / j; };
     // rounds of the entry lanes per tile: whole points side by side, or (fewer, where the
@@ -500,7 +555,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         if (mode == 0 || with_one < with_two) g.sequence_waves = 1;
     }
     {
-        const int forced_seq = env_int("SPHX_SEQUENCE_WAVES", 0);
+        const int forced_seq = switch_or(SW_SEQUENCE_WAVES, 0);
         if (forced_seq >= 1 && forced_seq <= 4) g.sequence_waves = static_cast<unsigned>(forced_seq);
     }
     entry_cost(g.sequence_waves, split_sides); // leaves `wide` as it will be
@@ -512,7 +567,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // float64 l_max = 14: 580 -> 426; with equal rounds, l_max = 32: 390 -> 423). It did not pay
     // with two points per tile (l_max = 32, three rounds instead of four: 387 -> 424 us) nor
     // where four points go side by side anyway (second derivatives float32 l_max = 8: 580 -> 631).
-    const int want_list = env_int("SPHX_JOB_LIST", -1);
+    const int want_list = switch_or(SW_JOB_LIST, -1);
     const bool saves_a_round = (S * g.jobs_per_point + wide - 1) / wide < rounds_by_point(g.jobs_per_point);
     if (want_list != 0 && saves_a_round && (want_list > 0 || (S >= 3 && g.points_per_pass <= 2))) {
         g.points_per_pass = 0;
@@ -552,7 +607,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // l_max = 8, 14 points, 632 against 561 for single tiles; cfg4 562 against 528).
     g.chunk_shift = 0;
     if (whole && S * nrow * esize >= 128u) {
-        const int want = env_int("SPHX_CHUNK_SHIFT", S >= 5 ? 0 : (S >= 3 ? 1 : (S == 2 ? 2 : 3)));
+        const int want = switch_or(SW_CHUNK_SHIFT, S >= 5 ? 0 : (S >= 3 ? 1 : (S == 2 ? 2 : 3)));
         g.chunk_shift = want < 0 ? 0u : (want > 10 ? 10u : static_cast<unsigned>(want));
     }
     unsigned per_cu = limit / out->lds_bytes;
@@ -585,6 +640,18 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
         return fail(SPHX_ERR_UNSUPPORTED, "too many samples for one launch");
     }
     const int hard = mode == 2 ? 1 : 6;
+    // The fused product contracts the staged rows in place of the flush and has one row buffer
+    // only: an override that asks for two is not for it (the flush stage of the two-buffer loop
+    // would write through the pointer that holds the caller's sph_grad).
+    struct WithoutRowBuffers {
+        bool active, saved;
+        explicit WithoutRowBuffers(bool on) : active(on), saved(t_switches.set[SW_ROW_BUFFERS]) {
+            if (active) t_switches.set[SW_ROW_BUFFERS] = false;
+        }
+        ~WithoutRowBuffers() {
+            if (active) t_switches.set[SW_ROW_BUFFERS] = saved;
+        }
+    } without_row_buffers(!lane_kernels);
     plan->lanes = false;
     plan->closed_only = l_max <= hard;
     plan->whole = true;
@@ -599,14 +666,14 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     }
     // Second derivatives at small l_max: one point per lane where that was measured to be faster
     // than the recursion kernel (SPHX_HESSIAN_LANES: 0 never, 2 wherever the rows fit).
-    const int hessian_lanes = env_int("SPHX_HESSIAN_LANES", 1);
+    const int hessian_lanes = switch_or(SW_HESSIAN_LANES, 1);
     const bool hessian_lanes_pay = elem == 4 ? l_max <= 5 : (l_max == 3 || (l_max == 5 && normalized));
     if (lane_kernels && mode == 2 && (hessian_lanes == 2 || (hessian_lanes == 1 && hessian_lanes_pay)) &&
         plan_hessian_lanes(n_samples, l_max, elem, lds_limit, &plan->closed)) {
         plan->lanes = true;
         return SPHX_OK;
     }
-    if (lane_kernels && mode == 1 && env_int("SPHX_GRADIENT_LANES", 1) != 0 &&
+    if (lane_kernels && mode == 1 && switch_or(SW_GRADIENT_LANES, 1) != 0 &&
         plan_gradient_lanes(n_samples, l_max, elem, lds_limit, &plan->closed)) {
         plan->lanes = true;
         return SPHX_OK;
@@ -618,7 +685,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // 479, l_max = 12: 545 -> 468; solid harmonics l_max = 4-12: 10-20 % less, l_max = 16, 100k
     // points: 580 -> 560).
     const int whole_cu = mode == 2 && elem == 8 ? lds_limit : 80 * 1024;
-    const unsigned budget = static_cast<unsigned>(env_int("SPHX_TILE_LDS_BUDGET", whole_cu));
+    const unsigned budget = static_cast<unsigned>(switch_or(SW_TILE_LDS_BUDGET, whole_cu));
     bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
                                &plan->split_sides, normalized);
     // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of
@@ -640,7 +707,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // 393, 407, 373, 399 us against 431, 451, 419, 424; l_max = 28, 30 (3) 396, 371 against 532,
     // 510; l_max = 32 (2) 462 against 389. Float32 gradients are therefore cut below three
     // points per tile only; values below eight, float64 gradients below four as before.)
-    const int split_below = env_int("SPHX_SPLIT_BELOW", mode == 0 ? 8 : (elem == 4 ? 3 : 4));
+    const int split_below = switch_or(SW_SPLIT_BELOW, mode == 0 ? 8 : (elem == 4 ? 3 : 4));
     const bool cut = plan->rec.g.tile < split_below;
     if (mode < 2 && (!fits || cut)) {
         Launch upper;
@@ -648,7 +715,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
                            &plan->split_sides)) {
             plan->whole = false;
             plan->rec = upper;
-            plan->rec.g.prefix_inside = lane_kernels && env_int("SPHX_PREFIX_INSIDE", 1) != 0 ? 1u : 0u;
+            plan->rec.g.prefix_inside = lane_kernels && switch_or(SW_PREFIX_INSIDE, 1) != 0 ? 1u : 0u;
             plan_closed(n_samples, l_max, hard, mode, elem, &plan->closed);
             fits = true;
         }
@@ -844,6 +911,90 @@ static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* d
     return hipErrorInvalidValue;
 }
 
+// What a call of a given shape launches, kept per thread so that a steady stream of equal calls
+// plans once: planning is a few hundred host instructions and, with overrides, a lock.
+struct PlannedCall {
+    // key
+    unsigned generation = 0; // of the overrides; 0 = empty slot
+    int kind = 0;            // 0: forward, 1: fused product
+    size_t n_samples = 0;
+    int l_max = 0, mode = 0, elem = 0, normalized = 0, device = 0;
+    // what was planned
+    Plan plan;
+    Launch lanes;         // fused product beyond l_max = 6: the lane kernels' launch
+    bool use_lanes = false;
+    bool lane_groups = false;
+};
+constexpr int kPlannedCalls = 16;
+static thread_local PlannedCall t_planned[kPlannedCalls];
+static thread_local unsigned t_planned_next = 0;
+static thread_local unsigned t_switches_generation = 0;
+
+// The slot for this shape; `*fresh` says that it has yet to be planned (by the caller, who then
+// sets `generation`; a failed plan leaves the slot empty).
+static PlannedCall* planned_call(int kind, size_t n_samples, int l_max, int mode, int elem,
+                                 int normalized, int device, bool* fresh) {
+    std::call_once(g_switch_env_once, read_switches_from_environment);
+    const unsigned generation = g_switch_generation.load(std::memory_order_acquire);
+    if (t_switches_generation != generation) {
+        std::lock_guard<std::mutex> lock(g_switch_mutex);
+        t_switches = g_switches;
+        t_switches_generation = g_switch_generation.load();
+    }
+    for (PlannedCall& c : t_planned) {
+        if (c.generation == t_switches_generation && c.kind == kind && c.n_samples == n_samples &&
+            c.l_max == l_max && c.mode == mode && c.elem == elem && c.normalized == normalized &&
+            c.device == device) {
+            *fresh = false;
+            return &c;
+        }
+    }
+    PlannedCall* c = &t_planned[t_planned_next++ % kPlannedCalls];
+    c->generation = 0;
+    c->kind = kind;
+    c->n_samples = n_samples;
+    c->l_max = l_max;
+    c->mode = mode;
+    c->elem = elem;
+    c->normalized = normalized;
+    c->device = device;
+    c->use_lanes = c->lane_groups = false;
+    *fresh = true;
+    return c;
+}
+
+// The evaluation proper, on `device`, which is the current one.
+template <typename T>
+static int forward_on(int device, const T* xyz, size_t n_samples, int l_max, int normalized, int mode,
+                      T* sph, T* dsph, T* ddsph, void* stream) {
+    int status = ensure_device_ready(device);
+    if (status != SPHX_OK) return status;
+    bool fresh = false;
+    PlannedCall* call = planned_call(0, n_samples, l_max, mode, sizeof(T), normalized != 0, device, &fresh);
+    if (fresh) {
+        status = make_plan(n_samples, l_max, mode, sizeof(T), g_lds_limit[device],
+                           g_compute_units[device], &call->plan, true, normalized != 0);
+        if (status != SPHX_OK) return status;
+        call->generation = t_switches_generation;
+    }
+    const Plan& plan = call->plan;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (normalized) {
+        e = mode == 0   ? dispatch<T, 0, true>(plan, xyz, sph, dsph, ddsph, s)
+            : mode == 1 ? dispatch<T, 1, true>(plan, xyz, sph, dsph, ddsph, s)
+                        : dispatch<T, 2, true>(plan, xyz, sph, dsph, ddsph, s);
+    } else {
+        e = mode == 0   ? dispatch<T, 0, false>(plan, xyz, sph, dsph, ddsph, s)
+            : mode == 1 ? dispatch<T, 1, false>(plan, xyz, sph, dsph, ddsph, s)
+                        : dispatch<T, 2, false>(plan, xyz, sph, dsph, ddsph, s);
+    }
+    if (e != hipSuccess) {
+        return fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
+    }
+    return SPHX_OK;
+}
+
 template <typename T>
 static int forward(const T* xyz, size_t n_samples, int l_max, int normalized, int mode, T* sph,
                    T* dsph, T* ddsph, void* stream) {
@@ -866,28 +1017,7 @@ static int forward(const T* xyz, size_t n_samples, int l_max, int normalized, in
         SPHX_HIP(hipSetDevice(device));
     }
 
-    int status = ensure_device_ready(device);
-    Plan plan;
-    if (status == SPHX_OK) {
-        status = make_plan(n_samples, l_max, mode, sizeof(T), g_lds_limit[device],
-                           g_compute_units[device], &plan, true, normalized != 0);
-    }
-    if (status == SPHX_OK) {
-        hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-        hipError_t e;
-        if (normalized) {
-            e = mode == 0   ? dispatch<T, 0, true>(plan, xyz, sph, dsph, ddsph, s)
-                : mode == 1 ? dispatch<T, 1, true>(plan, xyz, sph, dsph, ddsph, s)
-                            : dispatch<T, 2, true>(plan, xyz, sph, dsph, ddsph, s);
-        } else {
-            e = mode == 0   ? dispatch<T, 0, false>(plan, xyz, sph, dsph, ddsph, s)
-                : mode == 1 ? dispatch<T, 1, false>(plan, xyz, sph, dsph, ddsph, s)
-                            : dispatch<T, 2, false>(plan, xyz, sph, dsph, ddsph, s);
-        }
-        if (e != hipSuccess) {
-            status = fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
-        }
-    }
+    int status = forward_on<T>(device, xyz, n_samples, l_max, normalized, mode, sph, dsph, ddsph, stream);
 
     if (device != current) {
         hipError_t e = hipSetDevice(current);
@@ -966,24 +1096,37 @@ static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int
         SPHX_HIP(hipSetDevice(device));
     }
     int status = ensure_device_ready(device);
-    Plan plan;
-    Launch lanes;
-    bool use_lanes = false;
+    if (status == SPHX_OK && l_max > SPHX_TABLE_LMAX) {
+        status = fail(SPHX_ERR_UNSUPPORTED, "l_max = " + std::to_string(l_max) +
+                                                " exceeds the device prefactor tables (" +
+                                                std::to_string(SPHX_TABLE_LMAX) + ")");
+    }
+    const PlannedCall* planned = nullptr;
     if (status == SPHX_OK) {
-        if (l_max > SPHX_TABLE_LMAX) {
-            status = fail(SPHX_ERR_UNSUPPORTED, "l_max = " + std::to_string(l_max) +
-                                                    " exceeds the device prefactor tables (" +
-                                                    std::to_string(SPHX_TABLE_LMAX) + ")");
-        } else if (l_max > 6 && env_int("SPHX_VJP_LANES", 1) != 0) {
-            use_lanes = plan_values(n_samples, l_max, sizeof(T), g_lds_limit[device], &lanes, true);
+        bool fresh = false;
+        PlannedCall* call = planned_call(1, n_samples, l_max, 1, sizeof(T), normalized != 0, device, &fresh);
+        if (fresh) {
+            if (l_max > 6 && switch_or(SW_VJP_LANES, 1) != 0) {
+                call->use_lanes = plan_values(n_samples, l_max, sizeof(T), g_lds_limit[device], &call->lanes, true);
+                // groups of lanes with channels of their own pay off from tiles of 16 points down
+                // (200k points, float32 l_max = 24: 225 against 279 us; float64 l_max = 24: 665
+                // against 866; with tiles of 32 the scalar-unit kernel is ahead, float64 l_max = 12:
+                // 329 against 397)
+                call->lane_groups = call->use_lanes && call->lanes.g.tile <= switch_or(SW_VJP_GROUPS_BELOW, 16);
+            }
+            if (!call->use_lanes) {
+                // the closed-form or the recursion kernels with the contraction in place of the flush
+                status = make_plan(n_samples, l_max, 1, sizeof(T), g_lds_limit[device], g_compute_units[device],
+                                   &call->plan, false);
+            }
+            if (status == SPHX_OK) call->generation = t_switches_generation;
         }
-    }
-    if (status == SPHX_OK && !use_lanes) {
-        // the closed-form or the recursion kernels with the contraction in place of the flush
-        status = make_plan(n_samples, l_max, 1, sizeof(T), g_lds_limit[device], g_compute_units[device],
-                           &plan, false);
+        planned = call;
     }
     if (status == SPHX_OK) {
+        const Plan& plan = planned->plan;
+        const Launch& lanes = planned->lanes;
+        const bool use_lanes = planned->use_lanes;
         hipStream_t s = reinterpret_cast<hipStream_t>(stream);
         hipError_t e;
         if (use_lanes) {
@@ -998,11 +1141,7 @@ static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int
                                    lanes.g, xyz, sph_grad, xyz_grad, accumulate);
                 return hipGetLastError();
             };
-            // groups of lanes with channels of their own pay off from tiles of 16 points down
-            // (200k points, float32 l_max = 24: 225 against 279 us; float64 l_max = 24: 665
-            // against 866; with tiles of 32 the scalar-unit kernel is ahead, float64 l_max = 12:
-            // 329 against 397)
-            if (lanes.g.tile > env_int("SPHX_VJP_GROUPS_BELOW", 16)) {
+            if (!planned->lane_groups) {
                 e = normalized ? launch(vjp_lanes_kernel<T, true>) : launch(vjp_lanes_kernel<T, false>);
             } else {
                 e = normalized ? launch(vjp_groups_kernel<T, true>) : launch(vjp_groups_kernel<T, false>);
@@ -1068,11 +1207,8 @@ static size_t via_f64_bytes_per_point(int l_max, int mode) {
     return sizeof(double) * (3 + ny * components_of(mode));
 }
 
-static int forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, int normalized, int mode,
-                               float* sph, float* dsph, float* ddsph, void* workspace,
-                               size_t workspace_bytes, void* stream) {
-    t_error.clear();
-    if (n_samples == 0) return SPHX_OK;
+static int check_via_f64_arguments(const float* xyz, int l_max, int mode, const float* sph,
+                                   const float* dsph, const float* ddsph) {
     if (l_max < 0) return fail(SPHX_ERR_ARGUMENT, "l_max must be non-negative");
     if (mode < 0 || mode > 2) return fail(SPHX_ERR_ARGUMENT, "unknown derivative selector");
     if (l_max > SPHX_TABLE_LMAX) {
@@ -1084,38 +1220,24 @@ static int forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, in
     if (sph == nullptr) return fail(SPHX_ERR_ARGUMENT, "sph is a null pointer");
     if (mode >= 1 && dsph == nullptr) return fail(SPHX_ERR_ARGUMENT, "dsph is a null pointer");
     if (mode >= 2 && ddsph == nullptr) return fail(SPHX_ERR_ARGUMENT, "ddsph is a null pointer");
+    return SPHX_OK;
+}
 
-    hipPointerAttribute_t attr;
-    SPHX_HIP(hipPointerGetAttributes(&attr, xyz));
-    int current = 0;
-    SPHX_HIP(hipGetDevice(&current));
-    const int device = attr.device;
-    if (device != current) SPHX_HIP(hipSetDevice(device));
-
+// The points in chunks of as many as the workspace holds: widen, evaluate in float64, narrow.
+// `device` is current. Enqueues only.
+static int via_f64_chunks(int device, const float* xyz, size_t n_samples, int l_max, int normalized,
+                          int mode, float* sph, float* dsph, float* ddsph, void* workspace,
+                          size_t workspace_bytes, void* stream) {
     const size_t per_point = via_f64_bytes_per_point(l_max, mode);
     const size_t ny = static_cast<size_t>(l_max + 1) * (l_max + 1);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    int status = SPHX_OK;
-    void* owned = nullptr;
-    if (workspace == nullptr) {
-        // no workspace given: one of our own for at most 256 MiB worth of points at a time
-        size_t points = (size_t(256) << 20) / per_point;
-        if (points < 64) points = 64;
-        if (points > n_samples) points = n_samples;
-        workspace_bytes = points * per_point;
-        hipError_t e = hipMalloc(&owned, workspace_bytes);
-        if (e != hipSuccess) {
-            status = fail(SPHX_ERR_HIP, std::string("hipMalloc of the float64 workspace: ") + hipGetErrorString(e));
-        }
-        workspace = owned;
-    }
     size_t chunk = workspace_bytes / per_point;
-    if (status == SPHX_OK && chunk == 0) {
-        status = fail(SPHX_ERR_ARGUMENT, "the workspace holds no point: " + std::to_string(per_point) +
-                                             " bytes are needed per point");
+    if (chunk == 0) {
+        return fail(SPHX_ERR_ARGUMENT, "the workspace holds no point: " + std::to_string(per_point) +
+                                           " bytes are needed per point");
     }
-    if (status == SPHX_OK && (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
-        status = fail(SPHX_ERR_ARGUMENT, "the workspace must be aligned to 16 bytes");
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
+        return fail(SPHX_ERR_ARGUMENT, "the workspace must be aligned to 16 bytes");
     }
     if (chunk > n_samples) chunk = n_samples;
     if (chunk >= 64) chunk &= ~size_t(63); // whole tiles of the closed-form kernels
@@ -1124,13 +1246,14 @@ static int forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, in
     double* w_dsph = w_sph + chunk * ny;
     double* w_ddsph = w_dsph + (mode >= 1 ? chunk * 3 * ny : 0);
     double* w_xyz = w_ddsph + (mode >= 2 ? chunk * 9 * ny : 0);
-    for (size_t first = 0; status == SPHX_OK && first < n_samples; first += chunk) {
+    for (size_t first = 0; first < n_samples; first += chunk) {
         const size_t count = n_samples - first < chunk ? n_samples - first : chunk;
         hipLaunchKernelGGL(widen_kernel, dim3(convert_blocks(count * 3)), dim3(kConvertThreads), 0, s,
                            xyz + first * 3, w_xyz, static_cast<unsigned long long>(count * 3));
-        status = forward<double>(w_xyz, count, l_max, normalized, mode, w_sph, mode >= 1 ? w_dsph : nullptr,
-                                 mode >= 2 ? w_ddsph : nullptr, stream);
-        if (status != SPHX_OK) break;
+        const int status = forward_on<double>(device, w_xyz, count, l_max, normalized, mode, w_sph,
+                                              mode >= 1 ? w_dsph : nullptr, mode >= 2 ? w_ddsph : nullptr,
+                                              stream);
+        if (status != SPHX_OK) return status;
         hipLaunchKernelGGL(narrow_kernel, dim3(convert_blocks(count * ny)), dim3(kConvertThreads), 0, s,
                            w_sph, sph + first * ny, static_cast<unsigned long long>(count * ny));
         if (mode >= 1) {
@@ -1143,18 +1266,52 @@ static int forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, in
         }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) {
-            status = fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
+            return fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
         }
     }
-    if (owned != nullptr) {
-        // our own workspace: wait for the work that uses it, then give it back
-        hipError_t e = hipStreamSynchronize(s);
-        if (e != hipSuccess && status == SPHX_OK) {
-            status = fail(SPHX_ERR_HIP, std::string("hipStreamSynchronize: ") + hipGetErrorString(e));
+    return SPHX_OK;
+}
+
+static int forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, int normalized, int mode,
+                               float* sph, float* dsph, float* ddsph, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+    t_error.clear();
+    if (n_samples == 0) return SPHX_OK;
+    int status = check_via_f64_arguments(xyz, l_max, mode, sph, dsph, ddsph);
+    if (status != SPHX_OK) return status;
+
+    hipPointerAttribute_t attr;
+    SPHX_HIP(hipPointerGetAttributes(&attr, xyz));
+    int current = 0;
+    SPHX_HIP(hipGetDevice(&current));
+    const int device = attr.device;
+    if (device != current) SPHX_HIP(hipSetDevice(device));
+
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    void* owned = nullptr;
+    if (workspace == nullptr) {
+        // No workspace given: one of our own for at most 256 MiB worth of points at a time, taken
+        // from and returned to the device's memory pool in stream order, so that the call still
+        // only enqueues (an allocation that waits for the device would stall the caller).
+        const size_t per_point = via_f64_bytes_per_point(l_max, mode);
+        size_t points = (size_t(256) << 20) / per_point;
+        if (points < 64) points = 64;
+        if (points > n_samples) points = n_samples;
+        workspace_bytes = points * per_point;
+        hipError_t e = hipMallocAsync(&owned, workspace_bytes, s);
+        if (e != hipSuccess) {
+            status = fail(SPHX_ERR_HIP, std::string("hipMallocAsync of the float64 workspace: ") + hipGetErrorString(e));
         }
-        e = hipFree(owned);
+        workspace = owned;
+    }
+    if (status == SPHX_OK) {
+        status = via_f64_chunks(device, xyz, n_samples, l_max, normalized, mode, sph, dsph, ddsph, workspace,
+                                workspace_bytes, stream);
+    }
+    if (owned != nullptr) {
+        hipError_t e = hipFreeAsync(owned, s); // after the work enqueued above, in stream order
         if (e != hipSuccess && status == SPHX_OK) {
-            status = fail(SPHX_ERR_HIP, std::string("hipFree: ") + hipGetErrorString(e));
+            status = fail(SPHX_ERR_HIP, std::string("hipFreeAsync: ") + hipGetErrorString(e));
         }
     }
     if (device != current) {
@@ -1228,6 +1385,8 @@ int sphx_plan(size_t n_samples, int l_max, int derivatives, int is_f64, int* til
         (void)hipGetLastError();
     }
     sphx::Plan plan;
+    bool fresh = false; // only for the side effect: the overrides as this thread's plans see them
+    (void)sphx::planned_call(-1, 0, 0, 0, 0, 0, -1, &fresh);
     int status = sphx::make_plan(n_samples ? n_samples : 1, l_max, derivatives,
                                  is_f64 ? sizeof(double) : sizeof(float), lds, cus, &plan);
     if (status != SPHX_OK) return status;
@@ -1237,6 +1396,72 @@ int sphx_plan(size_t n_samples, int l_max, int derivatives, int is_f64, int* til
     if (lds_bytes) *lds_bytes = static_cast<int>(main.lds_bytes);
     if (workgroups) *workgroups = static_cast<int>(main.workgroups);
     return SPHX_OK;
+}
+
+int sphx_describe_plan(size_t n_samples, int l_max, int derivatives, int is_f64, int normalized,
+                       char* out, size_t capacity) {
+    sphx::t_error.clear();
+    if (out == nullptr || capacity == 0) return sphx::fail(SPHX_ERR_ARGUMENT, "no room for the description");
+    int device = 0, lds = 160 * 1024, cus = 256;
+    if (hipGetDevice(&device) == hipSuccess) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, device) == hipSuccess && v > 0) lds = v;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
+    } else {
+        (void)hipGetLastError();
+    }
+    sphx::Plan plan;
+    bool fresh = false;
+    (void)sphx::planned_call(-1, 0, 0, 0, 0, 0, -1, &fresh);
+    const int status = sphx::make_plan(n_samples ? n_samples : 1, l_max, derivatives,
+                                       is_f64 ? sizeof(double) : sizeof(float), lds, cus, &plan, true,
+                                       normalized != 0);
+    if (status != SPHX_OK) return status;
+    const std::string t = is_f64 ? "double" : "float";
+    const std::string head = t + ", " + std::to_string(derivatives) + ", " + (normalized ? "true" : "false");
+    auto geometry = [](const sphx::Launch& l) {
+        return " [" + std::to_string(l.g.tile) + " points per tile, " + std::to_string(l.threads) + " threads, " +
+               std::to_string(l.lds_bytes) + " B LDS, " + std::to_string(l.workgroups) + " workgroups]";
+    };
+    std::string text;
+    if (plan.closed_only) {
+        text = "closed_form_kernel<" + head + ", " + std::to_string(l_max) + ", false>" + geometry(plan.closed);
+    } else if (plan.lanes) {
+        const char* names[3] = {"values_kernel", "gradients_lanes_kernel", "hessians_lanes_kernel"};
+        text = std::string(names[derivatives]) + "<" + t + ", " + (normalized ? "true" : "false") + ">" +
+               geometry(plan.closed);
+    } else {
+        if (!plan.whole && plan.rec.g.prefix_inside == 0) {
+            text = "closed_form_kernel<" + head + ", 6, true>" + geometry(plan.closed) + " + ";
+        }
+        text += "recursion_kernel<" + head + ", " + (plan.whole ? "true" : "false") + ", " +
+                (plan.split_sides ? "true" : "false") + ", false, " +
+                (plan.rec.g.points_per_pass == 0 ? "true" : "false") + ">" + geometry(plan.rec);
+    }
+    std::snprintf(out, capacity, "%s", text.c_str());
+    return SPHX_OK;
+}
+
+int sphx_set_switch(const char* name, int value) {
+    sphx::t_error.clear();
+    if (name != nullptr) {
+        for (int i = 0; i < sphx::SW_COUNT; ++i) {
+            if (std::strcmp(name, sphx::kSwitchNames[i]) == 0) {
+                std::lock_guard<std::mutex> lock(sphx::g_switch_mutex);
+                sphx::g_switches.set[i] = true;
+                sphx::g_switches.value[i] = value;
+                sphx::g_switch_generation.fetch_add(1);
+                return SPHX_OK;
+            }
+        }
+    }
+    return sphx::fail(SPHX_ERR_ARGUMENT, std::string("unknown switch: ") + (name ? name : "(null)"));
+}
+
+void sphx_reset_switches(void) {
+    std::lock_guard<std::mutex> lock(sphx::g_switch_mutex);
+    sphx::g_switches = sphx::Switches();
+    sphx::g_switch_generation.fetch_add(1);
 }
 
 } // extern "C"

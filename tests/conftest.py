@@ -51,6 +51,19 @@ def library():
     return _c_lib.get_library()
 
 
+@pytest.fixture
+def switches(library):
+    """Override planning decisions of the library for one test (sphx_set_switch); all overrides
+    are dropped afterwards."""
+
+    def set_switch(name, value):
+        assert library.sphx_set_switch(name.encode(), int(value)) == 0, library.sphx_last_error()
+
+    library.sphx_reset_switches()
+    yield set_switch
+    library.sphx_reset_switches()
+
+
 def same_numbers(a, b):
     """Element-wise identity as numbers: equal values (so -0.0 == 0.0) or NaN in both."""
     a = np.asarray(a)

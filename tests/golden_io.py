@@ -30,3 +30,22 @@ def edge_cases(tag):
                         for label in ("sph", "dsph", "ddsph")
                     )
                     yield xyz, l_max, normalized, mode, want
+
+
+DEGENERATE_L_MAX = (1, 6, 7, 11)
+
+
+def degenerate_cases(tag):
+    """Yield (xyz, degenerate_at, l_max, normalized, mode, (sph, dsph, ddsph)): points for which the
+    reference returns infinities and NaN, between ordinary ones."""
+    with np.load(os.path.join(GOLDEN, f"degenerate_{tag}.npz"), allow_pickle=False) as f:
+        xyz, where = f["xyz"], f["degenerate_at"]
+        for l_max in DEGENERATE_L_MAX:
+            for normalized in (True, False):
+                kind = "spherical" if normalized else "solid"
+                for mode in ("values", "gradients", "hessians"):
+                    want = tuple(
+                        f[key] if (key := f"{kind}_l{l_max}_{mode}_{label}") in f.files else None
+                        for label in ("sph", "dsph", "ddsph")
+                    )
+                    yield xyz, where, l_max, normalized, mode, want

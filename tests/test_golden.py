@@ -2,7 +2,7 @@
 
 import pytest
 
-from golden_io import CONFIGS, config_case, edge_cases
+from golden_io import CONFIGS, config_case, degenerate_cases, edge_cases
 from helpers import same_numbers
 
 
@@ -28,6 +28,29 @@ def test_oracle_on_edge_cases(oracle, tag):
                 assert same_numbers(g, w).all(), (l_max, normalized, mode)
         count += 1
     assert count == 36
+
+
+@pytest.mark.parametrize("tag", ["f32", "f64"])
+def test_oracle_on_degenerate_points(oracle, tag):
+    """The origin, NaN, infinite, denormal and overflowing coordinates: the restatement returns
+    what the compiled reference returns, NaN for NaN, signed infinity for signed infinity, and the
+    fixture does hold such numbers (the reference has no guard, templates.hpp:392-400)."""
+    import numpy as np
+
+    count = 0
+    for xyz, where, l_max, normalized, mode, want in degenerate_cases(tag):
+        with np.errstate(all="ignore"):
+            got = oracle.compute(xyz, l_max, normalized, mode)
+        for g, w in zip(got, want):
+            assert (g is None) == (w is None)
+            if w is not None:
+                assert same_numbers(g, w).all(), (l_max, normalized, mode)
+        ordinary = np.setdiff1d(np.arange(xyz.shape[0]), where)
+        assert np.isfinite(want[0][ordinary]).all()
+        if normalized:
+            assert np.isnan(want[0][where[0], 1:]).all()  # the origin: 0 * inf
+        count += 1
+    assert count == 24
 
 
 def test_cfg5_golden_holds_the_float_overflow(oracle):

@@ -106,11 +106,11 @@ def test_many_tiles_per_workgroup_with_shifted_outputs(oracle, library, shift):
 
 @pytest.mark.parametrize("route", ["lanes", "recursion"])
 @pytest.mark.parametrize("dtype,tdtype", [(np.float32, torch.float32), (np.float64, torch.float64)])
-def test_second_derivatives_at_small_l_max_by_both_kernels(oracle, library, route, dtype, tdtype, monkeypatch):
+def test_second_derivatives_at_small_l_max_by_both_kernels(oracle, library, route, dtype, tdtype, switches):
     """l_max 2 ... 8 with Hessians through the one-point-per-lane kernel wherever its rows fit and
-    through the recursion kernel (the library picks per l_max by itself; the switch is read at
-    every call), sizes around a tile, shifted outputs with guard elements."""
-    monkeypatch.setenv("SPHX_HESSIAN_LANES", "2" if route == "lanes" else "0")
+    through the recursion kernel (the library picks per l_max by itself; the switch is set
+    for this test), sizes around a tile, shifted outputs with guard elements."""
+    switches("SPHX_HESSIAN_LANES", "2" if route == "lanes" else "0")
     rng = np.random.default_rng(17)
     for l_max in range(2, 9):
         for n, shift in ((1, 0), (31, 1), (64, 0), (65, 2), (2049, 0), (4133, 3)):
@@ -133,11 +133,11 @@ def test_second_derivatives_at_small_l_max_by_both_kernels(oracle, library, rout
 
 
 @pytest.mark.parametrize("launches", ["one", "two"])
-def test_rows_cut_at_l7_by_one_launch_and_by_two(oracle, library, launches, monkeypatch):
+def test_rows_cut_at_l7_by_one_launch_and_by_two(oracle, library, launches, switches):
     """Few points per tile: the recursion kernel stages l >= 7 and l <= 6 comes either from its
-    wave 0 (the default) or from a launch of the closed-form kernel before it (the switch is read
-    at every call). Sizes around the batches of 64 points, workgroups without tiles included."""
-    monkeypatch.setenv("SPHX_PREFIX_INSIDE", "1" if launches == "one" else "0")
+    wave 0 (the default) or from a launch of the closed-form kernel before it (switch set for this
+    test). Sizes around the batches of 64 points, workgroups without tiles included."""
+    switches("SPHX_PREFIX_INSIDE", "1" if launches == "one" else "0")
     rng = np.random.default_rng(23)
     cases = ((np.float32, torch.float32, 20, "gradients"), (np.float32, torch.float32, 32, "gradients"),
              (np.float64, torch.float64, 14, "gradients"), (np.float32, torch.float32, 36, "values"),
@@ -164,14 +164,14 @@ def test_rows_cut_at_l7_by_one_launch_and_by_two(oracle, library, launches, monk
 
 
 @pytest.mark.parametrize("tile", [3, 5, 7])
-def test_recursion_kernel_with_tiles_that_are_no_power_of_two(oracle, library, tile, monkeypatch):
+def test_recursion_kernel_with_tiles_that_are_no_power_of_two(oracle, library, tile, switches):
     """The planner takes as many points per tile as fit; here sizes it would not pick are forced
-    (the switches are read at every call), with the lane kernels off so that the recursion kernel
+    (switches set for this test), with the lane kernels off so that the recursion kernel
     runs at every l_max."""
-    monkeypatch.setenv("SPHX_TILE", str(tile))
-    monkeypatch.setenv("SPHX_GRADIENT_LANES", "0")
-    monkeypatch.setenv("SPHX_HESSIAN_LANES", "0")
-    monkeypatch.setenv("SPHX_VALUES_LDS", "1")
+    switches("SPHX_TILE", str(tile))
+    switches("SPHX_GRADIENT_LANES", "0")
+    switches("SPHX_HESSIAN_LANES", "0")
+    switches("SPHX_VALUES_LDS", "1")
     rng = np.random.default_rng(29 + tile)
     cases = ((np.float32, 9, "hessians"), (np.float64, 8, "hessians"), (np.float32, 12, "gradients"),
              (np.float64, 13, "gradients"), (np.float32, 20, "gradients"), (np.float64, 10, "values"))
@@ -189,14 +189,14 @@ def test_recursion_kernel_with_tiles_that_are_no_power_of_two(oracle, library, t
 
 
 @pytest.mark.parametrize("order", ["list", "points"])
-def test_entry_jobs_as_one_list_and_point_by_point(oracle, library, order, monkeypatch):
+def test_entry_jobs_as_one_list_and_point_by_point(oracle, library, order, switches):
     """The two variants of the recursion kernel's entry stage (the jobs of a tile as one list
     over the lanes, or whole points side by side; the planner picks per shape, the switch forces
     one wherever the other would save nothing), with enough points for full tiles."""
-    monkeypatch.setenv("SPHX_JOB_LIST", "1" if order == "list" else "0")
-    monkeypatch.setenv("SPHX_GRADIENT_LANES", "0")
-    monkeypatch.setenv("SPHX_HESSIAN_LANES", "0")
-    monkeypatch.setenv("SPHX_VALUES_LDS", "1")
+    switches("SPHX_JOB_LIST", "1" if order == "list" else "0")
+    switches("SPHX_GRADIENT_LANES", "0")
+    switches("SPHX_HESSIAN_LANES", "0")
+    switches("SPHX_VALUES_LDS", "1")
     rng = np.random.default_rng(31)
     cases = ((np.float32, 17, "gradients"), (np.float32, 20, "gradients"), (np.float64, 16, "gradients"),
              (np.float32, 14, "hessians"), (np.float64, 14, "hessians"), (np.float32, 34, "values"),

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from golden_io import CONFIGS, config_case, edge_cases
+from golden_io import CONFIGS, config_case, degenerate_cases, edge_cases
 from gpu_utils import announce, run_calculator, run_launch_layer
 from helpers import MODES, same_numbers, special_points, within_tolerance
 from sphericart_amd.workloads import WORKLOADS
@@ -58,6 +58,24 @@ def test_golden_edge_cases(tag):
     for xyz, l_max, normalized, mode, want in edge_cases(tag):
         announce("golden edge", tag, l_max, normalized, mode)
         check(run_calculator(xyz, l_max, normalized, mode), want, (tag, l_max, normalized, mode))
+
+
+@pytest.mark.parametrize("tag", ["f32", "f64"])
+def test_golden_degenerate_points(tag):
+    """The origin, NaN, infinite, denormal and overflowing coordinates, each between ordinary
+    points of the same tile: what the compiled reference returns (it has no guard around
+    1 / sqrt(x^2 + y^2 + z^2), sphericart/include/templates.hpp:392-400), number for number, NaN
+    for NaN and signed infinity for signed infinity; the ordinary neighbours are unaffected."""
+    for xyz, where, l_max, normalized, mode, want in degenerate_cases(tag):
+        announce("golden degenerate", tag, l_max, normalized, mode)
+        got = run_calculator(xyz, l_max, normalized, mode)
+        for g, w, label in zip(got, want, ("sph", "dsph", "ddsph")):
+            assert (g is None) == (w is None)
+            if w is not None:
+                same = same_numbers(g, w)
+                bad_points = np.unique(np.nonzero(~same)[0])
+                assert same.all(), (tag, l_max, normalized, mode, label, "points", bad_points[:10],
+                                    "of which degenerate", np.intersect1d(bad_points, where)[:10])
 
 
 @pytest.mark.parametrize("name", CONFIGS)

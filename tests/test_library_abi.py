@@ -84,6 +84,25 @@ def test_launch_plans(library):
     assert _plan(library, 10, 3, 7, False)[0] == 1
 
 
+def test_planner_overrides(library, switches):
+    """sphx_set_switch changes what the next call plans; sphx_reset_switches restores the default;
+    unknown names are refused. Environment variables alone change nothing."""
+    default = _plan(library, 50_000, 20, 1, False)
+    os.environ["SPHX_TILE"] = "3"
+    try:
+        assert _plan(library, 50_000, 20, 1, False) == default
+    finally:
+        del os.environ["SPHX_TILE"]
+    switches("SPHX_TILE", 3)
+    status, (tile, _, _, _) = _plan(library, 50_000, 20, 1, False)
+    assert status == 0 and tile == 3 and default[1][0] != 3
+    library.sphx_reset_switches()
+    assert _plan(library, 50_000, 20, 1, False) == default
+    assert library.sphx_set_switch(b"SPHX_NO_SUCH_SWITCH", 1) == 1
+    assert b"unknown switch" in library.sphx_last_error()
+    assert library.sphx_set_switch(None, 1) == 1
+
+
 def test_zero_samples_is_a_no_op(library):
     # returns before touching pointers or the GPU (reference: sphericart_cuda.cpp:85-89)
     assert library.sphx_forward_f32(None, 0, 4, 1, 2, None, None, None, None) == 0

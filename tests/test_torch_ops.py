@@ -118,13 +118,13 @@ def test_fused_vjp_equals_checker_number_for_number(library, oracle, normalized,
 @pytest.mark.parametrize("route", ["lanes", "rows"])
 @pytest.mark.parametrize("normalized", [True, False])
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-5), (np.float64, 1e-12)])
-def test_fused_vjp_beyond_the_closed_forms(library, oracle, normalized, dtype, tol, route, monkeypatch):
+def test_fused_vjp_beyond_the_closed_forms(library, oracle, normalized, dtype, tol, route, switches):
     """l_max > 6, two routes: one point per lane with the entries kept in registers ("lanes", the
     default wherever a tile of 8 points or more fits in LDS), or the recursion kernel contracting
     its staged rows ("rows"). Either adds the terms in another order than the checker's loop,
     so the comparison is relative to the sum of absolute terms."""
     if route == "rows":
-        monkeypatch.setenv("SPHX_VJP_LANES", "0")  # read by the library at every call
+        switches("SPHX_VJP_LANES", "0")
     rng = np.random.default_rng(12)
     fn = library.sphx_vjp_f32 if dtype == np.float32 else library.sphx_vjp_f64
     stream = torch.cuda.current_stream().cuda_stream
