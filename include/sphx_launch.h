@@ -138,6 +138,24 @@ SPHX_EXPORT int sphx_forward_f32_via_f64(const float* xyz, size_t n_samples, int
                                          void* stream);
 SPHX_EXPORT size_t sphx_forward_f32_via_f64_workspace(size_t n_samples, int l_max, int derivatives);
 
+/* sphx_forward_f32_via_f64 for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc. No counterpart in the reference. The float64 rows are staged in a
+ * scratch array of 32 MiB that is part of the library's device code (every GPU
+ * the library runs on holds its own copy until the process ends); the call
+ * allocates and frees nothing and only enqueues on `stream`. The whole call
+ * must fit into the scratch: more than
+ * sphx_forward_f32_via_f64_static_capacity(l_max, derivatives) points
+ * (32 MiB / (8 * (3 + (l_max+1)^2 * {1, 4, 13})); 0 for invalid arguments)
+ * return SPHX_ERR_UNSUPPORTED with a message that names the limit; larger
+ * batches are passed in slices. All calls on one GPU share that GPU's array:
+ * calls that overlap in time on one GPU (two streams, two threads) race and
+ * must be ordered by the caller. Same results as sphx_forward_f32_via_f64. */
+SPHX_EXPORT int sphx_forward_f32_via_f64_static(const float* xyz, size_t n_samples, int l_max,
+                                                int normalized, int derivatives, float* sph,
+                                                float* dsph, float* ddsph, void* stream);
+SPHX_EXPORT size_t sphx_forward_f32_via_f64_static_capacity(int l_max, int derivatives);
+
 /* Host copy of the prefactor table the kernels use for this l_max: the F_l^m
  * block followed by the Q_l^m-recursion block, (l_max+1)(l_max+2) numbers.
  * Replaces compute_sph_prefactors<T> (sphericart/include/templates.hpp:54-97)

@@ -32,6 +32,8 @@ LAUNCH_SYMBOLS = [
     "sphx_vjp_f64",
     "sphx_forward_f32_via_f64",
     "sphx_forward_f32_via_f64_workspace",
+    "sphx_forward_f32_via_f64_static",
+    "sphx_forward_f32_via_f64_static_capacity",
     "sphx_prefactors_f32",
     "sphx_prefactors_f64",
     "sphx_device_count",
@@ -82,6 +84,11 @@ def _declare(lib):
         c_void_p, c_size_t, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]
     lib.sphx_forward_f32_via_f64_workspace.restype = c_size_t
     lib.sphx_forward_f32_via_f64_workspace.argtypes = [c_size_t, c_int, c_int]
+    lib.sphx_forward_f32_via_f64_static.restype = c_int
+    lib.sphx_forward_f32_via_f64_static.argtypes = [
+        c_void_p, c_size_t, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.sphx_forward_f32_via_f64_static_capacity.restype = c_size_t
+    lib.sphx_forward_f32_via_f64_static_capacity.argtypes = [c_int, c_int]
     lib.sphx_describe_plan.restype = c_int
     lib.sphx_describe_plan.argtypes = [c_size_t, c_int, c_int, c_int, c_int, ctypes.c_char_p, c_size_t]
     lib.sphx_set_switch.restype = c_int

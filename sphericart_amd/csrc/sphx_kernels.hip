@@ -75,6 +75,8 @@ static bool g_tables_ready[kMaxDevices] = {};
 static int g_lds_limit[kMaxDevices] = {};
 static int g_compute_units[kMaxDevices] = {};
 
+static int find_scratch(int device);
+
 // Upload the tables to the constant memory of `device` (current) once.
 static int ensure_device_ready(int device) {
     if (device < 0 || device >= kMaxDevices) {
@@ -104,6 +106,10 @@ static int ensure_device_ready(int device) {
                      "sphericart_amd: device %d reports %d XCDs; the kernels' workgroup order is laid out "
                      "for the 8 XCDs of an MI355X in SPX mode and will be slower here\n",
                      device, xcds);
+    }
+    {
+        const int status = find_scratch(device);
+        if (status != SPHX_OK) return status;
     }
     g_lds_limit[device] = lds;
     g_compute_units[device] = cus;
@@ -1207,6 +1213,25 @@ static size_t via_f64_bytes_per_point(int l_max, int mode) {
     return sizeof(double) * (3 + ny * components_of(mode));
 }
 
+// The library's own scratch memory for sphx_forward_f32_via_f64_static: callers that must not
+// allocate (HIP graph capture, serving loops, harnesses that forbid it) get the float64 rows of one
+// call staged here. Every device the library runs on holds its own copy of the array, at its own
+// address, until the process ends; g_scratch[device] is that address, asked from the runtime once
+// per device (ensure_device_ready). In host code the array's name is only a handle for that
+// question, never an address to hand to a kernel.
+constexpr size_t kScratchBytes = size_t(32) << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+static void* g_scratch[kMaxDevices] = {};
+
+// with `device` current; called under g_init_mutex by ensure_device_ready
+static int find_scratch(int device) {
+    void* ptr = nullptr;
+    SPHX_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) return fail(SPHX_ERR_HIP, "hipGetSymbolAddress returned no address for the scratch array");
+    g_scratch[device] = ptr;
+    return SPHX_OK;
+}
+
 static int check_via_f64_arguments(const float* xyz, int l_max, int mode, const float* sph,
                                    const float* dsph, const float* ddsph) {
     if (l_max < 0) return fail(SPHX_ERR_ARGUMENT, "l_max must be non-negative");
@@ -1323,6 +1348,45 @@ static int forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, in
     return status;
 }
 
+// The same with the library's scratch array as the workspace: nothing is allocated. One chunk
+// only, so a call is a fixed, short sequence of launches; more points than fit are refused.
+static int forward_f32_via_f64_static(const float* xyz, size_t n_samples, int l_max, int normalized,
+                                      int mode, float* sph, float* dsph, float* ddsph, void* stream) {
+    t_error.clear();
+    if (n_samples == 0) return SPHX_OK;
+    int status = check_via_f64_arguments(xyz, l_max, mode, sph, dsph, ddsph);
+    if (status != SPHX_OK) return status;
+    const size_t per_point = via_f64_bytes_per_point(l_max, mode);
+    if (n_samples > kScratchBytes / per_point) {
+        return fail(SPHX_ERR_UNSUPPORTED,
+                    std::to_string(n_samples) + " points of " + std::to_string(per_point) +
+                        " bytes each exceed the library's scratch memory of " + std::to_string(kScratchBytes) +
+                        " bytes: at most " + std::to_string(kScratchBytes / per_point) +
+                        " points of this shape per call");
+    }
+    hipPointerAttribute_t attr;
+    SPHX_HIP(hipPointerGetAttributes(&attr, xyz));
+    int current = 0;
+    SPHX_HIP(hipGetDevice(&current));
+    const int device = attr.device;
+    if (device != current) SPHX_HIP(hipSetDevice(device));
+    status = ensure_device_ready(device); // finds this device's copy of the scratch array
+    if (status == SPHX_OK) {
+        // Every number of the part of the scratch this call uses is written (widen_kernel, the
+        // float64 kernels) before it is read (the kernels, narrow_kernel), whatever the last
+        // call left there: nothing has to be cleared.
+        status = via_f64_chunks(device, xyz, n_samples, l_max, normalized, mode, sph, dsph, ddsph,
+                                g_scratch[device], kScratchBytes, stream);
+    }
+    if (device != current) {
+        hipError_t e = hipSetDevice(current);
+        if (e != hipSuccess && status == SPHX_OK) {
+            status = fail(SPHX_ERR_HIP, std::string("hipSetDevice: ") + hipGetErrorString(e));
+        }
+    }
+    return status;
+}
+
 } // namespace sphx
 
 extern "C" {
@@ -1344,6 +1408,17 @@ int sphx_forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, int 
                              size_t workspace_bytes, void* stream) {
     return sphx::forward_f32_via_f64(xyz, n_samples, l_max, normalized, derivatives, sph, dsph, ddsph,
                                      workspace, workspace_bytes, stream);
+}
+
+int sphx_forward_f32_via_f64_static(const float* xyz, size_t n_samples, int l_max, int normalized,
+                                    int derivatives, float* sph, float* dsph, float* ddsph, void* stream) {
+    return sphx::forward_f32_via_f64_static(xyz, n_samples, l_max, normalized, derivatives, sph, dsph, ddsph,
+                                            stream);
+}
+
+size_t sphx_forward_f32_via_f64_static_capacity(int l_max, int derivatives) {
+    if (l_max < 0 || l_max > SPHX_TABLE_LMAX || derivatives < 0 || derivatives > 2) return 0;
+    return sphx::kScratchBytes / sphx::via_f64_bytes_per_point(l_max, derivatives);
 }
 
 size_t sphx_forward_f32_via_f64_workspace(size_t n_samples, int l_max, int derivatives) {

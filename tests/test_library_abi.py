@@ -103,6 +103,17 @@ def test_planner_overrides(library, switches):
     assert library.sphx_set_switch(None, 1) == 1
 
 
+def test_static_scratch_capacity(library):
+    # 32 MiB / (8 * (3 + (l_max + 1)^2 * {1, 4, 13}))
+    assert library.sphx_forward_f32_via_f64_static_capacity(6, 1) == (32 << 20) // (8 * (3 + 49 * 4))
+    assert library.sphx_forward_f32_via_f64_static_capacity(32, 2) == (32 << 20) // (8 * (3 + 1089 * 13))
+    assert library.sphx_forward_f32_via_f64_static_capacity(-1, 0) == 0
+    assert library.sphx_forward_f32_via_f64_static_capacity(4, 3) == 0
+    # zero points: nothing is looked at
+    assert library.sphx_forward_f32_via_f64_static(None, 0, 4, 1, 1, None, None, None, None) == 0
+    assert library.sphx_forward_f32_via_f64_static(None, 5, 4, 1, 0, None, None, None, None) == 1
+
+
 def test_zero_samples_is_a_no_op(library):
     # returns before touching pointers or the GPU (reference: sphericart_cuda.cpp:85-89)
     assert library.sphx_forward_f32(None, 0, 4, 1, 2, None, None, None, None) == 0
