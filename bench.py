@@ -9,18 +9,20 @@ preallocated outputs. The default workload is the configuration the headline
 metric is quoted on: real spherical harmonics, l_max = 6, float32, values and
 gradients, 1,000,000 points.
 
-The K timed steps are enqueued back to back between one pair of events and
-one pair of host clock readings (`value`, `ms_per_step`); a second pass of K
-steps with an event pair around every launch gives the duration of the single
-launch that `roofline` is computed from.
+The K timed steps are enqueued back to back between one pair of host clock
+readings (`value`, `ms_per_step`) and one pair of events on the launch stream,
+whose distance over K is the average launch duration that `roofline` is
+computed from. A second pass of K steps with an event pair around every launch
+records the spread; such a pair adds 2-4 us to the launch it brackets, which
+matters for the configurations whose launch takes 12 us.
 
 One JSON line is printed. Next to the contract fields it carries
 
   roofline      achieved HBM bandwidth of the kernel: algorithmic bytes per
                 launch (sizeof(T) * (3 + (l_max+1)^2 * components) per point)
                 divided by the average launch duration, measured with events
-                on the launch stream around every launch of the second pass,
-                against the 8 TB/s peak of MI355X;
+                on the launch stream around the timed region, against the
+                8 TB/s peak of MI355X;
   roofline_by_config
                 (default workload only) the same figure for the other four
                 configurations of the reference's benchmark set, each with the
@@ -287,8 +289,12 @@ def time_each_launch(step, steps, stream):
     return [b.elapsed_time(e) for b, e in events]
 
 
-def roofline_of(launch_ms, bytes_per_launch):
-    avg_s = sum(launch_ms) / len(launch_ms) / 1e3
+def roofline_of(device_ms, steps, launch_ms, bytes_per_launch):
+    """`device_ms`: between one event before the first and one after the last of `steps` launches
+    enqueued back to back; the average launch duration is that over `steps` (it agrees with the
+    profiler's kernel durations to a few percent at every size). `launch_ms`: every launch between
+    an event pair of its own, which adds 2-4 us to each (kept for the spread: median, minimum)."""
+    avg_s = device_ms / steps / 1e3
     achieved = bytes_per_launch / avg_s / 1e9
     return {
         "bound": "hbm",
@@ -298,9 +304,20 @@ def roofline_of(launch_ms, bytes_per_launch):
         "frac": achieved / PEAK_HBM_GBPS,
         "algorithmic_bytes_per_launch": bytes_per_launch,
         "avg_launch_us": avg_s * 1e6,
-        "median_launch_us": statistics.median(launch_ms) * 1e3,
-        "min_launch_us": min(launch_ms) * 1e3,
+        "back_to_back_us_per_launch": avg_s * 1e6,
+        "per_launch_events": {
+            "avg_us": sum(launch_ms) / len(launch_ms) * 1e3,
+            "median_us": statistics.median(launch_ms) * 1e3,
+            "min_us": min(launch_ms) * 1e3,
+        },
     }
+
+
+def measure(prepared, steps, settle_seconds, warmup):
+    settle(prepared.step, settle_seconds, warmup)
+    wall, device_ms = time_back_to_back(prepared.step, steps, prepared.stream)
+    launch_ms = time_each_launch(prepared.step, steps, prepared.stream)
+    return wall, roofline_of(device_ms, steps, launch_ms, prepared.bytes_per_launch)
 
 
 def measure_config(lib, name, steps, settle_seconds, with_cold):
@@ -313,33 +330,22 @@ def measure_config(lib, name, steps, settle_seconds, with_cold):
     w = WORKLOADS[name]
     steps = max(steps, 50)
     prepared = Prepared(lib, w)
-    settle(prepared.step, settle_seconds, 10)
-    wall, device_ms = time_back_to_back(prepared.step, steps, prepared.stream)
-    entry = roofline_of(time_each_launch(prepared.step, steps, prepared.stream), prepared.bytes_per_launch)
+    wall, entry = measure(prepared, steps, settle_seconds, 10)
     entry.update({
         "workload": f"{w.name}: {w.description}",
         "dtype": w.dtype,
         "kernels": prepared.kernels(),
         "launches_timed": steps,
         "points_per_s": w.n_samples * steps / wall,
-        "back_to_back_us_per_launch": device_ms / steps * 1e3,
         "traffic": MEASURED_TRAFFIC_BYTES.get(name),
     })
     del prepared
     torch.cuda.empty_cache()
     if with_cold:
         cold = Prepared(lib, w, rotate_mb=1024)
-        settle(cold.step, settle_seconds, 10)
-        launch_ms = time_each_launch(cold.step, steps, cold.stream)
-        r = roofline_of(launch_ms, cold.bytes_per_launch)
-        entry["cold"] = {
-            "rotate_mb": 1024,
-            "output_buffers": len(cold.outputs),
-            "avg_launch_us": r["avg_launch_us"],
-            "min_launch_us": r["min_launch_us"],
-            "achieved": r["achieved"],
-            "frac": r["frac"],
-        }
+        _, r = measure(cold, steps, settle_seconds, 10)
+        entry["cold"] = {"rotate_mb": 1024, "output_buffers": len(cold.outputs), "avg_launch_us": r["avg_launch_us"],
+                         "achieved": r["achieved"], "frac": r["frac"], "per_launch_events": r["per_launch_events"]}
         del cold
         torch.cuda.empty_cache()
     return entry
@@ -435,10 +441,9 @@ def main():
     # the timed region: K steps back to back
     wall, device_ms = time_back_to_back(step, args.steps, stream)
     # the single launch: K more steps, an event pair around each
-    roofline = roofline_of(time_each_launch(step, args.steps, stream), bytes_per_launch)
+    roofline = roofline_of(device_ms, args.steps, time_each_launch(step, args.steps, stream), bytes_per_launch)
     roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(
         args.workload if args.op == "forward" else f"{args.workload}:{args.op}")
-    roofline["back_to_back_us_per_launch"] = device_ms / args.steps * 1e3
     headline = args.workload == "cfg3" and args.op == "forward" and args.rotate_mb == 0
 
     result = {
@@ -479,11 +484,10 @@ def main():
             result["cpu_baseline"] = cpu_backward_baseline(dsph.cpu().numpy(), sph_grad.cpu().numpy())
     if headline and not args.no_by_config:
         cold = Prepared(lib, w, rotate_mb=1024)
-        settle(cold.step, args.settle_seconds, 10)
-        r = roofline_of(time_each_launch(cold.step, max(args.steps, 50), cold.stream), cold.bytes_per_launch)
+        _, r = measure(cold, max(args.steps, 50), args.settle_seconds, 10)
         result["roofline"]["cold"] = {
             "rotate_mb": 1024, "output_buffers": len(cold.outputs), "avg_launch_us": r["avg_launch_us"],
-            "min_launch_us": r["min_launch_us"], "achieved": r["achieved"], "frac": r["frac"],
+            "achieved": r["achieved"], "frac": r["frac"], "per_launch_events": r["per_launch_events"],
         }
         del cold, prepared, sph, dsph, ddsph
         torch.cuda.empty_cache()

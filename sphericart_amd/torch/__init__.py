@@ -4,8 +4,8 @@ Same two classes and methods as the reference's
 sphericart-torch/python/sphericart/torch/spherical_hamonics.py (``forward``,
 ``compute``, ``compute_with_gradients``, ``compute_with_hessians``, ``l_max``);
 the operators behind them are registered in :mod:`sphericart_amd.torch.ops`.
-Tensors must live on the GPU. ``omp_num_threads`` has no meaning here (there is
-no host evaluator) and is not offered.
+Tensors must live on the GPU. ``omp_num_threads`` reports 1: there is no host
+evaluator and no OpenMP team behind the operators.
 """
 
 from typing import Tuple
@@ -40,6 +40,10 @@ class SphericalHarmonics(torch.nn.Module):
     def compute_with_hessians(self, xyz: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
         return torch.ops.sphericart_amd.spherical_harmonics_with_hessians(xyz, self._l_max)
 
+    def omp_num_threads(self) -> int:
+        """Threads of the host evaluator in the reference; 1 here (GPU only)."""
+        return 1
+
     def l_max(self) -> int:
         return self._l_max
 
@@ -64,6 +68,10 @@ class SolidHarmonics(torch.nn.Module):
 
     def compute_with_hessians(self, xyz: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
         return torch.ops.sphericart_amd.solid_harmonics_with_hessians(xyz, self._l_max)
+
+    def omp_num_threads(self) -> int:
+        """See :py:meth:`SphericalHarmonics.omp_num_threads`."""
+        return 1
 
     def l_max(self) -> int:
         return self._l_max

@@ -6,6 +6,11 @@ and vmap rules from Python (sphericart-torch/python/sphericart/torch/register.py
 The same six live here in the ``sphericart_amd`` namespace with the same
 schemas; their device implementation calls ``sphx_forward_*`` on the tensor's
 current stream. Only the GPU key has an implementation: CPU tensors raise.
+Unless the reference's own extension already owns it, the ``sphericart_torch``
+namespace is defined as well, with the reference's eight schemas (the six
+operators and the two ``*_omp_num_threads``), each forwarding to its
+``sphericart_amd`` twin: code, scripted modules included, that names
+``torch.ops.sphericart_torch.*`` resolves against this library.
 
 The backward formulas are the reference's (register.py:82-175). Where it writes
 the vector-Jacobian products as ``torch.sum(grad.unsqueeze(1) * dsph, dim=2)``,
@@ -340,3 +345,36 @@ for _prefix in ("spherical_harmonics", "solid_harmonics"):
     _register_vmap(_prefix, 0)
     _register_vmap(f"{_prefix}_with_gradients", (0, 0))
     _register_vmap(f"{_prefix}_with_hessians", (0, 0, 0))
+
+
+# ---- the reference's namespace (sphericart-torch/src/torch.cpp:367-385) ---------------------
+#
+# Aliases: every operator forwards to its twin above through a composite implementation, so the
+# autograd, fake-tensor and vmap rules registered there apply unchanged. The two
+# *_omp_num_threads operators report 1: there is no host evaluator and no OpenMP team behind
+# these operators. Skipped when the namespace is taken (the reference's extension is loaded).
+
+REFERENCE_NAMESPACE = "sphericart_torch"
+reference_namespace_defined = False
+
+
+def _define_reference_namespace():
+    global _reference_lib, reference_namespace_defined
+    try:
+        _reference_lib = torch.library.Library(REFERENCE_NAMESPACE, "DEF")
+    except RuntimeError:
+        return  # another library owns the namespace
+    for prefix in ("spherical_harmonics", "solid_harmonics"):
+        _reference_lib.define(f"{prefix}(Tensor xyz, int l_max) -> Tensor")
+        _reference_lib.define(f"{prefix}_with_gradients(Tensor xyz, int l_max) -> (Tensor, Tensor)")
+        _reference_lib.define(f"{prefix}_with_hessians(Tensor xyz, int l_max) -> (Tensor, Tensor, Tensor)")
+        _reference_lib.define(f"{prefix}_omp_num_threads(int l_max) -> int")
+        for suffix in ("", "_with_gradients", "_with_hessians"):
+            twin = getattr(_ops, prefix + suffix)
+            _reference_lib.impl(prefix + suffix, (lambda op: lambda xyz, l_max: op(xyz, l_max))(twin),
+                                "CompositeImplicitAutograd")
+        _reference_lib.impl(f"{prefix}_omp_num_threads", lambda l_max: 1, "CompositeExplicitAutograd")
+    reference_namespace_defined = True
+
+
+_define_reference_namespace()

@@ -132,3 +132,45 @@ def test_inside_a_training_loop():
         opt.step()
         losses.append(float(loss.detach()))
     assert losses[-1] < losses[0]
+
+
+class ReferenceNames(torch.nn.Module):
+    """Names the operators as the reference registers them (sphericart-torch/src/torch.cpp:367-385)."""
+
+    def forward(self, xyz):
+        sph = torch.ops.sphericart_torch.spherical_harmonics(xyz, 8)
+        solid, dsolid = torch.ops.sphericart_torch.solid_harmonics_with_gradients(xyz, 4)
+        return sph, solid, dsolid
+
+
+def test_reference_namespace_resolves(oracle, tmp_path):
+    """A module written against `torch.ops.sphericart_torch.*`: eager, scripted, saved and loaded;
+    forward equal to the oracle number for number, xyz.grad equal to the oracle's gradients
+    contracted in float64 to rounding; the two *_omp_num_threads operators exist."""
+    import numpy as np
+
+    from sphericart_amd.torch import ops
+
+    assert ops.reference_namespace_defined
+    announce("reference namespace")
+    assert torch.ops.sphericart_torch.spherical_harmonics_omp_num_threads(8) == 1
+    assert torch.ops.sphericart_torch.solid_harmonics_omp_num_threads(4) == 1
+    assert sphericart_amd.torch.SolidHarmonics(4).omp_num_threads() == 1
+    xyz_host = _xyz(257, seed=3).cpu().numpy()
+    want_sph, want_dsph, _ = oracle.compute(xyz_host, 8, True, "gradients")
+    want_solid, want_dsolid, _ = oracle.compute(xyz_host, 4, False, "gradients")
+    script = torch.jit.script(ReferenceNames())
+    path = str(tmp_path / "reference_names.pt")
+    script.save(path)
+    for module in (ReferenceNames(), script, torch.jit.load(path)):
+        xyz = torch.from_numpy(xyz_host).cuda().requires_grad_()
+        sph, solid, dsolid = module(xyz)
+        np.testing.assert_array_equal(sph.detach().cpu().numpy(), want_sph)
+        np.testing.assert_array_equal(solid.detach().cpu().numpy(), want_solid)
+        np.testing.assert_array_equal(dsolid.detach().cpu().numpy(), want_dsolid)
+        (sph.sum() + solid.sum()).backward()
+        want_grad = want_dsph.sum(axis=2) + want_dsolid.sum(axis=2)
+        scale = np.abs(want_dsph).sum(axis=2) + np.abs(want_dsolid).sum(axis=2)
+        assert (np.abs(xyz.grad.cpu().numpy() - want_grad) <= 1e-12 * scale).all()
+    with pytest.raises(RuntimeError, match="GPU"):
+        torch.ops.sphericart_torch.spherical_harmonics(torch.zeros(2, 3), 3)
