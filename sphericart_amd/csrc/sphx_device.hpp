@@ -635,14 +635,19 @@ __device__ __forceinline__ void emit(V v, V* dst) {
 // as 16-byte stores at 16-byte aligned addresses, consecutive lanes to consecutive addresses;
 // at most three (float) or one (double) leading and trailing elements are stored one by one.
 // PADDED: the staged run has `pad` spare elements after every `row` elements (see staged_index).
-template <typename T, bool STREAMING, bool PADDED, int UNROLL = 1>
+// LINES: the 16-byte stores start at a 128-byte line of dst instead of at the first 16-byte
+// boundary, so that every store instruction of a wave (64 x 16 bytes) covers eight whole lines
+// and none is written in two parts by two instructions; up to 31 (float) or 15 (double)
+// leading elements are then stored one by one. Needs nthreads >= 34.
+template <typename T, bool STREAMING, bool PADDED, int UNROLL = 1, bool LINES = false>
 __device__ __forceinline__ void copy_out(const T* __restrict__ staged, T* __restrict__ dst,
                                          unsigned len, unsigned row, unsigned pad, unsigned magic,
                                          unsigned tid, unsigned nthreads) {
     using V = typename Pack<T>::type;
     constexpr unsigned W = Pack<T>::width;
-    const unsigned misalign = static_cast<unsigned>(reinterpret_cast<uintptr_t>(dst) & 15u);
-    unsigned head = ((16u - misalign) & 15u) / static_cast<unsigned>(sizeof(T));
+    constexpr unsigned ALIGN = LINES ? 128u : 16u;
+    const unsigned misalign = static_cast<unsigned>(reinterpret_cast<uintptr_t>(dst) & (ALIGN - 1u));
+    unsigned head = ((ALIGN - misalign) & (ALIGN - 1u)) / static_cast<unsigned>(sizeof(T));
     if (head > len) head = len;
     const unsigned nvec = (len - head) / W;
     V* out = reinterpret_cast<V*>(dst + head) + tid;

@@ -286,7 +286,8 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
 
 // gradients_lanes_kernel: 64, 32 or 16 points per workgroup with their four rows and tables in
 // LDS. Returns false when too few points would be resident on a CU for it to pay.
-static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int lds_limit, Launch* out) {
+static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int lds_limit, int cus,
+                                Launch* out) {
     Tiling& g = out->g;
     std::memset(&g, 0, sizeof(g));
     const unsigned esize = static_cast<unsigned>(elem);
@@ -304,14 +305,29 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     // l_max = 13 357 us with 3 x 16 against 433 with 32; l_max = 15 579 us with 32 against 651
     // with 2 x 16. Below 32 resident points (or 3 x 16) the recursion kernel is the faster one
     // (l_max = 18: 1 038 us against 1 236).
+    // Few points (one workgroup per CU can take them all): the time of the call is the time of
+    // one workgroup, and every workgroup beyond one per CU makes the waves of a CU queue for its
+    // vector ALUs with most of their lanes idle. Then the tile is N / CUs, rounded up to a
+    // multiple of four: cfg1 (10 000 points, float64 l_max = 8) 11.8 us with 632 tiles of 16,
+    // 16.1 us with 320 tiles of 32 (one per CU at a time: two rounds), see below for tiles of 40.
+    unsigned few = 0;
+    const unsigned forced_tile = static_cast<unsigned>(switch_or(SW_GRADIENT_LANES_TILE, 0));
+    if (cus > 0 && n_samples <= static_cast<size_t>(cus) * 64u) {
+        few = static_cast<unsigned>((n_samples + static_cast<size_t>(cus) - 1) / static_cast<size_t>(cus));
+        few = (few + 3u) & ~3u;
+        if (few < 8u) few = 8u;
+    }
+    if (forced_tile == 1u) few = 0; // 1: the throughput rule also for few points
     unsigned tile = 0, off_d = 0, off_t = 0, bytes = 0, best = 0, best_groups = 0;
-    for (unsigned t = 64; t >= 16; t /= 2) {
+    for (unsigned t : {64u, 32u, 16u, few}) {
+        if (t == 0) continue;
         const unsigned od = (t * s_stride + vec - 1u) / vec * vec;
         const unsigned ot = od + (t * d_stride + vec - 1u) / vec * vec;
         const unsigned b = (ot + t * table_stride) * esize;
         if (b > limit) continue;
         unsigned score = (limit / b) * t * (t >= 32 ? 4u : 3u);
-        if (static_cast<unsigned>(switch_or(SW_GRADIENT_LANES_TILE, 0)) == t) score = 1u << 30;
+        if (t == few) score = 1u << 29;
+        if (forced_tile == t) score = 1u << 30;
         if (score > best || (score == best && best_groups < 2)) {
             best = score;
             best_groups = limit / b;
@@ -339,7 +355,9 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     // are enough and leave room for more workgroups (1.5 GB of output: float64 l_max = 8 469 us
     // with eight waves, 345 with four; float32 l_max = 7, 8 286, 274 against 273, 261; from three
     // channels on eight waves are faster, l_max = 12: 357 against 411).
-    int waves = switch_or(SW_GRADIENT_LANES_WAVES, l_max <= 8 ? 4 : 8);
+    // (few points: one workgroup per CU, occupancy is no concern and eight waves shorten the
+    // longest chain of work in the workgroup)
+    int waves = switch_or(SW_GRADIENT_LANES_WAVES, l_max <= 8 && tile != few ? 4 : 8);
     waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
     out->threads = 64u * static_cast<unsigned>(waves);
     out->lds_bytes = bytes;
@@ -680,7 +698,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
         return SPHX_OK;
     }
     if (lane_kernels && mode == 1 && switch_or(SW_GRADIENT_LANES, 1) != 0 &&
-        plan_gradient_lanes(n_samples, l_max, elem, lds_limit, &plan->closed)) {
+        plan_gradient_lanes(n_samples, l_max, elem, lds_limit, cus, &plan->closed)) {
         plan->lanes = true;
         return SPHX_OK;
     }
@@ -713,7 +731,10 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // 393, 407, 373, 399 us against 431, 451, 419, 424; l_max = 28, 30 (3) 396, 371 against 532,
     // 510; l_max = 32 (2) 462 against 389. Float32 gradients are therefore cut below three
     // points per tile only; values below eight, float64 gradients below four as before.)
-    const int split_below = switch_or(SW_SPLIT_BELOW, mode == 0 ? 8 : (elem == 4 ? 3 : 4));
+    // (Since the float64 rows go out in whole lines, copy_out<LINES>, the cut rows gained 20 %
+    // there: l_max = 20, 100k points 491 -> 376 us, and with four points per tile they now win as
+    // well, l_max = 18: 291 us cut against 328 whole; with five, l_max = 16: 580 against 481.)
+    const int split_below = switch_or(SW_SPLIT_BELOW, mode == 0 ? 8 : (elem == 4 ? 3 : 5));
     const bool cut = plan->rec.g.tile < split_below;
     if (mode < 2 && (!fits || cut)) {
         Launch upper;

@@ -203,9 +203,21 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
     rows.dsph = lds + g.off_dsph + lane * g.off_ddsph;
     rows.ddsph = nullptr;
     T* tab = lds + g.off_pts + lane * g.off_iter; // [m][3]: c_m, s_m, 2(m+1)z
+    // Who does what. The channels above the closed forms go to the waves in snake order, the
+    // longest first; the eight slices of the closed forms to the waves that have no channel, or,
+    // when every wave has one, to the waves from the last backwards. No wave waits for another
+    // before the rows are complete: a wave with channels makes the (c_m, s_m, 2(m+1)z) tables
+    // itself (a tenth of a channel's work; the waves write the same numbers to the same places
+    // and each reads back what it wrote).
+    const unsigned channels = static_cast<unsigned>(L - H);
+    const bool has_channel = wave < channels;
+    const unsigned spare = waves > channels ? waves - channels : 0u; // waves without a channel
+    auto my_slice = [&](unsigned j) -> bool {
+        return spare != 0 ? wave == channels + j % spare : (waves - 1u - wave) == j % waves;
+    };
     if (lane < valid) {
         p = load_point<T, NORM>(xyz + (first + lane) * 3);
-        if (wave == 0) {
+        if (has_channel) {
             const T twoz = p.z + p.z;
             T cm = 1.0, sm = 0.0, tz = twoz;
             tab[0] = cm;
@@ -222,17 +234,15 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
                 tab[3 * m + 2] = tz;
             }
         }
-        const unsigned from_last = waves - 1u - wave;
-        if (0 % waves == from_last) closed_form_job<T, 1, NORM, H, 0, 9>(p, rows);
-        if (1 % waves == from_last) closed_form_job<T, 1, NORM, H, 9, 16>(p, rows);
-        if (2 % waves == from_last) closed_form_job<T, 1, NORM, H, 16, 25>(p, rows);
-        if (3 % waves == from_last) closed_form_job<T, 1, NORM, H, 25, 31>(p, rows);
-        if (4 % waves == from_last) closed_form_job<T, 1, NORM, H, 31, 36>(p, rows);
-        if (5 % waves == from_last) closed_form_job<T, 1, NORM, H, 36, 41>(p, rows);
-        if (6 % waves == from_last) closed_form_job<T, 1, NORM, H, 41, 45>(p, rows);
-        if (7 % waves == from_last) closed_form_job<T, 1, NORM, H, 45, 49>(p, rows);
+        if (my_slice(0)) closed_form_job<T, 1, NORM, H, 0, 9>(p, rows);
+        if (my_slice(1)) closed_form_job<T, 1, NORM, H, 9, 16>(p, rows);
+        if (my_slice(2)) closed_form_job<T, 1, NORM, H, 16, 25>(p, rows);
+        if (my_slice(3)) closed_form_job<T, 1, NORM, H, 25, 31>(p, rows);
+        if (my_slice(4)) closed_form_job<T, 1, NORM, H, 31, 36>(p, rows);
+        if (my_slice(5)) closed_form_job<T, 1, NORM, H, 36, 41>(p, rows);
+        if (my_slice(6)) closed_form_job<T, 1, NORM, H, 41, 45>(p, rows);
+        if (my_slice(7)) closed_form_job<T, 1, NORM, H, 45, 49>(p, rows);
     }
-    __syncthreads(); // the tables
     if (lane < valid) {
         const T x = p.x, y = p.y;
         const T rxy = p.x2 + p.y2;
