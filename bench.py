@@ -53,11 +53,13 @@ PEAK_HBM_GBPS = 8000.0
 # plain device-to-device copy of known size (`--calibrate-copy`: WRITE_SIZE
 # reads the copied bytes exactly, FETCH_SIZE half of them, so fetches are
 # doubled). KiB per dispatch * 1024 * factor, fetch + write, all kernels of one
-# call added up.
+# call added up; the five configurations as in profiles/*_cfgN.md.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg3": int((5930.6 * 2.0 + 765861.1) * 1024),
-    "cfg4": int((1323.1 * 2.0 + 2935253.2) * 1024),
-    "cfg5": int((2914.8 * 2.0 + 3785830.1) * 1024),
+    "cfg1": 26866092,
+    "cfg2": 76091891,
+    "cfg3": 796482282,
+    "cfg4": 3008449407,
+    "cfg5": 3881148774,
     "cfg3:backward": int((394551.2 * 2.0 + 11719.3) * 1024),
     "cfg3:vjp": int((101629.1 * 2.0 + 11718.8) * 1024),
     "cfg5:vjp": int((426681.8 * 2.0 + 2344.1) * 1024),
