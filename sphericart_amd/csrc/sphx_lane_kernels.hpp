@@ -57,7 +57,7 @@ __global__ __launch_bounds__(kValuesMaxThreads) void values_kernel(Tiling g, con
     T* lds = reinterpret_cast<T*>(lds_raw);
     const unsigned tid = threadIdx.x;
     const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6); // the same for all lanes: scalar
     const unsigned waves = blockDim.x >> 6;
     const int L = g.l_max;
     const unsigned ny = g.ny;
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
     T* lds = reinterpret_cast<T*>(lds_raw);
     const unsigned tid = threadIdx.x;
     const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6); // the same for all lanes: scalar
     const unsigned threads = blockDim.x;
     const unsigned waves = threads >> 6;
     const int L = g.l_max;
@@ -383,7 +383,7 @@ __global__ __launch_bounds__(kHessianLaneThreads) void hessians_lanes_kernel(Til
     T* lds = reinterpret_cast<T*>(lds_raw);
     const unsigned tid = threadIdx.x;
     const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6); // the same for all lanes: scalar
     const unsigned threads = blockDim.x;
     const unsigned waves = threads >> 6;
     const int L = g.l_max;
@@ -407,10 +407,12 @@ __global__ __launch_bounds__(kHessianLaneThreads) void hessians_lanes_kernel(Til
     T* tmz = sn + (L + 1);
     if (lane < valid) {
         p = load_point<T, NORM>(xyz + (first + lane) * 3);
-        if (wave == 0) azimuth_job<T>(p, L, c, sn, tmz);
+        // every wave has a channel and makes the tables for it itself (a few percent of a
+        // channel's work; the waves write the same numbers to the same places and each reads back
+        // what it wrote): no wave waits for another before the rows are complete
+        azimuth_job<T>(p, L, c, sn, tmz);
         if (wave == waves - 1) closed_form_job<T, 2, NORM, H>(p, rows);
     }
-    __syncthreads(); // the tables
     if (lane < valid) {
         const T rxy = p.x2 + p.y2;
         const T* cF = table_F<T>();

@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
     T* lds = reinterpret_cast<T*>(lds_raw);
     const unsigned tid = threadIdx.x;
     const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6); // the same for all lanes: scalar
     const int L = g.l_max;
     const unsigned S = g.tile;
     const unsigned ny = g.ny;
@@ -514,7 +514,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
             // points: 491 -> 381 us); in float32 that measured the same or 2 % worse.
             constexpr bool LINES = sizeof(T) == 8;
             const unsigned waves = count / 64;
-            for (unsigned r = ft >> 6; r < valid * components_of(MODE); r += waves) {
+            for (unsigned r = __builtin_amdgcn_readfirstlane(ft >> 6); r < valid * components_of(MODE); r += waves) {
                 // rows [0, valid) are values, the next 3 * valid are gradients
                 if (r < valid) {
                     copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL, LINES>(

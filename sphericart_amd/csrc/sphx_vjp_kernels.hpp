@@ -155,7 +155,7 @@ __global__ __launch_bounds__(kValuesMaxThreads) void vjp_lanes_kernel(Tiling g, 
     T* lds = reinterpret_cast<T*>(lds_raw);
     const unsigned tid = threadIdx.x;
     const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6); // the same for all lanes: scalar
     const unsigned threads = blockDim.x;
     const unsigned waves = threads >> 6;
     const int L = g.l_max;
@@ -388,7 +388,7 @@ __global__ __launch_bounds__(kValuesMaxThreads) void vjp_groups_kernel(Tiling g,
     T* lds = reinterpret_cast<T*>(lds_raw);
     const unsigned tid = threadIdx.x;
     const unsigned lane = tid & 63u;
-    const unsigned wave = tid >> 6;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6); // the same for all lanes: scalar
     const unsigned threads = blockDim.x;
     const unsigned waves = threads >> 6;
     const int L = g.l_max;
