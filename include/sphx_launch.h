@@ -121,6 +121,14 @@ SPHX_EXPORT int sphx_vjp_f64(const double* xyz, const double* sph_grad, size_t n
  * reference; never chosen implicitly, since parity with the reference is
  * defined on sphx_forward_f32.
  *
+ * Beyond the closed forms (l_max > 6; l_max > 1 with second derivatives) this
+ * is one launch of the recursion kernel in its mixed variant: it reads the
+ * float coordinates, keeps tables and iterates in float64 and stages float
+ * rows, each number rounded as it is stored. No workspace is read or written
+ * then, and nothing is allocated. At or below the closed forms, and where one
+ * point's float rows and float64 tables exceed a CU's LDS, the points are
+ * widened, evaluated into float64 rows in a workspace and narrowed:
+ *
  *   workspace        device memory, 16-byte aligned, of workspace_bytes bytes;
  *                    the points are processed in chunks of as many as it holds
  *                    (8 * (3 + (l_max+1)^2 * {1, 4, 13}) bytes each), enqueued
@@ -130,8 +138,7 @@ SPHX_EXPORT int sphx_vjp_f64(const double* xyz, const double* sph_grad, size_t n
  *                    (hipMallocAsync / hipFreeAsync): it still only enqueues.
  *
  * sphx_forward_f32_via_f64_workspace returns the size with which n_samples
- * points are one chunk (0 for invalid arguments). Costs the float64 evaluation
- * plus one pass over the float64 rows. */
+ * points are one chunk (0 for invalid arguments). */
 SPHX_EXPORT int sphx_forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max,
                                          int normalized, int derivatives, float* sph, float* dsph,
                                          float* ddsph, void* workspace, size_t workspace_bytes,

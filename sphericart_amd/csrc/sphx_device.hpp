@@ -46,11 +46,13 @@ template <> struct Pack<double> {
 
 // Where the staged outputs of one point live in LDS. Element (component a,
 // index k) of the point's gradient row is at dsph[a * ny + k], and so on; the
-// rows mirror the layout of the output arrays in HBM.
-template <typename T> struct Rows {
-    T* sph;
-    T* dsph;
-    T* ddsph;
+// rows mirror the layout of the output arrays in HBM. The rows may be of a
+// narrower type than the arithmetic (float rows filled from float64 results,
+// every number rounded once as it is stored).
+template <typename O> struct Rows {
+    O* sph;
+    O* dsph;
+    O* ddsph;
     int ny;
 };
 
@@ -60,11 +62,11 @@ template <typename T> struct Point {
 };
 
 // templates.hpp:156-173 / :386-400
-template <typename T, bool NORM> __device__ __forceinline__ Point<T> load_point(const T* xyz) {
+template <typename T, bool NORM, typename I> __device__ __forceinline__ Point<T> load_point(const I* xyz) {
     Point<T> p;
-    p.x = xyz[0];
-    p.y = xyz[1];
-    p.z = xyz[2];
+    p.x = static_cast<T>(xyz[0]); // exact when the coordinates are stored narrower than T
+    p.y = static_cast<T>(xyz[1]);
+    p.z = static_cast<T>(xyz[2]);
     p.x2 = p.x * p.x;
     p.y2 = p.y * p.y;
     p.z2 = p.z * p.z;
@@ -132,30 +134,31 @@ __device__ __forceinline__ Entry<T> finish(const Point<T>& p, Entry<T> e) {
 }
 
 // Store a finished entry into the point's staged rows.
-template <typename T, int MODE>
-__device__ __forceinline__ void put(const Rows<T>& out, int k, const Entry<T>& e) {
-    out.sph[k] = e.v;
+template <typename T, int MODE, typename O>
+__device__ __forceinline__ void put(const Rows<O>& out, int k, const Entry<T>& e) {
+    out.sph[k] = static_cast<O>(e.v);
     if constexpr (MODE >= 1) {
         const int ny = out.ny;
-        out.dsph[k] = e.gx;
-        out.dsph[ny + k] = e.gy;
-        out.dsph[2 * ny + k] = e.gz;
+        out.dsph[k] = static_cast<O>(e.gx);
+        out.dsph[ny + k] = static_cast<O>(e.gy);
+        out.dsph[2 * ny + k] = static_cast<O>(e.gz);
         if constexpr (MODE == 2) {
-            out.ddsph[k] = e.hxx;
-            out.ddsph[ny + k] = e.hxy;
-            out.ddsph[2 * ny + k] = e.hxz;
-            out.ddsph[3 * ny + k] = e.hxy;
-            out.ddsph[4 * ny + k] = e.hyy;
-            out.ddsph[5 * ny + k] = e.hyz;
-            out.ddsph[6 * ny + k] = e.hxz;
-            out.ddsph[7 * ny + k] = e.hyz;
-            out.ddsph[8 * ny + k] = e.hzz;
+            const O hxy = static_cast<O>(e.hxy), hxz = static_cast<O>(e.hxz), hyz = static_cast<O>(e.hyz);
+            out.ddsph[k] = static_cast<O>(e.hxx);
+            out.ddsph[ny + k] = hxy;
+            out.ddsph[2 * ny + k] = hxz;
+            out.ddsph[3 * ny + k] = hxy;
+            out.ddsph[4 * ny + k] = static_cast<O>(e.hyy);
+            out.ddsph[5 * ny + k] = hyz;
+            out.ddsph[6 * ny + k] = hxz;
+            out.ddsph[7 * ny + k] = hyz;
+            out.ddsph[8 * ny + k] = static_cast<O>(e.hzz);
         }
     }
 }
 
-template <typename T, int MODE, bool NORM>
-__device__ __forceinline__ void stage(const Rows<T>& out, int k, const Point<T>& p, Entry<T> e) {
+template <typename T, int MODE, bool NORM, typename O>
+__device__ __forceinline__ void stage(const Rows<O>& out, int k, const Point<T>& p, Entry<T> e) {
     put<T, MODE>(out, k, finish<T, MODE, NORM>(p, e));
 }
 
@@ -187,8 +190,8 @@ template <typename T> __device__ __forceinline__ void rotate4(unsigned turn, T& 
 }
 
 template <typename T, int MODE, bool NORM, int H, int KLO = 0, int KHI = (H + 1) * (H + 1),
-          bool ROTATE = false>
-__device__ __forceinline__ void closed_form_job(const Point<T>& p, const Rows<T>& out,
+          bool ROTATE = false, typename O = T>
+__device__ __forceinline__ void closed_form_job(const Point<T>& p, const Rows<O>& out,
                                                 [[maybe_unused]] unsigned turn = 0) {
     static_assert(MODE < 2 || H <= 1, "second derivatives in closed form stop at l = 1");
     static_assert(MODE < 2 || !ROTATE, "rotated stores are written for values and gradients");
@@ -201,14 +204,14 @@ __device__ __forceinline__ void closed_form_job(const Point<T>& p, const Rows<T>
         for (int k = KLO; k < KROT; k += 4) {
             T v0 = Y[k], v1 = Y[k + 1], v2 = Y[k + 2], v3 = Y[k + 3];
             rotate4<T>(turn, v0, v1, v2, v3);
-            out.sph[k + (turn & 3u)] = v0;
-            out.sph[k + ((turn + 1u) & 3u)] = v1;
-            out.sph[k + ((turn + 2u) & 3u)] = v2;
-            out.sph[k + ((turn + 3u) & 3u)] = v3;
+            out.sph[k + (turn & 3u)] = static_cast<O>(v0);
+            out.sph[k + ((turn + 1u) & 3u)] = static_cast<O>(v1);
+            out.sph[k + ((turn + 2u) & 3u)] = static_cast<O>(v2);
+            out.sph[k + ((turn + 3u) & 3u)] = static_cast<O>(v3);
         }
 #pragma unroll
         for (int k = KROT; k < KHI; ++k) {
-            out.sph[k] = Y[k];
+            out.sph[k] = static_cast<O>(Y[k]);
         }
     } else {
         T DX[NH], DY[NH], DZ[NH];
@@ -398,13 +401,13 @@ __device__ __forceinline__ void sequence_job(int l, int which, T z, T rxy,
 // reference's. SPLIT == false: one job computes both sides (the common factors are shared).
 // SPLIT == true: one job computes the side it is given, so that a tile with few (l, m) pairs
 // still spreads over all lanes.
-template <typename T, int MODE, bool NORM, bool SPLIT>
+template <typename T, int MODE, bool NORM, bool SPLIT, typename O>
 __device__ __forceinline__ void entry_job(int l, int m, int tri, int side, const Point<T>& p,
                                           const T* __restrict__ pk, const T* __restrict__ c,
                                           const T* __restrict__ s, const T* __restrict__ A,
                                           [[maybe_unused]] const T* __restrict__ B,
                                           [[maybe_unused]] const T* __restrict__ C,
-                                          const Rows<T>& out) {
+                                          const Rows<O>& out) {
     // tri = l(l+1)/2; pk, A, B, C already point at the (l, 0) entries of their triangular arrays
     constexpr bool GRAD = MODE >= 1;
     constexpr bool HESS = MODE == 2;

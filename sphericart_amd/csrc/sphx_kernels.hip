@@ -422,13 +422,17 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
 }
 
 // Tile size and LDS layout of the recursion kernel. Returns false when not even one point fits.
+// `elem` is the size of the numbers the kernel computes with, `out_elem` that of the coordinates
+// and the output arrays (and so of the staged rows): smaller when float arrays are evaluated in
+// float64, else the same (0).
 static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, size_t elem,
                            unsigned budget, int lds_limit, int cus, Launch* out, bool* split_sides,
-                           bool normalized = true) {
+                           bool normalized = true, size_t out_elem = 0) {
     Tiling& g = out->g;
     std::memset(&g, 0, sizeof(g));
     const int hard = mode == 2 ? 1 : 6;
     const unsigned esize = static_cast<unsigned>(elem);
+    const unsigned osize = out_elem == 0 ? esize : static_cast<unsigned>(out_elem);
     const unsigned ny = static_cast<unsigned>(l_max + 1) * (l_max + 1);
     const unsigned nyh = static_cast<unsigned>(hard + 1) * (hard + 1);
     const unsigned nrow = whole ? ny : ny - nyh;
@@ -443,18 +447,17 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // per point: the rows in every row buffer, point tables three times, iterates twice
     // staged rows are `row_stride` apart (recursion_kernel): nrow, or a little more when the rows
     // are cut so that they keep their position within 16 bytes
-    const unsigned row_stride = nrow + (whole ? 0u : nyh % (16u / esize));
+    const unsigned row_stride = nrow + (whole ? 0u : nyh % (16u / osize));
     const unsigned rows_per_point = components_of(mode) * row_stride;
     const unsigned rest_per_point = 3 * (8 + 3 * (l_max + 1)) + 2 * arrays * tri_all;
-    unsigned fixed = 0;
-    auto bytes_for = [&](unsigned S, unsigned buffers) {
-        return (S * (buffers * rows_per_point + rest_per_point) + fixed) * esize;
-    };
+    unsigned fixed = 0; // bytes
+    auto point_bytes = [&](unsigned buffers) { return buffers * rows_per_point * osize + rest_per_point * esize; };
+    auto bytes_for = [&](unsigned S, unsigned buffers) { return S * point_bytes(buffers) + fixed; };
     const unsigned limit = static_cast<unsigned>(lds_limit);
     for (;;) {
         // 24: alignment slack of the row arrays
         // + 3 lines: a staging region starts at a line boundary of its output array
-        fixed = 2 * tri_all + table_elems_for(may_split) + 24 + 2 * 3 * (128u / esize);
+        fixed = (2 * tri_all + table_elems_for(may_split) + 24) * esize + 2 * 3 * 128u;
         if (bytes_for(1, 1) <= limit || !may_split) break;
         may_split = false; // the longer job table is what does not fit
     }
@@ -466,7 +469,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     int want_buffers = switch_or(SW_ROW_BUFFERS, 0);
     if (want_buffers == 0) {
         const unsigned single = bytes_for(1, 1) <= budget
-                                    ? (budget / esize - fixed) / (rows_per_point + rest_per_point)
+                                    ? (budget - fixed) / point_bytes(1)
                                     : 1u;
         want_buffers = mode == 2 && single <= 2 ? 2 : 1;
     }
@@ -480,7 +483,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         // 611 with 7; l_max = 14: 705 with 4, 602 with 6; float32 l_max = 21: 639 with 4, 603
         // with 6; second derivatives, float64 l_max = 12: 783 with 2, 547 with 3; never more
         // than 4 % slower than the power of two below)
-        S = (budget / esize - fixed) / (buffers * rows_per_point + rest_per_point);
+        S = (budget - fixed) / point_bytes(buffers);
         if (switch_or(SW_TILE_POW2, 0) != 0) S = pow2_floor(S);
         if (S > 64) S = 64;
     }
@@ -599,14 +602,15 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
 
     // in front of every staging region, room for the part of a 128-byte line that precedes the
     // tile's run (recursion_kernel, flush_run)
-    const unsigned line = whole ? 128u / esize : 16u / esize;
+    const unsigned line = whole ? 128u / osize : 16u / osize;
     unsigned at = align4(S * row_stride + line);
     g.off_dsph = at;
     if (mode >= 1) at = align4(at + S * 3 * row_stride + line);
     g.off_ddsph = at;
     if (mode == 2) at = align4(at + S * 9 * row_stride + line);
     g.rows_elems = at;
-    at *= buffers;
+    g.tables_at = at * buffers * osize; // a multiple of 16: `at` is one of 4
+    at = 0; // from here on in numbers of the arithmetic type, counted from tables_at
     g.off_F = at;
     at += tri_all;
     g.off_Q = at;
@@ -617,7 +621,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     at += 2 * S * arrays * tri_all;
     g.off_jobs = at;
     at += table_elems_for(may_split);
-    out->lds_bytes = at * esize;
+    out->lds_bytes = g.tables_at + at * esize;
     out->threads = kRecursionThreads;
     if (out->lds_bytes > limit) return false;
 
@@ -630,7 +634,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // l_max = 16, 4 points per tile, 446 us in chunks of eight tiles, 394 in chunks of two;
     // l_max = 8, 14 points, 632 against 561 for single tiles; cfg4 562 against 528).
     g.chunk_shift = 0;
-    if (whole && S * nrow * esize >= 128u) {
+    if (whole && S * nrow * osize >= 128u) {
         const int want = switch_or(SW_CHUNK_SHIFT, S >= 5 ? 0 : (S >= 3 ? 1 : (S == 2 ? 2 : 3)));
         g.chunk_shift = want < 0 ? 0u : (want > 10 ? 10u : static_cast<unsigned>(want));
     }
@@ -828,16 +832,22 @@ static hipError_t launch_closed(const Launch& l, const T* xyz, T* sph, T* dsph, 
     return hipGetLastError();
 }
 
-template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false>
-static hipError_t launch_recursion(const Launch& l, const T* xyz, T* sph, T* dsph, T* ddsph,
-                                   hipStream_t stream) {
+template <typename X> struct AsGiven {
+    using type = X; // a parameter of this type takes no part in template argument deduction
+};
+
+template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false,
+          typename O = T>
+static hipError_t launch_recursion(const Launch& l, const typename AsGiven<O>::type* xyz,
+                                   typename AsGiven<O>::type* sph, typename AsGiven<O>::type* dsph,
+                                   typename AsGiven<O>::type* ddsph, hipStream_t stream) {
     if constexpr (!VJP && !LIST) {
         // the variant whose entry lanes take the jobs of a tile as one list
         if (l.g.points_per_pass == 0) {
-            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, false, true>(l, xyz, sph, dsph, ddsph, stream);
+            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, false, true, O>(l, xyz, sph, dsph, ddsph, stream);
         }
     }
-    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST>;
+    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O>;
     // The workgroups are persistent: launch exactly as many as are resident at once (registers
     // may allow fewer per CU than LDS does), or the last ones would run alone after the rest.
     unsigned workgroups = l.workgroups;
@@ -943,7 +953,7 @@ static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* d
 struct PlannedCall {
     // key
     unsigned generation = 0; // of the overrides; 0 = empty slot
-    int kind = 0;            // 0: forward, 1: fused product
+    int kind = 0;            // 0: forward, 1: fused product, 2: float arrays evaluated in float64
     size_t n_samples = 0;
     int l_max = 0, mode = 0, elem = 0, normalized = 0, device = 0;
     // what was planned
@@ -951,6 +961,7 @@ struct PlannedCall {
     Launch lanes;         // fused product beyond l_max = 6: the lane kernels' launch
     bool use_lanes = false;
     bool lane_groups = false;
+    bool wide = false;    // kind 2: the recursion kernel covers this shape
 };
 constexpr int kPlannedCalls = 16;
 static thread_local PlannedCall t_planned[kPlannedCalls];
@@ -1019,6 +1030,85 @@ static int forward_on(int device, const T* xyz, size_t n_samples, int l_max, int
     if (e != hipSuccess) {
         return fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
     }
+    return SPHX_OK;
+}
+
+// float arrays evaluated in float64 inside the recursion kernel (its O = float, T = double
+// variants): which shapes that covers, and the launch. Below the closed-form limit there is no
+// recursion kernel to run; the caller then evaluates into a float64 workspace and narrows.
+static bool make_wide_plan(size_t n_samples, int l_max, int mode, int lds_limit, int cus, Plan* plan,
+                           bool normalized) {
+    const int hard = mode == 2 ? 1 : 6;
+    if (l_max <= hard || l_max > SPHX_TABLE_LMAX || (n_samples + 63) / 64 > 0x7fffffffull) return false;
+    plan->lanes = false;
+    plan->closed_only = false;
+    plan->whole = true;
+    plan->split_sides = false;
+    const int whole_cu = mode == 2 ? lds_limit : 80 * 1024; // as for float64 arrays (make_plan)
+    const unsigned budget = static_cast<unsigned>(switch_or(SW_TILE_LDS_BUDGET, whole_cu));
+    bool fits = plan_recursion(n_samples, l_max, mode, true, 8, budget, lds_limit, cus, &plan->rec,
+                               &plan->split_sides, normalized, 4);
+    // rows cut at l = 7 where few points fit, by the rule for float rows (make_plan)
+    const int split_below = switch_or(SW_SPLIT_BELOW, mode == 0 ? 8 : 3);
+    if (mode < 2 && (!fits || plan->rec.g.tile < split_below)) {
+        Launch upper;
+        if (plan_recursion(n_samples, l_max, mode, false, 8, budget, lds_limit, cus, &upper,
+                           &plan->split_sides, normalized, 4)) {
+            plan->whole = false;
+            plan->rec = upper;
+            plan->rec.g.prefix_inside = 1u;
+            fits = true;
+        }
+    }
+    return fits;
+}
+
+template <int MODE, bool NORM>
+static hipError_t dispatch_wide(const Plan& plan, const float* xyz, float* sph, float* dsph, float* ddsph,
+                                hipStream_t stream) {
+    if constexpr (MODE == 2) {
+        if (plan.split_sides) {
+            return launch_recursion<double, 2, NORM, true, true, false, false, float>(plan.rec, xyz, sph, dsph, ddsph, stream);
+        }
+        return launch_recursion<double, 2, NORM, true, false, false, false, float>(plan.rec, xyz, sph, dsph, ddsph, stream);
+    } else {
+        if (plan.whole) {
+            return launch_recursion<double, MODE, NORM, true, false, false, false, float>(plan.rec, xyz, sph, dsph, ddsph, stream);
+        }
+        return launch_recursion<double, MODE, NORM, false, false, false, false, float>(plan.rec, xyz, sph, dsph, ddsph, stream);
+    }
+}
+
+// `device` is current. *taken = false: not a shape for this path, nothing was enqueued.
+static int forward_wide_on(int device, const float* xyz, size_t n_samples, int l_max, int normalized,
+                           int mode, float* sph, float* dsph, float* ddsph, void* stream, bool* taken) {
+    *taken = false;
+    int status = ensure_device_ready(device);
+    if (status != SPHX_OK) return status;
+    bool fresh = false;
+    PlannedCall* call = planned_call(2, n_samples, l_max, mode, 8, normalized != 0, device, &fresh);
+    if (fresh) {
+        call->wide = make_wide_plan(n_samples, l_max, mode, g_lds_limit[device], g_compute_units[device],
+                                    &call->plan, normalized != 0);
+        call->generation = t_switches_generation;
+    }
+    if (!call->wide) return SPHX_OK;
+    const Plan& plan = call->plan;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (normalized) {
+        e = mode == 0   ? dispatch_wide<0, true>(plan, xyz, sph, dsph, ddsph, s)
+            : mode == 1 ? dispatch_wide<1, true>(plan, xyz, sph, dsph, ddsph, s)
+                        : dispatch_wide<2, true>(plan, xyz, sph, dsph, ddsph, s);
+    } else {
+        e = mode == 0   ? dispatch_wide<0, false>(plan, xyz, sph, dsph, ddsph, s)
+            : mode == 1 ? dispatch_wide<1, false>(plan, xyz, sph, dsph, ddsph, s)
+                        : dispatch_wide<2, false>(plan, xyz, sph, dsph, ddsph, s);
+    }
+    if (e != hipSuccess) {
+        return fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
+    }
+    *taken = true;
     return SPHX_OK;
 }
 
@@ -1198,8 +1288,10 @@ static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int
 // and Q_l^l = (2l-1)!! leave the range of the type from l = 29 (NaN and inf in
 // the outputs) and high-|m| entries come out as exact zeros from l of about 20
 // (sphericart/include/templates.hpp:54-97 evaluated in float). This path, which
-// a caller must ask for, widens xyz, runs the float64 kernels into a workspace
-// and rounds every result once.
+// a caller must ask for, evaluates in float64 and rounds every result once:
+// beyond the closed forms in one launch of the recursion kernel's mixed variant
+// (forward_wide_on), else by widening xyz, running the float64 kernels into a
+// workspace and narrowing the rows (below).
 // ---------------------------------------------------------------------------
 constexpr unsigned kConvertThreads = 256;
 
@@ -1335,7 +1427,11 @@ static int forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, in
 
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     void* owned = nullptr;
-    if (workspace == nullptr) {
+    // Beyond the closed forms the recursion kernel does it all in one launch: it reads the float
+    // coordinates, computes in float64 and stages float rows. No workspace is touched then.
+    bool fused = false;
+    status = forward_wide_on(device, xyz, n_samples, l_max, normalized, mode, sph, dsph, ddsph, stream, &fused);
+    if (status == SPHX_OK && !fused && workspace == nullptr) {
         // No workspace given: one of our own for at most 256 MiB worth of points at a time, taken
         // from and returned to the device's memory pool in stream order, so that the call still
         // only enqueues (an allocation that waits for the device would stall the caller).
@@ -1350,7 +1446,7 @@ static int forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, in
         }
         workspace = owned;
     }
-    if (status == SPHX_OK) {
+    if (status == SPHX_OK && !fused) {
         status = via_f64_chunks(device, xyz, n_samples, l_max, normalized, mode, sph, dsph, ddsph, workspace,
                                 workspace_bytes, stream);
     }

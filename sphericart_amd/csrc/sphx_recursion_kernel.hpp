@@ -54,17 +54,27 @@ constexpr unsigned kRecursionThreads = 512;
 // and spill a few registers; with 170 registers and one workgroup per CU, l_max = 12 float64
 // gradients took 800 us instead of 513 us. The second-derivative kernels keep what they need
 // (forced to 128 they spill in the entry jobs: 918 us against 558 us at l_max = 10, float64).
-template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false>
-__global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling g, const T* __restrict__ xyz,
-                                                                     T* __restrict__ sph,
-                                                                     T* __restrict__ dsph,
-                                                                     T* __restrict__ ddsph) {
+//
+// O: the type of xyz and of the output arrays, T the type of the arithmetic. O = float with
+// T = double evaluates float arrays in float64: the coordinates are widened as they are read, the
+// tables and iterates are float64, and every result is rounded once, as it is staged. The staged
+// rows are rows of O, so a tile holds as many points as in the float kernel's and the flush is
+// that kernel's.
+template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false,
+          typename O = T>
+__global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling g, const O* __restrict__ xyz,
+                                                                     O* __restrict__ sph,
+                                                                     O* __restrict__ dsph,
+                                                                     O* __restrict__ ddsph) {
     static_assert(!VJP || (MODE == 1 && !SPLIT), "the fused product is built on the gradient kernel");
+    static_assert(!VJP || std::is_same<T, O>::value, "the fused product stages what it computes");
     constexpr int H = MODE == 2 ? 1 : 6;
     constexpr unsigned NYH = (H + 1) * (H + 1);
     constexpr unsigned ARRAYS = MODE + 1; // iterate arrays per point: A, B, C
     constexpr unsigned NT = kRecursionThreads;
-    T* lds = reinterpret_cast<T*>(lds_raw);
+    // the row buffers, rows of O, come first; everything else is T and counts from g.tables_at
+    O* row_lds = reinterpret_cast<O*>(lds_raw);
+    T* lds = reinterpret_cast<T*>(lds_raw + g.tables_at);
     const unsigned tid = threadIdx.x;
     const unsigned lane = tid & 63u;
     const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6); // the same for all lanes: scalar
@@ -77,7 +87,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
     // long; a stride that equals ny modulo 16 bytes, with the first row placed like its HBM
     // address modulo 16 bytes, puts every staged row at the same position within 16 bytes as
     // its destination, so that the copy is 16-byte loads and stores on both sides.
-    constexpr unsigned W16 = 16u / static_cast<unsigned>(sizeof(T));
+    constexpr unsigned W16 = 16u / static_cast<unsigned>(sizeof(O));
     const unsigned row_stride = nrow + skip % W16;
     const unsigned tri_all = (L + 1) * (L + 2) / 2;
 
@@ -165,7 +175,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
             const unsigned long long i = first + lane;
             if (i < g.n_samples) {
                 const Point<T> p = load_point<T, NORM>(xyz + i * 3);
-                Rows<T> rows;
+                Rows<O> rows;
                 rows.ny = static_cast<int>(ny);
                 rows.sph = sph + i * ny;
                 rows.dsph = MODE >= 1 ? dsph + i * 3 * ny : nullptr;
@@ -215,10 +225,10 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
         const unsigned n = (batch << g.az_shift) + lane / S;
         const unsigned s = lane % S;
         if (lane < batch_tiles * S && s < valid_in(n)) {
-            const T* src = xyz + (static_cast<unsigned long long>(tile_of(n)) * S + s) * 3;
-            rx = src[0];
-            ry = src[1];
-            rz = src[2];
+            const O* src = xyz + (static_cast<unsigned long long>(tile_of(n)) * S + s) * 3;
+            rx = static_cast<T>(src[0]);
+            ry = static_cast<T>(src[1]);
+            rz = static_cast<T>(src[2]);
         }
     };
     // stage one of a batch of tiles (wave 0; lane == tid there)
@@ -279,10 +289,10 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
     const unsigned wide_first = 64 * entry_first_wave;
     const unsigned wide_lanes = 64 * (entry_end_wave - entry_first_wave);
 
-    constexpr unsigned LINE = 128u / static_cast<unsigned>(sizeof(T)); // elements per 128-byte line
+    constexpr unsigned LINE = 128u / static_cast<unsigned>(sizeof(O)); // elements per 128-byte line
     // position within its 128-byte line of element `element` of an output array
-    auto phase_of = [](const T* array, unsigned long long element) -> unsigned {
-        return static_cast<unsigned>((reinterpret_cast<uintptr_t>(array) / sizeof(T) + element) % LINE);
+    auto phase_of = [](const O* array, unsigned long long element) -> unsigned {
+        return static_cast<unsigned>((reinterpret_cast<uintptr_t>(array) / sizeof(O) + element) % LINE);
     };
 
     // Where the rows of tile n start within their staging regions. WHOLE: element 0 of a region
@@ -308,7 +318,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
         if constexpr (WHOLE) {
             const unsigned valid = valid_in(n);
             if (lane < valid) {
-                T* staged = lds + buffer * g.rows_elems;
+                O* staged = row_lds + buffer * g.rows_elems;
                 const Phases ph = phases_of(n);
                 const T* rec = point_data(n, lane);
                 Point<T> p;
@@ -319,7 +329,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
                 p.y2 = rec[4];
                 p.z2 = rec[5];
                 p.ir = rec[6];
-                Rows<T> rows;
+                Rows<O> rows;
                 rows.ny = static_cast<int>(ny);
                 rows.sph = staged + ph.sph + lane * ny;
                 rows.dsph = staged + g.off_dsph + ph.dsph + lane * 3 * ny;
@@ -331,7 +341,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
                     // Not for float64 and not for values alone, where the selects cost registers
                     // that the kernel does not have to spare (values: 68 -> 89, and l_max = 9 lost
                     // its third workgroup per CU, 80 -> 106 us).
-                    constexpr bool MAY_ROTATE = sizeof(T) == 4 && MODE == 1;
+                    constexpr bool MAY_ROTATE = sizeof(T) == 4 && MODE == 1; // not where T and O differ
                     if (MAY_ROTATE && (ny & 31u) == 0) {
                         const unsigned turn = lane & 3u;
                         if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 8, true>(p, rows, turn);
@@ -360,7 +370,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
     // stage three of tile n, into row buffer `buffer` (the entry waves)
     auto entry_stage = [&](unsigned n, unsigned buffer) {
         const unsigned valid = valid_in(n);
-        T* staged = lds + buffer * g.rows_elems;
+        O* staged = row_lds + buffer * g.rows_elems;
         const unsigned t = tid - wide_first;
         const Phases ph = phases_of(n);
         const unsigned phase_sph = ph.sph, phase_dsph = ph.dsph, phase_ddsph = ph.ddsph;
@@ -372,7 +382,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
         const T* itA = nullptr;
         const T* itB = nullptr;
         const T* itC = nullptr;
-        Rows<T> rows;
+        Rows<O> rows;
         rows.ny = static_cast<int>(row_stride);
         rows.sph = rows.dsph = rows.ddsph = nullptr;
         auto take_point = [&](unsigned s) {
@@ -447,7 +457,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
         constexpr int WHOLE_UNROLL = decltype(lone)::value ? SPHX_FLUSH_UNROLL : 1;
         const unsigned valid = valid_in(n);
         const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
-        const T* staged = lds + buffer * g.rows_elems;
+        const O* staged = row_lds + buffer * g.rows_elems;
         if constexpr (WHOLE) {
             // The tile's run of `len` elements of one output array starts at element `at` of that
             // array. Only whole 128-byte lines go out with vector stores. The line in which the
@@ -456,13 +466,13 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
             // staged in; at the ends of a chunk the partial lines are stored element by element.
             const bool starts = (n & chunk_mask) == 0;
             const bool ends = (n & chunk_mask) == chunk_mask || valid_in(n + 1) == 0;
-            T* carry_to = lds + (streaming ? (buffer ^ 1u) : buffer) * g.rows_elems;
-            auto flush_run = [&](unsigned region_offset, T* array, unsigned long long at, unsigned len) {
-                using V = typename Pack<T>::type;
-                constexpr unsigned W = Pack<T>::width;
-                T* region = lds + buffer * g.rows_elems + region_offset;
+            O* carry_to = row_lds + (streaming ? (buffer ^ 1u) : buffer) * g.rows_elems;
+            auto flush_run = [&](unsigned region_offset, O* array, unsigned long long at, unsigned len) {
+                using V = typename Pack<O>::type;
+                constexpr unsigned W = Pack<O>::width;
+                O* region = row_lds + buffer * g.rows_elems + region_offset;
                 const unsigned phase = phase_of(array, at);
-                T* line0 = array + (at - phase); // HBM address of region element 0
+                O* line0 = array + (at - phase); // HBM address of region element 0
                 const unsigned lo = starts ? phase : 0u; // first element that holds data
                 const unsigned hi = phase + len;
                 const unsigned full_lo = (lo + LINE - 1u) / LINE * LINE;
@@ -480,12 +490,12 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
                             for (int u = 0; u < WHOLE_UNROLL; ++u) hold[u] = in[v + u * count];
 #pragma unroll
                             for (int u = 0; u < WHOLE_UNROLL; ++u) {
-                                emit<T, SPHX_STREAMING_STORES>(hold[u], out + v + u * count);
+                                emit<O, SPHX_STREAMING_STORES>(hold[u], out + v + u * count);
                             }
                         }
                     }
                     for (; v < nvec; v += count) {
-                        emit<T, SPHX_STREAMING_STORES>(in[v], out + v);
+                        emit<O, SPHX_STREAMING_STORES>(in[v], out + v);
                     }
                     tail_from = full_hi;
                 } else {
@@ -497,7 +507,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
                 // tail: stored if the chunk ends here, else handed to the next tile
                 const unsigned tail = hi - tail_from;
                 if (ft < tail) {
-                    const T value = region[tail_from + ft];
+                    const O value = region[tail_from + ft];
                     if (ends) {
                         line0[tail_from + ft] = value;
                     } else if (carry_to + region_offset != region || tail_from != 0) {
@@ -512,17 +522,17 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
             // one run per (point, component) row, dealt to the waves in turn. In float64 the
             // vector stores start at a line boundary of the row (l_max = 20 gradients, 100k
             // points: 491 -> 381 us); in float32 that measured the same or 2 % worse.
-            constexpr bool LINES = sizeof(T) == 8;
+            constexpr bool LINES = sizeof(O) == 8;
             const unsigned waves = count / 64;
             for (unsigned r = __builtin_amdgcn_readfirstlane(ft >> 6); r < valid * components_of(MODE); r += waves) {
                 // rows [0, valid) are values, the next 3 * valid are gradients
                 if (r < valid) {
-                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL, LINES>(
+                    copy_out<O, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL, LINES>(
                         staged + phase_of(sph, first * ny + skip) % W16 + r * row_stride,
                         sph + (first + r) * ny + skip, nrow, nrow, 0, 0, ft & 63u, 64);
                 } else {
                     const unsigned q = r - valid;
-                    copy_out<T, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL, LINES>(
+                    copy_out<O, SPHX_STREAMING_STORES, false, SPHX_FLUSH_UNROLL, LINES>(
                         staged + g.off_dsph + phase_of(dsph, first * 3 * ny + skip) % W16 + q * row_stride,
                         dsph + (first * 3 + q) * ny + skip, nrow, nrow, 0, 0, ft & 63u, 64);
                 }
@@ -540,7 +550,7 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
         if constexpr (VJP) {
             const unsigned valid = valid_in(n);
             const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
-            const T* staged = lds + buffer * g.rows_elems + g.off_dsph;
+            const T* staged = row_lds + buffer * g.rows_elems + g.off_dsph; // O is T here
             const T* upstream = sph;
             T* xyz_grad = dsph;
             if (wave == 0) return;

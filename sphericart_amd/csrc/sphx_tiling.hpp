@@ -49,8 +49,11 @@ struct Tiling {
     unsigned prefix_inside; // rows that start at l = 7: the recursion kernel writes l <= 6 too
     // LDS carve-up, in elements of T: the row buffers come first, rows_elems each, with the
     // gradient and second-derivative rows at off_dsph and off_ddsph inside a buffer; the other
-    // offsets count from the start of dynamic LDS
+    // offsets count from the start of dynamic LDS. (recursion_kernel: the row offsets are in
+    // elements of the output arrays, the others in numbers of the arithmetic type and count
+    // from byte tables_at.)
     unsigned rows_elems, off_dsph, off_ddsph, off_F, off_Q, off_pts, off_iter, off_jobs;
+    unsigned tables_at;
 };
 
 extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];

@@ -102,21 +102,26 @@ class _BaseHarmonics:
     def _compute_via_float64(self, xyz, sph, dsph, ddsph):
         derivatives = 2 if ddsph is not None else (1 if dsph is not None else 0)
         n_samples = xyz.shape[0]
-        # a workspace from torch's allocator keeps the call asynchronous; at most 256 MiB, the
-        # library walks over the points in chunks of what it holds
-        wanted = self._lib.sphx_forward_f32_via_f64_workspace(n_samples, self._l_max, derivatives)
-        floor = self._lib.sphx_forward_f32_via_f64_workspace(min(n_samples, 64), self._l_max, derivatives)
-        size = max(min(wanted, 256 << 20), floor)
-        workspace = torch.empty(size, dtype=torch.uint8, device=xyz.device)
+        # Beyond the closed forms the library evaluates in one launch and needs no workspace (if a
+        # shape should not fit that launch it takes one from the device's pool, in stream order).
+        # Below, a workspace from torch's allocator: at most 256 MiB, the library walks over the
+        # points in chunks of what it holds.
+        workspace, size = None, 0
+        if self._l_max <= (1 if derivatives == 2 else 6):
+            wanted = self._lib.sphx_forward_f32_via_f64_workspace(n_samples, self._l_max, derivatives)
+            floor = self._lib.sphx_forward_f32_via_f64_workspace(min(n_samples, 64), self._l_max, derivatives)
+            size = max(min(wanted, 256 << 20), floor)
+            workspace = torch.empty(size, dtype=torch.uint8, device=xyz.device)
         with torch.cuda.device(xyz.device):
             stream = torch.cuda.current_stream()
             status = self._lib.sphx_forward_f32_via_f64(
                 xyz.data_ptr(), n_samples, self._l_max, self._normalized, derivatives,
                 sph.data_ptr(), dsph.data_ptr() if dsph is not None else None,
                 ddsph.data_ptr() if ddsph is not None else None,
-                workspace.data_ptr(), size, stream.cuda_stream,
+                workspace.data_ptr() if workspace is not None else None, size, stream.cuda_stream,
             )
-            workspace.record_stream(stream)
+            if workspace is not None:
+                workspace.record_stream(stream)
         if status != 0:
             raise RuntimeError(self._lib.sphx_last_error().decode())
 

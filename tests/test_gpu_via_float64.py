@@ -70,6 +70,45 @@ def test_equals_the_rounded_float64_oracle(oracle, library, l_max, mode, normali
                 assert same_numbers(g.cpu().numpy(), w).all(), workspace_bytes
 
 
+@pytest.mark.parametrize("l_max,mode,n", [(7, "values", 20000), (9, "gradients", 6000), (2, "hessians", 9000),
+                                          (8, "hessians", 3000), (14, "hessians", 900), (17, "gradients", 3001),
+                                          (20, "gradients", 2500), (24, "values", 2000), (32, "gradients", 1200),
+                                          (40, "values", 700), (24, "hessians", 150), (48, "gradients", 130)])
+@pytest.mark.parametrize("normalized", [True, False])
+def test_one_launch_beyond_the_closed_forms(library, l_max, mode, normalized, n):
+    """Beyond the closed forms the recursion kernel itself computes in float64 and stages float
+    rows. Checked against the float64 arrays of ``sphx_forward_f64`` for the widened points
+    (pinned against the oracle in test_gpu_parity.py), rounded by torch: both conversions are
+    exact or correctly rounded, so the numbers must be the same. Sizes: many tiles per
+    workgroup, whole and cut rows, tiles of one point to dozens. The workspace handed in must
+    come back untouched."""
+    rng = np.random.default_rng(l_max * 3 + n)
+    xyz = special_points(np.float32, rng, n)
+    xyz_dev = torch.from_numpy(xyz).cuda()
+    k, ny = MODE_INDEX[mode], (l_max + 1) ** 2
+    announce("via float64 in one launch", l_max, mode, normalized, n)
+    status, want = run_launch_layer(library, xyz_dev.double(), l_max, normalized, mode)
+    assert status == 0, library.sphx_last_error()
+    workspace_bytes = 4096
+    workspace = torch.full((workspace_bytes,), 0xAB, dtype=torch.uint8, device="cuda")
+    opts = dict(dtype=torch.float32, device="cuda")
+    got = (
+        torch.full((n, ny), -7.0, **opts),
+        torch.full((n, 3, ny), -7.0, **opts) if k >= 1 else None,
+        torch.full((n, 3, 3, ny), -7.0, **opts) if k >= 2 else None,
+    )
+    status = library.sphx_forward_f32_via_f64(
+        xyz_dev.data_ptr(), n, l_max, int(bool(normalized)), k, got[0].data_ptr(),
+        got[1].data_ptr() if got[1] is not None else None, got[2].data_ptr() if got[2] is not None else None,
+        workspace.data_ptr(), workspace_bytes, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert status == 0, library.sphx_last_error()
+    assert bool((workspace == 0xAB).all())
+    for g, w in zip(got, want):
+        if g is not None:
+            assert same_numbers(g.cpu().numpy(), w.to(torch.float32).cpu().numpy()).all()
+
+
 def test_finite_where_float32_arithmetic_is_not(oracle, library):
     """l_max = 40, points on the unit sphere: the float32 kernels (and the reference) give NaN
     from l = 29 on, the float64 evaluation gives numbers of order one."""
