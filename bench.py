@@ -57,7 +57,7 @@ PEAK_HBM_GBPS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     "cfg1": 26866092,
     "cfg2": 76091891,
-    "cfg3": 796482282,
+    "cfg3": 796356224,
     "cfg4": 3008449407,
     "cfg5": 3881148774,
     "cfg3:backward": int((394551.2 * 2.0 + 11719.3) * 1024),

@@ -287,7 +287,7 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
 // gradients_lanes_kernel: 64, 32 or 16 points per workgroup with their four rows and tables in
 // LDS. Returns false when too few points would be resident on a CU for it to pay.
 static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int lds_limit, int cus,
-                                Launch* out) {
+                                Launch* out, bool normalized = true) {
     Tiling& g = out->g;
     std::memset(&g, 0, sizeof(g));
     const unsigned esize = static_cast<unsigned>(elem);
@@ -295,7 +295,8 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     const unsigned vec = 16u / esize;
     auto stride_of = [&](unsigned block) { return (block * (esize / 4u)) % 8u == 0 ? block + vec : block; };
     const unsigned s_stride = stride_of(ny), d_stride = stride_of(3u * ny);
-    const unsigned table_stride = (3u * static_cast<unsigned>(l_max + 1)) | 1u;
+    // (closed forms only, l_max <= 6: no tables)
+    const unsigned table_stride = l_max <= 6 ? 0u : (3u * static_cast<unsigned>(l_max + 1)) | 1u;
     const unsigned limit = static_cast<unsigned>(lds_limit);
     // Which tile: the one that keeps most points resident on a CU (tile times the workgroups
     // that fit), a tile of 16 counted at three quarters because it leaves three lanes in four
@@ -326,6 +327,11 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
         const unsigned b = (ot + t * table_stride) * esize;
         if (b > limit) continue;
         unsigned score = (limit / b) * t * (t >= 32 ? 4u : 3u);
+        // l_max = 6, closed forms only: 32 points per workgroup, half the lanes idle, but twice as
+        // many workgroups in different phases on a CU (1M points, float32: 127 us against 140 us
+        // with 64 points; a tile of 32 rows of 49 numbers is a whole number of 128-byte lines,
+        // tiles of 24, 28, 36, 40, 48 points took 143-164 us)
+        if (l_max == 6 && t == 32) score = 1u << 28;
         if (t == few) score = 1u << 29;
         if (forced_tile == t) score = 1u << 30;
         if (score > best || (score == best && best_groups < 2)) {
@@ -357,7 +363,11 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     // channels on eight waves are faster, l_max = 12: 357 against 411).
     // (few points: one workgroup per CU, occupancy is no concern and eight waves shorten the
     // longest chain of work in the workgroup)
-    int waves = switch_or(SW_GRADIENT_LANES_WAVES, l_max <= 8 && tile != few ? 4 : 8);
+    // (closed forms only, l_max <= 6: eight; six for normalised float32 at l_max = 6, 127 us
+    // against 130 us with eight and 136-138 us with four or five)
+    const int by_shape = l_max <= 6 ? (l_max == 6 && elem == 4 && normalized && tile != few ? 6 : 8)
+                                    : (l_max <= 8 && tile != few ? 4 : 8);
+    int waves = switch_or(SW_GRADIENT_LANES_WAVES, by_shape);
     waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
     out->threads = 64u * static_cast<unsigned>(waves);
     out->lds_bytes = bytes;
@@ -684,6 +694,21 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     plan->closed_only = l_max <= hard;
     plan->whole = true;
     plan->split_sides = false;
+    // Gradients in closed form, where the rows of a tile are so long that few single-wave
+    // workgroups of closed_form_kernel share a CU: the lanes kernel instead, which cuts the closed
+    // forms in slices for six or eight waves and flushes with all of them. Measured, us, against
+    // closed_form_kernel: l_max = 6 float32 1M points 127 against 134 (solid 133 against 134), 300k
+    // 43 against 49, 100k 17 against 23, 10k 5.0 against 6.8; float64 500k 125 against 148 (solid
+    // 131 against 152), 100k 29 against 42; l_max = 5 float64 680k 135 against 149; l_max = 4
+    // float32 2M 131 against 141, 100k 8.7 against 11.3. Not below: l_max = 3 float32 100k 8.0
+    // against 7.3, l_max = 4 float64 1M 139 against 132, l_max = 5 float32 140 against 142.
+    const bool in_slices = l_max == 6 || (l_max == 5 && elem == 8) || (l_max == 4 && elem == 4 && normalized);
+    if (plan->closed_only && lane_kernels && mode == 1 && in_slices && switch_or(SW_GRADIENT_LANES, 1) != 0 &&
+        plan_gradient_lanes(n_samples, l_max, elem, lds_limit, cus, &plan->closed, normalized)) {
+        plan->closed_only = false;
+        plan->lanes = true;
+        return SPHX_OK;
+    }
     if (plan->closed_only) {
         plan_closed(n_samples, l_max, l_max, mode, elem, &plan->closed);
         return SPHX_OK;
@@ -877,7 +902,10 @@ static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* d
         }
         if constexpr (MODE == 1) {
             const Launch& l = plan.closed;
-            auto kernel = gradients_lanes_kernel<T, NORM>;
+            if (l.g.l_max < 4) return hipErrorInvalidValue; // never planned
+            auto kernel = l.g.l_max >= 6   ? gradients_lanes_kernel<T, NORM, 6>
+                          : l.g.l_max == 5 ? gradients_lanes_kernel<T, NORM, 5>
+                                           : gradients_lanes_kernel<T, NORM, 4>;
             if (l.lds_bytes > 64u * 1024u) {
                 unsigned unused = 0;
                 hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &unused);

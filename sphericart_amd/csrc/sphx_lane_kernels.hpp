@@ -172,12 +172,39 @@ __global__ __launch_bounds__(kValuesMaxThreads) void values_kernel(Tiling g, con
 // g.rows_elems / g.off_dsph / g.off_ddsph: stride of a point's values row, start of
 // the gradient rows, stride of a point's three gradient rows; g.off_pts, g.off_iter:
 // the tables and their stride.
+//
+// l_max <= 6 (H = l_max): closed forms only, no channels, no tables. The same kernel then is the
+// closed forms of 16 to 64 points cut in slices for the waves of a workgroup, where
+// closed_form_kernel has one wave evaluate all of them and then flush alone: with rows of four
+// arrays in LDS few of its single-wave workgroups fit on a CU, and each is a long chain of
+// arithmetic followed by a long run of stores.
 // ---------------------------------------------------------------------------
-template <typename T, bool NORM>
+// where the eight slices of the closed forms begin: by l for H = 6 (a slice that ends with an l
+// evaluates nothing of the next), in equal parts below
+template <int H> __device__ constexpr int closed_slice_start(int j) {
+    constexpr int NH = (H + 1) * (H + 1);
+    if (H == 6) {
+        constexpr int by_l[9] = {0, 9, 16, 25, 31, 36, 41, 45, 49};
+        return by_l[j];
+    }
+    return j * NH / 8;
+}
+
+template <typename T, bool NORM, int H, int J = 0, typename Pick>
+__device__ __forceinline__ void closed_form_slices(const Point<T>& p, const Rows<T>& rows, Pick mine) {
+    if constexpr (J < 8) {
+        constexpr int LO = closed_slice_start<H>(J), HI = closed_slice_start<H>(J + 1);
+        if constexpr (HI > LO) {
+            if (mine(static_cast<unsigned>(J))) closed_form_job<T, 1, NORM, H, LO, HI>(p, rows);
+        }
+        closed_form_slices<T, NORM, H, J + 1>(p, rows, mine);
+    }
+}
+
+template <typename T, bool NORM, int H = 6>
 __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tiling g, const T* __restrict__ xyz,
                                                                            T* __restrict__ sph,
                                                                            T* __restrict__ dsph) {
-    constexpr int H = 6;
     using V = typename Pack<T>::type;
     constexpr unsigned W = Pack<T>::width;
     T* lds = reinterpret_cast<T*>(lds_raw);
@@ -209,7 +236,7 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
     // before the rows are complete: a wave with channels makes the (c_m, s_m, 2(m+1)z) tables
     // itself (a tenth of a channel's work; the waves write the same numbers to the same places
     // and each reads back what it wrote).
-    const unsigned channels = static_cast<unsigned>(L - H);
+    const unsigned channels = H == 6 ? static_cast<unsigned>(L - H) : 0u;
     const bool has_channel = wave < channels;
     const unsigned spare = waves > channels ? waves - channels : 0u; // waves without a channel
     auto my_slice = [&](unsigned j) -> bool {
@@ -234,16 +261,9 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
                 tab[3 * m + 2] = tz;
             }
         }
-        if (my_slice(0)) closed_form_job<T, 1, NORM, H, 0, 9>(p, rows);
-        if (my_slice(1)) closed_form_job<T, 1, NORM, H, 9, 16>(p, rows);
-        if (my_slice(2)) closed_form_job<T, 1, NORM, H, 16, 25>(p, rows);
-        if (my_slice(3)) closed_form_job<T, 1, NORM, H, 25, 31>(p, rows);
-        if (my_slice(4)) closed_form_job<T, 1, NORM, H, 31, 36>(p, rows);
-        if (my_slice(5)) closed_form_job<T, 1, NORM, H, 36, 41>(p, rows);
-        if (my_slice(6)) closed_form_job<T, 1, NORM, H, 41, 45>(p, rows);
-        if (my_slice(7)) closed_form_job<T, 1, NORM, H, 45, 49>(p, rows);
+        closed_form_slices<T, NORM, H>(p, rows, my_slice);
     }
-    if (lane < valid) {
+    if (H == 6 && lane < valid) {
         const T x = p.x, y = p.y;
         const T rxy = p.x2 + p.y2;
         const T zero = static_cast<T>(0.0);

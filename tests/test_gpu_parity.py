@@ -46,6 +46,28 @@ def test_sweep_against_oracle(oracle, dtype, normalized, mode):
         check(got, want, (l_max, normalized, mode))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("normalized", [True, False])
+def test_closed_form_gradients_by_both_kernels(oracle, library, switches, dtype, normalized):
+    """Gradients at l_max <= 6 have two kernels: one wave per 64 points, or the closed forms in
+    slices for the waves of a workgroup (the planner's choice at l_max = 4-6). Both against the
+    oracle, for every l_max, at sizes that leave tiles of 32, 64 and N / CUs points ragged."""
+    rng = np.random.default_rng(7)
+    for l_max in range(1, 7):
+        for n in (1, 33, 777, 20001):
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, normalized, "gradients")
+            xyz_dev = torch.from_numpy(xyz).cuda()
+            for lanes in (1, 0):
+                switches("SPHX_GRADIENT_LANES", lanes)
+                announce("closed-form gradients", np.dtype(dtype).name, normalized, l_max, n, "lanes", lanes)
+                status, got = run_launch_layer(library, xyz_dev, l_max, normalized, "gradients")
+                torch.cuda.synchronize()
+                assert status == 0, library.sphx_last_error()
+                got = tuple(None if g is None else g.cpu().numpy() for g in got)
+                check(got, want, (l_max, normalized, n, lanes))
+
+
 @pytest.mark.parametrize("name", CONFIGS)
 def test_golden_benchmark_configurations(name):
     xyz, l_max, normalized, mode, want = config_case(name)

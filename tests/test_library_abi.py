@@ -69,9 +69,14 @@ def _plan(library, n, l_max, mode, f64):
 
 
 def test_launch_plans(library):
+    # gradients at l_max = 6: the closed forms in slices for six waves, 32 points per workgroup
     status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 6, 1, False)
+    assert status == 0 and tile == 32 and threads == 384
+    assert lds == 32 * 4 * 49 * 4 and groups == 31256  # 8 XCD stretches of 3907 tiles
+    # values at l_max = 6: one wave per 64 points
+    status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 6, 0, False)
     assert status == 0 and tile == 64 and threads == 64
-    assert lds == 64 * 4 * 49 * 4 and groups == 15632  # 8 XCD stretches of 1954 tiles
+    assert lds == 64 * 49 * 4 and groups == 15632  # 8 XCD stretches of 1954 tiles
     for n, l_max, mode, f64 in ((10_000, 8, 1, True), (100_000, 16, 2, True), (200_000, 32, 1, False), (5, 20, 2, False)):
         status, (tile, threads, lds, groups) = _plan(library, n, l_max, mode, f64)
         assert status == 0
