@@ -123,14 +123,15 @@ static int ensure_device_ready(int device) {
 // only if SPHX_DEBUG_SWITCHES is set to something other than 0.
 enum Switch : int {
     SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_FLUSH_WAVES, SW_GRADIENT_LANES, SW_GRADIENT_LANES_TILE,
-    SW_GRADIENT_LANES_WAVES, SW_HESSIAN_LANES, SW_JOB_LIST, SW_PREFIX_INSIDE, SW_ROW_BUFFERS,
+    SW_GRADIENT_LANES_WAVES, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST, SW_PREFIX_INSIDE, SW_ROW_BUFFERS,
     SW_SEQUENCE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_TILE, SW_TILE_LDS_BUDGET,
     SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
     SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_COUNT
 };
 static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_FLUSH_WAVES", "SPHX_GRADIENT_LANES",
-    "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_HESSIAN_LANES", "SPHX_JOB_LIST",
+    "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_HESSIAN_LANES", "SPHX_HESSIAN_LANES_PARTS",
+    "SPHX_JOB_LIST",
     "SPHX_PREFIX_INSIDE", "SPHX_ROW_BUFFERS", "SPHX_SEQUENCE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
@@ -376,7 +377,8 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
 
 // hessians_lanes_kernel: 64 or 32 points per workgroup with their thirteen rows, tables and
 // iterates in LDS. Returns false when 32 points do not fit.
-static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds_limit, Launch* out) {
+static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds_limit, Launch* out,
+                               bool normalized = true) {
     Tiling& g = out->g;
     std::memset(&g, 0, sizeof(g));
     const unsigned esize = static_cast<unsigned>(elem);
@@ -386,8 +388,17 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
     const unsigned s_stride = stride_of(ny), d_stride = stride_of(3u * ny), dd_stride = stride_of(9u * ny);
     const unsigned table_stride = (3u * static_cast<unsigned>(l_max + 1)) | 1u;
     const unsigned channels = static_cast<unsigned>(l_max - 1);
-    const unsigned most = kHessianLaneThreads / 64u;
-    const unsigned waves = channels < most ? channels : most;
+    const unsigned most = (elem == 4 ? hessian_lane_threads<float>() : hessian_lane_threads<double>()) / 64u;
+    // Waves per channel, each with a part of its m: two where one or two channels would leave the
+    // workgroup with one or two waves (80 MB of output, us, one against two: float32 l_max = 3
+    // 99 against 83, solid 80 against 70, 20 000 points 10.9 against 9.1; l_max = 2 74 against 70,
+    // solid 58 against 61; float64 l_max = 3 solid 85 against 73, normalised 105 against 151).
+    const bool shared = (l_max == 3 && (elem == 4 || !normalized)) || (l_max == 2 && elem == 4 && normalized);
+    unsigned parts = static_cast<unsigned>(switch_or(SW_HESSIAN_LANES_PARTS, shared ? 2 : 1));
+    if (parts != 1 && parts != 2 && parts != 4) parts = 1;
+    while (parts > 1 && parts > most) parts /= 2;
+    const unsigned slots = channels * parts <= most ? channels : most / parts;
+    const unsigned waves = slots * parts;
     const unsigned limit = static_cast<unsigned>(lds_limit);
     unsigned tile = 0, off_d = 0, off_dd = 0, off_t = 0, off_s = 0, bytes = 0, best = 0, best_groups = 0;
     for (unsigned t = 64; t >= 32; t /= 2) {
@@ -426,6 +437,7 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
     g.off_jobs = off_s;
     g.jobs_per_point = table_stride;
     out->workgroups = g.tiles_per_xcd * 8u;
+    g.sequence_waves = parts;
     out->threads = 64u * waves;
     out->lds_bytes = bytes;
     return true;
@@ -722,7 +734,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     const int hessian_lanes = switch_or(SW_HESSIAN_LANES, 1);
     const bool hessian_lanes_pay = elem == 4 ? l_max <= 5 : (l_max == 3 || (l_max == 5 && normalized));
     if (lane_kernels && mode == 2 && (hessian_lanes == 2 || (hessian_lanes == 1 && hessian_lanes_pay)) &&
-        plan_hessian_lanes(n_samples, l_max, elem, lds_limit, &plan->closed)) {
+        plan_hessian_lanes(n_samples, l_max, elem, lds_limit, &plan->closed, normalized)) {
         plan->lanes = true;
         return SPHX_OK;
     }

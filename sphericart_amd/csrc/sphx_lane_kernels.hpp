@@ -389,11 +389,17 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
 // g.rows_elems, g.off_dsph, g.off_ddsph strides, g.off_F, g.off_Q starts of the gradient and
 // second-derivative rows; g.off_pts, g.off_iter: tables [c | s | 2(m+1)z] and their stride;
 // g.off_jobs, g.jobs_per_point: the waves' scratch [A | B | C] and a lane's share of it.
+// g.sequence_waves (1, 2 or 4): the waves that share one channel, each taking a part of its m.
 // ---------------------------------------------------------------------------
 constexpr unsigned kHessianLaneThreads = 256; // float64 entries need more than 128 registers
+template <typename T> constexpr unsigned hessian_lane_threads() {
+    // (float32 with 512 threads, 128 registers per lane: l_max = 2-5 5-15 % slower with the
+    // same number of waves)
+    return kHessianLaneThreads;
+}
 
 template <typename T, bool NORM>
-__global__ __launch_bounds__(kHessianLaneThreads) void hessians_lanes_kernel(Tiling g, const T* __restrict__ xyz,
+__global__ __launch_bounds__(hessian_lane_threads<T>()) void hessians_lanes_kernel(Tiling g, const T* __restrict__ xyz,
                                                                             T* __restrict__ sph,
                                                                             T* __restrict__ dsph,
                                                                             T* __restrict__ ddsph) {
@@ -440,15 +446,24 @@ __global__ __launch_bounds__(kHessianLaneThreads) void hessians_lanes_kernel(Til
         T* A = lds + g.off_jobs + (wave * tile + lane) * g.jobs_per_point;
         T* B = A + (L + 1);
         T* C = B + (L + 1);
+        // The waves that share a channel each run its three recursions (a few percent of the
+        // entries' work) and take a part of its m: few channels then still fill the workgroup.
+        const unsigned parts = g.sequence_waves;
+        const unsigned slots = waves / parts; // channels in work at a time
+        const unsigned slot = wave % slots, part = wave / slots;
         for (unsigned i = 0; static_cast<int>(i) < L - H; ++i) {
-            const unsigned pos = i % waves;
-            if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
+            const unsigned pos = i % slots;
+            if ((((i / slots) & 1u) ? slots - 1u - pos : pos) != slot) continue;
             const int l = L - static_cast<int>(i);
             const int tri = l * (l + 1) / 2;
             sequence_job<T>(l, 0, p.z, rxy, cQ, tmz, A);
             sequence_job<T>(l, 1, p.z, rxy, cQ, tmz, B);
             sequence_job<T>(l, 2, p.z, rxy, cQ, tmz, C);
-            for (int m = l; m >= 0; --m) {
+            // m = l .. 0 in `parts` runs of nearly equal length, the first from the top
+            const int count = l + 1;
+            const int m_hi = l - static_cast<int>(part) * count / static_cast<int>(parts);
+            const int m_lo = l + 1 - static_cast<int>(part + 1) * count / static_cast<int>(parts);
+            for (int m = m_hi; m >= m_lo; --m) {
                 entry_job<T, 2, NORM, false>(l, m, tri, 0, p, cF + tri, c, sn, A, B, C, rows);
             }
         }

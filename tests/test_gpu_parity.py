@@ -68,6 +68,28 @@ def test_closed_form_gradients_by_both_kernels(oracle, library, switches, dtype,
                 check(got, want, (l_max, normalized, n, lanes))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("normalized", [True, False])
+def test_second_derivative_lanes_with_shared_channels(oracle, library, switches, dtype, normalized):
+    """The one-point-per-lane kernel for second derivatives at l_max 2-5, with one, two and four
+    waves per l channel (each wave a part of the channel's m), against the oracle."""
+    rng = np.random.default_rng(9)
+    for l_max in range(2, 6):
+        for n in (3, 100, 4097):
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, normalized, "hessians")
+            xyz_dev = torch.from_numpy(xyz).cuda()
+            for parts in (1, 2, 4):
+                switches("SPHX_HESSIAN_LANES", 2)
+                switches("SPHX_HESSIAN_LANES_PARTS", parts)
+                announce("second derivatives, lanes", np.dtype(dtype).name, normalized, l_max, n, "parts", parts)
+                status, got = run_launch_layer(library, xyz_dev, l_max, normalized, "hessians")
+                torch.cuda.synchronize()
+                assert status == 0, library.sphx_last_error()
+                got = tuple(None if g is None else g.cpu().numpy() for g in got)
+                check(got, want, (l_max, normalized, n, parts))
+
+
 @pytest.mark.parametrize("name", CONFIGS)
 def test_golden_benchmark_configurations(name):
     xyz, l_max, normalized, mode, want = config_case(name)
