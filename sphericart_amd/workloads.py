@@ -2,9 +2,11 @@
 
 Points are generated on the host in float64 from a counter-based generator
 (SplitMix64 over the point index, so any slice of a cloud can be produced on its
-own and the numbers do not depend on the numpy version), rounded once to the
-working precision, and that one array is what both the GPU path and any CPU
-checker are fed with.
+own), rounded once to the working precision, and that one array is what both
+the GPU path and any CPU checker are fed with. Only integer arithmetic, +, -, *,
+/ and square roots are used, all of which IEEE 754 rounds correctly: no
+function of the C library or of numpy's vector math is involved, so the clouds
+are the same bits on every machine.
 """
 
 from dataclasses import dataclass
@@ -33,15 +35,33 @@ def uniform(seed, n, stream, first=0):
 
 
 def normal(seed, n, stream, first=0):
-    """Standard normal deviates by Box-Muller from two uniform streams."""
-    u1 = uniform(seed, n, 2 * stream, first)
-    u2 = uniform(seed, n, 2 * stream + 1, first)
-    return np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
+    """Deviates of mean 0 and variance 1: the sum of twelve uniform streams minus six
+    (Irwin-Hall; bell-shaped within +-6, which is all the point clouds need)."""
+    total = uniform(seed, n, 12 * stream, first)
+    for j in range(1, 12):
+        total = total + uniform(seed, n, 12 * stream + j, first)
+    return total - 6.0
 
 
 def _directions(seed, n, first):
-    v = np.stack([normal(seed, n, 10 + a, first) for a in range(3)], axis=1)
-    return v / np.linalg.norm(v, axis=1, keepdims=True)
+    """Uniform directions after Marsaglia (1972): (a, b) uniform in the unit disk, s = a^2 + b^2,
+    direction (2a sqrt(1-s), 2b sqrt(1-s), 1-2s). A point whose pair falls outside the disk takes
+    the pair of the next attempt's streams, so every point still depends on its index alone."""
+    a = np.zeros(n)
+    b = np.zeros(n)
+    s = np.full(n, 2.0)
+    for attempt in range(64):
+        todo = s >= 1.0
+        if not todo.any():
+            break
+        ta = 2.0 * uniform(seed, n, 100 + 2 * attempt, first) - 1.0
+        tb = 2.0 * uniform(seed, n, 101 + 2 * attempt, first) - 1.0
+        a = np.where(todo, ta, a)
+        b = np.where(todo, tb, b)
+        s = np.where(todo, ta * ta + tb * tb, s)
+    s = np.minimum(s, 1.0)  # (no point gets here unplaced: 0.215^64)
+    root = np.sqrt(1.0 - s)
+    return np.stack([2.0 * a * root, 2.0 * b * root, 1.0 - 2.0 * s], axis=1)
 
 
 def _on_axis(xyz, radius, every, first):
@@ -109,8 +129,10 @@ def _cfg4(seed, n, first):
 
 
 def _cfg5(seed, n, first):
-    lo, hi = np.log(1e-2), np.log(1e2)
-    radius = np.exp(lo + (hi - lo) * uniform(seed, n, 20, first))
+    # radii from 1e-2 over thirteen octaves (to 82), the same share of the points in each:
+    # 0.01 m 2^e with e uniform in 0 .. 12 and m uniform in [1, 2)
+    octave = np.floor(13.0 * uniform(seed, n, 21, first))
+    radius = 0.01 * np.ldexp(1.0 + uniform(seed, n, 20, first), octave.astype(np.int64))
     xyz = _directions(seed, n, first) * radius[:, None]
     return _on_axis(xyz, radius, 200, first)
 
@@ -120,7 +142,7 @@ _GENERATORS = {"cfg1": _cfg1, "cfg2": _cfg2, "cfg3": _cfg3, "cfg4": _cfg4, "cfg5
 
 WORKLOADS = {
     "cfg1": Workload(
-        "cfg1", "spherical, l_max=8, f64, values+gradients, 10k points, xyz ~ N(0,1)",
+        "cfg1", "spherical, l_max=8, f64, values+gradients, 10k points, xyz bell-shaped with variance 1",
         8, "f64", True, "gradients", 10_000, 1001,
     ),
     "cfg2": Workload(
@@ -140,7 +162,7 @@ WORKLOADS = {
     "cfg5": Workload(
         "cfg5",
         "spherical, l_max=32, f32, values+gradients, 200k points, uniform directions, "
-        "r log-uniform in [1e-2,1e2), 0.5% of the points on the +-z axis",
+        "r spread evenly over the 13 octaves of [1e-2, 82), 0.5% of the points on the +-z axis",
         32, "f32", True, "gradients", 200_000, 1005,
     ),
     # not one of the reference's configurations: values alone beyond the closed forms, the shape
