@@ -610,15 +610,38 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     entry_cost(g.sequence_waves, split_sides); // leaves `wide` as it will be
     g.jobs_per_point = *split_sides ? jobs_split : jobs;
     g.magic_jobs = magic_of(g.jobs_per_point);
+    {
+        // the kinds of jobs in the order of the job table (recursion_kernel)
+        const unsigned sides = *split_sides ? 2u : 1u;
+        const unsigned levels = static_cast<unsigned>(l_max - hard);
+        unsigned bulk = 0;
+        for (int l = hard + 1; l <= l_max; ++l) bulk += l >= 2 ? static_cast<unsigned>(l - 2) : 0u;
+        g.kind_jobs[0] = sides * bulk;
+        g.kind_jobs[1] = sides * levels;
+        g.kind_jobs[2] = levels;
+        for (int k = 0; k < 3; ++k) g.kind_magic[k] = g.kind_jobs[k] ? magic_of(g.kind_jobs[k]) : 0u;
+    }
     g.points_per_pass = per_pass(g.jobs_per_point);
-    // The list costs a few instructions per job: only where it saves a round (1.5 GB of output,
-    // gradients float32 l_max = 17, 20, 30: 466, 563, 442 -> 379, 453, 371 us; second derivatives
-    // float64 l_max = 14: 580 -> 426; with equal rounds, l_max = 32: 390 -> 423). It did not pay
-    // with two points per tile (l_max = 32, three rounds instead of four: 387 -> 424 us) nor
-    // where four points go side by side anyway (second derivatives float32 l_max = 8: 580 -> 631).
+    // The jobs of a tile as one list. Values: the list is point after point and costs a few
+    // instructions per job, so only where it saves a round and few points go side by side anyway
+    // (float32 l_max = 40, 48: 527, 477 -> 468, 428 us). With derivatives the list is ordered by
+    // kind of job first (recursion_kernel), which keeps the lanes of a wave on one branch of
+    // entry_job: side by side, the 77 one-sided jobs of a point at l_max = 8 with second
+    // derivatives put all seven kinds into every wave and 41 % of the lanes were active on
+    // average. 400 MB of output, us, points side by side against the list: second derivatives
+    // float32 l_max = 6, 8, 10, 12 (22, 14, 9, 6 points per tile) 164, 157, 138, 144 -> 115, 117,
+    // 117, 115 (solid 108, 97, 97, 97 -> 98, 84, 89, 93); float64 l_max = 4, 8, 12, 16 146, 165,
+    // 135, 123 -> 106, 104, 99, 96; gradients float32 l_max = 18, 24, 26 124, 123, 116 -> 109, 116,
+    // 108, float64 l_max = 12, 13, 14 122, 127, 127 -> 107, 111, 115. With one or two points per
+    // tile the list loses unless it saves a round (float32 gradients l_max = 32, 40: 113, 101 ->
+    // 117, 119; l_max = 36, five rounds instead of six, 111 -> 108, solid 127 -> 112), and so it
+    // does for solid second derivatives in float64 with four points (cfg4 535 -> 559 us).
     const int want_list = switch_or(SW_JOB_LIST, -1);
     const bool saves_a_round = (S * g.jobs_per_point + wide - 1) / wide < rounds_by_point(g.jobs_per_point);
-    if (want_list != 0 && saves_a_round && (want_list > 0 || (S >= 3 && g.points_per_pass <= 2))) {
+    const bool by_shape = mode == 0 ? saves_a_round && S >= 3 && g.points_per_pass <= 2
+                                    : (mode == 2 && elem == 8 && !normalized ? S >= 5 : S >= 3) ||
+                                          (saves_a_round && S >= 2);
+    if (want_list == 2 || (want_list == 1 && saves_a_round) || (want_list < 0 && by_shape)) {
         g.points_per_pass = 0;
     }
 
@@ -732,13 +755,22 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // Second derivatives at small l_max: one point per lane where that was measured to be faster
     // than the recursion kernel (SPHX_HESSIAN_LANES: 0 never, 2 wherever the rows fit).
     const int hessian_lanes = switch_or(SW_HESSIAN_LANES, 1);
-    const bool hessian_lanes_pay = elem == 4 ? l_max <= 5 : (l_max == 3 || (l_max == 5 && normalized));
+    // (Since the recursion kernel takes its jobs as a list ordered by kind it wins from l_max = 4
+    // on; 400 MB of output, us, lanes against recursion: float32 l_max = 2 87, 99 (solid 72, 82),
+    // l_max = 3 104, 108 (solid 89, 100), l_max = 4 147, 107 (solid 113, 87), l_max = 5 130, 112
+    // (solid 99, 86); float64 l_max = 3 129, 114 (solid 91, 102), l_max = 5 163, 107; 20 000 points
+    // float32 l_max = 3 9.0, 11.2, l_max = 4 17.9, 13.5.)
+    const bool hessian_lanes_pay = elem == 4 ? l_max <= 3 : (l_max == 3 && !normalized);
     if (lane_kernels && mode == 2 && (hessian_lanes == 2 || (hessian_lanes == 1 && hessian_lanes_pay)) &&
         plan_hessian_lanes(n_samples, l_max, elem, lds_limit, &plan->closed, normalized)) {
         plan->lanes = true;
         return SPHX_OK;
     }
-    if (lane_kernels && mode == 1 && switch_or(SW_GRADIENT_LANES, 1) != 0 &&
+    // (float32 from l_max = 14 on the recursion kernel with its jobs as a list ordered by kind is
+    // ahead: 600 MB of output, lanes against recursion, l_max = 13 151, 150 us; 14 169, 153; 15 189,
+    // 171; 16 174, 154; solid 14 152, 144; 16 160, 144. SPHX_GRADIENT_LANES=2: lanes wherever they fit.)
+    const int gradient_lanes = switch_or(SW_GRADIENT_LANES, 1);
+    if (lane_kernels && mode == 1 && gradient_lanes != 0 && (gradient_lanes == 2 || elem == 8 || l_max <= 13) &&
         plan_gradient_lanes(n_samples, l_max, elem, lds_limit, cus, &plan->closed)) {
         plan->lanes = true;
         return SPHX_OK;

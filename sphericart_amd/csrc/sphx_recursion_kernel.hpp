@@ -416,20 +416,50 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
         };
         const unsigned per_point = g.jobs_per_point;
         if constexpr (LIST) {
-            // The jobs of the tile's points as one list, point after point, dealt to the wide
-            // lanes round after round: only the last round can leave lanes idle. The host
-            // launches this variant where it saves rounds (l_max = 20: 203 jobs per point on 320
-            // lanes, seven points in five rounds instead of seven); a lane looks at every job's
-            // point. (Both loops in one kernel made either slower by some 5 %.)
+            // The jobs of the tile's points as one list, dealt to the wide lanes round after
+            // round: only the last round can leave lanes idle (l_max = 20: 203 jobs per point on
+            // 320 lanes, seven points in five rounds instead of seven); a lane looks at every
+            // job's point. (Both loops in one kernel made either slower by some 5 %.)
+            // With derivatives the list is ordered by kind first (the bulk of all points, then |m| = l of all
+            // points, |m| = l - 1, m = 0) and by point within a kind, so that the lanes of a wave
+            // share a branch of entry_job except where two kinds meet: three places per tile
+            // instead of three per point.
             const unsigned total = valid * per_point;
+            if constexpr (MODE == 0) {
+                // values: an entry is three multiplications, the order by kind does not pay
+                // (float32 l_max = 40, 400k points: 824 us point after point, 889 us by kind)
+                unsigned current = ~0u;
+                for (unsigned q = t; q < total; q += wide_lanes) {
+                    const unsigned s = __umulhi(q, g.magic_jobs); // exact: q * per_point < 2^32
+                    if (s != current) {
+                        current = s;
+                        take_point(s);
+                    }
+                    take_job(q - s * per_point);
+                }
+                return;
+            }
+            const unsigned b0 = g.kind_jobs[0], b1 = g.kind_jobs[1], b3 = g.kind_jobs[2];
+            const unsigned t1 = valid * b0, t2 = t1 + valid * b1, t3 = t2 + valid * b1;
             unsigned current = ~0u;
             for (unsigned q = t; q < total; q += wide_lanes) {
-                const unsigned s = __umulhi(q, g.magic_jobs); // exact: q * per_point < 2^32
+                unsigned r, b, first_job, magic;
+                if (q < t1) {
+                    r = q, b = b0, first_job = 0, magic = g.kind_magic[0];
+                } else if (q < t2) {
+                    r = q - t1, b = b1, first_job = b0, magic = g.kind_magic[1];
+                } else if (q < t3) {
+                    r = q - t2, b = b1, first_job = b0 + b1, magic = g.kind_magic[1];
+                } else {
+                    r = q - t3, b = b3, first_job = b0 + 2 * b1, magic = g.kind_magic[2];
+                }
+                // exact: r * b < 2^32; a single job per point has no such multiplier in 32 bits
+                const unsigned s = b == 1 ? r : __umulhi(r, magic);
                 if (s != current) {
                     current = s;
                     take_point(s);
                 }
-                take_job(q - s * per_point);
+                take_job(first_job + (r - s * b));
             }
         } else {
             // One pass takes the jobs of as many points as fit side by side in the wide lanes

@@ -54,6 +54,9 @@ struct Tiling {
     // from byte tables_at.)
     unsigned rows_elems, off_dsph, off_ddsph, off_F, off_Q, off_pts, off_iter, off_jobs;
     unsigned tables_at;
+    // recursion_kernel, job-list variant: jobs per point of the kinds bulk / |m| = l and l - 1 /
+    // m = 0 (the order of the job table), and ceil(2^32 / .) of each (0 where there are none)
+    unsigned kind_jobs[3], kind_magic[3];
 };
 
 extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];

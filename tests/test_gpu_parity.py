@@ -90,6 +90,36 @@ def test_second_derivative_lanes_with_shared_channels(oracle, library, switches,
                 check(got, want, (l_max, normalized, n, parts))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("mode", ["gradients", "hessians"])
+def test_job_list_by_kind_and_points_side_by_side(oracle, library, switches, dtype, mode):
+    """The recursion kernel deals the entry jobs of a tile either point by point, side by side,
+    or as one list ordered by kind of job. Both, with tiles of one to many points (single jobs
+    per kind at l_max = 2 and 3 included), against the oracle."""
+    rng = np.random.default_rng(13)
+    shapes = [(2, 0), (3, 0), (4, 3), (7, 0), (9, 5), (13, 0), (18, 2)] if mode == "hessians" else \
+        [(7, 0), (8, 3), (12, 0), (17, 0), (21, 4), (26, 0), (33, 1)]
+    for l_max, tile in shapes:
+        for normalized in (True, False):
+            n = 1500
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, normalized, mode)
+            xyz_dev = torch.from_numpy(xyz).cuda()
+            for job_list in (2, 0):
+                switches("SPHX_GRADIENT_LANES", 0)
+                switches("SPHX_HESSIAN_LANES", 0)
+                switches("SPHX_JOB_LIST", job_list)
+                if tile:
+                    switches("SPHX_TILE", tile)
+                announce("job list", np.dtype(dtype).name, mode, normalized, l_max, "tile", tile, "list", job_list)
+                status, got = run_launch_layer(library, xyz_dev, l_max, normalized, mode)
+                torch.cuda.synchronize()
+                assert status == 0, library.sphx_last_error()
+                got = tuple(None if g is None else g.cpu().numpy() for g in got)
+                check(got, want, (l_max, normalized, tile, job_list))
+            library.sphx_reset_switches()
+
+
 @pytest.mark.parametrize("name", CONFIGS)
 def test_golden_benchmark_configurations(name):
     xyz, l_max, normalized, mode, want = config_case(name)
