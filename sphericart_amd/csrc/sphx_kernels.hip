@@ -483,18 +483,14 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         if (bytes_for(1, 1) <= limit || !may_split) break;
         may_split = false; // the longer job table is what does not fit
     }
-    // Two row buffers (tile n flushed by a wave of its own while tile n+1 is computed) pay off
-    // where the rows of a point are so long that a single buffer holds one or two points and
-    // the flush of such a tile is long: measured with second derivatives (l_max = 16, float64:
-    // 770 us against 810 us). With many points per tile, or with the rows cut in two kernels,
-    // one buffer flushed by all waves measured faster.
-    int want_buffers = switch_or(SW_ROW_BUFFERS, 0);
-    if (want_buffers == 0) {
-        const unsigned single = bytes_for(1, 1) <= budget
-                                    ? (budget - fixed) / point_bytes(1)
-                                    : 1u;
-        want_buffers = mode == 2 && single <= 2 ? 2 : 1;
-    }
+    // Two row buffers (tile n flushed by a wave of its own while tile n+1 is computed) are built
+    // and tested but no longer chosen: they once paid where a single buffer holds one or two
+    // points (second derivatives l_max = 16, float64: 770 us against 810 us), but a wave that
+    // flushes alone waits for its own LDS loads most of the time and the entry waves lose a wave
+    // and half the points per tile. 400 MB of output, us, two buffers against one: second
+    // derivatives float32 l_max = 20, 22, 28 157, 122, 167 against 121, 100, 105 (solid 109, 96
+    // against 88, 79); float64 l_max = 20, 22 149, 134 against 126, 105; l_max = 24 the same.
+    int want_buffers = switch_or(SW_ROW_BUFFERS, 1);
     unsigned buffers = want_buffers == 2 ? 2u : 1u;
     if (bytes_for(1, buffers) > limit) buffers = 1;
     if (bytes_for(1, buffers) > limit) return false;
@@ -635,12 +631,20 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // 108, float64 l_max = 12, 13, 14 122, 127, 127 -> 107, 111, 115. With one or two points per
     // tile the list loses unless it saves a round (float32 gradients l_max = 32, 40: 113, 101 ->
     // 117, 119; l_max = 36, five rounds instead of six, 111 -> 108, solid 127 -> 112), and so it
-    // does for solid second derivatives in float64 with four points (cfg4 535 -> 559 us).
+    // does for solid second derivatives in float64 where the points side by side fill the lanes
+    // anyway (cfg4, four points, 94 % of the lanes: 535 -> 559 us; l_max = 15, 83 %: 98 -> 84 us).
+    // Second derivatives with two points per tile: the list unless the sides are split (float64
+    // l_max = 20, 22 156, 138 -> 126, 105 us; solid float32 l_max = 22 83 -> 79; float32 with split
+    // sides 100 -> 108).
     const int want_list = switch_or(SW_JOB_LIST, -1);
     const bool saves_a_round = (S * g.jobs_per_point + wide - 1) / wide < rounds_by_point(g.jobs_per_point);
-    const bool by_shape = mode == 0 ? saves_a_round && S >= 3 && g.points_per_pass <= 2
-                                    : (mode == 2 && elem == 8 && !normalized ? S >= 5 : S >= 3) ||
-                                          (saves_a_round && S >= 2);
+    // lanes that points side by side would fill, in percent
+    const unsigned fill = 100u * g.points_per_pass * g.jobs_per_point / wide;
+    const bool cheap_jobs = mode == 2 && elem == 8 && !normalized; // no chain rule, few branches
+    const bool by_shape = mode == 0   ? saves_a_round && S >= 3 && g.points_per_pass <= 2
+                          : mode == 1 ? S >= 3 || (saves_a_round && S >= 2)
+                                      : (S >= 3 && !(cheap_jobs && fill >= 90u)) || (S == 2 && !*split_sides) ||
+                                            (saves_a_round && S >= 2);
     if (want_list == 2 || (want_list == 1 && saves_a_round) || (want_list < 0 && by_shape)) {
         g.points_per_pass = 0;
     }
