@@ -582,7 +582,12 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // rounds of the entry waves per tile, in tenths of two-sided jobs, with `waves` sequence waves
     auto entry_cost = [&](unsigned waves, bool* split) {
         wide = kRecursionThreads - 64 * (1 + waves + g.flush_waves);
-        *split = may_split && one_side_costs * rounds(jobs_split) < 10 * rounds(jobs);
+        // (with two or more points per tile the jobs go as a list ordered by kind, which fills the
+        // lanes without splitting, and the two-sided job shares the common factors: 400 MB of
+        // output, us, split against not, normalised float32 l_max = 4, 8, 16, 20 110, 115, 108,
+        // 121 -> 104, 100, 96, 113; solid l_max = 6, 12 94, 92 -> 83, 83; with one point per tile
+        // splitting stays, l_max = 24, 28 117, 104 against 184, 166)
+        *split = may_split && S < 2 && one_side_costs * rounds(jobs_split) < 10 * rounds(jobs);
         return *split ? one_side_costs * rounds(jobs_split) : 10 * rounds(jobs);
     };
     // A second sequence wave takes a wave from the entries. One is enough where it saves the
