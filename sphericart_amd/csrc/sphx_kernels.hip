@@ -122,16 +122,17 @@ static int ensure_device_ready(int device) {
 // looked at. The variables of the same names are read once, when the library is first used, and
 // only if SPHX_DEBUG_SWITCHES is set to something other than 0.
 enum Switch : int {
-    SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_FLUSH_WAVES, SW_GRADIENT_LANES, SW_GRADIENT_LANES_TILE,
-    SW_GRADIENT_LANES_WAVES, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST, SW_PREFIX_INSIDE, SW_ROW_BUFFERS,
+    SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_FLUSH_WAVES, SW_GRADIENT_LANES, SW_GRADIENT_LANES_PARTS,
+    SW_GRADIENT_LANES_TILE, SW_GRADIENT_LANES_WAVES, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST,
+    SW_PREFIX_INSIDE, SW_ROW_BUFFERS,
     SW_SEQUENCE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_TILE, SW_TILE_LDS_BUDGET,
     SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
     SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_COUNT
 };
 static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_FLUSH_WAVES", "SPHX_GRADIENT_LANES",
-    "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_HESSIAN_LANES", "SPHX_HESSIAN_LANES_PARTS",
-    "SPHX_JOB_LIST",
+    "SPHX_GRADIENT_LANES_PARTS", "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_HESSIAN_LANES",
+    "SPHX_HESSIAN_LANES_PARTS", "SPHX_JOB_LIST",
     "SPHX_PREFIX_INSIDE", "SPHX_ROW_BUFFERS", "SPHX_SEQUENCE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
@@ -372,6 +373,17 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
     out->threads = 64u * static_cast<unsigned>(waves);
     out->lds_bytes = bytes;
+    // Few points, one or two channels: two waves per channel, each with half of its m (the longest
+    // chain of the one workgroup a CU has is then half a channel or two slices of the closed
+    // forms, not a whole channel). Measured on one device, one wave per channel against two, us:
+    // float64 10 000 points l_max = 8 10.0 against 9.0, l_max = 7 8.7 against 7.8; float32
+    // l_max = 8 7.6 against 6.7, 2 000 points 7.0 against 5.6. With three channels two waves are
+    // left for the eight slices and nothing is gained (float64 l_max = 9 10.2 against 10.5), with
+    // four channels none (l_max = 10: 9.5 against 9.1 in float32, 9.9 against 10.2 in float64).
+    const unsigned channels = l_max > 6 ? static_cast<unsigned>(l_max - 6) : 0u;
+    const bool halves = tile == few && channels >= 1 && channels <= 2 && waves == 8;
+    const int parts = switch_or(SW_GRADIENT_LANES_PARTS, halves ? 2 : 1);
+    g.sequence_waves = parts == 2 && 2u * channels <= static_cast<unsigned>(waves) ? 2u : 1u;
     return true;
 }
 

@@ -237,10 +237,15 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
     // itself (a tenth of a channel's work; the waves write the same numbers to the same places
     // and each reads back what it wrote).
     const unsigned channels = H == 6 ? static_cast<unsigned>(L - H) : 0u;
-    const bool has_channel = wave < channels;
-    const unsigned spare = waves > channels ? waves - channels : 0u; // waves without a channel
+    // g.sequence_waves = 2 (few points, the time of the call is that of one workgroup; the host sees
+    // to it that twice the channels leave waves over): two waves share a channel, the first
+    // takes the upper half of its m, the second runs the recursions bare down to the lower half.
+    const unsigned parts = g.sequence_waves == 2 ? 2u : 1u;
+    const unsigned channel_waves = channels * parts;
+    const bool has_channel = wave < channel_waves;
+    const unsigned spare = waves > channel_waves ? waves - channel_waves : 0u; // waves without a channel
     auto my_slice = [&](unsigned j) -> bool {
-        return spare != 0 ? wave == channels + j % spare : (waves - 1u - wave) == j % waves;
+        return spare != 0 ? wave == channel_waves + j % spare : (waves - 1u - wave) == j % waves;
     };
     if (lane < valid) {
         p = load_point<T, NORM>(xyz + (first + lane) * 3);
@@ -280,8 +285,12 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
         };
         for (unsigned i = 0; static_cast<int>(i) < L - H; ++i) {
             const unsigned pos = i % waves;
-            if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
+            if (parts == 1 ? (((i / waves) & 1u) ? waves - 1u - pos : pos) != wave : i != wave / 2u) continue;
             const int l = L - static_cast<int>(i);
+            // the values of m this wave turns into entries: all, or one half of l .. 0 (m = l and
+            // m = l - 1 cost less than the others, the lower half has the bare steps before it)
+            const int m_top = parts == 1 || (wave & 1u) == 0 ? l : l / 2 - 1;
+            const int m_bottom = parts == 1 || (wave & 1u) != 0 ? 0 : l / 2;
             const int tri = l * (l + 1) / 2;
             const int mid = 2 * tri;
             const T* pk = cF + tri;
@@ -293,7 +302,7 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
             T b1 = qk[-1];        // Q_{l-1}^{l-1} at m = l - 1
             T c1 = tab[3 * (l - 1)], s1 = tab[3 * (l - 1) + 1];
             T c0 = tab[3 * l], s0 = tab[3 * l + 1];
-            {
+            if (m_top >= l) {
                 // m = l (templates_core.hpp:122-152)
                 auto pq = a2 * pk[l];
                 const T vp = pq * c0, vn = pq * s0;
@@ -305,7 +314,7 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
             s0 = s1;
             c1 = tab[3 * (l - 2)];
             s1 = tab[3 * (l - 2) + 1];
-            {
+            if (m_top >= l - 1 && m_bottom <= l - 1) {
                 // m = l - 1 (:154-198)
                 const T pkm = pk[l - 1];
                 auto pq = a1 * pkm;
@@ -315,7 +324,7 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
                 stage<T, 1, NORM>(rows, mid + l - 1, p, entry(vp, pq * c1, pq * -s1, pdq * c0));
                 stage<T, 1, NORM>(rows, mid - (l - 1), p, entry(vn, pq * s1, pq * c1, pdq * s0));
             }
-            for (int m = l - 2; m >= 1; --m) {
+            for (int m = l - 2; m >= 1 && m >= m_bottom; --m) {
                 // :201-390
                 c0 = c1;
                 s0 = s1;
@@ -324,24 +333,26 @@ __global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tili
                 const T tz = tab[3 * m + 2];
                 const T a0 = qk[m] * (tz * a1 + rxy * a2);
                 const T b0 = kb[m] * (tz * b1 + rxy * b2);
-                const T pkm = pk[m];
-                auto pq = a0 * pkm;
-                const T vp = pq * c0, vn = pq * s0;
-                pq *= m;
-                auto pdq = pkm * b1;
-                auto pdqx = pdq * x;
-                auto pdqy = pdq * y;
-                auto pdz = pkm * (l + m) * b0;
-                stage<T, 1, NORM>(rows, mid + m, p,
-                                  entry(vp, (pdqx * c0 + pq * c1), (pdqy * c0 + pq * -s1), pdz * c0));
-                stage<T, 1, NORM>(rows, mid - m, p,
-                                  entry(vn, (pdqx * s0 + pq * s1), (pdqy * s0 + pq * c1), pdz * s0));
+                if (m <= m_top) {
+                    const T pkm = pk[m];
+                    auto pq = a0 * pkm;
+                    const T vp = pq * c0, vn = pq * s0;
+                    pq *= m;
+                    auto pdq = pkm * b1;
+                    auto pdqx = pdq * x;
+                    auto pdqy = pdq * y;
+                    auto pdz = pkm * (l + m) * b0;
+                    stage<T, 1, NORM>(rows, mid + m, p,
+                                      entry(vp, (pdqx * c0 + pq * c1), (pdqy * c0 + pq * -s1), pdz * c0));
+                    stage<T, 1, NORM>(rows, mid - m, p,
+                                      entry(vn, (pdqx * s0 + pq * s1), (pdqy * s0 + pq * c1), pdz * s0));
+                }
                 a2 = a1;
                 a1 = a0;
                 b2 = b1;
                 b1 = b0;
             }
-            {
+            if (m_bottom == 0) {
                 // m = 0 (:392-426)
                 const T tz = tab[2];
                 const T a0 = qk[0] * (tz * a1 + rxy * a2);

@@ -91,6 +91,30 @@ def test_second_derivative_lanes_with_shared_channels(oracle, library, switches,
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("normalized", [True, False])
+def test_gradient_lanes_with_shared_channels(oracle, library, switches, dtype, normalized):
+    """The one-point-per-lane kernel for gradients above the closed forms, with one and two waves
+    per l channel (each wave half of the channel's m), few points (where the planner picks two
+    waves for one or two channels) and many, against the oracle."""
+    rng = np.random.default_rng(21)
+    for l_max in (7, 8, 9, 10):
+        for n in (1, 50, 3000, 10000, 40000):
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, normalized, "gradients")
+            xyz_dev = torch.from_numpy(xyz).cuda()
+            for parts in (1, 2):
+                switches("SPHX_GRADIENT_LANES", 2)
+                switches("SPHX_GRADIENT_LANES_WAVES", 8)
+                switches("SPHX_GRADIENT_LANES_PARTS", parts)
+                announce("gradients, lanes", np.dtype(dtype).name, normalized, l_max, n, "parts", parts)
+                status, got = run_launch_layer(library, xyz_dev, l_max, normalized, "gradients")
+                torch.cuda.synchronize()
+                assert status == 0, library.sphx_last_error()
+                got = tuple(None if g is None else g.cpu().numpy() for g in got)
+                check(got, want, (l_max, normalized, n, parts))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("mode", ["gradients", "hessians"])
 def test_job_list_by_kind_and_points_side_by_side(oracle, library, switches, dtype, mode):
     """The recursion kernel deals the entry jobs of a tile either point by point, side by side,
