@@ -123,18 +123,19 @@ static int ensure_device_ready(int device) {
 // only if SPHX_DEBUG_SWITCHES is set to something other than 0.
 enum Switch : int {
     SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_FLUSH_WAVES, SW_GRADIENT_LANES, SW_GRADIENT_LANES_PARTS,
-    SW_GRADIENT_LANES_TILE, SW_GRADIENT_LANES_WAVES, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST,
+    SW_GRADIENT_LANES_TILE, SW_GRADIENT_LANES_WAVES, SW_GROUP_THREADS, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST,
     SW_PREFIX_INSIDE, SW_ROW_BUFFERS,
-    SW_SEQUENCE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_TILE, SW_TILE_LDS_BUDGET,
+    SW_SEQUENCE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
     SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
     SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_COUNT
 };
 static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_FLUSH_WAVES", "SPHX_GRADIENT_LANES",
-    "SPHX_GRADIENT_LANES_PARTS", "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_HESSIAN_LANES",
+    "SPHX_GRADIENT_LANES_PARTS", "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_GROUP_THREADS",
+    "SPHX_HESSIAN_LANES",
     "SPHX_HESSIAN_LANES_PARTS", "SPHX_JOB_LIST",
     "SPHX_PREFIX_INSIDE", "SPHX_ROW_BUFFERS", "SPHX_SEQUENCE_WAVES", "SPHX_SPLIT_BELOW",
-    "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
+    "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
     "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE",
 };
@@ -455,13 +456,35 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
     return true;
 }
 
+// Threads per workgroup of the recursion kernel: 512, two workgroups to a CU, or 1024, one
+// workgroup with all of the CU's LDS and tiles of twice as many points (gradients, and second
+// derivatives in float32; not the fused product, not values, whose entries are too cheap for
+// thirteen waves of them, not second derivatives in float64, whose entry jobs need more than the
+// 128 registers a lane of sixteen waves has). Two workgroups of 512 on a CU run their stages and
+// their flushes against each other as chance has it, and a tile of one or two points leaves the
+// entry lanes and the sequence lanes half idle in their last rounds; one workgroup of 1024
+// measured, 1.2 GB of output, us, 512 against 1024: gradients float32 l_max = 14, 20, 24, 28,
+// 32, 36 283, 306, 323, 329, 331, 342 against 245, 249, 259, 253, 267, 268 (l_max = 40 288
+// against 290); float64 l_max = 12, 16, 20, 24, 32 303, 307, 320, 271, 266 against 239, 233,
+// 252, 248, 249; second derivatives float32 l_max = 4, 8, 12, 16, 20, 24 252, 262, 271, 258,
+// 334, 361 against 231, 239, 238, 238, 245, 266; solid harmonics alike. With few points (below
+// 4 096) 512 threads stay: more workgroups have a tile then.
+// SPHX_GROUP_THREADS = 512 or 1024 overrides the rule.
+static unsigned group_threads(size_t n_samples, int mode, size_t elem, bool forward) {
+    const bool exists = forward && (mode == 1 || (mode == 2 && elem == 4));
+    if (!exists) return kRecursionThreads;
+    const int want = switch_or(SW_GROUP_THREADS, 0);
+    if (want == 512 || want == 1024) return static_cast<unsigned>(want);
+    return n_samples >= 4096 ? 2 * kRecursionThreads : kRecursionThreads;
+}
+
 // Tile size and LDS layout of the recursion kernel. Returns false when not even one point fits.
 // `elem` is the size of the numbers the kernel computes with, `out_elem` that of the coordinates
 // and the output arrays (and so of the staged rows): smaller when float arrays are evaluated in
 // float64, else the same (0).
 static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, size_t elem,
                            unsigned budget, int lds_limit, int cus, Launch* out, bool* split_sides,
-                           bool normalized = true, size_t out_elem = 0) {
+                           bool normalized = true, size_t out_elem = 0, unsigned threads = kRecursionThreads) {
     Tiling& g = out->g;
     std::memset(&g, 0, sizeof(g));
     const int hard = mode == 2 ? 1 : 6;
@@ -593,7 +616,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     };
     // rounds of the entry waves per tile, in tenths of two-sided jobs, with `waves` sequence waves
     auto entry_cost = [&](unsigned waves, bool* split) {
-        wide = kRecursionThreads - 64 * (1 + waves + g.flush_waves);
+        wide = threads - 64 * (1 + waves + g.flush_waves);
         // (with two or more points per tile the jobs go as a list ordered by kind, which fills the
         // lanes without splitting, and the two-sided job shares the common factors: 400 MB of
         // output, us, split against not, normalised float32 l_max = 4, 8, 16, 20 110, 115, 108,
@@ -610,7 +633,29 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // 48 468, 428 against 527, 477; with equal rounds two are faster by 2-3 % with derivatives).
     // Second derivatives in float64 follow no such rule (l_max = 6, 8, 10: 555, 437, 505 against
     // 449, 558, 445) and keep two.
-    if (g.sequence_waves == 2 && !(mode == 2 && elem == 8)) {
+    if (threads > kRecursionThreads) {
+        // Sixteen waves: the tile is larger, the recursions of a tile more, and the tile waits for
+        // them if they need many rounds. Measured with two, three and four sequence waves (1.2 GB
+        // of output, us): gradients float32 l_max = 12, 16, 20, 24, 28, 32 249, 257, 252, 265, 255,
+        // 272 / 238, 245, 249, 259, 253, 267 / 244, 248, 264, 272, 269, 281: three. Float64
+        // l_max = 9, 12, 16, 18, 20, 32 223, 244, 244, 248, 270, 251 / 218, 245, 240, 234, 252, 257 /
+        // 239, 239, 233, 239, 257, 253: as few rounds of recursions as four waves would need, with
+        // as few waves as that takes. Second derivatives, float32, l_max = 4, 8, 12, 16, 20, 24 240,
+        // 239, 240, 238, 245, 276 / 231, 248, 247, 246, 250, 266: the entries weigh more there, two,
+        // three at both ends.
+        const unsigned recursions = S * arrays * static_cast<unsigned>(l_max - hard);
+        if (mode == 1 && elem == 4) {
+            g.sequence_waves = 3;
+        } else if (mode == 1) {
+            const unsigned least = (recursions + 255u) / 256u;
+            g.sequence_waves = 2;
+            while (g.sequence_waves < 4 && (recursions + 64u * g.sequence_waves - 1u) / (64u * g.sequence_waves) > least) {
+                ++g.sequence_waves;
+            }
+        } else {
+            g.sequence_waves = l_max <= 4 || l_max >= 22 ? 3u : 2u;
+        }
+    } else if (g.sequence_waves == 2 && !(mode == 2 && elem == 8)) {
         bool split_one = false, split_two = false;
         const unsigned with_one = entry_cost(1, &split_one);
         const unsigned with_two = entry_cost(2, &split_two);
@@ -688,8 +733,55 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.off_jobs = at;
     at += table_elems_for(may_split);
     out->lds_bytes = g.tables_at + at * esize;
-    out->threads = kRecursionThreads;
+    out->threads = threads;
     if (out->lds_bytes > limit) return false;
+    // Jobs point by point, one point per pass, with derivatives: in the last round of a point the
+    // jobs with |m| = l, |m| = l - 1 and m = 0 are moved to wave boundaries of the entry lanes where
+    // the lanes of that round allow it, because a wave runs the branch of every kind of job it
+    // holds one after the other and the tile waits for the slowest wave. cfg5 (l_max = 32, 533 jobs
+    // on 320 lanes): the second round was 135 bulk jobs, then 26 + 26 + 26, all three in the third
+    // wave together with the end of the bulk; now m = 0 follows the bulk and the other two start
+    // the fourth and fifth wave. The gaps are places without a job at the end of the job table.
+    g.kind_at[0] = g.kind_at[1] = g.kind_at[2] = 0;
+    if (mode >= 1 && !*split_sides && g.points_per_pass == 1 && switch_or(SW_SPREAD_KINDS, 0) != 0) {
+        const unsigned levels = g.kind_jobs[1], bulk = g.kind_jobs[0], jobs_now = g.jobs_per_point;
+        const unsigned waves = wide / 64u;
+        const unsigned base = jobs_now / wide * wide; // first job of the last round
+        if (jobs_now % wide != 0 && bulk >= base && levels != 0) {
+            const unsigned bulk_waves = (bulk - base + 63u) / 64u;
+            const unsigned spare = bulk_waves * 64u - (bulk - base); // lanes free in the bulk's last wave
+            const unsigned level_waves = (levels + 63u) / 64u;
+            const unsigned after_bulk = base + bulk_waves * 64u;
+            unsigned at_l = 0, at_l1 = 0, at_0 = 0;
+            if (bulk_waves + 3u * level_waves <= waves) { // every kind its own waves
+                at_l = after_bulk;
+                at_l1 = at_l + level_waves * 64u;
+                at_0 = at_l1 + level_waves * 64u;
+            } else if (levels <= spare && bulk_waves + 2u * level_waves <= waves) {
+                at_0 = bulk; // m = 0, the cheapest, shares the bulk's last wave
+                at_l = after_bulk;
+                at_l1 = at_l + level_waves * 64u;
+            } else if (2u * levels <= 64u && bulk_waves + 2u <= waves) {
+                at_l = after_bulk; // m = 0 shares a wave with |m| = l
+                at_0 = at_l + levels;
+                at_l1 = at_l + 64u;
+            }
+            if (at_l != 0) {
+                unsigned padded = at_l + levels;
+                if (at_l1 + levels > padded) padded = at_l1 + levels;
+                if (at_0 + levels > padded) padded = at_0 + levels;
+                const unsigned more = ((padded - jobs_now) * 4u + esize - 1u) / esize * esize; // bytes
+                if (padded <= base + wide && out->lds_bytes + more <= limit) {
+                    g.kind_at[0] = at_l;
+                    g.kind_at[1] = at_l1;
+                    g.kind_at[2] = at_0;
+                    g.jobs_per_point = padded;
+                    g.magic_jobs = magic_of(padded);
+                    out->lds_bytes += more;
+                }
+            }
+        }
+    }
 
     g.n_tiles = static_cast<unsigned>((n_samples + S - 1) / S);
     g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
@@ -706,7 +798,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     }
     unsigned per_cu = limit / out->lds_bytes;
     if (per_cu < 1) per_cu = 1;
-    if (per_cu > 4) per_cu = 4; // 512 threads each: 2048 lanes per CU
+    if (per_cu > 2048u / threads) per_cu = 2048u / threads; // 2048 lanes per CU
     unsigned want = (static_cast<unsigned>(cus) * per_cu + 7u) & ~7u;
     // Few points: shorter chunks, down to single tiles, until every resident workgroup has one
     // (10 000 points at l_max = 8 are 625 tiles of 16: in chunks of 8 they kept 80 workgroups
@@ -790,8 +882,16 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // (float32 from l_max = 14 on the recursion kernel with its jobs as a list ordered by kind is
     // ahead: 600 MB of output, lanes against recursion, l_max = 13 151, 150 us; 14 169, 153; 15 189,
     // 171; 16 174, 154; solid 14 152, 144; 16 160, 144. SPHX_GRADIENT_LANES=2: lanes wherever they fit.)
+    // (With workgroups of 1024 threads the recursion kernel is ahead earlier when there are points
+    // enough for them: 1.2 GB of output, us, lanes against recursion, float32 l_max = 8 214, 206; 9
+    // 256, 217; 10 241, 227; 11 256, 286; 12 306, 238; 13 301, 246; float64 l_max = 7 224, 507; 8
+    // 246, 214; 9 307, 218; 10 293, 226; 11 309, 292. The lanes keep l_max <= 8 and 11 in float32,
+    // l_max = 7 in float64, and every call of fewer than 65 536 points.)
     const int gradient_lanes = switch_or(SW_GRADIENT_LANES, 1);
-    if (lane_kernels && mode == 1 && gradient_lanes != 0 && (gradient_lanes == 2 || elem == 8 || l_max <= 13) &&
+    const bool large_groups = group_threads(n_samples, mode, elem, lane_kernels) > kRecursionThreads && n_samples >= 65536;
+    const bool lanes_by_shape = large_groups ? (elem == 4 ? l_max <= 8 || l_max == 11 : l_max <= 7)
+                                             : elem == 8 || l_max <= 13;
+    if (lane_kernels && mode == 1 && gradient_lanes != 0 && (gradient_lanes == 2 || lanes_by_shape) &&
         plan_gradient_lanes(n_samples, l_max, elem, lds_limit, cus, &plan->closed)) {
         plan->lanes = true;
         return SPHX_OK;
@@ -802,10 +902,11 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // the tile takes all of it (1.5 GB of output, l_max = 6: 694 -> 473 us, l_max = 10: 582 ->
     // 479, l_max = 12: 545 -> 468; solid harmonics l_max = 4-12: 10-20 % less, l_max = 16, 100k
     // points: 580 -> 560).
-    const int whole_cu = mode == 2 && elem == 8 ? lds_limit : 80 * 1024;
+    const unsigned threads = group_threads(n_samples, mode, elem, lane_kernels);
+    const int whole_cu = (mode == 2 && elem == 8) || threads > kRecursionThreads ? lds_limit : 80 * 1024;
     const unsigned budget = static_cast<unsigned>(switch_or(SW_TILE_LDS_BUDGET, whole_cu));
     bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
-                               &plan->split_sides, normalized);
+                               &plan->split_sides, normalized, 0, threads);
     // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of
     // the lanes idle for some two thousand instructions per tile: then the recursion kernel
     // stages l >= 7 only and its wave 0, which mostly waits, writes l <= 6 straight from
@@ -833,7 +934,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     if (mode < 2 && (!fits || cut)) {
         Launch upper;
         if (plan_recursion(n_samples, l_max, mode, false, elem, budget, lds_limit, cus, &upper,
-                           &plan->split_sides)) {
+                           &plan->split_sides, true, 0, threads)) {
             plan->whole = false;
             plan->rec = upper;
             plan->rec.g.prefix_inside = lane_kernels && switch_or(SW_PREFIX_INSIDE, 1) != 0 ? 1u : 0u;
@@ -844,7 +945,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     if (fits && !lane_kernels && plan->rec.g.points_per_pass == 0) {
         // the fused product has no job-list variant of the kernel: whole points side by side
         const Tiling& g = plan->rec.g;
-        const unsigned wide = kRecursionThreads - 64 * (1 + g.sequence_waves + g.flush_waves);
+        const unsigned wide = plan->rec.threads - 64 * (1 + g.sequence_waves + g.flush_waves);
         plan->rec.g.points_per_pass = g.jobs_per_point >= wide ? 1u : wide / g.jobs_per_point;
     }
     if (!fits) {
@@ -926,18 +1027,31 @@ template <typename X> struct AsGiven {
     using type = X; // a parameter of this type takes no part in template argument deduction
 };
 
+// Workgroups of 1024 threads (one per CU, all of its LDS) exist for gradients and for second
+// derivatives in float32: the other kernels need more registers than sixteen waves leave a lane,
+// or gain nothing.
+template <typename T, int MODE, bool VJP>
+constexpr bool kLargeGroups = !VJP && (MODE == 1 || (MODE == 2 && sizeof(T) == 4));
+
 template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false,
-          typename O = T>
+          typename O = T, unsigned NT = kRecursionThreads>
 static hipError_t launch_recursion(const Launch& l, const typename AsGiven<O>::type* xyz,
                                    typename AsGiven<O>::type* sph, typename AsGiven<O>::type* dsph,
                                    typename AsGiven<O>::type* ddsph, hipStream_t stream) {
     if constexpr (!VJP && !LIST) {
         // the variant whose entry lanes take the jobs of a tile as one list
         if (l.g.points_per_pass == 0) {
-            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, false, true, O>(l, xyz, sph, dsph, ddsph, stream);
+            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, false, true, O, NT>(l, xyz, sph, dsph, ddsph, stream);
         }
     }
-    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O>;
+    if constexpr (NT == kRecursionThreads && kLargeGroups<T, MODE, VJP>) {
+        if (l.threads == 2 * kRecursionThreads) {
+            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O, 2 * kRecursionThreads>(
+                l, xyz, sph, dsph, ddsph, stream);
+        }
+    }
+    if (l.threads != NT) return hipErrorInvalidValue; // never planned
+    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O, NT>;
     // The workgroups are persistent: launch exactly as many as are resident at once (registers
     // may allow fewer per CU than LDS does), or the last ones would run alone after the rest.
     unsigned workgroups = l.workgroups;
@@ -1137,16 +1251,17 @@ static bool make_wide_plan(size_t n_samples, int l_max, int mode, int lds_limit,
     plan->closed_only = false;
     plan->whole = true;
     plan->split_sides = false;
-    const int whole_cu = mode == 2 ? lds_limit : 80 * 1024; // as for float64 arrays (make_plan)
+    const unsigned threads = group_threads(n_samples, mode, 8, true);
+    const int whole_cu = mode == 2 || threads > kRecursionThreads ? lds_limit : 80 * 1024; // as for float64 arrays (make_plan)
     const unsigned budget = static_cast<unsigned>(switch_or(SW_TILE_LDS_BUDGET, whole_cu));
     bool fits = plan_recursion(n_samples, l_max, mode, true, 8, budget, lds_limit, cus, &plan->rec,
-                               &plan->split_sides, normalized, 4);
+                               &plan->split_sides, normalized, 4, threads);
     // rows cut at l = 7 where few points fit, by the rule for float rows (make_plan)
     const int split_below = switch_or(SW_SPLIT_BELOW, mode == 0 ? 8 : 3);
     if (mode < 2 && (!fits || plan->rec.g.tile < split_below)) {
         Launch upper;
         if (plan_recursion(n_samples, l_max, mode, false, 8, budget, lds_limit, cus, &upper,
-                           &plan->split_sides, normalized, 4)) {
+                           &plan->split_sides, normalized, 4, threads)) {
             plan->whole = false;
             plan->rec = upper;
             plan->rec.g.prefix_inside = 1u;

@@ -61,8 +61,8 @@ constexpr unsigned kRecursionThreads = 512;
 // rows are rows of O, so a tile holds as many points as in the float kernel's and the flush is
 // that kernel's.
 template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false,
-          typename O = T>
-__global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling g, const O* __restrict__ xyz,
+          typename O = T, unsigned NT = kRecursionThreads>
+__global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling g, const O* __restrict__ xyz,
                                                                      O* __restrict__ sph,
                                                                      O* __restrict__ dsph,
                                                                      O* __restrict__ ddsph) {
@@ -71,7 +71,6 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
     constexpr int H = MODE == 2 ? 1 : 6;
     constexpr unsigned NYH = (H + 1) * (H + 1);
     constexpr unsigned ARRAYS = MODE + 1; // iterate arrays per point: A, B, C
-    constexpr unsigned NT = kRecursionThreads;
     // the row buffers, rows of O, come first; everything else is T and counts from g.tables_at
     O* row_lds = reinterpret_cast<O*>(lds_raw);
     T* lds = reinterpret_cast<T*>(lds_raw + g.tables_at);
@@ -110,6 +109,17 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
         };
         // one thread per l fills that l's places (a single thread writing all of them took
         // 10 us at l_max = 32, a third of the time of a small evaluation)
+        // Jobs point by point, a point's jobs in more rounds than one: in a point's last round
+        // the kinds other than the bulk start with a wave of their own where the lanes allow it
+        // (the host says where), and the places in between hold no job. A wave runs the branch
+        // of every kind it holds, one after the other: at l_max = 32 the third of five entry
+        // waves held the end of the bulk and all three other kinds, and every tile waited for it
+        // (7 100 cycles against 3 300-4 900 for the other four).
+        const bool spread = !SPLIT && !LIST && g.kind_at[0] != 0;
+        if (spread) {
+            for (unsigned i = tid; i < g.jobs_per_point; i += NT) job_table[i] = kNoJob;
+            __syncthreads();
+        }
         if (static_cast<int>(tid) < L - H) {
             constexpr unsigned SIDES = SPLIT ? 2u : 1u;
             const int l = L - static_cast<int>(tid);
@@ -121,10 +131,12 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
             for (unsigned side = 0; side < SIDES; ++side) {
                 unsigned at = side * bulk_all + bulk_above(l);
                 for (int m = l - 2; m >= 1; --m) job_table[at++] = pack(l, m, static_cast<int>(side));
-                job_table[SIDES * bulk_all + side * levels + tid] = pack(l, l, static_cast<int>(side));
-                job_table[SIDES * (bulk_all + levels) + side * levels + tid] = pack(l, l - 1, static_cast<int>(side));
+                const unsigned at_l = spread ? g.kind_at[0] : SIDES * bulk_all + side * levels;
+                const unsigned at_l1 = spread ? g.kind_at[1] : SIDES * (bulk_all + levels) + side * levels;
+                job_table[at_l + tid] = pack(l, l, static_cast<int>(side));
+                job_table[at_l1 + tid] = pack(l, l - 1, static_cast<int>(side));
             }
-            job_table[SIDES * (bulk_all + 2 * levels) + tid] = pack(l, 0, 0);
+            job_table[(spread ? g.kind_at[2] : SIDES * (bulk_all + 2 * levels)) + tid] = pack(l, 0, 0);
         }
     }
 
@@ -407,6 +419,9 @@ __global__ __launch_bounds__(kRecursionThreads, MODE < 2 ? 4 : 1) void recursion
         };
         auto take_job = [&](unsigned e) {
             const unsigned packed = job_table[e];
+            if constexpr (!LIST && !SPLIT) {
+                if (packed == kNoJob) return;
+            }
             const int m = static_cast<int>(packed & 0x7fu);
             const int side = static_cast<int>((packed >> 7) & 1u);
             const int l = static_cast<int>((packed >> 8) & 0xffu);

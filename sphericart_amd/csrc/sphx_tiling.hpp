@@ -57,7 +57,14 @@ struct Tiling {
     // recursion_kernel, job-list variant: jobs per point of the kinds bulk / |m| = l and l - 1 /
     // m = 0 (the order of the job table), and ceil(2^32 / .) of each (0 where there are none)
     unsigned kind_jobs[3], kind_magic[3];
+    // recursion_kernel, jobs point by point: where the jobs with |m| = l, |m| = l - 1 and m = 0 start
+    // in the job table when they are moved to wave boundaries of the entry lanes (0: they follow
+    // the bulk without gaps); jobs_per_point then counts the gaps too
+    unsigned kind_at[3];
 };
+
+// a place in the job table of recursion_kernel that holds no job
+constexpr unsigned kNoJob = 0xffffffffu;
 
 extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 

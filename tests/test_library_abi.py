@@ -80,7 +80,7 @@ def test_launch_plans(library):
     for n, l_max, mode, f64 in ((10_000, 8, 1, True), (100_000, 16, 2, True), (200_000, 32, 1, False), (5, 20, 2, False)):
         status, (tile, threads, lds, groups) = _plan(library, n, l_max, mode, f64)
         assert status == 0
-        assert 1 <= tile <= 64 and threads in (256, 512) and lds <= 160 * 1024
+        assert 1 <= tile <= 64 and threads in (256, 512, 1024) and lds <= 160 * 1024
         assert groups % 8 == 0 and groups >= 8
     assert _plan(library, 10, 65, 0, False)[0] == 2       # beyond the tables
     assert _plan(library, 10, 64, 2, True)[0] == 2        # one point's rows no longer fit in LDS
