@@ -125,7 +125,7 @@ enum Switch : int {
     SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_FLUSH_WAVES, SW_GRADIENT_LANES, SW_GRADIENT_LANES_PARTS,
     SW_GRADIENT_LANES_TILE, SW_GRADIENT_LANES_WAVES, SW_GROUP_THREADS, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST,
     SW_PREFIX_INSIDE, SW_ROW_BUFFERS,
-    SW_SEQUENCE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
+    SW_SEQUENCE_WAVES, SW_SLICE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
     SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
     SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_COUNT
 };
@@ -134,7 +134,7 @@ static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_GRADIENT_LANES_PARTS", "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_GROUP_THREADS",
     "SPHX_HESSIAN_LANES",
     "SPHX_HESSIAN_LANES_PARTS", "SPHX_JOB_LIST",
-    "SPHX_PREFIX_INSIDE", "SPHX_ROW_BUFFERS", "SPHX_SEQUENCE_WAVES", "SPHX_SPLIT_BELOW",
+    "SPHX_PREFIX_INSIDE", "SPHX_ROW_BUFFERS", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
     "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE",
@@ -591,6 +591,21 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.flush_waves = buffers == 2 ? static_cast<unsigned>(switch_or(SW_FLUSH_WAVES, 1)) : 0u;
     if (g.flush_waves > 2) g.flush_waves = 2;
     if (buffers == 2 && g.flush_waves < 1) g.flush_waves = 1;
+    // Waves of their own for the closed forms of l <= 6 (whole rows): with sixteen waves and
+    // float32 gradients, where the tile otherwise waits for the entry waves that carry a slice on
+    // top of their jobs; one of them up to eight points per tile, two from nine on, three from 28
+    // on (l_max = 8, 9, 10, 12, 13 with two 224, 226, 226, 233, 244 us, with three 209, 216, 222,
+    // 231, 241). 1.2 GB of
+    // output, us, three sequence waves and the slices on all waves against two sequence waves and
+    // one / two slice waves: l_max = 14, 18, 24, 28, 32, 36, 40 252, 253, 263, 256, 270, 270, 296
+    // against 250, 241, 253, 248, 254, 260, 275 / 237, 237, 248, 254, 255, 262, 271. In float64 the
+    // closed forms are too much for two or three waves (l_max = 16: 258 against 340 / 300 us).
+    g.slice_waves = 0;
+    const bool slices_apart = threads > kRecursionThreads && mode == 1 && elem == 4;
+    if (whole && mode < 2 && buffers == 1) {
+        const int want = switch_or(SW_SLICE_WAVES, slices_apart ? (S >= 28 ? 3 : (S >= 9 ? 2 : 1)) : 0);
+        g.slice_waves = want < 0 ? 0u : (want > 4 ? 4u : static_cast<unsigned>(want));
+    }
     g.sequence_waves = S * arrays * static_cast<unsigned>(l_max - hard) > 64 ? 2u : 1u;
     // Split the sides when that lets the entries of a tile go through the entry waves in fewer
     // rounds than it costs, a one-sided job being about 0.6 of a two-sided one. Normalised
@@ -616,7 +631,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     };
     // rounds of the entry waves per tile, in tenths of two-sided jobs, with `waves` sequence waves
     auto entry_cost = [&](unsigned waves, bool* split) {
-        wide = threads - 64 * (1 + waves + g.flush_waves);
+        wide = threads - 64 * (1 + waves + g.flush_waves + g.slice_waves);
         // (with two or more points per tile the jobs go as a list ordered by kind, which fills the
         // lanes without splitting, and the two-sided job shares the common factors: 400 MB of
         // output, us, split against not, normalised float32 l_max = 4, 8, 16, 20 110, 115, 108,
@@ -645,7 +660,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         // three at both ends.
         const unsigned recursions = S * arrays * static_cast<unsigned>(l_max - hard);
         if (mode == 1 && elem == 4) {
-            g.sequence_waves = 3;
+            g.sequence_waves = g.slice_waves != 0 ? 2 : 3; // (two with slice waves, see above)
         } else if (mode == 1) {
             const unsigned least = (recursions + 255u) / 256u;
             g.sequence_waves = 2;
@@ -738,12 +753,19 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // Jobs point by point, one point per pass, with derivatives: in the last round of a point the
     // jobs with |m| = l, |m| = l - 1 and m = 0 are moved to wave boundaries of the entry lanes where
     // the lanes of that round allow it, because a wave runs the branch of every kind of job it
-    // holds one after the other and the tile waits for the slowest wave. cfg5 (l_max = 32, 533 jobs
-    // on 320 lanes): the second round was 135 bulk jobs, then 26 + 26 + 26, all three in the third
-    // wave together with the end of the bulk; now m = 0 follows the bulk and the other two start
-    // the fourth and fifth wave. The gaps are places without a job at the end of the job table.
+    // holds one after the other and the tile waits for the slowest wave. Float32 l_max = 32, 533
+    // jobs on 320 lanes: the second round was 135 bulk jobs, then 26 + 26 + 26, all three in the
+    // third wave together with the end of the bulk; moved, m = 0 follows the bulk and the other two
+    // start the fourth and fifth wave. The gaps are places without a job at the end of the job
+    // table. With one workgroup of 1024 threads on a CU this pays (float64 gradients l_max = 32,
+    // two points per tile: 290 -> 249 us per 1.2 GB). With two workgroups of 512 the slowest wave of
+    // a tile of cfg5 went from 7 400 to 5 900 cycles and a launch from 979 to 926 us for the first
+    // few launches after a pause, but from 896 to 947 us in a long series of launches, and builds
+    // of the kernel that differ in a few scalar instructions moved either number by 5 %: how the
+    // stages and flushes of the two workgroups of a CU fall against each other decides there,
+    // and nothing in the kernel controls that. Off for 512 threads (SPHX_SPREAD_KINDS).
     g.kind_at[0] = g.kind_at[1] = g.kind_at[2] = 0;
-    if (mode >= 1 && !*split_sides && g.points_per_pass == 1 && switch_or(SW_SPREAD_KINDS, 0) != 0) {
+    if (mode >= 1 && !*split_sides && g.points_per_pass == 1 && switch_or(SW_SPREAD_KINDS, threads > kRecursionThreads ? 1 : 0) != 0) {
         const unsigned levels = g.kind_jobs[1], bulk = g.kind_jobs[0], jobs_now = g.jobs_per_point;
         const unsigned waves = wide / 64u;
         const unsigned base = jobs_now / wide * wide; // first job of the last round
@@ -886,9 +908,10 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // enough for them: 1.2 GB of output, us, lanes against recursion, float32 l_max = 8 214, 206; 9
     // 256, 217; 10 241, 227; 11 256, 286; 12 306, 238; 13 301, 246; float64 l_max = 7 224, 507; 8
     // 246, 214; 9 307, 218; 10 293, 226; 11 309, 292. The lanes keep l_max <= 8 and 11 in float32,
-    // l_max = 7 in float64, and every call of fewer than 65 536 points.)
+    // l_max = 7 in float64, and every call of fewer than 32 768 points (50 000 points, lanes against
+    // recursion: float64 l_max = 9 54, 43 us, float32 l_max = 12 42, 38 us; 20 000 points 25, 22 and 21, 24).)
     const int gradient_lanes = switch_or(SW_GRADIENT_LANES, 1);
-    const bool large_groups = group_threads(n_samples, mode, elem, lane_kernels) > kRecursionThreads && n_samples >= 65536;
+    const bool large_groups = group_threads(n_samples, mode, elem, lane_kernels) > kRecursionThreads && n_samples >= 32768;
     const bool lanes_by_shape = large_groups ? (elem == 4 ? l_max <= 8 || l_max == 11 : l_max <= 7)
                                              : elem == 8 || l_max <= 13;
     if (lane_kernels && mode == 1 && gradient_lanes != 0 && (gradient_lanes == 2 || lanes_by_shape) &&
@@ -945,7 +968,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     if (fits && !lane_kernels && plan->rec.g.points_per_pass == 0) {
         // the fused product has no job-list variant of the kernel: whole points side by side
         const Tiling& g = plan->rec.g;
-        const unsigned wide = plan->rec.threads - 64 * (1 + g.sequence_waves + g.flush_waves);
+        const unsigned wide = plan->rec.threads - 64 * (1 + g.sequence_waves + g.flush_waves + g.slice_waves);
         plan->rec.g.points_per_pass = g.jobs_per_point >= wide ? 1u : wide / g.jobs_per_point;
     }
     if (!fits) {

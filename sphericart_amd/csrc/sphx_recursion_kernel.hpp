@@ -297,7 +297,7 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
     // The waves between the sequence waves and the flush waves compute entries.
     const bool streaming = g.row_buffers == 2;
     const unsigned entry_first_wave = 1 + g.sequence_waves;
-    const unsigned entry_end_wave = NT / 64 - (streaming ? g.flush_waves : 0u);
+    const unsigned entry_end_wave = NT / 64 - (streaming ? g.flush_waves : g.slice_waves);
     const unsigned wide_first = 64 * entry_first_wave;
     const unsigned wide_lanes = 64 * (entry_end_wave - entry_first_wave);
 
@@ -669,8 +669,13 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
         for (unsigned n = 0; valid_in(n) != 0; ++n) {
             __syncthreads(); // tables of tile n+1, iterates of tile n in place; rows of tile n-1 flushed
             // the closed-form slices go round all waves: those that make tables and iterates
-            // have time to spare
-            closed_stage(n, 0, wave, NT / 64);
+            // have time to spare; or to wave 0 and the waves set aside for them, when the entry
+            // waves that had a slice on top of their jobs were what the tile waited for
+            if (g.slice_waves == 0) {
+                closed_stage(n, 0, wave, NT / 64);
+            } else if (wave == 0 || wave >= entry_end_wave) {
+                closed_stage(n, 0, wave == 0 ? 0u : wave - entry_end_wave + 1u, g.slice_waves + 1u);
+            }
             if (wave == 0) {
                 if ((n & (batch_tiles - 1u)) == 0) {
                     azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
@@ -679,7 +684,7 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
                 if (prefix_wave) prefix_slice();
             } else if (wave < entry_first_wave) {
                 recursion_stage(n + 1);
-            } else {
+            } else if (wave < entry_end_wave) {
                 entry_stage(n, 0);
             }
             __syncthreads(); // rows of tile n complete

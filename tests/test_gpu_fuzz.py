@@ -24,7 +24,7 @@ OVERRIDES = (
     ("SPHX_ROW_BUFFERS", (1, 2)), ("SPHX_SEQUENCE_WAVES", (1, 2)), ("SPHX_CHUNK_SHIFT", (0, 1, 2, 3)),
     ("SPHX_AZ_SHIFT", (0, 1, 2, 3)), ("SPHX_SPLIT_SIDES", (0,)), ("SPHX_TILE_POW2", (1,)),
     ("SPHX_SPLIT_BELOW", (0, 64)), ("SPHX_GRADIENT_LANES_PARTS", (1, 2)), ("SPHX_GROUP_THREADS", (512, 1024)),
-    ("SPHX_GROUP_THREADS", (1024,)), ("SPHX_SPREAD_KINDS", (1,)),
+    ("SPHX_GROUP_THREADS", (1024,)), ("SPHX_SPREAD_KINDS", (0, 1)), ("SPHX_SLICE_WAVES", (0, 1, 2, 3)),
 )
 
 
