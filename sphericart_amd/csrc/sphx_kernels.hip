@@ -457,21 +457,22 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
 }
 
 // Threads per workgroup of the recursion kernel: 512, two workgroups to a CU, or 1024, one
-// workgroup with all of the CU's LDS and tiles of twice as many points (gradients, and second
-// derivatives in float32; not the fused product, not values, whose entries are too cheap for
-// thirteen waves of them, not second derivatives in float64, whose entry jobs need more than the
-// 128 registers a lane of sixteen waves has). Two workgroups of 512 on a CU run their stages and
+// workgroup with all of the CU's LDS and tiles of twice as many points (not the fused product,
+// and not second derivatives in float64, whose entry jobs need more than the 128 registers a
+// lane of sixteen waves has). Two workgroups of 512 on a CU run their stages and
 // their flushes against each other as chance has it, and a tile of one or two points leaves the
 // entry lanes and the sequence lanes half idle in their last rounds; one workgroup of 1024
 // measured, 1.2 GB of output, us, 512 against 1024: gradients float32 l_max = 14, 20, 24, 28,
 // 32, 36 283, 306, 323, 329, 331, 342 against 245, 249, 259, 253, 267, 268 (l_max = 40 288
 // against 290); float64 l_max = 12, 16, 20, 24, 32 303, 307, 320, 271, 266 against 239, 233,
 // 252, 248, 249; second derivatives float32 l_max = 4, 8, 12, 16, 20, 24 252, 262, 271, 258,
-// 334, 361 against 231, 239, 238, 238, 245, 266; solid harmonics alike. With few points (below
-// 4 096) 512 threads stay: more workgroups have a tile then.
+// 334, 361 against 231, 239, 238, 238, 245, 266; solid harmonics alike; values, whose entries
+// are three multiplications, gain less: float32 l_max = 24, 32, 40 405, 383, 378 against 396,
+// 377, 376, float64 l_max = 24, 28, 32 317, 322, 335 against 292, 305, 297. With few points
+// (below 4 096) 512 threads stay: more workgroups have a tile then.
 // SPHX_GROUP_THREADS = 512 or 1024 overrides the rule.
 static unsigned group_threads(size_t n_samples, int mode, size_t elem, bool forward) {
-    const bool exists = forward && (mode == 1 || (mode == 2 && elem == 4));
+    const bool exists = forward && (mode <= 1 || (mode == 2 && elem == 4));
     if (!exists) return kRecursionThreads;
     const int want = switch_or(SW_GROUP_THREADS, 0);
     if (want == 512 || want == 1024) return static_cast<unsigned>(want);
@@ -667,8 +668,13 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
             while (g.sequence_waves < 4 && (recursions + 64u * g.sequence_waves - 1u) / (64u * g.sequence_waves) > least) {
                 ++g.sequence_waves;
             }
-        } else {
+        } else if (mode == 2) {
             g.sequence_waves = l_max <= 4 || l_max >= 22 ? 3u : 2u;
+        } else {
+            // values, two against three: float32 l_max = 24, 28, 32, 40, 48 381, 436, 373, 420, 355
+            // against 396, 392, 377, 376, 366; float64 l_max = 24, 28, 32 295, 326, 293 against
+            // 292, 305, 297
+            g.sequence_waves = 3;
         }
     } else if (g.sequence_waves == 2 && !(mode == 2 && elem == 8)) {
         bool split_one = false, split_two = false;
@@ -1050,11 +1056,10 @@ template <typename X> struct AsGiven {
     using type = X; // a parameter of this type takes no part in template argument deduction
 };
 
-// Workgroups of 1024 threads (one per CU, all of its LDS) exist for gradients and for second
-// derivatives in float32: the other kernels need more registers than sixteen waves leave a lane,
-// or gain nothing.
+// Workgroups of 1024 threads (one per CU, all of its LDS) exist for all but second derivatives
+// in float64, which need more registers than sixteen waves leave a lane, and the fused product.
 template <typename T, int MODE, bool VJP>
-constexpr bool kLargeGroups = !VJP && (MODE == 1 || (MODE == 2 && sizeof(T) == 4));
+constexpr bool kLargeGroups = !VJP && (MODE <= 1 || (MODE == 2 && sizeof(T) == 4));
 
 template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false,
           typename O = T, unsigned NT = kRecursionThreads>

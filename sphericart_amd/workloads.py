@@ -171,14 +171,14 @@ WORKLOADS = {
         "val10", "spherical, l_max=10, f32, values, 1M points, uniform directions, r ~ U[0.5,5)",
         10, "f32", True, "values", 1_000_000, 1010,
     ),
-    # likewise for the gradients kernel of l_max just above the closed forms
+    # likewise gradients at l_max just above the closed forms
     "grad10": Workload(
         "grad10",
         "spherical, l_max=10, f32, values+gradients, 1M points, uniform directions, r ~ U[0.5,5), "
         "1% of the points exactly on the +-z axis",
         10, "f32", True, "gradients", 1_000_000, 1011,
     ),
-    # and for the kernel of second derivatives at small l_max
+    # and second derivatives at small l_max
     "hess5": Workload(
         "hess5",
         "spherical, l_max=5, f32, values+gradients+Hessians, 500k points, uniform directions, r ~ U[0.5,5), "
