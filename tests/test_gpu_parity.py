@@ -115,6 +115,39 @@ def test_gradient_lanes_with_shared_channels(oracle, library, switches, dtype, n
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("mode", ["values", "gradients", "hessians"])
+def test_workgroups_of_512_and_1024_threads(oracle, library, switches, dtype, mode):
+    """The recursion kernel in workgroups of 512 threads (two to a CU) and of 1024 (one, with all of
+    its LDS, larger tiles, waves of their own for the closed forms, kinds of jobs at wave
+    boundaries), many points and few, against the oracle. Second derivatives in float64 exist
+    with 512 threads only; the switch is then ignored."""
+    rng = np.random.default_rng(31)
+    l_values = {"values": (9, 23, 31, 46), "gradients": (9, 12, 21, 32, 44), "hessians": (4, 7, 13, 22)}[mode]
+    for l_max in l_values:
+        for normalized in (True, False):
+            n = 3001 if l_max < 30 else 1201
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, normalized, mode)
+            xyz_dev = torch.from_numpy(xyz).cuda()
+            for threads, extra in ((512, {}), (1024, {}), (1024, {"SPHX_SLICE_WAVES": 3, "SPHX_SEQUENCE_WAVES": 4}),
+                                   (1024, {"SPHX_SLICE_WAVES": 0, "SPHX_SPREAD_KINDS": 0, "SPHX_JOB_LIST": 0})):
+                library.sphx_reset_switches()
+                switches("SPHX_GRADIENT_LANES", 0)
+                switches("SPHX_HESSIAN_LANES", 0)
+                switches("SPHX_VALUES_LDS", 1)
+                switches("SPHX_GROUP_THREADS", threads)
+                for name, value in extra.items():
+                    switches(name, value)
+                announce("workgroup size", np.dtype(dtype).name, mode, normalized, l_max, threads, extra)
+                status, got = run_launch_layer(library, xyz_dev, l_max, normalized, mode)
+                torch.cuda.synchronize()
+                assert status == 0, library.sphx_last_error()
+                got = tuple(None if g is None else g.cpu().numpy() for g in got)
+                check(got, want, (l_max, normalized, threads, extra))
+    library.sphx_reset_switches()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("mode", ["gradients", "hessians"])
 def test_job_list_by_kind_and_points_side_by_side(oracle, library, switches, dtype, mode):
     """The recursion kernel deals the entry jobs of a tile either point by point, side by side,

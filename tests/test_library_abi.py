@@ -82,6 +82,14 @@ def test_launch_plans(library):
         assert status == 0
         assert 1 <= tile <= 64 and threads in (256, 512, 1024) and lds <= 160 * 1024
         assert groups % 8 == 0 and groups >= 8
+    # cfg5: one workgroup of 1024 threads per CU with all of its LDS, five points per tile;
+    # the same shape with few points: workgroups of 512 threads
+    status, (tile, threads, lds, groups) = _plan(library, 200_000, 32, 1, False)
+    assert status == 0 and (tile, threads, groups) == (5, 1024, 256) and 150_000 < lds <= 160 * 1024
+    status, (tile, threads, lds, groups) = _plan(library, 2_000, 32, 1, False)
+    assert status == 0 and threads == 512 and lds <= 80 * 1024
+    # second derivatives in float64 keep 512 threads (more than 128 registers per lane)
+    assert _plan(library, 100_000, 16, 2, True)[1][1] == 512
     assert _plan(library, 10, 65, 0, False)[0] == 2       # beyond the tables
     assert _plan(library, 10, 64, 2, True)[0] == 2        # one point's rows no longer fit in LDS
     assert b"LDS" in library.sphx_last_error()
