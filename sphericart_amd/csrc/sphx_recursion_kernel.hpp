@@ -454,19 +454,27 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
                 }
                 return;
             }
-            const unsigned b0 = g.kind_jobs[0], b1 = g.kind_jobs[1], b3 = g.kind_jobs[2];
+            // (read into scalar registers here: picked by index inside the loop, the members of g
+            // would be copied to scratch memory and fetched from there job by job, and a wave that
+            // waits for such a load also waits for the stores of its last flush)
+            const unsigned b0 = __builtin_amdgcn_readfirstlane(g.kind_jobs[0]);
+            const unsigned b1 = __builtin_amdgcn_readfirstlane(g.kind_jobs[1]);
+            const unsigned b3 = __builtin_amdgcn_readfirstlane(g.kind_jobs[2]);
+            const unsigned magic0 = __builtin_amdgcn_readfirstlane(g.kind_magic[0]);
+            const unsigned magic1 = __builtin_amdgcn_readfirstlane(g.kind_magic[1]);
+            const unsigned magic3 = __builtin_amdgcn_readfirstlane(g.kind_magic[2]);
             const unsigned t1 = valid * b0, t2 = t1 + valid * b1, t3 = t2 + valid * b1;
             unsigned current = ~0u;
             for (unsigned q = t; q < total; q += wide_lanes) {
                 unsigned r, b, first_job, magic;
                 if (q < t1) {
-                    r = q, b = b0, first_job = 0, magic = g.kind_magic[0];
+                    r = q, b = b0, first_job = 0, magic = magic0;
                 } else if (q < t2) {
-                    r = q - t1, b = b1, first_job = b0, magic = g.kind_magic[1];
+                    r = q - t1, b = b1, first_job = b0, magic = magic1;
                 } else if (q < t3) {
-                    r = q - t2, b = b1, first_job = b0 + b1, magic = g.kind_magic[1];
+                    r = q - t2, b = b1, first_job = b0 + b1, magic = magic1;
                 } else {
-                    r = q - t3, b = b3, first_job = b0 + 2 * b1, magic = g.kind_magic[2];
+                    r = q - t3, b = b3, first_job = b0 + 2 * b1, magic = magic3;
                 }
                 // exact: r * b < 2^32; a single job per point has no such multiplier in 32 bits
                 const unsigned s = b == 1 ? r : __umulhi(r, magic);
