@@ -13,14 +13,14 @@
 namespace sphx {
 
 // ---------------------------------------------------------------------------
-// l > H through the recursion. 512 threads, persistent workgroups that walk
-// over tiles of `tile` consecutive points, four tiles in flight per workgroup,
-// every wave with a role of its own and one barrier per tile:
+// l > H through the recursion. NT = 512 or 1024 threads, persistent workgroups
+// that walk over tiles of `tile` consecutive points, four tiles in flight per
+// workgroup, every wave with a role of its own and one barrier per tile:
 //
 //   wave 0       one batch of up to eight tiles ahead, one lane per point:
 //                normalised coordinates, c_m, s_m, 2(m+1)z into LDS (azimuth_job);
-//   wave 1 (, 2) tile i+1, one lane per (point, l, sequence): the bare Q recursions,
-//                every iterate into LDS (sequence_job);
+//   waves 1 ..   tile i+1, one lane per (point, l, sequence): the bare Q recursions,
+//                every iterate into LDS (sequence_job); g.sequence_waves of them;
 //   entry waves  tile i, one job per (point, l, m >= 0): the entries (l, +-m) of
 //                every requested array, chain rule included, staged in LDS in
 //                HBM layout (entry_job). Neighbouring lanes take neighbouring m
@@ -33,9 +33,14 @@ namespace sphx {
 // takes them off the critical path. The last stage is bound by HBM, the entry
 // stage by the vector ALUs: side by side, neither waits for the other. The
 // point tables are kept in three buffers, the iterates and the staged rows in
-// two. When the rows of a single point are too long for two row buffers there
-// is one, no wave is set aside for flushing, and all waves flush tile i after
-// a second barrier.
+// two. With one row buffer (what the host plans; two are kept for tests) no
+// wave is set aside for flushing and all waves flush tile i after a second
+// barrier.
+//
+// NT = 512: two workgroups share a CU, half of its LDS each. NT = 1024: one
+// workgroup has the CU and all of its LDS, its tiles are more than twice as
+// large, and with g.slice_waves the closed forms of l <= H have waves of their
+// own (the last ones) next to wave 0.
 //
 // SPLIT == true (second derivatives, so few points per tile that the (l, m)
 // pairs of a tile leave lanes idle): the entries (l, +m) and (l, -m) are two
@@ -49,8 +54,8 @@ namespace sphx {
 // ---------------------------------------------------------------------------
 constexpr unsigned kRecursionThreads = 512;
 
-// Values and gradients: at most 128 registers, so that two workgroups share a CU (four waves
-// per SIMD) wherever their LDS allows. Only the float64 closed forms exceed that on their own
+// Values and gradients: at most 128 registers, so that two workgroups of 512 threads or one of
+// 1024 fit on a CU (four waves per SIMD) wherever their LDS allows. Only the float64 closed forms exceed that on their own
 // and spill a few registers; with 170 registers and one workgroup per CU, l_max = 12 float64
 // gradients took 800 us instead of 513 us. The second-derivative kernels keep what they need
 // (forced to 128 they spill in the entry jobs: 918 us against 558 us at l_max = 10, float64).
