@@ -507,7 +507,8 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // are cut so that they keep their position within 16 bytes
     const unsigned row_stride = nrow + (whole ? 0u : nyh % (16u / osize));
     const unsigned rows_per_point = components_of(mode) * row_stride;
-    const unsigned rest_per_point = 3 * (8 + 3 * (l_max + 1)) + 2 * arrays * tri_all;
+    // (the records of a point and its sequences of iterates are an odd number of words apart)
+    const unsigned rest_per_point = 3 * ((8 + 3 * (l_max + 1)) | 1u) + 2 * arrays * (tri_all | 1u);
     unsigned fixed = 0; // bytes
     auto point_bytes = [&](unsigned buffers) { return buffers * rows_per_point * osize + rest_per_point * esize; };
     auto bytes_for = [&](unsigned S, unsigned buffers) { return S * point_bytes(buffers) + fixed; };
@@ -566,7 +567,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // Point tables for several tiles at a time (recursion_kernel, az_shift): as many tiles as
     // wave 0 has lanes for, eight at most, as long as the larger table area keeps the workgroup
     // within the budget (or within what it needs anyway).
-    const unsigned point_record = 8 + 3 * static_cast<unsigned>(l_max + 1);
+    const unsigned point_record = (8 + 3 * static_cast<unsigned>(l_max + 1)) | 1u;
     unsigned az_shift = 0;
     {
         const unsigned allowed = bytes_for(S, buffers) > budget ? bytes_for(S, buffers) : budget;
@@ -750,7 +751,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.off_pts = at;
     at += table_slots * S * point_record;
     g.off_iter = at;
-    at += 2 * S * arrays * tri_all;
+    at += 2 * S * arrays * (tri_all | 1u);
     g.off_jobs = at;
     at += table_elems_for(may_split);
     out->lds_bytes = g.tables_at + at * esize;

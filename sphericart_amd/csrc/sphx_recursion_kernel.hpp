@@ -146,7 +146,11 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
     }
 
     // per point: 8 numbers (x, y, z, x^2, y^2, z^2, 1/r, x^2 + y^2), then c, s, 2(m+1)z
-    const unsigned point_stride = 8 + 3 * (L + 1);
+    // (both strides odd: lanes of the sequence waves work on different points and sequences
+    // at once, and a stride with a power of two in it puts them on a few LDS banks: at l_max = 31
+    // the iterates of neighbouring sequences were 528 words apart, 16 modulo the 32 banks)
+    const unsigned point_stride = (8 + 3 * (L + 1)) | 1u;
+    const unsigned iterate_stride = tri_all | 1u;
     // The tables are made for 2^az_shift tiles at a time (a batch), one lane per point, so that
     // the recurrences, a chain of dependent operations that few lanes share, run once per batch
     // instead of once per tile. Single tiles are made two rounds ahead and kept in three
@@ -159,7 +163,7 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
         return lds + g.off_pts + (slot * S + s) * point_stride;
     };
     auto iterates = [&](unsigned buffer, unsigned s, unsigned which, int l) -> T* {
-        return lds + g.off_iter + ((buffer * S + s) * ARRAYS + which) * tri_all + l * (l + 1) / 2;
+        return lds + g.off_iter + ((buffer * S + s) * ARRAYS + which) * iterate_stride + l * (l + 1) / 2;
     };
 
     // same XCD-contiguous walk as the closed-form kernel
@@ -358,7 +362,12 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
                     // Not for float64 and not for values alone, where the selects cost registers
                     // that the kernel does not have to spare (values: 68 -> 89, and l_max = 9 lost
                     // its third workgroup per CU, 80 -> 106 us).
-                    constexpr bool MAY_ROTATE = sizeof(T) == 4 && MODE == 1; // not where T and O differ
+                    // Nor in workgroups of 1024 threads: their tiles beyond l_max = 15 hold few enough
+                    // points for the conflicts to cost less than the selects (us per 1.2 GB, rotated
+                    // against not: l_max = 15, 23 points, 270, 298; l_max = 23, 31, 39 with 10, 6, 4
+                    // points 269, 312, 345 against 266, 258, 269), and without this code the whole
+                    // kernel needs fewer registers (l_max = 32: 732 -> 710 us).
+                    constexpr bool MAY_ROTATE = sizeof(T) == 4 && MODE == 1 && NT == kRecursionThreads; // not where T and O differ
                     if (MAY_ROTATE && (ny & 31u) == 0) {
                         const unsigned turn = lane & 3u;
                         if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 8, true>(p, rows, turn);
