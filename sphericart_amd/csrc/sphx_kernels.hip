@@ -725,7 +725,9 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // lanes that points side by side would fill, in percent
     const unsigned fill = 100u * g.points_per_pass * g.jobs_per_point / wide;
     const bool cheap_jobs = mode == 2 && elem == 8 && !normalized; // no chain rule, few branches
-    const bool by_shape = mode == 0   ? saves_a_round && S >= 3 && g.points_per_pass <= 2
+    // (values in workgroups of 1024 threads: always the list, us per 1.2 GB without and with:
+    // float32 l_max = 26 475, 391; float64 l_max = 26, 36 353, 307 and 351, 299; the same elsewhere)
+    const bool by_shape = mode == 0   ? (threads > kRecursionThreads ? S >= 2 : saves_a_round && S >= 3 && g.points_per_pass <= 2)
                           : mode == 1 ? S >= 3 || (saves_a_round && S >= 2)
                                       : (S >= 3 && !(cheap_jobs && fill >= 90u)) || (S == 2 && !*split_sides) ||
                                             (saves_a_round && S >= 2);
