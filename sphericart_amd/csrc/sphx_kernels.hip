@@ -528,7 +528,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // derivatives float32 l_max = 20, 22, 28 157, 122, 167 against 121, 100, 105 (solid 109, 96
     // against 88, 79); float64 l_max = 20, 22 149, 134 against 126, 105; l_max = 24 the same.
     int want_buffers = switch_or(SW_ROW_BUFFERS, 1);
-    unsigned buffers = want_buffers == 2 ? 2u : 1u;
+    unsigned buffers = want_buffers == 2 && threads == kRecursionThreads ? 2u : 1u; // (none with 1024 threads)
     if (bytes_for(1, buffers) > limit) buffers = 1;
     if (bytes_for(1, buffers) > limit) return false;
     unsigned S = 1;

@@ -304,7 +304,8 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
     };
 
     // The waves between the sequence waves and the flush waves compute entries.
-    const bool streaming = g.row_buffers == 2;
+    // (two row buffers exist in workgroups of 512 threads only; the host plans none for 1024)
+    const bool streaming = NT == kRecursionThreads && g.row_buffers == 2;
     const unsigned entry_first_wave = 1 + g.sequence_waves;
     const unsigned entry_end_wave = NT / 64 - (streaming ? g.flush_waves : g.slice_waves);
     const unsigned wide_first = 64 * entry_first_wave;
@@ -658,7 +659,7 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
         recursion_stage(0);
     }
 
-    if (streaming) {
+    if (NT == kRecursionThreads && streaming) {
         // Two row buffers: while the entry waves fill one with tile n, the flush waves send the
         // other, tile n - 1, to HBM; one barrier per tile, and the stores never pause for the
         // arithmetic. One more round after the last tile flushes it.
