@@ -55,11 +55,11 @@ PEAK_HBM_GBPS = 8000.0
 # doubled). KiB per dispatch * 1024 * factor, fetch + write, all kernels of one
 # call added up; the five configurations as in profiles/*_cfgN.md.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg1": 26795740,
+    "cfg1": 26804978,
     "cfg2": 76110936,
     "cfg3": 796269808,
     "cfg4": 3008426691,
-    "cfg5": 3513243065,
+    "cfg5": 3487694887,
     "cfg3:backward": int((394551.2 * 2.0 + 11719.3) * 1024),
     "cfg3:vjp": int((101629.1 * 2.0 + 11718.8) * 1024),
     "cfg5:vjp": int((426681.8 * 2.0 + 2344.1) * 1024),
