@@ -122,19 +122,19 @@ static int ensure_device_ready(int device) {
 // looked at. The variables of the same names are read once, when the library is first used, and
 // only if SPHX_DEBUG_SWITCHES is set to something other than 0.
 enum Switch : int {
-    SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_FLUSH_WAVES, SW_GRADIENT_LANES, SW_GRADIENT_LANES_PARTS,
+    SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_GRADIENT_LANES, SW_GRADIENT_LANES_PARTS,
     SW_GRADIENT_LANES_TILE, SW_GRADIENT_LANES_WAVES, SW_GROUP_THREADS, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST,
-    SW_PREFIX_INSIDE, SW_ROW_BUFFERS,
+    SW_PREFIX_INSIDE,
     SW_SEQUENCE_WAVES, SW_SLICE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
     SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
     SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_COUNT
 };
 static const char* const kSwitchNames[SW_COUNT] = {
-    "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_FLUSH_WAVES", "SPHX_GRADIENT_LANES",
+    "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_GRADIENT_LANES",
     "SPHX_GRADIENT_LANES_PARTS", "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_GROUP_THREADS",
     "SPHX_HESSIAN_LANES",
     "SPHX_HESSIAN_LANES_PARTS", "SPHX_JOB_LIST",
-    "SPHX_PREFIX_INSIDE", "SPHX_ROW_BUFFERS", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
+    "SPHX_PREFIX_INSIDE", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
     "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE",
@@ -510,35 +510,33 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // (the records of a point and its sequences of iterates are an odd number of words apart)
     const unsigned rest_per_point = 3 * ((8 + 3 * (l_max + 1)) | 1u) + 2 * arrays * (tri_all | 1u);
     unsigned fixed = 0; // bytes
-    auto point_bytes = [&](unsigned buffers) { return buffers * rows_per_point * osize + rest_per_point * esize; };
-    auto bytes_for = [&](unsigned S, unsigned buffers) { return S * point_bytes(buffers) + fixed; };
+    const unsigned point_bytes = rows_per_point * osize + rest_per_point * esize;
+    auto bytes_for = [&](unsigned S) { return S * point_bytes + fixed; };
     const unsigned limit = static_cast<unsigned>(lds_limit);
     for (;;) {
         // 24: alignment slack of the row arrays
         // + 3 lines: a staging region starts at a line boundary of its output array
         fixed = (2 * tri_all + table_elems_for(may_split) + 24) * esize + 2 * 3 * 128u;
-        if (bytes_for(1, 1) <= limit || !may_split) break;
+        if (bytes_for(1) <= limit || !may_split) break;
         may_split = false; // the longer job table is what does not fit
     }
-    // Two row buffers (tile n flushed by a wave of its own while tile n+1 is computed) are built
-    // and tested but no longer chosen: they once paid where a single buffer holds one or two
-    // points (second derivatives l_max = 16, float64: 770 us against 810 us), but a wave that
-    // flushes alone waits for its own LDS loads most of the time and the entry waves lose a wave
-    // and half the points per tile. 400 MB of output, us, two buffers against one: second
-    // derivatives float32 l_max = 20, 22, 28 157, 122, 167 against 121, 100, 105 (solid 109, 96
-    // against 88, 79); float64 l_max = 20, 22 149, 134 against 126, 105; l_max = 24 the same.
-    int want_buffers = switch_or(SW_ROW_BUFFERS, 1);
-    unsigned buffers = want_buffers == 2 && threads == kRecursionThreads ? 2u : 1u; // (none with 1024 threads)
-    if (bytes_for(1, buffers) > limit) buffers = 1;
-    if (bytes_for(1, buffers) > limit) return false;
+    // (One row buffer. A second one, flushed by a wave of its own while the next tile is computed,
+    // was built and measured: it once paid where a single buffer holds one or two points (second
+    // derivatives l_max = 16, float64: 770 us against 810 us), but a wave that flushes alone waits
+    // for its own LDS loads most of the time and the entry waves lose a wave and half the points
+    // per tile. 400 MB of output, us, two buffers against one: second derivatives float32
+    // l_max = 20, 22, 28 157, 122, 167 against 121, 100, 105 (solid 109, 96 against 88, 79);
+    // float64 l_max = 20, 22 149, 134 against 126, 105. Its loop is no longer in the kernel,
+    // which is 1-4 % faster without it.)
+    if (bytes_for(1) > limit) return false;
     unsigned S = 1;
-    if (bytes_for(1, buffers) <= budget) {
+    if (bytes_for(1) <= budget) {
         // as many points as the budget holds, a power of two or not: fewer barrier rounds per
         // point (2 GB of output, gradients, float64 l_max = 13: 824 us with 4 points per tile,
         // 611 with 7; l_max = 14: 705 with 4, 602 with 6; float32 l_max = 21: 639 with 4, 603
         // with 6; second derivatives, float64 l_max = 12: 783 with 2, 547 with 3; never more
         // than 4 % slower than the power of two below)
-        S = (budget - fixed) / point_bytes(buffers);
+        S = (budget - fixed) / point_bytes;
         if (switch_or(SW_TILE_POW2, 0) != 0) S = pow2_floor(S);
         if (S > 64) S = 64;
     }
@@ -548,7 +546,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // too much). 500 points, us: second derivatives float64 l_max = 6 16.1 -> 10.2, l_max = 16
     // 16.6 -> 12.6, float32 l_max = 12 17.5 -> 11.2; gradients float32 l_max = 20 23.9 -> 12.7.
     if (S > 1 && switch_or(SW_TILE_SMALL_N, 1) != 0) {
-        unsigned per_cu = limit / bytes_for(S, buffers);
+        unsigned per_cu = limit / bytes_for(S);
         per_cu = per_cu < 1 ? 1u : (per_cu > 2 ? 2u : per_cu);
         if (mode == 2 && elem == 8) per_cu = 1; // more than 128 registers per lane
         const unsigned long long resident = static_cast<unsigned long long>(cus > 0 ? cus : 1) * per_cu;
@@ -560,7 +558,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         }
     }
     const int forced = switch_or(SW_TILE, 0);
-    if (forced > 0 && forced <= 64 && bytes_for(forced, buffers) <= limit) {
+    if (forced > 0 && forced <= 64 && bytes_for(forced) <= limit) {
         S = static_cast<unsigned>(forced);
     }
 
@@ -570,13 +568,13 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     const unsigned point_record = (8 + 3 * static_cast<unsigned>(l_max + 1)) | 1u;
     unsigned az_shift = 0;
     {
-        const unsigned allowed = bytes_for(S, buffers) > budget ? bytes_for(S, buffers) : budget;
+        const unsigned allowed = bytes_for(S) > budget ? bytes_for(S) : budget;
         const int cap = switch_or(SW_AZ_SHIFT, 3);
         for (unsigned shift = cap < 0 ? 0u : (cap > 6 ? 6u : static_cast<unsigned>(cap)); shift >= 1; --shift) {
             const unsigned tiles = 1u << shift;
             if (tiles * S > 64) continue;
             const unsigned extra = (2 * tiles - 3) * S * point_record * esize;
-            if (bytes_for(S, buffers) + extra <= allowed || bytes_for(S, buffers) + extra <= budget) {
+            if (bytes_for(S) + extra <= allowed || bytes_for(S) + extra <= budget) {
                 az_shift = shift;
                 break;
             }
@@ -589,10 +587,6 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.ny = static_cast<int>(ny);
     g.tile = static_cast<int>(S);
     g.az_shift = az_shift;
-    g.row_buffers = buffers;
-    g.flush_waves = buffers == 2 ? static_cast<unsigned>(switch_or(SW_FLUSH_WAVES, 1)) : 0u;
-    if (g.flush_waves > 2) g.flush_waves = 2;
-    if (buffers == 2 && g.flush_waves < 1) g.flush_waves = 1;
     // Waves of their own for the closed forms of l <= 6 (whole rows): with sixteen waves and
     // float32 gradients, where the tile otherwise waits for the entry waves that carry a slice on
     // top of their jobs; one of them up to eight points per tile, two from nine on, three from 28
@@ -604,7 +598,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // closed forms are too much for two or three waves (l_max = 16: 258 against 340 / 300 us).
     g.slice_waves = 0;
     const bool slices_apart = threads > kRecursionThreads && mode == 1 && elem == 4;
-    if (whole && mode < 2 && buffers == 1) {
+    if (whole && mode < 2) {
         const int want = switch_or(SW_SLICE_WAVES, slices_apart ? (S >= 28 ? 3 : (S >= 9 ? 2 : 1)) : 0);
         g.slice_waves = want < 0 ? 0u : (want > 4 ? 4u : static_cast<unsigned>(want));
     }
@@ -633,7 +627,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     };
     // rounds of the entry waves per tile, in tenths of two-sided jobs, with `waves` sequence waves
     auto entry_cost = [&](unsigned waves, bool* split) {
-        wide = threads - 64 * (1 + waves + g.flush_waves + g.slice_waves);
+        wide = threads - 64 * (1 + waves + g.slice_waves);
         // (with two or more points per tile the jobs go as a list ordered by kind, which fills the
         // lanes without splitting, and the two-sided job shares the common factors: 400 MB of
         // output, us, split against not, normalised float32 l_max = 4, 8, 16, 20 110, 115, 108,
@@ -744,7 +738,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.off_ddsph = at;
     if (mode == 2) at = align4(at + S * 9 * row_stride + line);
     g.rows_elems = at;
-    g.tables_at = at * buffers * osize; // a multiple of 16: `at` is one of 4
+    g.tables_at = at * osize; // a multiple of 16: `at` is one of 4
     at = 0; // from here on in numbers of the arithmetic type, counted from tables_at
     g.off_F = at;
     at += tri_all;
@@ -857,18 +851,6 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
         return fail(SPHX_ERR_UNSUPPORTED, "too many samples for one launch");
     }
     const int hard = mode == 2 ? 1 : 6;
-    // The fused product contracts the staged rows in place of the flush and has one row buffer
-    // only: an override that asks for two is not for it (the flush stage of the two-buffer loop
-    // would write through the pointer that holds the caller's sph_grad).
-    struct WithoutRowBuffers {
-        bool active, saved;
-        explicit WithoutRowBuffers(bool on) : active(on), saved(t_switches.set[SW_ROW_BUFFERS]) {
-            if (active) t_switches.set[SW_ROW_BUFFERS] = false;
-        }
-        ~WithoutRowBuffers() {
-            if (active) t_switches.set[SW_ROW_BUFFERS] = saved;
-        }
-    } without_row_buffers(!lane_kernels);
     plan->lanes = false;
     plan->closed_only = l_max <= hard;
     plan->whole = true;
@@ -977,7 +959,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     if (fits && !lane_kernels && plan->rec.g.points_per_pass == 0) {
         // the fused product has no job-list variant of the kernel: whole points side by side
         const Tiling& g = plan->rec.g;
-        const unsigned wide = plan->rec.threads - 64 * (1 + g.sequence_waves + g.flush_waves + g.slice_waves);
+        const unsigned wide = plan->rec.threads - 64 * (1 + g.sequence_waves + g.slice_waves);
         plan->rec.g.points_per_pass = g.jobs_per_point >= wide ? 1u : wide / g.jobs_per_point;
     }
     if (!fits) {

@@ -26,16 +26,16 @@ namespace sphx {
 //                HBM layout (entry_job). Neighbouring lanes take neighbouring m
 //                of one (point, l), so their LDS traffic falls on neighbouring
 //                banks;
-//   flush waves  tile i-1: stream its staged rows to HBM with 16-byte stores.
+//   all waves    after a second barrier: stream the staged rows of tile i to HBM
+//                with 16-byte stores.
 //
 // The first two stages are short chains of dependent operations that only a
 // few lanes can share; running them one and two tiles ahead of the wide stage
-// takes them off the critical path. The last stage is bound by HBM, the entry
-// stage by the vector ALUs: side by side, neither waits for the other. The
-// point tables are kept in three buffers, the iterates and the staged rows in
-// two. With one row buffer (what the host plans; two are kept for tests) no
-// wave is set aside for flushing and all waves flush tile i after a second
-// barrier.
+// takes them off the critical path. The point tables are kept in three
+// buffers, the iterates in two, the staged rows in one. (A second row buffer,
+// flushed by waves of their own while the next tile is computed, was built and
+// measured slower on every shape: waves that only flush wait for their own LDS
+// loads most of the time, and the tile has to be half as large.)
 //
 // NT = 512: two workgroups share a CU, half of its LDS each. NT = 1024: one
 // workgroup has the CU and all of its LDS, its tiles are more than twice as
@@ -303,11 +303,9 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
         }
     };
 
-    // The waves between the sequence waves and the flush waves compute entries.
-    // (two row buffers exist in workgroups of 512 threads only; the host plans none for 1024)
-    const bool streaming = NT == kRecursionThreads && g.row_buffers == 2;
+    // The waves between the sequence waves and the slice waves compute entries.
     const unsigned entry_first_wave = 1 + g.sequence_waves;
-    const unsigned entry_end_wave = NT / 64 - (streaming ? g.flush_waves : g.slice_waves);
+    const unsigned entry_end_wave = NT / 64 - g.slice_waves;
     const unsigned wide_first = 64 * entry_first_wave;
     const unsigned wide_lanes = 64 * (entry_end_wave - entry_first_wave);
 
@@ -333,14 +331,14 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
         return ph;
     };
 
-    // WHOLE: the closed forms of tile n, one lane per point, into row buffer `buffer`. The
+    // WHOLE: the closed forms of tile n, one lane per point, into the staged rows. The
     // entries of a point are cut in slices (by l), dealt to `among` waves of which this is number
     // `who`, so that no single wave carries all of the chain rule and staging.
-    auto closed_stage = [&](unsigned n, unsigned buffer, unsigned who, unsigned among) {
+    auto closed_stage = [&](unsigned n, unsigned who, unsigned among) {
         if constexpr (WHOLE) {
             const unsigned valid = valid_in(n);
             if (lane < valid) {
-                O* staged = row_lds + buffer * g.rows_elems;
+                O* staged = row_lds;
                 const Phases ph = phases_of(n);
                 const T* rec = point_data(n, lane);
                 Point<T> p;
@@ -394,10 +392,10 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
         }
     };
 
-    // stage three of tile n, into row buffer `buffer` (the entry waves)
-    auto entry_stage = [&](unsigned n, unsigned buffer) {
+    // stage three of tile n (the entry waves)
+    auto entry_stage = [&](unsigned n) {
         const unsigned valid = valid_in(n);
-        O* staged = row_lds + buffer * g.rows_elems;
+        O* staged = row_lds;
         const unsigned t = tid - wide_first;
         const Phases ph = phases_of(n);
         const unsigned phase_sph = ph.sph, phase_dsph = ph.dsph, phase_ddsph = ph.ddsph;
@@ -517,15 +515,13 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
         }
     };
 
-    // last stage of tile n: row buffer `buffer` to HBM, by `count` threads of which this is
-    // number `ft`. `lone` (a std::integral_constant): the copy of a run is the work of a single
-    // wave, which then keeps several LDS loads in flight; with all waves of the workgroup on one
-    // run, loads and stores alternating one by one measured faster.
-    auto flush_stage = [&](unsigned n, unsigned buffer, unsigned ft, unsigned count, auto lone) {
-        constexpr int WHOLE_UNROLL = decltype(lone)::value ? SPHX_FLUSH_UNROLL : 1;
+    // last stage of tile n: the staged rows to HBM, by `count` threads of which this is number
+    // `ft`. (With all waves of the workgroup on one run, loads and stores alternating one by one
+    // measured faster than several loads in flight per wave.)
+    auto flush_stage = [&](unsigned n, unsigned ft, unsigned count) {
         const unsigned valid = valid_in(n);
         const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
-        const O* staged = row_lds + buffer * g.rows_elems;
+        const O* staged = row_lds;
         if constexpr (WHOLE) {
             // The tile's run of `len` elements of one output array starts at element `at` of that
             // array. Only whole 128-byte lines go out with vector stores. The line in which the
@@ -534,11 +530,11 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
             // staged in; at the ends of a chunk the partial lines are stored element by element.
             const bool starts = (n & chunk_mask) == 0;
             const bool ends = (n & chunk_mask) == chunk_mask || valid_in(n + 1) == 0;
-            O* carry_to = row_lds + (streaming ? (buffer ^ 1u) : buffer) * g.rows_elems;
+            O* carry_to = row_lds;
             auto flush_run = [&](unsigned region_offset, O* array, unsigned long long at, unsigned len) {
                 using V = typename Pack<O>::type;
                 constexpr unsigned W = Pack<O>::width;
-                O* region = row_lds + buffer * g.rows_elems + region_offset;
+                O* region = row_lds + region_offset;
                 const unsigned phase = phase_of(array, at);
                 O* line0 = array + (at - phase); // HBM address of region element 0
                 const unsigned lo = starts ? phase : 0u; // first element that holds data
@@ -550,19 +546,7 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
                     const unsigned nvec = (full_hi - full_lo) / W;
                     const V* in = reinterpret_cast<const V*>(region + full_lo);
                     V* out = reinterpret_cast<V*>(line0 + full_lo);
-                    unsigned v = ft;
-                    if constexpr (WHOLE_UNROLL > 1) {
-                        for (; v + (WHOLE_UNROLL - 1) * count < nvec; v += WHOLE_UNROLL * count) {
-                            V hold[WHOLE_UNROLL];
-#pragma unroll
-                            for (int u = 0; u < WHOLE_UNROLL; ++u) hold[u] = in[v + u * count];
-#pragma unroll
-                            for (int u = 0; u < WHOLE_UNROLL; ++u) {
-                                emit<O, SPHX_STREAMING_STORES>(hold[u], out + v + u * count);
-                            }
-                        }
-                    }
-                    for (; v < nvec; v += count) {
+                    for (unsigned v = ft; v < nvec; v += count) {
                         emit<O, SPHX_STREAMING_STORES>(in[v], out + v);
                     }
                     tail_from = full_hi;
@@ -614,11 +598,11 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
     // and a butterfly adds the lanes' sums up. With WHOLE == false the staged rows begin at
     // l = H + 1 and closed_form_vjp_kernel has already stored the sum over l <= H, so the
     // result is added to what xyz_grad holds. Wave 0 stays out: it has loads in flight.
-    auto contract_stage = [&](unsigned n, unsigned buffer) {
+    auto contract_stage = [&](unsigned n) {
         if constexpr (VJP) {
             const unsigned valid = valid_in(n);
             const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
-            const T* staged = row_lds + buffer * g.rows_elems + g.off_dsph; // O is T here
+            const T* staged = row_lds + g.off_dsph; // O is T here
             const T* upstream = sph;
             T* xyz_grad = dsph;
             if (wave == 0) return;
@@ -659,63 +643,33 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
         recursion_stage(0);
     }
 
-    if (NT == kRecursionThreads && streaming) {
-        // Two row buffers: while the entry waves fill one with tile n, the flush waves send the
-        // other, tile n - 1, to HBM; one barrier per tile, and the stores never pause for the
-        // arithmetic. One more round after the last tile flushes it.
-        for (unsigned n = 0;; ++n) {
-            __syncthreads(); // tables of tile n+1, iterates of tile n, rows of tile n-1 complete
-            const unsigned valid = valid_in(n);
-            const unsigned before = n > 0 ? valid_in(n - 1) : 0u;
-            if (valid == 0 && before == 0) break;
-            if (wave == 0) {
-                if ((n & (batch_tiles - 1u)) == 0) {
-                    azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
-                    fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz); // for the next batch
-                }
-                if (prefix_wave) prefix_slice();
-            } else if (wave < entry_first_wave) {
-                recursion_stage(n + 1);
-            } else if (wave < entry_end_wave) {
-                if (valid != 0) {
-                    closed_stage(n, n & 1u, wave - entry_first_wave, entry_end_wave - entry_first_wave);
-                    entry_stage(n, n & 1u);
-                }
-            } else if (before != 0) {
-                flush_stage(n - 1, (n - 1) & 1u, tid - 64 * entry_end_wave, 64 * g.flush_waves,
-                            std::true_type{});
-            }
+    // every wave takes part in the flush, after a second barrier
+    for (unsigned n = 0; valid_in(n) != 0; ++n) {
+        __syncthreads(); // tables of tile n+1, iterates of tile n in place; rows of tile n-1 flushed
+        // the closed-form slices go round all waves: those that make tables and iterates
+        // have time to spare; or to wave 0 and the waves set aside for them, when the entry
+        // waves that had a slice on top of their jobs were what the tile waited for
+        if (g.slice_waves == 0) {
+            closed_stage(n, wave, NT / 64);
+        } else if (wave == 0 || wave >= entry_end_wave) {
+            closed_stage(n, wave == 0 ? 0u : wave - entry_end_wave + 1u, g.slice_waves + 1u);
         }
-    } else {
-        // One row buffer (the rows of one point fill most of LDS): every wave takes part in the
-        // flush, after a second barrier.
-        for (unsigned n = 0; valid_in(n) != 0; ++n) {
-            __syncthreads(); // tables of tile n+1, iterates of tile n in place; rows of tile n-1 flushed
-            // the closed-form slices go round all waves: those that make tables and iterates
-            // have time to spare; or to wave 0 and the waves set aside for them, when the entry
-            // waves that had a slice on top of their jobs were what the tile waited for
-            if (g.slice_waves == 0) {
-                closed_stage(n, 0, wave, NT / 64);
-            } else if (wave == 0 || wave >= entry_end_wave) {
-                closed_stage(n, 0, wave == 0 ? 0u : wave - entry_end_wave + 1u, g.slice_waves + 1u);
+        if (wave == 0) {
+            if ((n & (batch_tiles - 1u)) == 0) {
+                azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
+                fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz);
             }
-            if (wave == 0) {
-                if ((n & (batch_tiles - 1u)) == 0) {
-                    azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
-                    fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz);
-                }
-                if (prefix_wave) prefix_slice();
-            } else if (wave < entry_first_wave) {
-                recursion_stage(n + 1);
-            } else if (wave < entry_end_wave) {
-                entry_stage(n, 0);
-            }
-            __syncthreads(); // rows of tile n complete
-            if constexpr (VJP) {
-                contract_stage(n, 0);
-            } else {
-                flush_stage(n, 0, tid, NT, std::false_type{});
-            }
+            if (prefix_wave) prefix_slice();
+        } else if (wave < entry_first_wave) {
+            recursion_stage(n + 1);
+        } else if (wave < entry_end_wave) {
+            entry_stage(n);
+        }
+        __syncthreads(); // rows of tile n complete
+        if constexpr (VJP) {
+            contract_stage(n);
+        } else {
+            flush_stage(n, tid, NT);
         }
     }
     // what is left of this workgroup's share of the batches (no barrier follows)

@@ -44,12 +44,10 @@ struct Tiling {
     unsigned vjp_accumulate; // fused product: add to xyz_grad instead of overwriting it
     unsigned az_shift;      // the point tables are made for 2^az_shift tiles at a time
     unsigned chunk_shift;   // a workgroup takes 2^chunk_shift consecutive tiles at a time
-    unsigned row_buffers;   // 2: tile n is flushed while tile n+1 is computed; 1: one after the other
-    unsigned flush_waves;   // waves that do nothing but flush (row_buffers == 2)
     unsigned prefix_inside; // rows that start at l = 7: the recursion kernel writes l <= 6 too
     unsigned slice_waves;   // not 0: wave 0 and this many waves of their own evaluate the closed forms
                             // of l <= 6 (whole rows, one row buffer); 0: the slices go round all waves
-    // LDS carve-up, in elements of T: the row buffers come first, rows_elems each, with the
+    // LDS carve-up, in elements of T: the staged rows come first, rows_elems of them, with the
     // gradient and second-derivative rows at off_dsph and off_ddsph inside a buffer; the other
     // offsets count from the start of dynamic LDS. (recursion_kernel: the row offsets are in
     // elements of the output arrays, the others in numbers of the arithmetic type and count

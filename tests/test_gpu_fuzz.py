@@ -21,7 +21,7 @@ OVERRIDES = (
     None, None, None,
     ("SPHX_GRADIENT_LANES", (0,)), ("SPHX_HESSIAN_LANES", (0, 2)), ("SPHX_VALUES_LDS", (1,)),
     ("SPHX_JOB_LIST", (0, 1, 2)), ("SPHX_PREFIX_INSIDE", (0,)), ("SPHX_TILE", (1, 2, 3, 5, 7, 8)),
-    ("SPHX_ROW_BUFFERS", (1, 2)), ("SPHX_SEQUENCE_WAVES", (1, 2)), ("SPHX_CHUNK_SHIFT", (0, 1, 2, 3)),
+    ("SPHX_SEQUENCE_WAVES", (1, 2, 3, 4)), ("SPHX_CHUNK_SHIFT", (0, 1, 2, 3)),
     ("SPHX_AZ_SHIFT", (0, 1, 2, 3)), ("SPHX_SPLIT_SIDES", (0,)), ("SPHX_TILE_POW2", (1,)),
     ("SPHX_SPLIT_BELOW", (0, 64)), ("SPHX_GRADIENT_LANES_PARTS", (1, 2)), ("SPHX_GROUP_THREADS", (512, 1024)),
     ("SPHX_GROUP_THREADS", (1024,)), ("SPHX_SPREAD_KINDS", (0, 1)), ("SPHX_SLICE_WAVES", (0, 1, 2, 3)),
