@@ -171,46 +171,15 @@ __device__ __forceinline__ void stage(const Rows<O>& out, int k, const Point<T>&
 // lower l but hardly any gradients of lower l, so what a slice does not stage the compiler
 // drops: several waves can share the entries of a point, each evaluating little more than its
 // own slice.
-//
-// ROTATE: the lanes of a wave hold one point each and store entry k of their points with one
-// instruction, at addresses one row length apart. When the row length is a multiple of 8 words
-// these fall on few LDS banks (a multiple of 32 words: on one, and the store takes 32 times as
-// long). The entries then go out four at a time, lane by lane in a different order
-// (k + turn, k + turn + 1, ... modulo 4, turn in 0..3 chosen by the caller so that lanes whose
-// rows share banks differ in it), which spreads one instruction over four times as many banks
-// for two selects per stored number.
-// (a0, a1, a2, a3) -> (a_turn, a_turn+1, a_turn+2, a_turn+3), indices modulo 4
-template <typename T> __device__ __forceinline__ void rotate4(unsigned turn, T& a0, T& a1, T& a2, T& a3) {
-    const bool one = (turn & 1u) != 0, two = (turn & 2u) != 0;
-    const T b0 = one ? a1 : a0, b1 = one ? a2 : a1, b2 = one ? a3 : a2, b3 = one ? a0 : a3;
-    a0 = two ? b2 : b0;
-    a1 = two ? b3 : b1;
-    a2 = two ? b0 : b2;
-    a3 = two ? b1 : b3;
-}
-
-template <typename T, int MODE, bool NORM, int H, int KLO = 0, int KHI = (H + 1) * (H + 1),
-          bool ROTATE = false, typename O = T>
-__device__ __forceinline__ void closed_form_job(const Point<T>& p, const Rows<O>& out,
-                                                [[maybe_unused]] unsigned turn = 0) {
+template <typename T, int MODE, bool NORM, int H, int KLO = 0, int KHI = (H + 1) * (H + 1), typename O = T>
+__device__ __forceinline__ void closed_form_job(const Point<T>& p, const Rows<O>& out) {
     static_assert(MODE < 2 || H <= 1, "second derivatives in closed form stop at l = 1");
-    static_assert(MODE < 2 || !ROTATE, "rotated stores are written for values and gradients");
     constexpr int NH = (H + 1) * (H + 1);
-    constexpr int KROT = ROTATE ? KLO + (KHI - KLO) / 4 * 4 : KLO; // [KLO, KROT) in rotated fours
     T Y[NH];
     low_values<T, H>(p.x, p.y, p.z, p.x2, p.y2, p.z2, Y);
     if constexpr (MODE == 0) {
 #pragma unroll
-        for (int k = KLO; k < KROT; k += 4) {
-            T v0 = Y[k], v1 = Y[k + 1], v2 = Y[k + 2], v3 = Y[k + 3];
-            rotate4<T>(turn, v0, v1, v2, v3);
-            out.sph[k + (turn & 3u)] = static_cast<O>(v0);
-            out.sph[k + ((turn + 1u) & 3u)] = static_cast<O>(v1);
-            out.sph[k + ((turn + 2u) & 3u)] = static_cast<O>(v2);
-            out.sph[k + ((turn + 3u) & 3u)] = static_cast<O>(v3);
-        }
-#pragma unroll
-        for (int k = KROT; k < KHI; ++k) {
+        for (int k = KLO; k < KHI; ++k) {
             out.sph[k] = static_cast<O>(Y[k]);
         }
     } else {
@@ -226,19 +195,7 @@ __device__ __forceinline__ void closed_form_job(const Point<T>& p, const Rows<O>
             return finish<T, MODE, NORM>(p, e);
         };
 #pragma unroll
-        for (int k = KLO; k < KROT; k += 4) {
-            Entry<T> e0 = finished(k), e1 = finished(k + 1), e2 = finished(k + 2), e3 = finished(k + 3);
-            rotate4<T>(turn, e0.v, e1.v, e2.v, e3.v);
-            rotate4<T>(turn, e0.gx, e1.gx, e2.gx, e3.gx);
-            rotate4<T>(turn, e0.gy, e1.gy, e2.gy, e3.gy);
-            rotate4<T>(turn, e0.gz, e1.gz, e2.gz, e3.gz);
-            put<T, MODE>(out, k + static_cast<int>(turn & 3u), e0);
-            put<T, MODE>(out, k + static_cast<int>((turn + 1u) & 3u), e1);
-            put<T, MODE>(out, k + static_cast<int>((turn + 2u) & 3u), e2);
-            put<T, MODE>(out, k + static_cast<int>((turn + 3u) & 3u), e3);
-        }
-#pragma unroll
-        for (int k = KROT; k < KHI; ++k) {
+        for (int k = KLO; k < KHI; ++k) {
             put<T, MODE>(out, k, finished(k));
         }
     }

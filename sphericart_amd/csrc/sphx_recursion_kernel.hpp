@@ -355,36 +355,20 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
                 rows.dsph = staged + g.off_dsph + ph.dsph + lane * 3 * ny;
                 rows.ddsph = staged + g.off_ddsph + ph.ddsph + lane * 9 * ny;
                 if constexpr (H == 6) {
-                    // float32 rows a multiple of 32 words long (l_max = 7, 15, 23, ...): the
-                    // stores of all lanes would fall on one LDS bank; stored in rotated fours
-                    // instead (closed_form_job; l_max = 7, 500k points, gradients: 343 -> 216 us).
-                    // Not for float64 and not for values alone, where the selects cost registers
-                    // that the kernel does not have to spare (values: 68 -> 89, and l_max = 9 lost
-                    // its third workgroup per CU, 80 -> 106 us).
-                    // Nor in workgroups of 1024 threads: their tiles beyond l_max = 15 hold few enough
-                    // points for the conflicts to cost less than the selects (us per 1.2 GB, rotated
-                    // against not: l_max = 15, 23 points, 270, 298; l_max = 23, 31, 39 with 10, 6, 4
-                    // points 269, 312, 345 against 266, 258, 269), and without this code the whole
-                    // kernel needs fewer registers (l_max = 32: 732 -> 710 us).
-                    constexpr bool MAY_ROTATE = sizeof(T) == 4 && MODE == 1 && NT == kRecursionThreads; // not where T and O differ
-                    if (MAY_ROTATE && (ny & 31u) == 0) {
-                        const unsigned turn = lane & 3u;
-                        if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 8, true>(p, rows, turn);
-                        if (1 % among == who) closed_form_job<T, MODE, NORM, H, 8, 16, true>(p, rows, turn);
-                        if (2 % among == who) closed_form_job<T, MODE, NORM, H, 16, 24, true>(p, rows, turn);
-                        if (3 % among == who) closed_form_job<T, MODE, NORM, H, 24, 32, true>(p, rows, turn);
-                        if (4 % among == who) closed_form_job<T, MODE, NORM, H, 32, 40, true>(p, rows, turn);
-                        if (5 % among == who) closed_form_job<T, MODE, NORM, H, 40, 49, true>(p, rows, turn);
-                    } else {
-                        if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows);
-                        if (1 % among == who) closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows);
-                        if (2 % among == who) closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows);
-                        if (3 % among == who) closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows);
-                        if (4 % among == who) closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows);
-                        if (5 % among == who) closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows);
-                        if (6 % among == who) closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows);
-                        if (7 % among == who) closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows);
-                    }
+                    // (Rows a multiple of 32 words long, l_max = 7, 15, 23, ...: the stores of all
+                    // lanes fall on one LDS bank. Storing in rotated fours, two selects per number,
+                    // paid for tiles of many points, l_max = 15 with 23 points 270 us against 298
+                    // per 1.2 GB, and cost more than the conflicts from ten points down, l_max = 23,
+                    // 31, 39 269, 312, 345 us against 266, 258, 269; without that code the kernel
+                    // needs fewer registers, l_max = 32: 732 -> 710 us. It is gone.)
+                    if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows);
+                    if (1 % among == who) closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows);
+                    if (2 % among == who) closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows);
+                    if (3 % among == who) closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows);
+                    if (4 % among == who) closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows);
+                    if (5 % among == who) closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows);
+                    if (6 % among == who) closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows);
+                    if (7 % among == who) closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows);
                 } else {
                     if (who == 0) closed_form_job<T, MODE, NORM, H>(p, rows);
                 }
