@@ -127,7 +127,7 @@ enum Switch : int {
     SW_PREFIX_INSIDE,
     SW_SEQUENCE_WAVES, SW_SLICE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
     SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
-    SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_COUNT
+    SW_VALUES_TILE_STEP, SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_COUNT
 };
 static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_GRADIENT_LANES",
@@ -137,7 +137,7 @@ static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_PREFIX_INSIDE", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
-    "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE",
+    "SPHX_VALUES_TILE_STEP", "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE",
 };
 struct Switches {
     bool set[SW_COUNT] = {};
@@ -213,7 +213,7 @@ static void plan_closed(size_t n_samples, int l_max, int hard, int mode, size_t 
     out->lds_bytes = at * static_cast<unsigned>(elem);
 }
 
-// values_kernel: 64 (or 32) points per workgroup, their rows and tables in LDS. Returns false
+// values_kernel: up to 64 points per workgroup, their rows and tables in LDS. Returns false
 // when that does not fit, and the recursion kernel takes over.
 static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit, Launch* out,
                         bool with_sums = false) {
@@ -226,28 +226,33 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     const unsigned row_stride = (ny * (esize / 4u)) % 8u == 0 ? ny + vec : ny;
     const unsigned table_stride = (3u * static_cast<unsigned>(l_max + 1)) | 1u;
     const unsigned tri_all = static_cast<unsigned>(l_max + 1) * (l_max + 2) / 2;
-    // float32 values whose 32 rows need more than half a CU's LDS (l_max >= 23) are left to the
-    // recursion kernel, which with its job-list variant is faster there (1 GB of output, l_max =
-    // 24, 28, 32: 508, 505, 472 us against 574, 567, 543; l_max = 26 is the exception, 627
-    // against 546); in float64 the values kernel still wins with a whole CU's LDS (l_max = 18,
-    // 20, 22: 426, 401, 380 against 483, 436, 429).
-    unsigned allowed = static_cast<unsigned>(
-        switch_or(SW_VALUES_LDS, with_sums || elem == 8 ? 160 * 1024 : 80 * 1024));
+    unsigned allowed = static_cast<unsigned>(switch_or(SW_VALUES_LDS, 160 * 1024));
     if (allowed > static_cast<unsigned>(lds_limit)) allowed = static_cast<unsigned>(lds_limit);
-    // Fewer than 64 points per workgroup leave lanes idle: with 32 the values kernel still beats
-    // the recursion kernel (l_max = 32 float32, 500k points: 781 against 1 077 us; l_max = 20
-    // float64: 470 against 710), with 16 it does not (l_max = 28 float64: 1 404 against 1 089).
+    // Fewer than 64 points per workgroup leave lanes idle, and from some tile on the recursion
+    // kernel with its job list is faster. Values, 1 GB of output, us, values kernel against
+    // recursion kernel: float32 with two workgroups per CU l_max = 24 (28 points) 306 against 397,
+    // l_max = 26 (24 points) 338 against 392; with one workgroup per CU l_max = 28 (44 points) 355
+    // against 393, l_max = 29 (40) 370 against 390, l_max = 30 (38) 419 against 391; float64
+    // l_max = 22 (32 points) 297 against 305, l_max = 23 (30) 319 against 302.
     // The product keeps no rows for HBM in LDS and has far more arithmetic per point to win:
     // it goes down to 8 points (l_max = 24 float64, 200k points: 830 us with 16 points per
     // workgroup against 1 456 us through the recursion kernel).
     const unsigned smallest = static_cast<unsigned>(
-        with_sums ? switch_or(SW_VJP_MIN_TILE, 8) : switch_or(SW_VALUES_MIN_TILE, 32));
+        with_sums ? switch_or(SW_VJP_MIN_TILE, 8) : switch_or(SW_VALUES_MIN_TILE, elem == 4 ? 24 : 32));
+    const unsigned smallest_alone = !with_sums && elem == 4 && smallest < 40 ? 40 : smallest;
+    // Values: the tile goes down in steps of 4 points, so that as many lanes work as rows fit
+    // (l_max = 16: 60 points where halving leaves 32, 202 against 278 us in float32, 240 against
+    // 352 in float64; steps of 1 or 2 gain nothing more and some odd sizes lose). The product halves.
+    const unsigned step = with_sums ? 0u : static_cast<unsigned>(switch_or(SW_VALUES_TILE_STEP, 4));
     // Two workgroups per CU (80 KB each) overlap one's tables and flush with the other's
-    // arithmetic: preferred, also at half the lanes, over one workgroup with all of LDS
-    // (l_max = 16 float32, 500k points: 142 against 164 us; l_max = 12 float64: 115 against 146).
+    // arithmetic: preferred, also with fewer lanes at work, over one workgroup with all of LDS
+    // (l_max = 16 float32, 500k points, 32 points against 64: 142 against 164 us; l_max = 12
+    // float64: 115 against 146).
+    const unsigned half = 80u * 1024u;
     unsigned tile = 0, rows = 0, bytes = 0;
-    for (unsigned limit : {allowed < 80u * 1024u ? allowed : 80u * 1024u, allowed}) {
-        for (unsigned t = 64; t >= smallest && t >= 8 && tile == 0; t /= 2) {
+    for (unsigned limit : {allowed < half ? allowed : half, allowed}) {
+        const unsigned least = limit > half ? smallest_alone : smallest;
+        for (unsigned t = 64; t >= least && t >= 8 && tile == 0; t = step == 0 ? t / 2 : t - step) {
             rows = (t * row_stride + vec - 1u) / vec * vec;
             // the product: the waves' sums; with fewer than 64 points also copies of the
             // prefactor tables (vjp_groups_kernel)

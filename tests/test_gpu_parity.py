@@ -115,6 +115,32 @@ def test_gradient_lanes_with_shared_channels(oracle, library, switches, dtype, n
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_values_kernel_with_tiles_of_any_size(oracle, library, switches, dtype):
+    """values_kernel takes as many points per workgroup as fit in LDS, in steps of four: tiles
+    of 60, 44, 28 points and others, a last tile that is not full, two workgroups per CU and
+    one with all of LDS (float32 l_max = 28), steps of one and halving, against the oracle."""
+    rng = np.random.default_rng(47)
+    for l_max in (11, 16, 19, 21, 24, 28):
+        for normalized in (True, False):
+            for n in (1, 59, 1201):
+                xyz = special_points(dtype, rng, n)
+                want = oracle.compute(xyz, l_max, normalized, "values")
+                xyz_dev = torch.from_numpy(xyz).cuda()
+                for step, least in ((None, None), (1, 8), (0, 32)):
+                    library.sphx_reset_switches()
+                    if step is not None:
+                        switches("SPHX_VALUES_TILE_STEP", step)
+                        switches("SPHX_VALUES_MIN_TILE", least)
+                    announce("values, tiles", np.dtype(dtype).name, normalized, l_max, n, "step", step)
+                    status, got = run_launch_layer(library, xyz_dev, l_max, normalized, "values")
+                    torch.cuda.synchronize()
+                    assert status == 0, library.sphx_last_error()
+                    got = tuple(None if g is None else g.cpu().numpy() for g in got)
+                    check(got, want, (l_max, normalized, n, step))
+    library.sphx_reset_switches()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("mode", ["values", "gradients", "hessians"])
 def test_workgroups_of_512_and_1024_threads(oracle, library, switches, dtype, mode):
     """The recursion kernel in workgroups of 512 threads (two to a CU) and of 1024 (one, with all of

@@ -90,6 +90,15 @@ def test_launch_plans(library):
     assert status == 0 and threads == 512 and lds <= 80 * 1024
     # second derivatives in float64 keep 512 threads (more than 128 registers per lane)
     assert _plan(library, 100_000, 16, 2, True)[1][1] == 512
+    # values: as many points per workgroup as fit in half a CU's LDS, in steps of four; in float32
+    # one workgroup with all of LDS while 40 points fit, then the recursion kernel
+    status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 16, 0, False)
+    assert status == 0 and (tile, threads) == (60, 512) and lds == 60 * (289 + 51) * 4
+    status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 28, 0, False)
+    assert status == 0 and (tile, threads) == (44, 512) and 80 * 1024 < lds <= 160 * 1024
+    assert _plan(library, 1_000_000, 30, 0, False)[1][1] == 1024
+    assert _plan(library, 1_000_000, 22, 0, True)[1][:2] == [32, 512]
+    assert _plan(library, 1_000_000, 23, 0, True)[1][1] == 1024
     assert _plan(library, 10, 65, 0, False)[0] == 2       # beyond the tables
     assert _plan(library, 10, 64, 2, True)[0] == 2        # one point's rows no longer fit in LDS
     assert b"LDS" in library.sphx_last_error()
