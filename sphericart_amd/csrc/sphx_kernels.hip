@@ -126,8 +126,8 @@ enum Switch : int {
     SW_GRADIENT_LANES_TILE, SW_GRADIENT_LANES_WAVES, SW_GROUP_THREADS, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST,
     SW_PREFIX_INSIDE,
     SW_SEQUENCE_WAVES, SW_SLICE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
-    SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
-    SW_VALUES_TILE_STEP, SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_COUNT
+    SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_ALONE, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
+    SW_VALUES_PACK, SW_VALUES_TILE_STEP, SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_COUNT
 };
 static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_GRADIENT_LANES",
@@ -136,8 +136,8 @@ static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_HESSIAN_LANES_PARTS", "SPHX_JOB_LIST",
     "SPHX_PREFIX_INSIDE", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
-    "SPHX_TILE_SMALL_N", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
-    "SPHX_VALUES_TILE_STEP", "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE",
+    "SPHX_TILE_SMALL_N", "SPHX_VALUES_ALONE", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
+    "SPHX_VALUES_PACK", "SPHX_VALUES_TILE_STEP", "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE",
 };
 struct Switches {
     bool set[SW_COUNT] = {};
@@ -219,6 +219,7 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
                         bool with_sums = false) {
     Tiling& g = out->g;
     std::memset(&g, 0, sizeof(g));
+    if (!with_sums && l_max > 63) return false; // a channel's prefactors: one per lane of a wave
     const unsigned esize = static_cast<unsigned>(elem);
     const unsigned ny = static_cast<unsigned>(l_max + 1) * (l_max + 1);
     const unsigned vec = 16u / esize;
@@ -239,7 +240,35 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // workgroup against 1 456 us through the recursion kernel).
     const unsigned smallest = static_cast<unsigned>(
         with_sums ? switch_or(SW_VJP_MIN_TILE, 8) : switch_or(SW_VALUES_MIN_TILE, elem == 4 ? 24 : 32));
-    const unsigned smallest_alone = !with_sums && elem == 4 && smallest < 40 ? 40 : smallest;
+    // Between tiles of 24-44 points, with lanes idle, and the recursion kernel lie two more forms
+    // of the values kernel: one workgroup per CU with all of its LDS and up to 64 points, and
+    // tiles of 32 or 16 points whose waves evaluate two or four channels side by side, all lanes
+    // at work. Which is fastest goes by the shape, not by a rule (row lengths, channels per wave
+    // and workgroups per CU all change with l_max). 1 GB of values, us, in the order tile that fits
+    // half of LDS / one workgroup with all of LDS / two channels, 32 points / four channels, 16
+    // points / recursion kernel, float32:
+    //   l_max 18 218 288 216 249 412      l_max 19 249 301 291 289 418      l_max 20 239 273 250 279 403
+    //   l_max 21 255 272 248 268 397      l_max 22 271 263 238 260 389      l_max 23 321 289   - 341 425
+    //   l_max 24 286 289   - 296 398      l_max 25 319 295   - 286 397      l_max 26 318 301   - 275 393
+    //   l_max 27   - 343 390 393 419      l_max 28   - 329 365 354 393      l_max 29   - 340 369 342 389
+    //   l_max 30   - 364 367 332 391      l_max 31   - 378 372 348 389      l_max 32   - 391 349 313 378
+    //   l_max 33   - 388 350 305 386      l_max 34   - 432   - 532 383
+    // float64:
+    //   l_max 13 221 244 283 310 313      l_max 14 227 214 239 309 310      l_max 15 258 234 257 326 347
+    //   l_max 16   - 241 361 335 322      l_max 20   - 273 300 363 313      l_max 21   - 292 303 365 296
+    //   l_max 22   - 295 282 328 303      l_max 23   - 337   - 582 301
+    unsigned pack_by_shape = 1;
+    bool alone_by_shape = false;
+    if (!with_sums && elem == 4) {
+        if (l_max == 21 || l_max == 22) pack_by_shape = 2;
+        if (l_max == 25 || l_max == 26 || (l_max >= 30 && l_max <= 33)) pack_by_shape = 4;
+        alone_by_shape = l_max == 23;
+    } else if (!with_sums) {
+        if (l_max == 22) pack_by_shape = 2;
+        alone_by_shape = l_max == 14 || l_max == 15;
+    }
+    const bool alone = !with_sums && switch_or(SW_VALUES_ALONE, alone_by_shape ? 1 : 0) != 0;
+    const unsigned smallest_alone = !with_sums && elem == 4 && smallest < 40 && !alone ? 40 : smallest;
     // Values: the tile goes down in steps of 4 points, so that as many lanes work as rows fit
     // (l_max = 16: 60 points where halving leaves 32, 202 against 278 us in float32, 240 against
     // 352 in float64; steps of 1 or 2 gain nothing more and some odd sizes lose). The product halves.
@@ -250,16 +279,26 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // float64: 115 against 146).
     const unsigned half = 80u * 1024u;
     unsigned tile = 0, rows = 0, bytes = 0;
-    for (unsigned limit : {allowed < half ? allowed : half, allowed}) {
-        const unsigned least = limit > half ? smallest_alone : smallest;
-        for (unsigned t = 64; t >= least && t >= 8 && tile == 0; t = step == 0 ? t / 2 : t - step) {
-            rows = (t * row_stride + vec - 1u) / vec * vec;
-            // the product: the waves' sums; with fewer than 64 points also copies of the
-            // prefactor tables (vjp_groups_kernel)
-            const unsigned extra = !with_sums ? 0u : (t == 64 ? 8u * 3u * 64u : 8u * 3u * 64u + 2u * tri_all);
-            bytes = (rows + t * table_stride + extra) * esize;
-            if (bytes <= limit) tile = t;
+    unsigned pack = with_sums ? 1u : static_cast<unsigned>(switch_or(SW_VALUES_PACK, static_cast<int>(pack_by_shape)));
+    if (pack != 2 && pack != 4) pack = 1;
+    auto search = [&]() {
+        for (unsigned limit : {alone ? 0u : (allowed < half ? allowed : half), allowed}) {
+            const unsigned least = pack > 1 ? 8u : (limit > half ? smallest_alone : smallest);
+            for (unsigned t = 64 / pack; t >= least && t >= 8 && tile == 0; t = step == 0 ? t / 2 : t - step) {
+                if (pack > 1 && t != 64 / pack) break;
+                rows = (t * row_stride + vec - 1u) / vec * vec;
+                // the product: the waves' sums; with fewer than 64 points also copies of the
+                // prefactor tables (vjp_groups_kernel)
+                const unsigned extra = !with_sums ? 0u : (t == 64 ? 8u * 3u * 64u : 8u * 3u * 64u + 2u * tri_all);
+                bytes = (rows + t * table_stride + extra) * esize;
+                if (bytes <= limit) tile = t;
+            }
         }
+    };
+    search();
+    if (tile == 0 && pack > 1) { // (a smaller LDS than the shapes above were measured with)
+        pack = 1;
+        search();
     }
     if (tile == 0) return false;
     g.n_samples = n_samples;
@@ -275,13 +314,14 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     g.off_jobs = rows + tile * table_stride; // the product: the waves' sums,
     g.off_F = g.off_jobs + 8u * 3u * 64u;    // and (fewer than 64 points) the prefactor tables
     g.off_Q = g.off_F + tri_all;
+    g.points_per_pass = with_sums ? 0u : pack; // values_kernel: channels a wave evaluates side by side
     out->workgroups = g.tiles_per_xcd * 8u;
     // one wave per l channel above the closed forms, eight at most
     int waves = switch_or(SW_VALUES_WAVES, 8);
     waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
     // (the product's closed-form slices want at least four; values: one for the tables, one for
     // the closed forms)
-    int want = l_max - 6;
+    int want = (l_max - 6 + static_cast<int>(pack) - 1) / static_cast<int>(pack);
     // the product, 0.8 GB of sph_grad, us: l_max = 9, 10 (three and four channels) 266, 310 with
     // four waves, 207, 282 with three (float64 279, 333 against 233, 304); l_max = 12 350 with six,
     // 316 with four (float64 385 against 321); one or two channels are best with four
@@ -1088,7 +1128,9 @@ static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* d
     if (plan.lanes) {
         if constexpr (MODE == 0) {
             const Launch& l = plan.closed;
-            auto kernel = values_kernel<T, NORM>;
+            auto kernel = l.g.points_per_pass == 4   ? values_kernel<T, NORM, 4>
+                          : l.g.points_per_pass == 2 ? values_kernel<T, NORM, 2>
+                                                     : values_kernel<T, NORM, 1>;
             if (l.lds_bytes > 64u * 1024u) {
                 unsigned unused = 0;
                 hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &unused);
@@ -1846,7 +1888,8 @@ int sphx_describe_plan(size_t n_samples, int l_max, int derivatives, int is_f64,
         text = "closed_form_kernel<" + head + ", " + std::to_string(l_max) + ", false>" + geometry(plan.closed);
     } else if (plan.lanes) {
         const char* names[3] = {"values_kernel", "gradients_lanes_kernel", "hessians_lanes_kernel"};
-        text = std::string(names[derivatives]) + "<" + t + ", " + (normalized ? "true" : "false") + ">" +
+        text = std::string(names[derivatives]) + "<" + t + ", " + (normalized ? "true" : "false") +
+               (derivatives == 0 ? ", " + std::to_string(plan.closed.g.points_per_pass) : std::string()) + ">" +
                geometry(plan.closed);
     } else {
         if (!plan.whole && plan.rec.g.prefix_inside == 0) {

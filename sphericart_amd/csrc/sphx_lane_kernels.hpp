@@ -13,26 +13,38 @@
 namespace sphx {
 
 // ---------------------------------------------------------------------------
-// Values only, l_max > 6, rows short enough that those of 64 points fit in LDS:
-// 64 points per workgroup, one point per lane, one to eight waves that share
-// the l channels of the same 64 points.
+// Values only, l_max > 6, rows short enough that those of 16 to 64 points fit
+// in LDS: one point per lane, one to eight waves that share the l channels of
+// the same points.
 //
 // Without derivatives an entry is three multiplications, so what counts is what
 // surrounds them. With one point per lane l and m are the same for the whole
-// wave: the prefactors come from constant memory through the scalar unit, no
-// job has to be decoded and no iterate passes through LDS, about 15
-// instructions per (l, +-m) pair of entries in all, a tenth of what the
-// recursion kernel spends on them. (With derivatives the entries themselves
-// dominate and rows are four and thirteen times as long, so that far fewer
-// than 64 points fit: gradients_lanes_kernel takes l_max up to about 16, the
-// recursion kernel the rest.)
+// wave: no job has to be decoded and no iterate passes through LDS. The
+// prefactors of a channel, m = 0..l, are loaded once, one per lane, and the
+// recursion takes each from its lane (v_readlane), so that its loop touches no
+// memory but the point's table in LDS, whose entries for the next m are fetched
+// before the arithmetic of this one: about 25 instructions per (l, +-m) pair of
+// entries, a fraction of what the recursion kernel spends on them. (Prefactors
+// through scalar loads inside the loop made every step wait for them: LDS and
+// scalar loads share one counter, so nothing could be fetched ahead. 1 GB of
+// values, float32, l_max = 22, 26, 28: 288, 341, 355 us then, 270, 315, 327 so.)
+// (With derivatives the entries themselves dominate and rows are four and
+// thirteen times as long, so that far fewer than 64 points fit:
+// gradients_lanes_kernel takes l_max up to about 16, the recursion kernel the
+// rest.)
 //
 // The rows of 64 points take most of a CU's LDS from l_max of about 12 on, and
 // one wave would leave three of the four SIMDs idle: the l channels are dealt
 // to the waves of the workgroup (in snake order, long and short ones mixed),
-// each wave evaluating its channels for all 64 points (l_max = 15 float32,
-// 500k points: 245 us with one wave, 113 with four, 106 with six). When not
-// even 64 rows fit, 32 points per workgroup and half the lanes idle.
+// each wave evaluating its channels for all points of the tile (l_max = 15
+// float32, 500k points: 245 us with one wave, 113 with four, 106 with six).
+// When 64 rows do not fit the tile is smaller, any number of points, and the
+// lanes beyond it idle; or (K = 2, 4) the tile is 32 or 16 points and a wave
+// evaluates K channels l0, l0 - 1, .. side by side, lane = side * (64 / K) +
+// point: it walks m down from l0 for all of them, each lane picks the
+// prefactors of its own channel, and the lanes of a shorter channel join when
+// m reaches their l. All lanes work then, for about 40 instructions per step
+// of two channels (the host picks by shape, see plan_values).
 //
 // Same operations in the same order as the reference: c_m, s_m, 2(m+1)z as in
 // templates.hpp:451-466, l <= 6 in closed form, then per l the recursion of
@@ -47,7 +59,33 @@ namespace sphx {
 // ---------------------------------------------------------------------------
 constexpr unsigned kValuesMaxThreads = 512;
 
-template <typename T, bool NORM>
+// The value a given lane holds, for the whole wave (the lane number is the same for all lanes).
+__device__ __forceinline__ float from_lane(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+__device__ __forceinline__ double from_lane(double v, int lane) {
+    const long long bits = __double_as_longlong(v);
+    const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(bits), lane));
+    const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(bits >> 32), lane));
+    return __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo));
+}
+
+// Prefactors of one l channel, m = 0..l: lane j of the wave holds that of m = j (one load for the
+// whole channel; all lanes must be active), and the recursion takes them from there with no
+// memory access in its loop. For l <= 63.
+template <typename T> struct ChannelPrefactors {
+    T lanes;
+    __device__ __forceinline__ ChannelPrefactors() : lanes(0) {}
+    __device__ __forceinline__ ChannelPrefactors(const T* row, int l, unsigned lane)
+        : lanes(row[static_cast<int>(lane) < l ? static_cast<int>(lane) : l]) {
+        // keeps the load here, where all lanes are active: its only uses are the reads of single
+        // lanes, and it would otherwise be moved to them, into code that only some lanes run
+        asm volatile("" : "+v"(lanes));
+    }
+    __device__ __forceinline__ T operator[](int m) const { return from_lane(lanes, m); }
+};
+
+template <typename T, bool NORM, unsigned K = 1>
 __global__ __launch_bounds__(kValuesMaxThreads) void values_kernel(Tiling g, const T* __restrict__ xyz,
                                                                   T* __restrict__ sph) {
     constexpr int H = 6;
@@ -68,12 +106,15 @@ __global__ __launch_bounds__(kValuesMaxThreads) void values_kernel(Tiling g, con
     const unsigned long long left = g.n_samples - first;
     const unsigned valid = left < tile ? static_cast<unsigned>(left) : tile;
 
+    // K > 1: the tile is 64 / K points, and lane = side * (64 / K) + point
+    const unsigned point = K == 1 ? lane : lane & (64u / K - 1u);
+    const unsigned side = K == 1 ? 0u : lane / (64u / K);
     Point<T> p;
     p.x = p.y = p.z = p.x2 = p.y2 = p.z2 = p.ir = 0;
-    T* row = lds + lane * g.rows_elems;
-    T* tab = lds + g.off_pts + lane * g.off_iter; // [m][3]: c_m, s_m, 2(m+1)z
-    if (lane < valid) {
-        p = load_point<T, NORM>(xyz + (first + lane) * 3);
+    T* row = lds + point * g.rows_elems;
+    T* tab = lds + g.off_pts + point * g.off_iter; // [m][3]: c_m, s_m, 2(m+1)z
+    if (point < valid) p = load_point<T, NORM>(xyz + (first + point) * 3);
+    if (point < valid && side == 0) {
         if (wave == 0) {
             const T twoz = p.z + p.z;
             T cm = 1.0, sm = 0.0, tz = twoz;
@@ -99,18 +140,76 @@ __global__ __launch_bounds__(kValuesMaxThreads) void values_kernel(Tiling g, con
         }
     }
     __syncthreads(); // the tables
-    if (lane < valid) {
+    if constexpr (K > 1) {
         const T rxy = p.x2 + p.y2;
-        const T* cF = table_F<T>();
-        const T* cQ = table_Q<T>();
+        // K channels side by side, l0, l0 - 1, ..: the wave walks m from l0 down for all of them,
+        // the lanes of a shorter channel join when m reaches their l (what they hold before that
+        // is not used: the first two steps of a channel take nothing from earlier ones); bundles
+        // of K channels go to the waves like single channels below
+        const unsigned bundles = (static_cast<unsigned>(L - H) + K - 1u) / K;
+        for (unsigned i = 0; i < bundles; ++i) {
+            const unsigned pos = i % waves;
+            if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
+            const int l0 = L - static_cast<int>(i * K); // >= H + 1, so l0 - (K - 1) >= 0
+            ChannelPrefactors<T> pk[K], qk[K];
+#pragma unroll
+            for (unsigned k = 0; k < K; ++k) {
+                const int lk = l0 - static_cast<int>(k);
+                pk[k] = ChannelPrefactors<T>(table_F<T>() + lk * (lk + 1) / 2, lk, lane);
+                qk[k] = ChannelPrefactors<T>(table_Q<T>() + lk * (lk + 1) / 2, lk, lane);
+            }
+            if (point >= valid) continue; // (all lanes are back at the next bundle's loads)
+            const int l = l0 - static_cast<int>(side);
+            const bool live = l > H;
+            T* mid = row + l * l + l;
+            auto prefactors = [&](int m, T& f, T& q) {
+                f = pk[0][m];
+                q = qk[0][m];
+#pragma unroll
+                for (unsigned k = 1; k < K; ++k) {
+                    const T fk = pk[k][m], qk_ = qk[k][m];
+                    if (side == k) {
+                        f = fk;
+                        q = qk_;
+                    }
+                }
+            };
+            T v1 = 0, v2 = 0;
+            T c = tab[3 * l0], s = tab[3 * l0 + 1], tz = tab[3 * l0 + 2];
+            for (int m = l0; m >= 1; --m) {
+                const T c0 = c, s0 = s, tz0 = tz;
+                c = tab[3 * m - 3];
+                s = tab[3 * m - 2];
+                tz = tab[3 * m - 1];
+                T f, q;
+                prefactors(m, f, q);
+                T v0 = q * (tz0 * v1 + rxy * v2);
+                if (m == l - 1) v0 = -p.z * v1;
+                if (m == l) v0 = q;
+                const T pq = v0 * f;
+                if (live && m <= l) {
+                    mid[m] = pq * c0;
+                    mid[-m] = pq * s0;
+                }
+                v2 = v1;
+                v1 = v0;
+            }
+            T f, q;
+            prefactors(0, f, q);
+            const T v0 = q * (tz * v1 + rxy * v2);
+            if (live) mid[0] = v0 * f;
+        }
+    } else {
+        const T rxy = p.x2 + p.y2;
         // channel number i = L - l goes to wave i % waves in even rounds, backwards in odd ones
         for (unsigned i = 0; static_cast<int>(i) < L - H; ++i) {
             const unsigned pos = i % waves;
             if ((((i / waves) & 1u) ? waves - 1u - pos : pos) != wave) continue;
             const int l = L - static_cast<int>(i);
             const int tri = l * (l + 1) / 2;
-            const T* pk = cF + tri;
-            const T* qk = cQ + tri;
+            const ChannelPrefactors<T> pk(table_F<T>() + tri, l, lane);
+            const ChannelPrefactors<T> qk(table_Q<T>() + tri, l, lane);
+            if (lane >= valid) continue; // (all lanes are back at the next channel's loads)
             T* mid = row + l * l + l;
             T v2 = qk[l];
             T v1 = -p.z * v2;
@@ -124,15 +223,21 @@ __global__ __launch_bounds__(kValuesMaxThreads) void values_kernel(Tiling g, con
                 mid[l - 1] = pq * tab[3 * (l - 1)];
                 mid[-(l - 1)] = pq * tab[3 * (l - 1) + 1];
             }
+            // the table entries of the next m are fetched before the arithmetic of this one
+            T c = tab[3 * (l - 2)], s = tab[3 * (l - 2) + 1], tz = tab[3 * (l - 2) + 2];
             for (int m = l - 2; m >= 1; --m) {
-                const T v0 = qk[m] * (tab[3 * m + 2] * v1 + rxy * v2);
+                const T c0 = c, s0 = s, tz0 = tz;
+                c = tab[3 * m - 3];
+                s = tab[3 * m - 2];
+                tz = tab[3 * m - 1];
+                const T v0 = qk[m] * (tz0 * v1 + rxy * v2);
                 const T pq = v0 * pk[m];
-                mid[m] = pq * tab[3 * m];
-                mid[-m] = pq * tab[3 * m + 1];
+                mid[m] = pq * c0;
+                mid[-m] = pq * s0;
                 v2 = v1;
                 v1 = v0;
             }
-            const T v0 = qk[0] * (tab[2] * v1 + rxy * v2);
+            const T v0 = qk[0] * (tz * v1 + rxy * v2);
             mid[0] = v0 * pk[0];
         }
     }

@@ -118,25 +118,30 @@ def test_gradient_lanes_with_shared_channels(oracle, library, switches, dtype, n
 def test_values_kernel_with_tiles_of_any_size(oracle, library, switches, dtype):
     """values_kernel takes as many points per workgroup as fit in LDS, in steps of four: tiles
     of 60, 44, 28 points and others, a last tile that is not full, two workgroups per CU and
-    one with all of LDS (float32 l_max = 28), steps of one and halving, against the oracle."""
+    one with all of LDS, steps of one and halving; and tiles of 32 and 16 points with two and
+    four channels side by side in a wave (channels that do not fill the last bundle, l_max =
+    7-9, included). All against the oracle."""
     rng = np.random.default_rng(47)
-    for l_max in (11, 16, 19, 21, 24, 28):
+    for l_max in (7, 8, 9, 11, 16, 19, 22, 23, 24, 26, 28, 32):
         for normalized in (True, False):
             for n in (1, 59, 1201):
                 xyz = special_points(dtype, rng, n)
                 want = oracle.compute(xyz, l_max, normalized, "values")
                 xyz_dev = torch.from_numpy(xyz).cuda()
-                for step, least in ((None, None), (1, 8), (0, 32)):
+                for step, least, pack, alone in ((None, None, None, None), (1, 8, 1, 0), (0, 32, 1, 0), (4, 8, 1, 1),
+                                                 (4, 8, 2, 0), (4, 8, 4, 0), (4, 8, 2, 1)):
                     library.sphx_reset_switches()
                     if step is not None:
                         switches("SPHX_VALUES_TILE_STEP", step)
                         switches("SPHX_VALUES_MIN_TILE", least)
-                    announce("values, tiles", np.dtype(dtype).name, normalized, l_max, n, "step", step)
+                        switches("SPHX_VALUES_PACK", pack)
+                        switches("SPHX_VALUES_ALONE", alone)
+                    announce("values, tiles", np.dtype(dtype).name, normalized, l_max, n, "step", step, "pack", pack, "alone", alone)
                     status, got = run_launch_layer(library, xyz_dev, l_max, normalized, "values")
                     torch.cuda.synchronize()
                     assert status == 0, library.sphx_last_error()
                     got = tuple(None if g is None else g.cpu().numpy() for g in got)
-                    check(got, want, (l_max, normalized, n, step))
+                    check(got, want, (l_max, normalized, n, step, pack, alone))
     library.sphx_reset_switches()
 
 
