@@ -137,8 +137,8 @@ def _cfg5(seed, n, first):
     return _on_axis(xyz, radius, 200, first)
 
 
-_GENERATORS = {"cfg1": _cfg1, "cfg2": _cfg2, "cfg3": _cfg3, "cfg4": _cfg4, "cfg5": _cfg5, "val10": _cfg2, "grad10": _cfg3,
-               "hess5": _cfg3}
+_GENERATORS = {"cfg1": _cfg1, "cfg2": _cfg2, "cfg3": _cfg3, "cfg4": _cfg4, "cfg5": _cfg5, "val10": _cfg2, "val22": _cfg2,
+               "grad10": _cfg3, "hess5": _cfg3}
 
 WORKLOADS = {
     "cfg1": Workload(
@@ -170,6 +170,12 @@ WORKLOADS = {
     "val10": Workload(
         "val10", "spherical, l_max=10, f32, values, 1M points, uniform directions, r ~ U[0.5,5)",
         10, "f32", True, "values", 1_000_000, 1010,
+    ),
+    # and at an l_max where 64 rows no longer fit in LDS (tiles of 32 points, two channels side by
+    # side in a wave)
+    "val22": Workload(
+        "val22", "spherical, l_max=22, f32, values, 500k points, uniform directions, r ~ U[0.5,5)",
+        22, "f32", True, "values", 500_000, 1013,
     ),
     # likewise gradients at l_max just above the closed forms
     "grad10": Workload(
