@@ -241,30 +241,33 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     const unsigned smallest = static_cast<unsigned>(
         with_sums ? switch_or(SW_VJP_MIN_TILE, 8) : switch_or(SW_VALUES_MIN_TILE, elem == 4 ? 24 : 32));
     // Between tiles of 24-44 points, with lanes idle, and the recursion kernel lie two more forms
-    // of the values kernel: one workgroup per CU with all of its LDS and up to 64 points, and
-    // tiles of 32 or 16 points whose waves evaluate two or four channels side by side, all lanes
-    // at work. Which is fastest goes by the shape, not by a rule (row lengths, channels per wave
-    // and workgroups per CU all change with l_max). 1 GB of values, us, in the order tile that fits
-    // half of LDS / one workgroup with all of LDS / two channels, 32 points / four channels, 16
-    // points / recursion kernel, float32:
-    //   l_max 18 218 288 216 249 412      l_max 19 249 301 291 289 418      l_max 20 239 273 250 279 403
-    //   l_max 21 255 272 248 268 397      l_max 22 271 263 238 260 389      l_max 23 321 289   - 341 425
-    //   l_max 24 286 289   - 296 398      l_max 25 319 295   - 286 397      l_max 26 318 301   - 275 393
-    //   l_max 27   - 343 390 393 419      l_max 28   - 329 365 354 393      l_max 29   - 340 369 342 389
-    //   l_max 30   - 364 367 332 391      l_max 31   - 378 372 348 389      l_max 32   - 391 349 313 378
-    //   l_max 33   - 388 350 305 386      l_max 34   - 432   - 532 383
+    // of the values kernel: one workgroup per CU with all of its LDS, up to 64 points and up to
+    // sixteen waves, and tiles of 32 or 16 points whose waves evaluate two or four channels side
+    // by side, all lanes at work. Which is fastest goes by the shape, not by a rule (row lengths,
+    // channels per wave and workgroups per CU all change with l_max). 1 GB of values, us, in the
+    // order: tile that fits half of LDS / one workgroup with all of LDS / two channels, 32 points,
+    // in half of LDS / the same with all of LDS / four channels, 16 points / recursion kernel.
+    // float32:
+    //   l_max 18 216 263 216 224 249 412    l_max 19 248 285 291 290 289 418    l_max 20 238 270 250 250 279 403
+    //   l_max 21 254 262 248 252 268 397    l_max 22 271 260 238 239 260 389    l_max 23 319 288   - 427 341 425
+    //   l_max 24 285 287   - 373 296 398    l_max 25 319 295   - 366 286 397    l_max 26 317 300   - 350 275 393
+    //   l_max 27   - 333   - 359 393 419    l_max 28   - 317   - 334 354 393    l_max 29   - 329   - 326 342 389
+    //   l_max 30   - 357   - 317 332 391    l_max 31   - 360   - 324 348 389    l_max 32   - 368   - 300 313 378
+    //   l_max 33   - 365   - 297 305 386    l_max 34   - 404   - 418   - 383
     // float64:
-    //   l_max 13 221 244 283 310 313      l_max 14 227 214 239 309 310      l_max 15 258 234 257 326 347
-    //   l_max 16   - 241 361 335 322      l_max 20   - 273 300 363 313      l_max 21   - 292 303 365 296
-    //   l_max 22   - 295 282 328 303      l_max 23   - 337   - 582 301
+    //   l_max 13 220 243   - 282 310 313    l_max 14 224 212   - 239 309 310    l_max 15 258 225   - 257 326 347
+    //   l_max 16   - 228   - 360 335 322    l_max 20   - 252   - 299 363 313    l_max 21   - 273   - 303 365 296
+    //   l_max 22   - 273   - 281 328 303    l_max 23   - 326   -   - 582 301
+    // (Sixteen waves for a workgroup alone on its CU: float64 l_max = 16-21 239, 255, 248, 268, 272, 291 us
+    // with eight, 228, 236, 228, 259, 252, 273 with up to sixteen; float32 l_max = 27, 28 340, 327 with
+    // eight, 337, 326 with sixteen, 333, 317 with twelve.)
     unsigned pack_by_shape = 1;
     bool alone_by_shape = false;
     if (!with_sums && elem == 4) {
-        if (l_max == 21 || l_max == 22) pack_by_shape = 2;
-        if (l_max == 25 || l_max == 26 || (l_max >= 30 && l_max <= 33)) pack_by_shape = 4;
+        if (l_max == 21 || l_max == 22 || (l_max >= 29 && l_max <= 33)) pack_by_shape = 2;
+        if (l_max == 25 || l_max == 26) pack_by_shape = 4;
         alone_by_shape = l_max == 23;
     } else if (!with_sums) {
-        if (l_max == 22) pack_by_shape = 2;
         alone_by_shape = l_max == 14 || l_max == 15;
     }
     const bool alone = !with_sums && switch_or(SW_VALUES_ALONE, alone_by_shape ? 1 : 0) != 0;
@@ -317,8 +320,10 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     g.points_per_pass = with_sums ? 0u : pack; // values_kernel: channels a wave evaluates side by side
     out->workgroups = g.tiles_per_xcd * 8u;
     // one wave per l channel above the closed forms, eight at most
-    int waves = switch_or(SW_VALUES_WAVES, 8);
-    waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
+    // (alone on its CU: up to sixteen; twelve for one channel per wave in float32)
+    const int most = !with_sums && bytes > half ? (elem == 4 && pack == 1 ? 12 : 16) : 8;
+    int waves = switch_or(SW_VALUES_WAVES, most);
+    waves = waves < 1 ? 1 : (waves > most ? most : waves);
     // (the product's closed-form slices want at least four; values: one for the tables, one for
     // the closed forms)
     int want = (l_max - 6 + static_cast<int>(pack) - 1) / static_cast<int>(pack);
@@ -1129,7 +1134,8 @@ static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* d
         if constexpr (MODE == 0) {
             const Launch& l = plan.closed;
             auto kernel = l.g.points_per_pass == 4   ? values_kernel<T, NORM, 4>
-                          : l.g.points_per_pass == 2 ? values_kernel<T, NORM, 2>
+                          : l.g.points_per_pass == 2 ? (l.threads > 512 ? values_kernel<T, NORM, 2, 1024> : values_kernel<T, NORM, 2>)
+                          : l.threads > 512          ? values_kernel<T, NORM, 1, 1024>
                                                      : values_kernel<T, NORM, 1>;
             if (l.lds_bytes > 64u * 1024u) {
                 unsigned unused = 0;

@@ -85,8 +85,8 @@ template <typename T> struct ChannelPrefactors {
     __device__ __forceinline__ T operator[](int m) const { return from_lane(lanes, m); }
 };
 
-template <typename T, bool NORM, unsigned K = 1>
-__global__ __launch_bounds__(kValuesMaxThreads) void values_kernel(Tiling g, const T* __restrict__ xyz,
+template <typename T, bool NORM, unsigned K = 1, unsigned NT = kValuesMaxThreads>
+__global__ __launch_bounds__(NT) void values_kernel(Tiling g, const T* __restrict__ xyz,
                                                                   T* __restrict__ sph) {
     constexpr int H = 6;
     constexpr unsigned NYH = (H + 1) * (H + 1);

@@ -95,12 +95,13 @@ def test_launch_plans(library):
     status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 16, 0, False)
     assert status == 0 and (tile, threads) == (60, 512) and lds == 60 * (289 + 51) * 4
     status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 28, 0, False)
-    assert status == 0 and (tile, threads) == (44, 512) and 80 * 1024 < lds <= 160 * 1024
+    assert status == 0 and (tile, threads) == (44, 768) and 80 * 1024 < lds <= 160 * 1024
     # tiles of 32 and 16 points: two and four channels side by side in a wave
     assert _plan(library, 1_000_000, 22, 0, False)[1][:2] == [32, 512]
-    assert _plan(library, 1_000_000, 32, 0, False)[1][:2] == [16, 448]
+    assert _plan(library, 1_000_000, 26, 0, False)[1][:2] == [16, 320]
+    assert _plan(library, 1_000_000, 32, 0, False)[1][:2] == [32, 832]
     assert _plan(library, 1_000_000, 34, 0, False)[1][1] == 1024
-    assert _plan(library, 1_000_000, 22, 0, True)[1][:2] == [32, 512]
+    assert _plan(library, 1_000_000, 22, 0, True)[1][:2] == [32, 1024]
     assert _plan(library, 1_000_000, 23, 0, True)[1][1] == 1024
     assert _plan(library, 10, 65, 0, False)[0] == 2       # beyond the tables
     assert _plan(library, 10, 64, 2, True)[0] == 2        # one point's rows no longer fit in LDS
