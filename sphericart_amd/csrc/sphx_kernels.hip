@@ -418,10 +418,17 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     // longest chain of work in the workgroup)
     // (closed forms only, l_max <= 6: eight; six for normalised float32 at l_max = 6, 127 us
     // against 130 us with eight and 136-138 us with four or five)
+    // (few points, three channels or more, or float64 tiles of up to 16 points: sixteen waves, two
+    // to a channel where that leaves four for the closed forms; 10 000 points, us, eight waves
+    // against sixteen: float32 l_max = 10 9.5 against 8.6, l_max = 12 11.8 against 10.9; float64
+    // l_max = 8 with 2 000 points 8.0 against 6.2; one or two channels at 40 points per tile gain
+    // nothing, float64 l_max = 8 9.2 against 9.1, l_max = 7 7.9 against 8.3)
+    const bool many = tile == few && l_max > 6 && (l_max >= 9 || (elem == 8 && tile <= 16));
     const int by_shape = l_max <= 6 ? (l_max == 6 && elem == 4 && normalized && tile != few ? 6 : 8)
-                                    : (l_max <= 8 && tile != few ? 4 : 8);
+                                    : (l_max <= 8 && tile != few ? 4 : (many ? 16 : 8));
     int waves = switch_or(SW_GRADIENT_LANES_WAVES, by_shape);
-    waves = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
+    const int most = l_max >= 6 ? 16 : 8; // (the kernels of l_max = 4, 5 exist for 512 threads)
+    waves = waves < 1 ? 1 : (waves > most ? most : waves);
     out->threads = 64u * static_cast<unsigned>(waves);
     out->lds_bytes = bytes;
     // Few points, one or two channels: two waves per channel, each with half of its m (the longest
@@ -432,7 +439,7 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     // left for the eight slices and nothing is gained (float64 l_max = 9 10.2 against 10.5), with
     // four channels none (l_max = 10: 9.5 against 9.1 in float32, 9.9 against 10.2 in float64).
     const unsigned channels = l_max > 6 ? static_cast<unsigned>(l_max - 6) : 0u;
-    const bool halves = tile == few && channels >= 1 && channels <= 2 && waves == 8;
+    const bool halves = tile == few && channels >= 1 && (channels <= 2 ? waves >= 8 : 2u * channels + 4u <= static_cast<unsigned>(waves));
     const int parts = switch_or(SW_GRADIENT_LANES_PARTS, halves ? 2 : 1);
     g.sequence_waves = parts == 2 && 2u * channels <= static_cast<unsigned>(waves) ? 2u : 1u;
     return true;
@@ -1148,7 +1155,8 @@ static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* d
         if constexpr (MODE == 1) {
             const Launch& l = plan.closed;
             if (l.g.l_max < 4) return hipErrorInvalidValue; // never planned
-            auto kernel = l.g.l_max >= 6   ? gradients_lanes_kernel<T, NORM, 6>
+            auto kernel = l.g.l_max >= 6   ? (l.threads > 512 ? gradients_lanes_kernel<T, NORM, 6, 1024>
+                                                              : gradients_lanes_kernel<T, NORM, 6>)
                           : l.g.l_max == 5 ? gradients_lanes_kernel<T, NORM, 5>
                                            : gradients_lanes_kernel<T, NORM, 4>;
             if (l.lds_bytes > 64u * 1024u) {

@@ -306,8 +306,8 @@ __device__ __forceinline__ void closed_form_slices(const Point<T>& p, const Rows
     }
 }
 
-template <typename T, bool NORM, int H = 6>
-__global__ __launch_bounds__(kValuesMaxThreads) void gradients_lanes_kernel(Tiling g, const T* __restrict__ xyz,
+template <typename T, bool NORM, int H = 6, unsigned NT = kValuesMaxThreads>
+__global__ __launch_bounds__(NT) void gradients_lanes_kernel(Tiling g, const T* __restrict__ xyz,
                                                                            T* __restrict__ sph,
                                                                            T* __restrict__ dsph) {
     using V = typename Pack<T>::type;

@@ -94,24 +94,25 @@ def test_second_derivative_lanes_with_shared_channels(oracle, library, switches,
 @pytest.mark.parametrize("normalized", [True, False])
 def test_gradient_lanes_with_shared_channels(oracle, library, switches, dtype, normalized):
     """The one-point-per-lane kernel for gradients above the closed forms, with one and two waves
-    per l channel (each wave half of the channel's m), few points (where the planner picks two
-    waves for one or two channels) and many, against the oracle."""
+    per l channel (each wave half of the channel's m), in workgroups of eight, twelve and sixteen
+    waves, few points (where the planner picks two waves per channel while waves are left for the
+    closed forms) and many, against the oracle."""
     rng = np.random.default_rng(21)
-    for l_max in (7, 8, 9, 10):
+    for l_max in (7, 8, 9, 10, 12):
         for n in (1, 50, 3000, 10000, 40000):
             xyz = special_points(dtype, rng, n)
             want = oracle.compute(xyz, l_max, normalized, "gradients")
             xyz_dev = torch.from_numpy(xyz).cuda()
-            for parts in (1, 2):
+            for parts, waves in ((1, 8), (2, 8), (1, 16), (2, 16), (2, 12)):
                 switches("SPHX_GRADIENT_LANES", 2)
-                switches("SPHX_GRADIENT_LANES_WAVES", 8)
+                switches("SPHX_GRADIENT_LANES_WAVES", waves)
                 switches("SPHX_GRADIENT_LANES_PARTS", parts)
-                announce("gradients, lanes", np.dtype(dtype).name, normalized, l_max, n, "parts", parts)
+                announce("gradients, lanes", np.dtype(dtype).name, normalized, l_max, n, "parts", parts, "waves", waves)
                 status, got = run_launch_layer(library, xyz_dev, l_max, normalized, "gradients")
                 torch.cuda.synchronize()
                 assert status == 0, library.sphx_last_error()
                 got = tuple(None if g is None else g.cpu().numpy() for g in got)
-                check(got, want, (l_max, normalized, n, parts))
+                check(got, want, (l_max, normalized, n, parts, waves))
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
