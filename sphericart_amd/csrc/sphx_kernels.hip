@@ -270,7 +270,28 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     } else if (!with_sums) {
         alone_by_shape = l_max == 14 || l_max == 15;
     }
-    const bool alone = !with_sums && switch_or(SW_VALUES_ALONE, alone_by_shape ? 1 : 0) != 0;
+    // The product: tiles halve, and where 32 points no longer fit half of LDS the next is 16 with
+    // groups of lanes (vjp_groups_kernel). Up to 64 points in one workgroup with all of LDS are
+    // faster on some shapes, with a number of waves that goes by the shape as well (the channels
+    // and the eight closed-form slices share the waves). 200k points (400k to l_max = 16), us,
+    // tiles in half of LDS against one workgroup per CU with 8 / 10 / 12 / 16 waves, float64:
+    //   l_max 13 257 261 261 260 261    l_max 14 498 287 287 287 287    l_max 15 520 408 474 474 473
+    //   l_max 16 540 460 526 526 526    l_max 17 290 274 259 285 285    l_max 18 299 301 294 313 313
+    //   l_max 19 316 327 316 283 329    l_max 20 331 356 353 317 370    l_max 21 590 621 621 621 622
+    //   l_max 22 615 559 560 559 560    l_max 23 626 591 591 590 590    l_max 24 640 611 611 611 611
+    //   l_max 25 661 649 648 649 650    l_max 26 678 690 691 690 690
+    // float32: l_max 19 146 152 148 135 158, l_max 21 181 178 182 172 162, others at best equal.
+    int waves_by_shape = 0;
+    if (with_sums && elem == 8) {
+        if ((l_max >= 14 && l_max <= 16) || (l_max >= 22 && l_max <= 25)) waves_by_shape = 8;
+        if (l_max == 17) waves_by_shape = 10;
+        if (l_max == 19 || l_max == 20) waves_by_shape = 12;
+    } else if (with_sums) {
+        if (l_max == 19) waves_by_shape = 12;
+        if (l_max == 21) waves_by_shape = 16;
+    }
+    if (waves_by_shape != 0) alone_by_shape = true;
+    const bool alone = switch_or(SW_VALUES_ALONE, alone_by_shape ? 1 : 0) != 0;
     const unsigned smallest_alone = !with_sums && elem == 4 && smallest < 40 && !alone ? 40 : smallest;
     // Values: the tile goes down in steps of 4 points, so that as many lanes work as rows fit
     // (l_max = 16: 60 points where halving leaves 32, 202 against 278 us in float32, 240 against
@@ -281,7 +302,8 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // (l_max = 16 float32, 500k points, 32 points against 64: 142 against 164 us; l_max = 12
     // float64: 115 against 146).
     const unsigned half = 80u * 1024u;
-    unsigned tile = 0, rows = 0, bytes = 0;
+    unsigned tile = 0, rows = 0, bytes = 0, sums_elems = 0;
+    const unsigned groups_below = static_cast<unsigned>(switch_or(SW_VJP_GROUPS_BELOW, 16)); // (vjp_groups_kernel: eight waves)
     unsigned pack = with_sums ? 1u : static_cast<unsigned>(switch_or(SW_VALUES_PACK, static_cast<int>(pack_by_shape)));
     if (pack != 2 && pack != 4) pack = 1;
     auto search = [&]() {
@@ -292,9 +314,14 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
                 rows = (t * row_stride + vec - 1u) / vec * vec;
                 // the product: the waves' sums; with fewer than 64 points also copies of the
                 // prefactor tables (vjp_groups_kernel)
-                const unsigned extra = !with_sums ? 0u : (t == 64 ? 8u * 3u * 64u : 8u * 3u * 64u + 2u * tri_all);
+                // (a workgroup alone on its CU with more than 16 points: up to sixteen waves)
+                const unsigned sums = (with_sums && limit > half && t > groups_below ? 16u : 8u) * 3u * 64u;
+                const unsigned extra = !with_sums ? 0u : (t == 64 ? sums : sums + 2u * tri_all);
                 bytes = (rows + t * table_stride + extra) * esize;
-                if (bytes <= limit) tile = t;
+                if (bytes <= limit) {
+                    tile = t;
+                    sums_elems = sums;
+                }
             }
         }
     };
@@ -315,14 +342,15 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     g.off_pts = rows;
     g.off_iter = table_stride;
     g.off_jobs = rows + tile * table_stride; // the product: the waves' sums,
-    g.off_F = g.off_jobs + 8u * 3u * 64u;    // and (fewer than 64 points) the prefactor tables
+    g.off_F = g.off_jobs + sums_elems;       // and (fewer than 64 points) the prefactor tables
     g.off_Q = g.off_F + tri_all;
     g.points_per_pass = with_sums ? 0u : pack; // values_kernel: channels a wave evaluates side by side
     out->workgroups = g.tiles_per_xcd * 8u;
     // one wave per l channel above the closed forms, eight at most
     // (alone on its CU: up to sixteen; twelve for one channel per wave in float32)
-    const int most = !with_sums && bytes > half ? (elem == 4 && pack == 1 ? 12 : 16) : 8;
-    int waves = switch_or(SW_VALUES_WAVES, most);
+    const int most = with_sums ? (sums_elems > 8u * 3u * 64u ? 16 : 8)
+                               : (bytes > half ? (elem == 4 && pack == 1 ? 12 : 16) : 8);
+    int waves = switch_or(SW_VALUES_WAVES, waves_by_shape != 0 && alone ? waves_by_shape : most);
     waves = waves < 1 ? 1 : (waves > most ? most : waves);
     // (the product's closed-form slices want at least four; values: one for the tables, one for
     // the closed forms)
@@ -1541,7 +1569,11 @@ static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int
                 return hipGetLastError();
             };
             if (!planned->lane_groups) {
-                e = normalized ? launch(vjp_lanes_kernel<T, true>) : launch(vjp_lanes_kernel<T, false>);
+                if (lanes.threads > 512) {
+                    e = normalized ? launch(vjp_lanes_kernel<T, true, 1024>) : launch(vjp_lanes_kernel<T, false, 1024>);
+                } else {
+                    e = normalized ? launch(vjp_lanes_kernel<T, true>) : launch(vjp_lanes_kernel<T, false>);
+                }
             } else {
                 e = normalized ? launch(vjp_groups_kernel<T, true>) : launch(vjp_groups_kernel<T, false>);
             }

@@ -143,8 +143,8 @@ __global__ __launch_bounds__(64, 3) void closed_form_vjp_kernel(Tiling g, const 
 // g.rows_elems: row stride of the staged weights, g.off_pts: tables,
 // g.off_iter: table stride, g.off_jobs: the waves' sums.
 // ---------------------------------------------------------------------------
-template <typename T, bool NORM>
-__global__ __launch_bounds__(kValuesMaxThreads) void vjp_lanes_kernel(Tiling g, const T* __restrict__ xyz,
+template <typename T, bool NORM, unsigned NT = kValuesMaxThreads>
+__global__ __launch_bounds__(NT) void vjp_lanes_kernel(Tiling g, const T* __restrict__ xyz,
                                                                      const T* __restrict__ sph_grad,
                                                                      T* __restrict__ xyz_grad,
                                                                      int accumulate) {

@@ -128,7 +128,8 @@ def test_fused_vjp_beyond_the_closed_forms(library, oracle, normalized, dtype, t
     rng = np.random.default_rng(12)
     fn = library.sphx_vjp_f32 if dtype == np.float32 else library.sphx_vjp_f64
     stream = torch.cuda.current_stream().cuda_stream
-    for l_max in (7, 8, 11, 16, 24, 32):
+    # (14-25: shapes where the lanes kernel has a CU to itself, with eight to sixteen waves)
+    for l_max in (7, 8, 11, 14, 16, 17, 19, 21, 24, 32):
         for n in (1, 17, 1000, 5003):
             if l_max == 32 and n > 1000:
                 continue
