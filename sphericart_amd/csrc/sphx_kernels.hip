@@ -127,7 +127,7 @@ enum Switch : int {
     SW_PREFIX_INSIDE,
     SW_SEQUENCE_WAVES, SW_SLICE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
     SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_ALONE, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
-    SW_VALUES_PACK, SW_VALUES_TILE_STEP, SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_COUNT
+    SW_VALUES_PACK, SW_VALUES_TILE_STEP, SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_VJP_TILE_STEP, SW_COUNT
 };
 static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_GRADIENT_LANES",
@@ -137,7 +137,7 @@ static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_PREFIX_INSIDE", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_ALONE", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
-    "SPHX_VALUES_PACK", "SPHX_VALUES_TILE_STEP", "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE",
+    "SPHX_VALUES_PACK", "SPHX_VALUES_TILE_STEP", "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE", "SPHX_VJP_TILE_STEP",
 };
 struct Switches {
     bool set[SW_COUNT] = {};
@@ -270,25 +270,29 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     } else if (!with_sums) {
         alone_by_shape = l_max == 14 || l_max == 15;
     }
-    // The product: tiles halve, and where 32 points no longer fit half of LDS the next is 16 with
-    // groups of lanes (vjp_groups_kernel). Up to 64 points in one workgroup with all of LDS are
-    // faster on some shapes, with a number of waves that goes by the shape as well (the channels
-    // and the eight closed-form slices share the waves). 200k points (400k to l_max = 16), us,
-    // tiles in half of LDS against one workgroup per CU with 8 / 10 / 12 / 16 waves, float64:
-    //   l_max 13 257 261 261 260 261    l_max 14 498 287 287 287 287    l_max 15 520 408 474 474 473
-    //   l_max 16 540 460 526 526 526    l_max 17 290 274 259 285 285    l_max 18 299 301 294 313 313
-    //   l_max 19 316 327 316 283 329    l_max 20 331 356 353 317 370    l_max 21 590 621 621 621 622
-    //   l_max 22 615 559 560 559 560    l_max 23 626 591 591 590 590    l_max 24 640 611 611 611 611
-    //   l_max 25 661 649 648 649 650    l_max 26 678 690 691 690 690
-    // float32: l_max 19 146 152 148 135 158, l_max 21 181 178 182 172 162, others at best equal.
+    // The product: tiles go down in steps of four points to 32 and halve from there, to 16 and 8
+    // points with groups of lanes (vjp_groups_kernel). One workgroup with all of LDS is faster on
+    // some shapes, with a number of waves that goes by the shape as well (the channels and the
+    // eight closed-form slices share the waves). 200k points (400k to l_max = 16), us, tiles in
+    // half of LDS against one workgroup per CU with 8 / 12 / 16 waves, float64:
+    //   l_max 13 256 260 260 260    l_max 14 497 286 286 287    l_max 15 519 341 322 342    l_max 16 538 393 360 393
+    //   l_max 17 289 236 216 229    l_max 18 299 274 240 239    l_max 19 315 310 273 272    l_max 20 330 356 317 317
+    //   l_max 21 589 620 619 619    l_max 22 615 558 558 558    l_max 23 626 589 590 589    l_max 24 641 610 610 611
+    //   l_max 25 660 649 649 649    l_max 26 676 690 690 690
+    // float32:
+    //   l_max 19 145 153 135 135    l_max 20 155 168 154 181    l_max 21 182 178 172 162    l_max 22 212 200 186 207
+    //   l_max 23 217 212 201 217    l_max 24 222 245 226 250    l_max 25 336 274 254 288    l_max 26 340 294 277 313
+    //   l_max 27 348 335 312 346    l_max 28 356 383 342 379    l_max 29 385 404 369 411    l_max 30 397 468 422 464
+    //   l_max 31 477 436 442 422    l_max 32 500 646 645 646
+    // (Tiles that halved all the way: float64 l_max = 10, 15, 16, 17 153, 405, 459, 259 us against 139, 340,
+    // 393, 230; float32 l_max = 15, 17, 18 166, 118, 135 against 153, 97, 114.)
     int waves_by_shape = 0;
     if (with_sums && elem == 8) {
-        if ((l_max >= 14 && l_max <= 16) || (l_max >= 22 && l_max <= 25)) waves_by_shape = 8;
-        if (l_max == 17) waves_by_shape = 10;
-        if (l_max == 19 || l_max == 20) waves_by_shape = 12;
+        if (l_max >= 14 && l_max <= 20) waves_by_shape = 12;
+        if (l_max >= 22 && l_max <= 25) waves_by_shape = 8;
     } else if (with_sums) {
-        if (l_max == 19) waves_by_shape = 12;
-        if (l_max == 21) waves_by_shape = 16;
+        if (l_max == 19 || l_max == 22 || l_max == 23 || (l_max >= 25 && l_max <= 29)) waves_by_shape = 12;
+        if (l_max == 21 || l_max == 31) waves_by_shape = 16;
     }
     if (waves_by_shape != 0) alone_by_shape = true;
     const bool alone = switch_or(SW_VALUES_ALONE, alone_by_shape ? 1 : 0) != 0;
@@ -296,7 +300,9 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // Values: the tile goes down in steps of 4 points, so that as many lanes work as rows fit
     // (l_max = 16: 60 points where halving leaves 32, 202 against 278 us in float32, 240 against
     // 352 in float64; steps of 1 or 2 gain nothing more and some odd sizes lose). The product halves.
-    const unsigned step = with_sums ? 0u : static_cast<unsigned>(switch_or(SW_VALUES_TILE_STEP, 4));
+    // (the product: the same above 32 points, halves from there down, for the groups of lanes of
+    // vjp_groups_kernel)
+    const unsigned step = static_cast<unsigned>(with_sums ? switch_or(SW_VJP_TILE_STEP, 4) : switch_or(SW_VALUES_TILE_STEP, 4));
     // Two workgroups per CU (80 KB each) overlap one's tables and flush with the other's
     // arithmetic: preferred, also with fewer lanes at work, over one workgroup with all of LDS
     // (l_max = 16 float32, 500k points, 32 points against 64: 142 against 164 us; l_max = 12
@@ -309,7 +315,8 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     auto search = [&]() {
         for (unsigned limit : {alone ? 0u : (allowed < half ? allowed : half), allowed}) {
             const unsigned least = pack > 1 ? 8u : (limit > half ? smallest_alone : smallest);
-            for (unsigned t = 64 / pack; t >= least && t >= 8 && tile == 0; t = step == 0 ? t / 2 : t - step) {
+            for (unsigned t = 64 / pack; t >= least && t >= 8 && tile == 0;
+                 t = step == 0 || (with_sums && t <= 32) ? t / 2 : t - step) {
                 if (pack > 1 && t != 64 / pack) break;
                 rows = (t * row_stride + vec - 1u) / vec * vec;
                 // the product: the waves' sums; with fewer than 64 points also copies of the
