@@ -273,26 +273,31 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // The product: tiles go down in steps of four points to 32 and halve from there, to 16 and 8
     // points with groups of lanes (vjp_groups_kernel). One workgroup with all of LDS is faster on
     // some shapes, with a number of waves that goes by the shape as well (the channels and the
-    // eight closed-form slices share the waves). 200k points (400k to l_max = 16), us, tiles in
-    // half of LDS against one workgroup per CU with 8 / 12 / 16 waves, float64:
-    //   l_max 13 256 260 260 260    l_max 14 497 286 286 287    l_max 15 519 341 322 342    l_max 16 538 393 360 393
-    //   l_max 17 289 236 216 229    l_max 18 299 274 240 239    l_max 19 315 310 273 272    l_max 20 330 356 317 317
-    //   l_max 21 589 620 619 619    l_max 22 615 558 558 558    l_max 23 626 589 590 589    l_max 24 641 610 610 611
-    //   l_max 25 660 649 649 649    l_max 26 676 690 690 690
-    // float32:
-    //   l_max 19 145 153 135 135    l_max 20 155 168 154 181    l_max 21 182 178 172 162    l_max 22 212 200 186 207
-    //   l_max 23 217 212 201 217    l_max 24 222 245 226 250    l_max 25 336 274 254 288    l_max 26 340 294 277 313
-    //   l_max 27 348 335 312 346    l_max 28 356 383 342 379    l_max 29 385 404 369 411    l_max 30 397 468 422 464
-    //   l_max 31 477 436 442 422    l_max 32 500 646 645 646
+    // eight closed-form slices share the waves; more than eight waves need twice the room for
+    // their sums, which can cost points). 200k points (400k to l_max = 16), us, tiles in half of LDS /
+    // one workgroup per CU with 8 / with up to 12 waves, float64:
+    //   l_max 13 257 261 261    l_max 14 498 287 286    l_max 15 519 328 324    l_max 16 538 383 360
+    //   l_max 17 289 228 214    l_max 18 299 261 240    l_max 19 315 290 272    l_max 20 330 336 316
+    //   l_max 21 588 375 620    l_max 22 613 556 557    l_max 23 627 588 589    l_max 24 640 610 610
+    //   l_max 25 660 649 650    l_max 26 675 689 690    l_max 29 804 804 804
+    // float32 (l_max = 21, 31 with 16 waves 162, 423):
+    //   l_max 19 144 153 135    l_max 20 155 168 154    l_max 21 181 178 172    l_max 22 211 168 185
+    //   l_max 23 216 212 201    l_max 24 222 244 224    l_max 25 335 274 255    l_max 26 340 294 276
+    //   l_max 27 348 289 313    l_max 28 356 318 342    l_max 29 385 404 370    l_max 30 397 381 422
+    //   l_max 31 477 436 442    l_max 32 500 470 645    l_max 33 510 675 676    l_max 34 518 694 695
+    //   l_max 35 789 725 726    l_max 36 807 748 748    l_max 37 820 773 773    l_max 40 874 852 851
     // (Tiles that halved all the way: float64 l_max = 10, 15, 16, 17 153, 405, 459, 259 us against 139, 340,
-    // 393, 230; float32 l_max = 15, 17, 18 166, 118, 135 against 153, 97, 114.)
+    // 393, 230 with the same number of waves; float32 l_max = 15, 17, 18 166, 118, 135 against 153, 97, 114.)
     int waves_by_shape = 0;
     if (with_sums && elem == 8) {
         if (l_max >= 14 && l_max <= 20) waves_by_shape = 12;
-        if (l_max >= 22 && l_max <= 25) waves_by_shape = 8;
+        if (l_max >= 21 && l_max <= 25) waves_by_shape = 8;
     } else if (with_sums) {
-        if (l_max == 19 || l_max == 22 || l_max == 23 || (l_max >= 25 && l_max <= 29)) waves_by_shape = 12;
+        if (l_max == 19 || l_max == 23 || l_max == 25 || l_max == 26 || l_max == 29) waves_by_shape = 12;
         if (l_max == 21 || l_max == 31) waves_by_shape = 16;
+        if (l_max == 22 || l_max == 27 || l_max == 28 || l_max == 30 || l_max == 32 || (l_max >= 35 && l_max <= 40)) {
+            waves_by_shape = 8;
+        }
     }
     if (waves_by_shape != 0) alone_by_shape = true;
     const bool alone = switch_or(SW_VALUES_ALONE, alone_by_shape ? 1 : 0) != 0;
@@ -309,6 +314,7 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // float64: 115 against 146).
     const unsigned half = 80u * 1024u;
     unsigned tile = 0, rows = 0, bytes = 0, sums_elems = 0;
+    const int sum_waves = switch_or(SW_VALUES_WAVES, waves_by_shape != 0 ? waves_by_shape : 16);
     const unsigned groups_below = static_cast<unsigned>(switch_or(SW_VJP_GROUPS_BELOW, 16)); // (vjp_groups_kernel: eight waves)
     unsigned pack = with_sums ? 1u : static_cast<unsigned>(switch_or(SW_VALUES_PACK, static_cast<int>(pack_by_shape)));
     if (pack != 2 && pack != 4) pack = 1;
@@ -321,8 +327,9 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
                 rows = (t * row_stride + vec - 1u) / vec * vec;
                 // the product: the waves' sums; with fewer than 64 points also copies of the
                 // prefactor tables (vjp_groups_kernel)
-                // (a workgroup alone on its CU with more than 16 points: up to sixteen waves)
-                const unsigned sums = (with_sums && limit > half && t > groups_below ? 16u : 8u) * 3u * 64u;
+                // (a workgroup alone on its CU with more than 16 points: room for the sums of
+                // up to sixteen waves, unless eight are asked for)
+                const unsigned sums = (with_sums && limit > half && t > groups_below && sum_waves > 8 ? 16u : 8u) * 3u * 64u;
                 const unsigned extra = !with_sums ? 0u : (t == 64 ? sums : sums + 2u * tri_all);
                 bytes = (rows + t * table_stride + extra) * esize;
                 if (bytes <= limit) {
