@@ -127,7 +127,7 @@ enum Switch : int {
     SW_PREFIX_INSIDE,
     SW_SEQUENCE_WAVES, SW_SLICE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
     SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_ALONE, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
-    SW_VALUES_PACK, SW_VALUES_TILE_STEP, SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_VJP_TILE_STEP, SW_COUNT
+    SW_VALUES_PACK, SW_VALUES_TILE_STEP, SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_VJP_STEP_FLOOR, SW_VJP_TILE_STEP, SW_COUNT
 };
 static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_GRADIENT_LANES",
@@ -137,7 +137,7 @@ static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_PREFIX_INSIDE", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_ALONE", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
-    "SPHX_VALUES_PACK", "SPHX_VALUES_TILE_STEP", "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE", "SPHX_VJP_TILE_STEP",
+    "SPHX_VALUES_PACK", "SPHX_VALUES_TILE_STEP", "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE", "SPHX_VJP_STEP_FLOOR", "SPHX_VJP_TILE_STEP",
 };
 struct Switches {
     bool set[SW_COUNT] = {};
@@ -288,16 +288,27 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     //   l_max 35 789 725 726    l_max 36 807 748 748    l_max 37 820 773 773    l_max 40 874 852 851
     // (Tiles that halved all the way: float64 l_max = 10, 15, 16, 17 153, 405, 459, 259 us against 139, 340,
     // 393, 230 with the same number of waves; float32 l_max = 15, 17, 18 166, 118, 135 against 153, 97, 114.)
+    // (On some shapes the steps of four go on below 32 points, to tiles of 28, 24 and 20 for the
+    // lanes kernel, before the groups of lanes take over. With that, one workgroup per CU with 8 /
+    // 12 waves against the best of the above: float64 l_max = 21 375 364 against 375, l_max = 22 444
+    // 405 against 559, l_max = 23 468 464 against 589, l_max = 24 565 564 against 611, l_max = 25 598
+    // 602 against 649, l_max = 26 719 661 against 677; float32 l_max = 35 692 642 against 725,
+    // l_max = 36 678 667 against 749, l_max = 37 718 792 against 773, l_max = 43 866 868 against 909.)
     int waves_by_shape = 0;
+    unsigned floor_by_shape = 32;
     if (with_sums && elem == 8) {
-        if (l_max >= 14 && l_max <= 20) waves_by_shape = 12;
-        if (l_max >= 21 && l_max <= 25) waves_by_shape = 8;
+        if (l_max >= 14 && l_max <= 26) waves_by_shape = l_max == 25 ? 8 : 12;
+        if (l_max >= 21 && l_max <= 26) floor_by_shape = 16;
     } else if (with_sums) {
-        if (l_max == 19 || l_max == 23 || l_max == 25 || l_max == 26 || l_max == 29) waves_by_shape = 12;
+        if (l_max == 19 || l_max == 23 || l_max == 25 || l_max == 26 || l_max == 29 || l_max == 35 || l_max == 36) {
+            waves_by_shape = 12;
+        }
         if (l_max == 21 || l_max == 31) waves_by_shape = 16;
-        if (l_max == 22 || l_max == 27 || l_max == 28 || l_max == 30 || l_max == 32 || (l_max >= 35 && l_max <= 40)) {
+        if (l_max == 22 || l_max == 27 || l_max == 28 || l_max == 30 || l_max == 32 || (l_max >= 37 && l_max <= 40) ||
+            l_max == 43) {
             waves_by_shape = 8;
         }
+        if ((l_max >= 35 && l_max <= 37) || l_max == 43) floor_by_shape = 16;
     }
     if (waves_by_shape != 0) alone_by_shape = true;
     const bool alone = switch_or(SW_VALUES_ALONE, alone_by_shape ? 1 : 0) != 0;
@@ -314,6 +325,7 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // float64: 115 against 146).
     const unsigned half = 80u * 1024u;
     unsigned tile = 0, rows = 0, bytes = 0, sums_elems = 0;
+    const unsigned step_floor = static_cast<unsigned>(switch_or(SW_VJP_STEP_FLOOR, static_cast<int>(floor_by_shape)));
     const int sum_waves = switch_or(SW_VALUES_WAVES, waves_by_shape != 0 ? waves_by_shape : 16);
     const unsigned groups_below = static_cast<unsigned>(switch_or(SW_VJP_GROUPS_BELOW, 16)); // (vjp_groups_kernel: eight waves)
     unsigned pack = with_sums ? 1u : static_cast<unsigned>(switch_or(SW_VALUES_PACK, static_cast<int>(pack_by_shape)));
@@ -322,7 +334,7 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
         for (unsigned limit : {alone ? 0u : (allowed < half ? allowed : half), allowed}) {
             const unsigned least = pack > 1 ? 8u : (limit > half ? smallest_alone : smallest);
             for (unsigned t = 64 / pack; t >= least && t >= 8 && tile == 0;
-                 t = step == 0 || (with_sums && t <= 32) ? t / 2 : t - step) {
+                 t = step == 0 || (with_sums && t <= step_floor) ? t / 2 : t - step) {
                 if (pack > 1 && t != 64 / pack) break;
                 rows = (t * row_stride + vec - 1u) / vec * vec;
                 // the product: the waves' sums; with fewer than 64 points also copies of the
