@@ -1,20 +1,24 @@
 """Build the HIP library in-tree: ``python -m sphericart_amd.build``.
 
-One ``hipcc`` call compiles the kernels for gfx950 together with the host-side
-C and C++ API into ``sphericart_amd/libsphericart_amd.so``. hipcc cross-compiles,
-so this works on a machine without a GPU.
+``hipcc`` compiles the kernels for gfx950 and the host-side C and C++ API, one
+translation unit per process, and links them into
+``sphericart_amd/libsphericart_amd.so``. hipcc cross-compiles, so this works on a
+machine without a GPU.
 """
 
 import os
 import shutil
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBRARY = os.path.join(HERE, "libsphericart_amd.so")
 
-SOURCES = ["sphx_kernels.hip", "sphx_backward.hip", "sphx_tables.cpp", "device_api.cpp", "capi.cpp"]
+OBJECTS = os.path.join(HERE, "build")
+
+SOURCES = ["sphx_kernels.hip", "sphx_pairs.hip", "sphx_backward.hip", "sphx_tables.cpp", "device_api.cpp", "capi.cpp"]
 
 # -ffp-contract=off: one rounding per source-level operation, on device and
 #   host alike; results then match the reference CPU evaluator built the same
@@ -27,7 +31,6 @@ FLAGS = [
     "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-fPIC",
-    "-shared",
     "-fvisibility=hidden",
 ]
 
@@ -43,17 +46,29 @@ def hipcc():
     return found
 
 
-def build(verbose=False, extra_flags=()):
+def build(verbose=False, extra_flags=(), jobs=None):
     """Compile ``libsphericart_amd.so``; raises ``RuntimeError`` with the compiler output on failure."""
-    command = [hipcc(), *FLAGS, *extra_flags, *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIBRARY]
+    os.makedirs(OBJECTS, exist_ok=True)
+
+    def compile_one(source):
+        target = os.path.join(OBJECTS, os.path.splitext(source)[0] + ".o")
+        command = [hipcc(), *FLAGS, *extra_flags, "-c", os.path.join(CSRC, source), "-o", target]
+        if verbose:
+            print(" ".join(command), flush=True)
+        done = subprocess.run(command, capture_output=True, text=True)
+        if done.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {source} ({done.returncode}):\n{done.stdout}\n{done.stderr}")
+        return target
+
+    workers = jobs or min(len(SOURCES), os.cpu_count() or 1, 16)
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        objects = list(pool.map(compile_one, SOURCES))
+    command = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-o", LIBRARY]
     if verbose:
         print(" ".join(command), flush=True)
     done = subprocess.run(command, capture_output=True, text=True)
     if done.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({done.returncode}):\n{done.stdout}\n{done.stderr}")
-    if verbose and done.stderr:
-        # hipcc's host pass does not know the packed-fp32 feature and says so
-        print(done.stderr, file=sys.stderr)
+        raise RuntimeError(f"hipcc failed to link ({done.returncode}):\n{done.stdout}\n{done.stderr}")
     build_example(verbose)
     return LIBRARY
 

@@ -270,7 +270,9 @@ __device__ __forceinline__ void azimuth_job(const Point<T>& p, int L, T* c, T* s
 // then independent jobs (entry_job) for all lanes of the workgroup. Same
 // operations in the same order as the reference's fused loop, hence the same
 // numbers.
-template <typename T>
+// STRIDE: distance in `out` between the iterates of consecutive m (1: an array of its own per
+// sequence; more: the sequences of one l interleaved, `out` then points at this sequence's m = 0).
+template <typename T, int STRIDE = 1>
 __device__ __forceinline__ void sequence_job(int l, int which, T z, T rxy,
                                              const T* __restrict__ Q,
                                              const T* __restrict__ tmz, T* __restrict__ out) {
@@ -288,13 +290,13 @@ __device__ __forceinline__ void sequence_job(int l, int which, T z, T rxy,
         v2 = 0.0;
         v1 = 0.0;
     }
-    out[l] = v2;
-    out[l - 1] = v1;
+    out[l * STRIDE] = v2;
+    out[(l - 1) * STRIDE] = v1;
     int m = l - 2;
     if (which == 2) {
         // first step of the Q_{l-2} sequence: its start value itself (:228-231, :404-406)
         const T v0 = qk[-l - 1];
-        out[m] = v0;
+        out[m * STRIDE] = v0;
         v2 = v1;
         v1 = v0;
         --m;
@@ -307,7 +309,7 @@ __device__ __forceinline__ void sequence_job(int l, int which, T z, T rxy,
     constexpr int DEPTH = 4;
     for (int odd = (m + 1) & (DEPTH - 1); odd > 0; --odd, --m) {
         const T v0 = k[m] * (tmz[m] * v1 + rxy * v2);
-        out[m] = v0;
+        out[m * STRIDE] = v0;
         v2 = v1;
         v1 = v0;
     }
@@ -331,7 +333,7 @@ __device__ __forceinline__ void sequence_job(int l, int which, T z, T rxy,
 #pragma unroll
         for (int j = DEPTH - 1; j >= 0; --j) {
             const T v0 = km[j] * (tz[j] * v1 + rxy * v2);
-            out[base + j] = v0;
+            out[(base + j) * STRIDE] = v0;
             v2 = v1;
             v1 = v0;
         }

@@ -47,6 +47,7 @@
 #include "sphx_lane_kernels.hpp"
 #include "sphx_vjp_kernels.hpp"
 #include "sphx_recursion_kernel.hpp"
+#include "sphx_pairs.hpp"
 
 namespace sphx {
 
@@ -74,6 +75,12 @@ static std::mutex g_init_mutex;
 static bool g_tables_ready[kMaxDevices] = {};
 static int g_lds_limit[kMaxDevices] = {};
 static int g_compute_units[kMaxDevices] = {};
+// where the constant tables of a device live, for kernels of other translation units
+struct TableAddresses {
+    const float *F32, *Q32;
+    const double *F64, *Q64;
+};
+static TableAddresses g_table_addresses[kMaxDevices] = {};
 
 static int find_scratch(int device);
 
@@ -92,6 +99,15 @@ static int ensure_device_ready(int device) {
     SPHX_HIP(hipMemcpyToSymbol(HIP_SYMBOL(kQ32), t.f32.data() + n, n * sizeof(float)));
     SPHX_HIP(hipMemcpyToSymbol(HIP_SYMBOL(kF64), t.f64.data(), n * sizeof(double)));
     SPHX_HIP(hipMemcpyToSymbol(HIP_SYMBOL(kQ64), t.f64.data() + n, n * sizeof(double)));
+    {
+        void *f32 = nullptr, *q32 = nullptr, *f64 = nullptr, *q64 = nullptr;
+        SPHX_HIP(hipGetSymbolAddress(&f32, HIP_SYMBOL(kF32)));
+        SPHX_HIP(hipGetSymbolAddress(&q32, HIP_SYMBOL(kQ32)));
+        SPHX_HIP(hipGetSymbolAddress(&f64, HIP_SYMBOL(kF64)));
+        SPHX_HIP(hipGetSymbolAddress(&q64, HIP_SYMBOL(kQ64)));
+        g_table_addresses[device] = TableAddresses{static_cast<const float*>(f32), static_cast<const float*>(q32),
+                                                   static_cast<const double*>(f64), static_cast<const double*>(q64)};
+    }
     int lds = 0, cus = 0;
     SPHX_HIP(hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device));
     SPHX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
@@ -124,6 +140,7 @@ static int ensure_device_ready(int device) {
 enum Switch : int {
     SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_GRADIENT_LANES, SW_GRADIENT_LANES_PARTS,
     SW_GRADIENT_LANES_TILE, SW_GRADIENT_LANES_WAVES, SW_GROUP_THREADS, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST,
+    SW_PAIRS, SW_PAIRS_BATCH, SW_PAIRS_CHUNK, SW_PAIRS_PREP_WAVES, SW_PAIRS_SEQUENCE_WAVES, SW_PAIRS_TILE,
     SW_PREFIX_INSIDE,
     SW_SEQUENCE_WAVES, SW_SLICE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
     SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_ALONE, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
@@ -134,6 +151,7 @@ static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_GRADIENT_LANES_PARTS", "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_GROUP_THREADS",
     "SPHX_HESSIAN_LANES",
     "SPHX_HESSIAN_LANES_PARTS", "SPHX_JOB_LIST",
+    "SPHX_PAIRS", "SPHX_PAIRS_BATCH", "SPHX_PAIRS_CHUNK", "SPHX_PAIRS_PREP_WAVES", "SPHX_PAIRS_SEQUENCE_WAVES", "SPHX_PAIRS_TILE",
     "SPHX_PREFIX_INSIDE", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_ALONE", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
@@ -181,8 +199,10 @@ struct Plan {
     bool whole;       // recursion_kernel evaluates the closed forms too: one launch
                       // otherwise closed_form_kernel<PREFIX> + recursion_kernel: two launches
     bool split_sides; // recursion_kernel takes the entries (l, +m) and (l, -m) as two jobs
+    bool pairs;       // values and gradients at large l_max: one launch of pairs_kernel (uses `pairs_launch`)
     Launch closed;
     Launch rec;
+    PairsLaunch pairs_launch;
 };
 
 static unsigned pow2_floor(unsigned v) {
@@ -966,6 +986,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     plan->closed_only = l_max <= hard;
     plan->whole = true;
     plan->split_sides = false;
+    plan->pairs = false;
     // Gradients in closed form, where the rows of a tile are so long that few single-wave
     // workgroups of closed_form_kernel share a CU: the lanes kernel instead, which cuts the closed
     // forms in slices for six or eight waves and flushes with all of them. Measured, us, against
@@ -1012,6 +1033,29 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // 246, 214; 9 307, 218; 10 293, 226; 11 309, 292. The lanes keep l_max <= 8 and 11 in float32,
     // l_max = 7 in float64, and every call of fewer than 32 768 points (50 000 points, lanes against
     // recursion: float64 l_max = 9 54, 43 us, float32 l_max = 12 42, 38 us; 20 000 points 25, 22 and 21, 24).)
+    // Values and gradients where the rows of few points fill LDS: pairs_kernel, whose entry lanes keep one
+    // (l, m) pair for the whole launch and whose other work runs while the rows are flushed. 1.2 GB of
+    // output, us, pairs_kernel against recursion_kernel: float32 l_max = 16, 20, 24, 28, 32, 36 299, 274,
+    // 267, 269, 253, 262 against 289, 286, 291, 288, 285, 286; float64 l_max = 14, 16, 20, 24, 28, 32, 36 289,
+    // 280, 265, 251, 268, 268, 248 against 283, 289, 288, 290, 285, 285, 274; cfg5 (l_max = 32, 200 000 points)
+    // 595 against 700. Below, a point's pairs leave most of the entry lanes idle and it loses (float32
+    // l_max = 12: 383 against 277). SPHX_PAIRS: 0 never, 2 wherever it fits.
+    {
+        const int pairs = switch_or(SW_PAIRS, 1);
+        const bool pairs_by_shape = n_samples >= 32768 && (elem == 4 ? l_max >= 20 : l_max >= 16);
+        if (lane_kernels && mode == 1 && (pairs == 2 || (pairs == 1 && pairs_by_shape))) {
+            PairsChoice want;
+            want.tile = static_cast<unsigned>(switch_or(SW_PAIRS_TILE, 0));
+            want.batch_tiles = static_cast<unsigned>(switch_or(SW_PAIRS_BATCH, 0));
+            want.prep_waves = static_cast<unsigned>(switch_or(SW_PAIRS_PREP_WAVES, 0));
+            want.sequence_waves = static_cast<unsigned>(switch_or(SW_PAIRS_SEQUENCE_WAVES, 0));
+            want.chunk_shift_plus_one = static_cast<unsigned>(switch_or(SW_PAIRS_CHUNK, -1) + 1);
+            if (plan_pairs(n_samples, l_max, elem, elem, lds_limit, cus, want, &plan->pairs_launch)) {
+                plan->pairs = true;
+                return SPHX_OK;
+            }
+        }
+    }
     const int gradient_lanes = switch_or(SW_GRADIENT_LANES, 1);
     const bool large_groups = group_threads(n_samples, mode, elem, lane_kernels) > kRecursionThreads && n_samples >= 32768;
     const bool lanes_by_shape = large_groups ? (elem == 4 ? l_max <= 8 || l_max == 11 : l_max <= 7)
@@ -1188,9 +1232,24 @@ static hipError_t launch_recursion(const Launch& l, const typename AsGiven<O>::t
     return hipGetLastError();
 }
 
+template <typename T> static const T* table_address(int device, bool q);
+template <> const float* table_address<float>(int device, bool q) {
+    return q ? g_table_addresses[device].Q32 : g_table_addresses[device].F32;
+}
+template <> const double* table_address<double>(int device, bool q) {
+    return q ? g_table_addresses[device].Q64 : g_table_addresses[device].F64;
+}
+
 template <typename T, int MODE, bool NORM>
-static hipError_t dispatch(const Plan& plan, const T* xyz, T* sph, T* dsph, T* ddsph,
+static hipError_t dispatch(const Plan& plan, int device, const T* xyz, T* sph, T* dsph, T* ddsph,
                            hipStream_t stream) {
+    if (plan.pairs) {
+        if constexpr (MODE == 1) {
+            return launch_pairs(plan.pairs_launch, NORM, table_address<T>(device, false), table_address<T>(device, true),
+                                xyz, sph, dsph, stream);
+        }
+        return hipErrorInvalidValue; // never planned
+    }
     if (plan.lanes) {
         if constexpr (MODE == 0) {
             const Launch& l = plan.closed;
@@ -1354,13 +1413,13 @@ static int forward_on(int device, const T* xyz, size_t n_samples, int l_max, int
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     hipError_t e;
     if (normalized) {
-        e = mode == 0   ? dispatch<T, 0, true>(plan, xyz, sph, dsph, ddsph, s)
-            : mode == 1 ? dispatch<T, 1, true>(plan, xyz, sph, dsph, ddsph, s)
-                        : dispatch<T, 2, true>(plan, xyz, sph, dsph, ddsph, s);
+        e = mode == 0   ? dispatch<T, 0, true>(plan, device, xyz, sph, dsph, ddsph, s)
+            : mode == 1 ? dispatch<T, 1, true>(plan, device, xyz, sph, dsph, ddsph, s)
+                        : dispatch<T, 2, true>(plan, device, xyz, sph, dsph, ddsph, s);
     } else {
-        e = mode == 0   ? dispatch<T, 0, false>(plan, xyz, sph, dsph, ddsph, s)
-            : mode == 1 ? dispatch<T, 1, false>(plan, xyz, sph, dsph, ddsph, s)
-                        : dispatch<T, 2, false>(plan, xyz, sph, dsph, ddsph, s);
+        e = mode == 0   ? dispatch<T, 0, false>(plan, device, xyz, sph, dsph, ddsph, s)
+            : mode == 1 ? dispatch<T, 1, false>(plan, device, xyz, sph, dsph, ddsph, s)
+                        : dispatch<T, 2, false>(plan, device, xyz, sph, dsph, ddsph, s);
     }
     if (e != hipSuccess) {
         return fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
@@ -1379,6 +1438,7 @@ static bool make_wide_plan(size_t n_samples, int l_max, int mode, int lds_limit,
     plan->closed_only = false;
     plan->whole = true;
     plan->split_sides = false;
+    plan->pairs = false;
     const unsigned threads = group_threads(n_samples, mode, 8, true);
     const int whole_cu = mode == 2 || threads > kRecursionThreads ? lds_limit : 80 * 1024; // as for float64 arrays (make_plan)
     const unsigned budget = static_cast<unsigned>(switch_or(SW_TILE_LDS_BUDGET, whole_cu));
@@ -1922,6 +1982,13 @@ int sphx_plan(size_t n_samples, int l_max, int derivatives, int is_f64, int* til
     int status = sphx::make_plan(n_samples ? n_samples : 1, l_max, derivatives,
                                  is_f64 ? sizeof(double) : sizeof(float), lds, cus, &plan);
     if (status != SPHX_OK) return status;
+    if (plan.pairs) {
+        if (tile_samples) *tile_samples = static_cast<int>(plan.pairs_launch.g.tile);
+        if (threads) *threads = static_cast<int>(plan.pairs_launch.threads);
+        if (lds_bytes) *lds_bytes = static_cast<int>(plan.pairs_launch.lds_bytes);
+        if (workgroups) *workgroups = static_cast<int>(plan.pairs_launch.workgroups);
+        return SPHX_OK;
+    }
     const sphx::Launch& main = plan.closed_only || plan.lanes ? plan.closed : plan.rec;
     if (tile_samples) *tile_samples = main.g.tile;
     if (threads) *threads = static_cast<int>(main.threads);
@@ -1956,7 +2023,12 @@ int sphx_describe_plan(size_t n_samples, int l_max, int derivatives, int is_f64,
                std::to_string(l.lds_bytes) + " B LDS, " + std::to_string(l.workgroups) + " workgroups]";
     };
     std::string text;
-    if (plan.closed_only) {
+    if (plan.pairs) {
+        const sphx::PairsLaunch& l = plan.pairs_launch;
+        text = "pairs_kernel<" + t + ", " + (normalized ? "true" : "false") + "> [" + std::to_string(l.g.tile) +
+               " points per tile, " + std::to_string(l.threads) + " threads, " + std::to_string(l.lds_bytes) +
+               " B LDS, " + std::to_string(l.workgroups) + " workgroups]";
+    } else if (plan.closed_only) {
         text = "closed_form_kernel<" + head + ", " + std::to_string(l_max) + ", false>" + geometry(plan.closed);
     } else if (plan.lanes) {
         const char* names[3] = {"values_kernel", "gradients_lanes_kernel", "hessians_lanes_kernel"};

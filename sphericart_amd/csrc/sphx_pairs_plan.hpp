@@ -1,0 +1,147 @@
+// Host side of pairs_kernel: tile, batch, wave roles, LDS layout and the table that gives every
+// entry lane its (l, m) pair, from the shape of a call. Plain C++, no HIP: the planner can be
+// compiled and tested without a device.
+#ifndef SPHX_PAIRS_PLAN_HPP
+#define SPHX_PAIRS_PLAN_HPP
+
+#include <cstddef>
+#include <cstring>
+
+#include "sphx_pairs_tiling.hpp"
+
+namespace sphx {
+
+// What the caller may fix (0 = let the planner choose).
+struct PairsChoice {
+    unsigned tile = 0, batch_tiles = 0, prep_waves = 0, sequence_waves = 0, chunk_shift_plus_one = 0;
+};
+
+struct PairsLaunch {
+    PairsTiling g;
+    unsigned lds_bytes = 0, threads = 0, workgroups = 0;
+};
+
+// The lane table: the pairs (l, m >= 1) of one point in a row, l and m descending, over as few waves as
+// hold them. (A table that kept the lanes of a half-wave on different LDS banks, at the price of one more
+// wave, measured 1-3 % slower: the stage is bound by instruction issue, not by LDS.) Returns the number
+// of waves, 0 if `waves` do not hold the pairs.
+inline unsigned pairs_lane_table(int l_max, int hard, unsigned waves, unsigned short* table) {
+    for (unsigned i = 0; i < kPairsThreads; ++i) table[i] = static_cast<unsigned short>(kPairsNoJob);
+    if (waves > kPairsThreads / 64u) waves = kPairsThreads / 64u;
+    unsigned at = 0;
+    for (int l = l_max; l > hard; --l) {
+        if (at + static_cast<unsigned>(l) > waves * 64u) return 0;
+        for (int m = l; m >= 1; --m) table[at++] = static_cast<unsigned short>((l << 8) | m);
+    }
+    return (at + 63u) / 64u;
+}
+
+// false: this shape is not for pairs_kernel (the pairs of a point do not fit the waves, or the rows of
+// a tile and the tables do not fit LDS).
+inline bool plan_pairs(size_t n_samples, int l_max, size_t elem, size_t out_elem, int lds_limit, int cus,
+                       const PairsChoice& want, PairsLaunch* out) {
+    constexpr int H = 6;
+    constexpr unsigned NYH = 49, COMP = 4, IT = 2, ITEMS = 9, WAVES = kPairsThreads / 64u;
+    if (l_max <= H || l_max > 64 || n_samples == 0) return false;
+    PairsTiling& g = out->g;
+    std::memset(&g, 0, sizeof(g));
+    const unsigned esize = static_cast<unsigned>(elem), osize = static_cast<unsigned>(out_elem);
+    const unsigned L = static_cast<unsigned>(l_max);
+    const unsigned ny = (L + 1) * (L + 1);
+    const unsigned tri_all = (L + 1) * (L + 2) / 2;
+    const unsigned levels = L - H;
+
+    const unsigned line = 128u / osize;
+    auto align4 = [](unsigned v) { return (v + 3u) & ~3u; };
+    // a point's record: x, y, z, 1/r, x^2 + y^2, three spare; the (c_m, s_m) pairs; 2(m+1)z from a multiple of
+    // four numbers on, and the records a multiple of four apart (16-byte reads of four steps' constants)
+    const unsigned tmz_at = align4(8u + 2u * (L + 1));
+    const unsigned point_stride = align4(tmz_at + (L + 1));
+    const unsigned q_stride = align4(L + 1);
+    const unsigned q_elems = (L + 1) * q_stride;
+    const unsigned f0_elems = align4(L + 1);
+    const unsigned park_stride = COMP * NYH + 1u; // odd: the lanes of a prep wave, one point each, spread over the banks
+    const unsigned iter_stride = align4(IT * tri_all + IT); // one group past the end is read, never used
+    auto bytes_for = [&](unsigned S, unsigned tpb) {
+        const unsigned rows = align4(S * ny + line) + align4(S * 3 * ny + line);
+        const unsigned tables = q_elems + f0_elems + 2 * tpb * S * (point_stride + park_stride) + 4u + S * iter_stride;
+        return rows * osize + tables * esize;
+    };
+
+    // as many points per tile as LDS holds next to a batch of three tiles, twelve at most (1.2 GB of
+    // output, l_max = 20 - 36: within 3 % of the best tile size on every shape)
+    unsigned S = want.tile ? want.tile : 12u;
+    if (S > 16) S = 16;
+    while (S > 1 && bytes_for(S, 3) > static_cast<unsigned>(lds_limit)) --S;
+    // batches: as many tiles as a wave has lanes for and LDS holds; at least three, so that the nine work
+    // items of a batch fit its tile rounds with the prep waves there are
+    unsigned tpb = want.batch_tiles ? want.batch_tiles : 64u / S;
+    if (tpb * S > 64u) tpb = 64u / S;
+    while (tpb > 3 && bytes_for(S, tpb) > static_cast<unsigned>(lds_limit)) --tpb;
+    if (tpb < 3 || bytes_for(S, tpb) > static_cast<unsigned>(lds_limit)) return false;
+    unsigned P = want.prep_waves ? want.prep_waves : (ITEMS + tpb - 1u) / tpb;
+    if (P * tpb < ITEMS) P = (ITEMS + tpb - 1u) / tpb;
+    // one recursion per lane and tile where four waves suffice for that
+    unsigned NSEQ = want.sequence_waves ? want.sequence_waves : (S * 2u * levels + 63u) / 64u;
+    if (NSEQ < 1) NSEQ = 1;
+    if (NSEQ > 4) NSEQ = 4;
+    if (P + NSEQ >= WAVES) return false;
+    const unsigned room = WAVES - P - NSEQ;
+    // the waves that hold a point's pairs, and as many points side by side as the entry waves allow
+    const unsigned slot_waves = pairs_lane_table(l_max, H, room, g.lane_job);
+    if (slot_waves == 0) return false;
+    unsigned slots = room / slot_waves;
+    if (slots > S) slots = S;
+    const unsigned E = slots * slot_waves;
+
+    g.n_samples = n_samples;
+    g.l_max = l_max;
+    g.ny = static_cast<int>(ny);
+    g.tile = S;
+    g.batch_tiles = tpb;
+    g.magic_batch = static_cast<unsigned>(((1ull << 32) + tpb - 1) / tpb);
+    g.prep_waves = P;
+    g.sequence_waves = NSEQ;
+    g.entry_waves = E;
+    g.slot_waves = slot_waves;
+    unsigned at = align4(S * ny + line);
+    g.off_dsph = at;
+    at = align4(at + S * 3 * ny + line);
+    g.tables_at = at * osize;
+    at = 0;
+    g.off_Q = at;
+    at += q_elems;
+    g.off_F0 = at;
+    at += f0_elems;
+    g.off_pts = at;
+    at += 2 * tpb * S * point_stride;
+    g.off_park = at;
+    at += 2 * tpb * S * park_stride;
+    at = align4(at);
+    g.off_iter = at;
+    at += S * iter_stride;
+    g.point_stride = point_stride;
+    g.park_stride = park_stride;
+    g.iter_stride = iter_stride;
+    g.tmz_at = tmz_at;
+    g.q_stride = q_stride;
+    out->lds_bytes = g.tables_at + at * esize;
+    out->threads = 64u * (P + NSEQ + E);
+    if (out->lds_bytes > static_cast<unsigned>(lds_limit)) return false;
+
+    g.n_tiles = static_cast<unsigned>((n_samples + S - 1) / S);
+    g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
+    // about eight points per chunk of consecutive tiles
+    g.chunk_shift = want.chunk_shift_plus_one ? want.chunk_shift_plus_one - 1u : (S >= 5 ? 0u : (S >= 3 ? 1u : (S == 2 ? 2u : 3u)));
+    const unsigned resident = (static_cast<unsigned>(cus > 0 ? cus : 8) + 7u) & ~7u;
+    auto chunks_in_xcd = [&]() { return (g.tiles_per_xcd + (1u << g.chunk_shift) - 1u) >> g.chunk_shift; };
+    while (g.chunk_shift > 0 && chunks_in_xcd() * 8u < resident) --g.chunk_shift;
+    const unsigned need = chunks_in_xcd() * 8u;
+    out->workgroups = resident < need ? resident : need;
+    if (out->workgroups < 8) out->workgroups = 8;
+    return true;
+}
+
+} // namespace sphx
+
+#endif

@@ -80,12 +80,13 @@ def test_launch_plans(library):
     for n, l_max, mode, f64 in ((10_000, 8, 1, True), (100_000, 16, 2, True), (200_000, 32, 1, False), (5, 20, 2, False)):
         status, (tile, threads, lds, groups) = _plan(library, n, l_max, mode, f64)
         assert status == 0
-        assert 1 <= tile <= 64 and threads in (256, 512, 1024) and lds <= 160 * 1024
+        assert 1 <= tile <= 64 and threads % 64 == 0 and 256 <= threads <= 1024 and lds <= 160 * 1024
         assert groups % 8 == 0 and groups >= 8
-    # cfg5: one workgroup of 1024 threads per CU with all of its LDS, five points per tile;
-    # the same shape with few points: workgroups of 512 threads
+    # cfg5: pairs_kernel, one workgroup per CU with nearly all of its LDS, five points per tile (three prep
+    # waves, four sequence waves, eight entry waves for the 507 pairs of a point);
+    # the same shape with few points: recursion_kernel in workgroups of 512 threads
     status, (tile, threads, lds, groups) = _plan(library, 200_000, 32, 1, False)
-    assert status == 0 and (tile, threads, groups) == (5, 1024, 256) and 150_000 < lds <= 160 * 1024
+    assert status == 0 and (tile, threads, groups) == (5, 960, 256) and 140_000 < lds <= 160 * 1024
     status, (tile, threads, lds, groups) = _plan(library, 2_000, 32, 1, False)
     assert status == 0 and threads == 512 and lds <= 80 * 1024
     # second derivatives in float64 keep 512 threads (more than 128 registers per lane)
