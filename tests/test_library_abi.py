@@ -114,15 +114,24 @@ def test_launch_plans(library):
 def test_planner_overrides(library, switches):
     """sphx_set_switch changes what the next call plans; sphx_reset_switches restores the default;
     unknown names are refused. Environment variables alone change nothing."""
-    default = _plan(library, 50_000, 20, 1, False)
+    default = _plan(library, 50_000, 14, 1, False)
     os.environ["SPHX_TILE"] = "3"
     try:
-        assert _plan(library, 50_000, 20, 1, False) == default
+        assert _plan(library, 50_000, 14, 1, False) == default
     finally:
         del os.environ["SPHX_TILE"]
     switches("SPHX_TILE", 3)
+    status, (tile, _, _, _) = _plan(library, 50_000, 14, 1, False)
+    assert status == 0 and tile == 3 and default[1][0] != 3
+    library.sphx_reset_switches()
+    assert _plan(library, 50_000, 14, 1, False) == default
+    # the same for pairs_kernel, which takes values and gradients from l_max = 20 on in float32
+    default = _plan(library, 50_000, 20, 1, False)
+    switches("SPHX_PAIRS_TILE", 3)
     status, (tile, _, _, _) = _plan(library, 50_000, 20, 1, False)
     assert status == 0 and tile == 3 and default[1][0] != 3
+    switches("SPHX_PAIRS", 0)
+    assert _plan(library, 50_000, 20, 1, False)[1][1] in (512, 1024)  # recursion_kernel again
     library.sphx_reset_switches()
     assert _plan(library, 50_000, 20, 1, False) == default
     assert library.sphx_set_switch(b"SPHX_NO_SUCH_SWITCH", 1) == 1
