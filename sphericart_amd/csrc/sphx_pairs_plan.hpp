@@ -133,6 +133,7 @@ inline bool plan_pairs(size_t n_samples, int l_max, size_t elem, size_t out_elem
     g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
     // about eight points per chunk of consecutive tiles
     g.chunk_shift = want.chunk_shift_plus_one ? want.chunk_shift_plus_one - 1u : (S >= 5 ? 0u : (S >= 3 ? 1u : (S == 2 ? 2u : 3u)));
+    if (g.chunk_shift > 10u) g.chunk_shift = 10u;
     const unsigned resident = (static_cast<unsigned>(cus > 0 ? cus : 8) + 7u) & ~7u;
     auto chunks_in_xcd = [&]() { return (g.tiles_per_xcd + (1u << g.chunk_shift) - 1u) >> g.chunk_shift; };
     while (g.chunk_shift > 0 && chunks_in_xcd() * 8u < resident) --g.chunk_shift;

@@ -1,0 +1,133 @@
+"""pairs_kernel (values and gradients, every entry lane bound to one (l, m) pair) against the oracle,
+number for number.
+
+The planner gives it float32 from l_max = 20 and float64 from l_max = 16 when a call has 32 768 points or
+more; here SPHX_PAIRS = 2 sends every shape it can hold through it, with the tile, batch and wave counts
+the planner would pick and with forced ones, so that every path of the kernel runs at sizes the oracle
+finishes in seconds: partial last tiles, fewer tiles than workgroups, several points side by side in the
+entry waves, several rounds of recursions per tile, outputs that start anywhere inside a 128-byte line.
+"""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_utils import announce
+from helpers import same_numbers, special_points
+
+pytestmark = pytest.mark.gpu
+
+
+def _evaluate(library, xyz, l_max, normalized, shift=0):
+    """sphx_forward_* with gradients into buffers with NaN guard bands; returns (sph, dsph, guards intact)."""
+    n = xyz.shape[0]
+    ny = (l_max + 1) ** 2
+    tdtype = torch.float32 if xyz.dtype == np.float32 else torch.float64
+    sizes = (n * ny, 3 * n * ny)
+    raw = [torch.full((size + 64,), float("nan"), dtype=tdtype, device="cuda") for size in sizes]
+    out = [raw[0][shift:shift + sizes[0]].view(n, ny), raw[1][shift:shift + sizes[1]].view(n, 3, ny)]
+    forward = library.sphx_forward_f32 if xyz.dtype == np.float32 else library.sphx_forward_f64
+    xyz_dev = torch.from_numpy(xyz).cuda()
+    status = forward(xyz_dev.data_ptr(), n, l_max, int(normalized), 1, out[0].data_ptr(), out[1].data_ptr(), None,
+                     torch.cuda.current_stream().cuda_stream)
+    assert status == 0, library.sphx_last_error()
+    torch.cuda.synchronize()
+    guards = all(bool(torch.isnan(raw[i][:shift]).all() and torch.isnan(raw[i][shift + sizes[i]:]).all())
+                 for i in range(2))
+    return out[0].cpu().numpy(), out[1].cpu().numpy(), guards
+
+
+def _plan_text(library, n, l_max, f64, normalized):
+    text = ctypes.create_string_buffer(512)
+    assert library.sphx_describe_plan(n, l_max, 1, int(f64), int(normalized), text, 512) == 0
+    return text.value.decode()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("normalized", [True, False])
+def test_every_l_max_it_holds(oracle, library, switches, dtype, normalized):
+    """l_max 7 .. 40 at a ragged number of points (a partial last tile, tiles of up to twelve points)."""
+    rng = np.random.default_rng(7)
+    switches("SPHX_PAIRS", 2)
+    ran = 0
+    for l_max in (7, 8, 9, 13, 16, 19, 20, 23, 24, 27, 31, 32, 33, 36, 40):
+        n = 389 if l_max < 30 else 167
+        text = _plan_text(library, n, l_max, dtype == np.float64, normalized)
+        announce("pairs", np.dtype(dtype).name, "normalized", normalized, "l_max", l_max, "n", n, text)
+        if not text.startswith("pairs_kernel"):
+            continue  # more pairs than the entry waves have lanes, or rows too long for LDS
+        ran += 1
+        xyz = special_points(dtype, rng, n)
+        want = oracle.compute(xyz, l_max, normalized, "gradients")
+        sph, dsph, guards = _evaluate(library, xyz, l_max, normalized)
+        assert same_numbers(sph, want[0]).all(), (l_max, "values")
+        assert same_numbers(dsph, want[1]).all(), (l_max, "gradients")
+        assert guards
+    assert ran >= 10
+
+
+def test_forced_tiles_batches_and_waves(oracle, library, switches):
+    """Plans the planner would not make: every tile size, small and large batches, one to four sequence
+    waves (several rounds of recursions per tile), one to three prep waves, chunks of one to eight tiles."""
+    rng = np.random.default_rng(11)
+    cases = [
+        (np.float32, 32, {"SPHX_PAIRS_TILE": 1}),
+        (np.float32, 32, {"SPHX_PAIRS_TILE": 2, "SPHX_PAIRS_SEQUENCE_WAVES": 1}),
+        (np.float32, 32, {"SPHX_PAIRS_TILE": 3, "SPHX_PAIRS_BATCH": 3, "SPHX_PAIRS_PREP_WAVES": 3}),
+        (np.float32, 32, {"SPHX_PAIRS_TILE": 4, "SPHX_PAIRS_CHUNK": 3}),
+        (np.float32, 24, {"SPHX_PAIRS_TILE": 7, "SPHX_PAIRS_SEQUENCE_WAVES": 2}),
+        (np.float32, 20, {"SPHX_PAIRS_TILE": 12, "SPHX_PAIRS_BATCH": 4}),
+        (np.float32, 12, {"SPHX_PAIRS_TILE": 16, "SPHX_PAIRS_PREP_WAVES": 1}),
+        (np.float32, 9, {"SPHX_PAIRS_TILE": 5, "SPHX_PAIRS_CHUNK": 0}),
+        (np.float64, 28, {"SPHX_PAIRS_TILE": 1, "SPHX_PAIRS_CHUNK": 2}),
+        (np.float64, 24, {"SPHX_PAIRS_TILE": 3, "SPHX_PAIRS_SEQUENCE_WAVES": 4}),
+        (np.float64, 16, {"SPHX_PAIRS_TILE": 6, "SPHX_PAIRS_BATCH": 10}),
+        (np.float64, 10, {"SPHX_PAIRS_TILE": 9, "SPHX_PAIRS_PREP_WAVES": 2, "SPHX_PAIRS_SEQUENCE_WAVES": 1}),
+    ]
+    for dtype, l_max, overrides in cases:
+        library.sphx_reset_switches()
+        switches("SPHX_PAIRS", 2)
+        for name, value in overrides.items():
+            switches(name, value)
+        for n, normalized in ((1201, True), (77, False)):
+            text = _plan_text(library, n, l_max, dtype == np.float64, normalized)
+            announce("pairs forced", np.dtype(dtype).name, "l_max", l_max, overrides, "n", n, text)
+            assert text.startswith("pairs_kernel"), text
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, normalized, "gradients")
+            sph, dsph, guards = _evaluate(library, xyz, l_max, normalized, shift=int(rng.integers(0, 33)))
+            assert same_numbers(sph, want[0]).all(), (l_max, overrides, n, "values")
+            assert same_numbers(dsph, want[1]).all(), (l_max, overrides, n, "gradients")
+            assert guards, (l_max, overrides, n)
+
+
+def test_few_points_and_shifted_outputs(oracle, library, switches):
+    """One point to a few tiles (most workgroups have no tile), outputs shifted by 0 .. 33 elements."""
+    rng = np.random.default_rng(13)
+    switches("SPHX_PAIRS", 2)
+    for dtype, l_max in ((np.float32, 21), (np.float64, 17)):
+        for n in (1, 2, 3, 4, 5, 11, 12, 13, 25, 64, 100):
+            shift = int(rng.integers(0, 34))
+            announce("pairs few points", np.dtype(dtype).name, "l_max", l_max, "n", n, "shift", shift)
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, True, "gradients")
+            sph, dsph, guards = _evaluate(library, xyz, l_max, True, shift=shift)
+            assert same_numbers(sph, want[0]).all(), (l_max, n, "values")
+            assert same_numbers(dsph, want[1]).all(), (l_max, n, "gradients")
+            assert guards, (l_max, n)
+
+
+def test_planned_by_shape(library):
+    """What the planner picks without overrides."""
+    assert _plan_text(library, 200_000, 32, False, True).startswith("pairs_kernel<float, true>")
+    assert _plan_text(library, 100_000, 20, False, False).startswith("pairs_kernel<float, false>")
+    assert _plan_text(library, 100_000, 16, True, True).startswith("pairs_kernel<double, true>")
+    assert _plan_text(library, 100_000, 19, False, True).startswith("recursion_kernel")
+    assert _plan_text(library, 100_000, 15, True, True).startswith("recursion_kernel")
+    assert _plan_text(library, 20_000, 32, False, True).startswith("recursion_kernel")  # few points
+    # second derivatives and values alone stay where they were
+    text = ctypes.create_string_buffer(512)
+    assert library.sphx_describe_plan(200_000, 32, 0, 0, 1, text, 512) == 0 and not text.value.startswith(b"pairs")
+    assert library.sphx_describe_plan(200_000, 24, 2, 0, 1, text, 512) == 0 and not text.value.startswith(b"pairs")
