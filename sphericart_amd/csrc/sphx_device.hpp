@@ -360,14 +360,15 @@ __device__ __forceinline__ void sequence_job(int l, int which, T z, T rxy,
 // reference's. SPLIT == false: one job computes both sides (the common factors are shared).
 // SPLIT == true: one job computes the side it is given, so that a tile with few (l, m) pairs
 // still spreads over all lanes.
-template <typename T, int MODE, bool NORM, bool SPLIT, typename O>
-__device__ __forceinline__ void entry_job(int l, int m, int tri, int side, const Point<T>& p,
-                                          const T* __restrict__ pk, const T* __restrict__ c,
-                                          const T* __restrict__ s, const T* __restrict__ A,
-                                          [[maybe_unused]] const T* __restrict__ B,
-                                          [[maybe_unused]] const T* __restrict__ C,
-                                          const Rows<O>& out) {
-    // tri = l(l+1)/2; pk, A, B, C already point at the (l, 0) entries of their triangular arrays
+//
+// The inputs come through `in`, addressed relative to the job's own m: in.pk() is the prefactor F_l^m,
+// in.c(d) / in.s(d) are c_{m+d} / s_{m+d}, in.A(d) / in.B(d) / in.C(d) the iterates of the three recursions at
+// m + d, with d a literal everywhere. A caller that holds them in arrays indexes those (EntryArrays below); a
+// caller that holds them in registers answers each d with a register.
+template <typename T, int MODE, bool NORM, bool SPLIT, typename In, typename O>
+__device__ __forceinline__ void entry_job_from(int l, int m, int tri, int side, const Point<T>& p, const In& in,
+                                               const Rows<O>& out) {
+    // tri = l(l+1)/2
     constexpr bool GRAD = MODE >= 1;
     constexpr bool HESS = MODE == 2;
     const T x = p.x, y = p.y;
@@ -397,20 +398,20 @@ __device__ __forceinline__ void entry_job(int l, int m, int tri, int side, const
 
     if (m == l) {
         // :122-152
-        const T qlm_2 = A[l];
-        const T cl = c[l], sl = s[l];
+        const T qlm_2 = in.A(0);
+        const T cl = in.c(0), sl = in.s(0);
         [[maybe_unused]] T cl1 = 0, sl1 = 0, cl2 = 0, sl2 = 0;
         if constexpr (GRAD) {
-            cl1 = c[l - 1];
-            sl1 = s[l - 1];
+            cl1 = in.c(-1);
+            sl1 = in.s(-1);
         }
         if constexpr (HESS) {
-            cl2 = c[l - 2];
-            sl2 = s[l - 2];
+            cl2 = in.c(-2);
+            sl2 = in.s(-2);
         }
         emit_sides([&](bool minus) {
             Entry<T> e = blank();
-            auto pq = qlm_2 * pk[l];
+            auto pq = qlm_2 * in.pk();
             e.v = pq * (minus ? sl : cl);
             if constexpr (GRAD) {
                 pq *= l;
@@ -427,20 +428,20 @@ __device__ __forceinline__ void entry_job(int l, int m, int tri, int side, const
         });
     } else if (m == l - 1) {
         // :154-198
-        [[maybe_unused]] const T qlm_2 = A[l];
-        const T qlm_1 = A[l - 1];
-        const T pkm = pk[l - 1];
-        const T cm = c[l - 1], sm = s[l - 1];
+        [[maybe_unused]] const T qlm_2 = in.A(1);
+        const T qlm_1 = in.A(0);
+        const T pkm = in.pk();
+        const T cm = in.c(0), sm = in.s(0);
         [[maybe_unused]] T cm1 = 0, sm1 = 0, cm2 = 0, sm2 = 0, ql1m_1 = 0;
         if constexpr (GRAD) {
-            cm1 = c[l - 2];
-            sm1 = s[l - 2];
-            ql1m_1 = B[l - 1];
+            cm1 = in.c(-1);
+            sm1 = in.s(-1);
+            ql1m_1 = in.B(0);
         }
         if constexpr (HESS) {
             if (l != 2) {
-                cm2 = c[l - 3];
-                sm2 = s[l - 3];
+                cm2 = in.c(-2);
+                sm2 = in.s(-2);
             }
         }
         emit_sides([&](bool minus) {
@@ -473,26 +474,26 @@ __device__ __forceinline__ void entry_job(int l, int m, int tri, int side, const
         });
     } else if (m > 0) {
         // :201-390
-        const T cm = c[m], sm = s[m], pkm = pk[m];
-        const T qlm_0 = A[m];
+        const T cm = in.c(0), sm = in.s(0), pkm = in.pk();
+        const T qlm_0 = in.A(0);
         [[maybe_unused]] T cm1 = 0, sm1 = 0, cm2 = 0, sm2 = 0, ql1m_2 = 0, ql1m_1 = 0;
         [[maybe_unused]] T ql2m_2 = 0, ql2m_1 = 0, ql2m_0 = 0;
         if constexpr (GRAD) {
-            cm1 = c[m - 1];
-            sm1 = s[m - 1];
+            cm1 = in.c(-1);
+            sm1 = in.s(-1);
             // the reference reads these after its shift: ql1m_2 is the iterate of step m + 1
             // (or the start value), ql1m_1 the iterate of step m
-            ql1m_2 = B[m + 1];
-            ql1m_1 = B[m];
+            ql1m_2 = in.B(1);
+            ql1m_1 = in.B(0);
         }
         if constexpr (HESS) {
             // ... and these before its shift: the iterates of steps m + 2, m + 1 and m
-            ql2m_2 = C[m + 2];
-            ql2m_1 = C[m + 1];
-            ql2m_0 = C[m];
+            ql2m_2 = in.C(2);
+            ql2m_1 = in.C(1);
+            ql2m_0 = in.C(0);
             if (m != 1) {
-                cm2 = c[m - 2];
-                sm2 = s[m - 2];
+                cm2 = in.c(-2);
+                sm2 = in.s(-2);
             }
         }
         emit_sides([&](bool minus) {
@@ -541,22 +542,23 @@ __device__ __forceinline__ void entry_job(int l, int m, int tri, int side, const
     } else {
         // m = 0, :392-426
         Entry<T> pos = blank();
-        const T qlm_0 = A[0];
-        pos.v = qlm_0 * pk[0];
+        const T qlm_0 = in.A(0);
+        const T pk0 = in.pk();
+        pos.v = qlm_0 * pk0;
         if constexpr (GRAD) {
-            const T ql1m_1 = B[1];
-            const T ql1m_0 = B[0];
-            pos.gx = pk[0] * x * ql1m_1;
-            pos.gy = pk[0] * y * ql1m_1;
-            pos.gz = pk[0] * l * ql1m_0;
+            const T ql1m_1 = in.B(1);
+            const T ql1m_0 = in.B(0);
+            pos.gx = pk0 * x * ql1m_1;
+            pos.gy = pk0 * y * ql1m_1;
+            pos.gz = pk0 * l * ql1m_0;
             if constexpr (HESS) {
-                const T ql2m_2 = C[2];
-                const T ql2m_1 = C[1];
-                const T ql2m_0 = C[0];
-                auto pql1m_1 = pk[0] * ql1m_1;
-                auto pql2m_2 = pk[0] * ql2m_2;
-                auto pql2m_0 = pk[0] * ql2m_0;
-                auto pql2m_1 = pk[0] * ql2m_1;
+                const T ql2m_2 = in.C(2);
+                const T ql2m_1 = in.C(1);
+                const T ql2m_0 = in.C(0);
+                auto pql1m_1 = pk0 * ql1m_1;
+                auto pql2m_2 = pk0 * ql2m_2;
+                auto pql2m_0 = pk0 * ql2m_0;
+                auto pql2m_1 = pk0 * ql2m_1;
                 pos.hxx = pql1m_1 + x2 * pql2m_2;
                 pos.hyy = pql1m_1 + y2 * pql2m_2;
                 pos.hzz = (l) * (l - 1) * pql2m_0;
@@ -567,6 +569,34 @@ __device__ __forceinline__ void entry_job(int l, int m, int tri, int side, const
         }
         stage<T, MODE, NORM>(out, mid, p, pos);
     }
+}
+
+// The inputs of entry_job_from in arrays: pk, A, B, C point at the (l, 0) entries of their triangular
+// arrays, c / s at the point's azimuthal tables.
+template <typename T> struct EntryArrays {
+    int m;
+    const T* __restrict__ pk_;
+    const T* __restrict__ c_;
+    const T* __restrict__ s_;
+    const T* __restrict__ A_;
+    const T* __restrict__ B_;
+    const T* __restrict__ C_;
+    __device__ __forceinline__ T pk() const { return pk_[m]; }
+    __device__ __forceinline__ T c(int d) const { return c_[m + d]; }
+    __device__ __forceinline__ T s(int d) const { return s_[m + d]; }
+    __device__ __forceinline__ T A(int d) const { return A_[m + d]; }
+    __device__ __forceinline__ T B(int d) const { return B_[m + d]; }
+    __device__ __forceinline__ T C(int d) const { return C_[m + d]; }
+};
+
+template <typename T, int MODE, bool NORM, bool SPLIT, typename O>
+__device__ __forceinline__ void entry_job(int l, int m, int tri, int side, const Point<T>& p,
+                                          const T* __restrict__ pk, const T* __restrict__ c,
+                                          const T* __restrict__ s, const T* __restrict__ A,
+                                          const T* __restrict__ B, const T* __restrict__ C,
+                                          const Rows<O>& out) {
+    const EntryArrays<T> in{m, pk, c, s, A, B, C};
+    entry_job_from<T, MODE, NORM, SPLIT>(l, m, tri, side, p, in, out);
 }
 
 // ---- LDS -> HBM ------------------------------------------------------------

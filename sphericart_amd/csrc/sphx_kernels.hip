@@ -1033,24 +1033,27 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // 246, 214; 9 307, 218; 10 293, 226; 11 309, 292. The lanes keep l_max <= 8 and 11 in float32,
     // l_max = 7 in float64, and every call of fewer than 32 768 points (50 000 points, lanes against
     // recursion: float64 l_max = 9 54, 43 us, float32 l_max = 12 42, 38 us; 20 000 points 25, 22 and 21, 24).)
-    // Values and gradients where the rows of few points fill LDS: pairs_kernel, whose entry lanes keep one
-    // (l, m) pair for the whole launch and whose other work runs while the rows are flushed. 1.2 GB of
-    // output, us, pairs_kernel against recursion_kernel: float32 l_max = 16, 20, 24, 28, 32, 36 299, 274,
-    // 267, 269, 253, 262 against 289, 286, 291, 288, 285, 286; float64 l_max = 14, 16, 20, 24, 28, 32, 36 289,
-    // 280, 265, 251, 268, 268, 248 against 283, 289, 288, 290, 285, 285, 274; cfg5 (l_max = 32, 200 000 points)
-    // 595 against 700. Below, a point's pairs leave most of the entry lanes idle and it loses (float32
-    // l_max = 12: 383 against 277). SPHX_PAIRS: 0 never, 2 wherever it fits.
+    // Derivatives where the rows of few points fill LDS: pairs_kernel, whose entry lanes keep one (l, m) pair for
+    // the whole launch and whose other work runs while the rows are flushed. 1.2 GB of output, us, pairs_kernel
+    // against recursion_kernel. Gradients: float32 l_max = 16, 20, 24, 28, 32, 36 299, 274, 267, 269, 253, 262
+    // against 289, 286, 291, 288, 285, 286; float64 l_max = 14, 16, 20, 24, 28, 32, 36 289, 280, 265, 251, 268, 268,
+    // 248 against 283, 289, 288, 290, 285, 285, 274; cfg5 (l_max = 32, 200 000 points) 570-620 against 700. Below,
+    // a point's pairs leave most of the entry lanes idle and it loses (float32 l_max = 12: 383 against 277).
+    // Second derivatives: float64 l_max = 12, 16, 20, 24 287, 299, 296, 318 against 290, 290, 333, 352; float32
+    // l_max = 12, 16, 20, 24 350, 303, 318, 307 against 289, 285, 294, 304 (the recursion kernel's job list by
+    // kind fills sixteen waves better). SPHX_PAIRS: 0 never, 2 wherever it fits.
     {
         const int pairs = switch_or(SW_PAIRS, 1);
-        const bool pairs_by_shape = n_samples >= 32768 && (elem == 4 ? l_max >= 20 : l_max >= 16);
-        if (lane_kernels && mode == 1 && (pairs == 2 || (pairs == 1 && pairs_by_shape))) {
+        const bool pairs_by_shape = n_samples >= 32768 && (mode == 1 ? (elem == 4 ? l_max >= 20 : l_max >= 16)
+                                                                     : (elem == 8 && l_max >= 20));
+        if (lane_kernels && mode >= 1 && l_max > hard && (pairs == 2 || (pairs == 1 && pairs_by_shape))) {
             PairsChoice want;
             want.tile = static_cast<unsigned>(switch_or(SW_PAIRS_TILE, 0));
             want.batch_tiles = static_cast<unsigned>(switch_or(SW_PAIRS_BATCH, 0));
             want.prep_waves = static_cast<unsigned>(switch_or(SW_PAIRS_PREP_WAVES, 0));
             want.sequence_waves = static_cast<unsigned>(switch_or(SW_PAIRS_SEQUENCE_WAVES, 0));
             want.chunk_shift_plus_one = static_cast<unsigned>(switch_or(SW_PAIRS_CHUNK, -1) + 1);
-            if (plan_pairs(n_samples, l_max, elem, elem, lds_limit, cus, want, &plan->pairs_launch)) {
+            if (plan_pairs(n_samples, l_max, mode, elem, elem, lds_limit, cus, want, &plan->pairs_launch)) {
                 plan->pairs = true;
                 return SPHX_OK;
             }
@@ -1244,9 +1247,9 @@ template <typename T, int MODE, bool NORM>
 static hipError_t dispatch(const Plan& plan, int device, const T* xyz, T* sph, T* dsph, T* ddsph,
                            hipStream_t stream) {
     if (plan.pairs) {
-        if constexpr (MODE == 1) {
-            return launch_pairs(plan.pairs_launch, NORM, table_address<T>(device, false), table_address<T>(device, true),
-                                xyz, sph, dsph, stream);
+        if constexpr (MODE >= 1) {
+            return launch_pairs(plan.pairs_launch, MODE, NORM, table_address<T>(device, false),
+                                table_address<T>(device, true), xyz, sph, dsph, ddsph, stream);
         }
         return hipErrorInvalidValue; // never planned
     }
@@ -2025,7 +2028,7 @@ int sphx_describe_plan(size_t n_samples, int l_max, int derivatives, int is_f64,
     std::string text;
     if (plan.pairs) {
         const sphx::PairsLaunch& l = plan.pairs_launch;
-        text = "pairs_kernel<" + t + ", " + (normalized ? "true" : "false") + "> [" + std::to_string(l.g.tile) +
+        text = "pairs_kernel<" + head + "> [" + std::to_string(l.g.tile) +
                " points per tile, " + std::to_string(l.threads) + " threads, " + std::to_string(l.lds_bytes) +
                " B LDS, " + std::to_string(l.workgroups) + " workgroups]";
     } else if (plan.closed_only) {

@@ -1,5 +1,5 @@
-// pairs_kernel: values and gradients beyond the closed forms, every entry lane bound to one
-// (l, m) pair for the whole launch.
+// pairs_kernel: derivatives beyond the closed forms, every entry lane bound to one (l, m) pair for the
+// whole launch. MODE 1: values and gradients; MODE 2: second derivatives too.
 #ifndef SPHX_PAIRS_KERNEL_HPP
 #define SPHX_PAIRS_KERNEL_HPP
 
@@ -41,7 +41,9 @@ namespace sphx {
 // Arithmetic: templates_core.hpp:122-152, :154-198, :201-294 and :392-426 of the reference
 // through the same expressions as entry_job (sphx_device.hpp), the chain rule of
 // templates.hpp:553-614 through finish(); same operations in the same order, hence the same
-// numbers.
+// numbers. With second derivatives (closed forms only to l = 1, three recursions per l, thirteen
+// rows per point) the entries are entry_job itself, fed from registers, and nothing is parked: the
+// prep waves evaluate the closed forms of l <= 1 straight into the rows.
 // ---------------------------------------------------------------------------
 extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 
@@ -65,6 +67,20 @@ __device__ __forceinline__ void azimuth_pairs_job(const Point<T>& p, int L, T* c
     }
 }
 
+// The inputs of entry_job_from (sphx_device.hpp) in registers: what a lane has read around its own m.
+template <typename T> struct EntryWindow {
+    T pk_;
+    T c_[3], s_[3];   // at m - 2, m - 1, m
+    T A_[2], B_[2];   // at m, m + 1
+    T C_[3];          // at m, m + 1, m + 2
+    __device__ __forceinline__ T pk() const { return pk_; }
+    __device__ __forceinline__ T c(int d) const { return c_[2 + d]; }
+    __device__ __forceinline__ T s(int d) const { return s_[2 + d]; }
+    __device__ __forceinline__ T A(int d) const { return A_[d]; }
+    __device__ __forceinline__ T B(int d) const { return B_[d]; }
+    __device__ __forceinline__ T C(int d) const { return C_[d]; }
+};
+
 template <typename T> struct Pair2;
 template <> struct Pair2<float> {
     typedef float type __attribute__((ext_vector_type(2)));
@@ -73,22 +89,25 @@ template <> struct Pair2<double> {
     typedef double type __attribute__((ext_vector_type(2)));
 };
 
-template <typename T, bool NORM, typename O = T>
-__global__ __launch_bounds__(kPairsThreads, 1) void pairs_kernel(PairsTiling g, const T* __restrict__ table_F,
-                                                                const T* __restrict__ table_Q,
-                                                                const O* __restrict__ xyz, O* __restrict__ sph,
-                                                                O* __restrict__ dsph
+// NT: the most threads a workgroup may have. 1024 leaves a lane 128 registers; the entries with second
+// derivatives need more and run in workgroups of 512.
+template <typename T, int MODE, bool NORM, unsigned NT = kPairsThreads, typename O = T>
+__global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __restrict__ table_F,
+                                                     const T* __restrict__ table_Q, const O* __restrict__ xyz,
+                                                     O* __restrict__ sph, O* __restrict__ dsph,
+                                                     O* __restrict__ ddsph
 #ifdef SPHX_PAIRS_CLOCKS
                                                                 ,
                                                                 unsigned long long* clocks
 #endif
 ) {
-    constexpr int MODE = 1;
-    constexpr int H = 6;
+    static_assert(MODE == 1 || MODE == 2, "values alone have kernels of their own");
+    constexpr int H = MODE == 2 ? 1 : 6;
     constexpr unsigned NYH = (H + 1) * (H + 1);
-    constexpr unsigned COMP = 4;   // component rows per point: values, three gradient rows
-    constexpr unsigned IT = 2;     // the two sequences of one l interleaved: (A_m, B_m) pairs
-    constexpr unsigned ITEMS = 9;  // work items of a batch: the records, eight slices of closed forms
+    constexpr unsigned COMP = MODE == 2 ? 13 : 4;  // component rows per point
+    constexpr unsigned SEQS = MODE + 1;            // recursions per (point, l): Q_l^m, the Q_{l-1} and Q_{l-2} sequences
+    constexpr unsigned IT = MODE == 2 ? 4 : 2;     // ... interleaved in LDS: (A_m, B_m) pairs, (A_m, B_m, C_m, -) fours
+    constexpr unsigned ITEMS = MODE == 2 ? 1 : 9;  // work items of a batch: the records, eight slices of closed forms
     using P2 = typename Pair2<T>::type;
     using V4 = T __attribute__((ext_vector_type(4)));
 
@@ -159,14 +178,23 @@ __global__ __launch_bounds__(kPairsThreads, 1) void pairs_kernel(PairsTiling g, 
     // Where the rows of tile n start within their staging regions: element 0 of a region stands for
     // the start of the 128-byte line in which the tile's run begins in HBM.
     struct Phases {
-        unsigned sph, dsph;
+        unsigned sph, dsph, ddsph;
     };
     auto phases_of = [&](unsigned n) -> Phases {
         const unsigned long long first_point = static_cast<unsigned long long>(tile_of(n)) * S;
         Phases ph;
         ph.sph = phase_of(sph, first_point * ny);
         ph.dsph = phase_of(dsph, first_point * 3 * ny);
+        ph.ddsph = MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
         return ph;
+    };
+    [[maybe_unused]] auto staged_rows = [&](const Phases& ph, unsigned s) -> Rows<O> {
+        Rows<O> rows;
+        rows.ny = static_cast<int>(ny);
+        rows.sph = row_lds + ph.sph + s * ny;
+        rows.dsph = row_lds + g.off_dsph + ph.dsph + s * 3 * ny;
+        rows.ddsph = MODE == 2 ? row_lds + g.off_ddsph + ph.ddsph + s * 9 * ny : nullptr;
+        return rows;
     };
 
 #ifdef SPHX_PAIRS_CLOCKS
@@ -222,26 +250,28 @@ __global__ __launch_bounds__(kPairsThreads, 1) void pairs_kernel(PairsTiling g, 
                 azimuth_pairs_job<T>(p, L, rec + 8, rec + g.tmz_at);
                 return;
             }
-            Rows<T> rows;
-            rows.ny = static_cast<int>(NYH);
-            rows.sph = parked(n, s);
-            rows.dsph = rows.sph + NYH;
-            rows.ddsph = nullptr;
-            switch (item) {
-            case 1: closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows); break;
-            case 2: closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows); break;
-            case 3: closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows); break;
-            case 4: closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows); break;
-            case 5: closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows); break;
-            case 6: closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows); break;
-            case 7: closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows); break;
-            default: closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows); break;
+            if constexpr (MODE == 1) {
+                Rows<T> rows;
+                rows.ny = static_cast<int>(NYH);
+                rows.sph = parked(n, s);
+                rows.dsph = rows.sph + NYH;
+                rows.ddsph = nullptr;
+                switch (item) {
+                case 1: closed_form_job<T, MODE, NORM, H, 0, 9>(p, rows); break;
+                case 2: closed_form_job<T, MODE, NORM, H, 9, 16>(p, rows); break;
+                case 3: closed_form_job<T, MODE, NORM, H, 16, 25>(p, rows); break;
+                case 4: closed_form_job<T, MODE, NORM, H, 25, 31>(p, rows); break;
+                case 5: closed_form_job<T, MODE, NORM, H, 31, 36>(p, rows); break;
+                case 6: closed_form_job<T, MODE, NORM, H, 36, 41>(p, rows); break;
+                case 7: closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows); break;
+                default: closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows); break;
+                }
             }
         };
         const unsigned prep_lanes = 64u * P;
-        // the closed forms of tile n from the parking area into its rows: point after point, a lane takes
-        // the same entries of every point
-        auto unpark_stage = [&](unsigned n, unsigned valid, O* rows_v, O* rows_g) {
+        // MODE 1: the closed forms of tile n from the parking area into its rows: point after point, a lane
+        // takes the same entries of every point
+        [[maybe_unused]] auto unpark_stage = [&](unsigned n, unsigned valid, O* rows_v, O* rows_g) {
             for (unsigned r = tid; r < COMP * NYH; r += prep_lanes) {
                 const unsigned comp = r / NYH;
                 const unsigned k = r - comp * NYH;
@@ -255,8 +285,23 @@ __global__ __launch_bounds__(kPairsThreads, 1) void pairs_kernel(PairsTiling g, 
                 }
             }
         };
+        // MODE 2: the closed forms of l <= 1 are a handful of operations: one lane per point, straight into the rows
+        [[maybe_unused]] auto low_stage = [&](unsigned n, unsigned valid, const Phases& ph) {
+            if (tid < valid) {
+                const T* rec = record(n, tid);
+                Point<T> p;
+                p.x = rec[0];
+                p.y = rec[1];
+                p.z = rec[2];
+                p.ir = rec[3];
+                p.x2 = p.x * p.x;
+                p.y2 = p.y * p.y;
+                p.z2 = p.z * p.z;
+                closed_form_job<T, MODE, NORM, H>(p, staged_rows(ph, tid));
+            }
+        };
         // the entries with m = 0 of tile n, one lane per (point, l); templates_core.hpp:392-426
-        auto axial_stage = [&](unsigned n, unsigned valid, O* rows_v, O* rows_g) {
+        auto axial_stage = [&](unsigned n, unsigned valid, const Phases& ph) {
             for (unsigned a = tid; a < valid * levels; a += prep_lanes) {
                 const unsigned s = a / levels;
                 const int l = L - static_cast<int>(a - s * levels);
@@ -264,30 +309,47 @@ __global__ __launch_bounds__(kPairsThreads, 1) void pairs_kernel(PairsTiling g, 
                 const T* it = iterates(s) + IT * (l * (l + 1) / 2);
                 const P2 xy = *reinterpret_cast<const P2*>(rec);
                 const P2 zi = *reinterpret_cast<const P2*>(rec + 2);
-                const P2 it0 = *reinterpret_cast<const P2*>(it);      // Q_l^0 and the Q_{l-1} sequence at 0
-                const P2 it1 = *reinterpret_cast<const P2*>(it + IT); // ... at 1
-                const T pk = F0[l];
                 Point<T> p;
                 p.x = xy[0];
                 p.y = xy[1];
                 p.z = zi[0];
                 p.ir = zi[1];
                 p.x2 = p.y2 = p.z2 = 0;
-                Entry<T> e;
-                e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = static_cast<T>(0.0);
-                e.v = it0[0] * pk;
-                e.gx = pk * p.x * it1[1];
-                e.gy = pk * p.y * it1[1];
-                e.gz = pk * l * it0[1];
-                e = finish<T, MODE, NORM>(p, e);
-                const unsigned k = static_cast<unsigned>(l * (l + 1));
-                O* out_v = rows_v + s * ny + k;
-                O* out_g = rows_g + s * 3 * ny + k;
-                out_v[0] = static_cast<O>(e.v);
-                out_g[0] = static_cast<O>(e.gx);
-                out_g[ny] = static_cast<O>(e.gy);
-                out_g[2 * ny] = static_cast<O>(e.gz);
-                asm volatile("" ::"v"(it1[0])); // see pair_entries
+                const T pk = F0[l];
+                if constexpr (MODE == 1) {
+                    const P2 it0 = *reinterpret_cast<const P2*>(it);      // Q_l^0 and the Q_{l-1} sequence at 0
+                    const P2 it1 = *reinterpret_cast<const P2*>(it + IT); // ... at 1
+                    Entry<T> e;
+                    e.hxx = e.hxy = e.hxz = e.hyy = e.hyz = e.hzz = static_cast<T>(0.0);
+                    e.v = it0[0] * pk;
+                    e.gx = pk * p.x * it1[1];
+                    e.gy = pk * p.y * it1[1];
+                    e.gz = pk * l * it0[1];
+                    e = finish<T, MODE, NORM>(p, e);
+                    const unsigned k = static_cast<unsigned>(l * (l + 1));
+                    O* out_v = row_lds + ph.sph + s * ny + k;
+                    O* out_g = row_lds + g.off_dsph + ph.dsph + s * 3 * ny + k;
+                    out_v[0] = static_cast<O>(e.v);
+                    out_g[0] = static_cast<O>(e.gx);
+                    out_g[ny] = static_cast<O>(e.gy);
+                    out_g[2 * ny] = static_cast<O>(e.gz);
+                    asm volatile("" ::"v"(it1[0])); // see pair_entries
+                } else {
+                    const V4 q0 = *reinterpret_cast<const V4*>(it);
+                    const V4 q1 = *reinterpret_cast<const V4*>(it + IT);
+                    const V4 q2 = *reinterpret_cast<const V4*>(it + 2 * IT);
+                    EntryWindow<T> in;
+                    in.pk_ = pk;
+                    in.c_[0] = in.c_[1] = in.c_[2] = in.s_[0] = in.s_[1] = in.s_[2] = 0; // m = 0 uses neither
+                    in.A_[0] = q0[0];
+                    in.A_[1] = q1[0];
+                    in.B_[0] = q0[1];
+                    in.B_[1] = q1[1];
+                    in.C_[0] = q0[2];
+                    in.C_[1] = q1[2];
+                    in.C_[2] = q2[2];
+                    entry_job_from<T, MODE, NORM, false>(l, 0, l * (l + 1) / 2, 0, p, in, staged_rows(ph, s));
+                }
             }
         };
 
@@ -305,10 +367,12 @@ __global__ __launch_bounds__(kPairsThreads, 1) void pairs_kernel(PairsTiling g, 
             SPHX_MARK(c_wait_a);
             {
                 const Phases ph = phases_of(n);
-                O* rows_v = row_lds + ph.sph;
-                O* rows_g = row_lds + g.off_dsph + ph.dsph;
-                unpark_stage(n, valid, rows_v, rows_g);
-                axial_stage(n, valid, rows_v, rows_g);
+                if constexpr (MODE == 1) {
+                    unpark_stage(n, valid, row_lds + ph.sph, row_lds + g.off_dsph + ph.dsph);
+                } else {
+                    low_stage(n, valid, ph);
+                }
+                axial_stage(n, valid, ph);
             }
             SPHX_MARK(c_work);
             __syncthreads(); // rows of tile n complete
@@ -329,36 +393,49 @@ __global__ __launch_bounds__(kPairsThreads, 1) void pairs_kernel(PairsTiling g, 
         // Same operations in the same order as sequence_job (sphx_device.hpp).
         const unsigned seq_tid = tid - 64u * P;
         const unsigned seq_lanes = 64u * NSEQ;
-        const unsigned seq_jobs = 2u * S * levels;
-        // job j: l from l_max down, the points of a tile and their two sequences side by side
+        const unsigned seq_jobs = SEQS * S * levels;
+        // job j: l from l_max down, the points of a tile and their sequences side by side
         auto run_chain = [&](unsigned n, unsigned j, unsigned valid) {
-            const unsigned per_l = 2u * S;
+            const unsigned per_l = SEQS * S;
             const unsigned step = j / per_l;
             const unsigned rest = j - step * per_l;
-            const unsigned s = rest >> 1, which = rest & 1u;
+            const unsigned s = rest / SEQS, which = rest - s * SEQS;
             if (s >= valid) return;
             const int l = L - static_cast<int>(step);
             const T* rec = record(n, s);
             const T z = rec[2];
             const T rxy = rec[4];
-            // row l for Q_l^m, row l - 1 for the Q_{l-1} sequence
+            // row l for Q_l^m, row l - 1 for the Q_{l-1} sequence, row l - 2 for the Q_{l-2} sequence
             const T* row = Qt + (static_cast<unsigned>(l) - which) * QS;
-            int base = (l - 2) & ~3; // the block of four that holds step l - 2
-            const T* pt = rec + g.tmz_at + base;
-            const T* pk = row + base;
-            T* po = iterates(s) + IT * (l * (l + 1) / 2) + which + IT * base;
-            V4 tz = *reinterpret_cast<const V4*>(pt);
-            V4 km = *reinterpret_cast<const V4*>(pk);
+            T* out = iterates(s) + IT * (l * (l + 1) / 2) + which;
+            // start values (templates_core.hpp:122-123, 135, 150, 155, 167, 196 and :228-231) and the first step
             T v1, v2;
+            int top = l - 2;
             if (which == 0) {
                 v2 = row[l];
                 v1 = -z * v2;
-            } else {
+                out[l * IT] = v2;
+                out[(l - 1) * IT] = v1;
+            } else if (which == 1) {
                 v2 = 0;
                 v1 = row[l - 1];
+                out[l * IT] = v2;
+                out[(l - 1) * IT] = v1;
+            } else {
+                v2 = 0;
+                v1 = row[l - 2];
+                out[l * IT] = v2;
+                out[(l - 1) * IT] = v2;
+                out[(l - 2) * IT] = v1;
+                top = l - 3;
             }
-            po[(l - base) * IT] = v2;
-            po[(l - 1 - base) * IT] = v1;
+            if (top < 0) return;
+            int base = top & ~3; // the block of four that holds the first step
+            const T* pt = rec + g.tmz_at + base;
+            const T* pk = row + base;
+            T* po = out + IT * base;
+            V4 tz = *reinterpret_cast<const V4*>(pt);
+            V4 km = *reinterpret_cast<const V4*>(pk);
             // (below m = 0 the reads fetch, unused, what precedes the tables: the pairs of the record,
             // the end of the row before)
             V4 tz_next = *reinterpret_cast<const V4*>(pt - 4);
@@ -370,7 +447,7 @@ __global__ __launch_bounds__(kPairsThreads, 1) void pairs_kernel(PairsTiling g, 
         v2 = v1;                                                \
         v1 = v0;                                                \
     } while (0)
-            switch ((l - 2) & 3) {
+            switch (top & 3) {
             case 3: SPHX_STEP(tz, km, 3); [[fallthrough]];
             case 2: SPHX_STEP(tz, km, 2); [[fallthrough]];
             case 1: SPHX_STEP(tz, km, 1); [[fallthrough]];
@@ -425,13 +502,16 @@ __global__ __launch_bounds__(kPairsThreads, 1) void pairs_kernel(PairsTiling g, 
         }
     } else {
         // ================================== entry waves ===================================
+        // MODE 1: the waves of a slot share a point, which is then the same for a whole wave (its addresses are
+        // scalars). MODE 2: the table deals the lanes to the points lane by lane.
         const unsigned ew = wave - entry_first;
-        const unsigned slot = ew / g.slot_waves;
-        const unsigned slots = g.entry_waves / g.slot_waves;
-        const unsigned job = g.lane_job[(ew - slot * g.slot_waves) * 64u + lane];
+        const unsigned wave_slot = MODE == 1 ? ew / g.slot_waves : 0u;
+        const unsigned job = g.lane_job[(ew - wave_slot * g.slot_waves) * 64u + lane];
         const bool has_job = job != kPairsNoJob;
-        const int e_l = has_job ? static_cast<int>(job >> 8) : H + 1;
-        const int e_m = has_job ? static_cast<int>(job & 0xffu) : 1;
+        const unsigned slot = MODE == 1 ? wave_slot : (has_job ? job >> 14 : 0u);
+        const unsigned slots = MODE == 1 ? g.entry_waves / g.slot_waves : g.lane_slots;
+        const int e_l = has_job ? static_cast<int>((job >> 7) & 127u) : H + 1;
+        const int e_m = has_job ? static_cast<int>(job & 127u) : 1;
         const bool no_pdq = e_m >= e_l - 1; // |m| = l and l - 1: no Q_{l-1}^{m+1} term in d/dx, d/dy
         const bool no_dz = e_m == e_l;      // |m| = l: no d/dz
         const int e_tri = e_l * (e_l + 1) / 2;
@@ -514,6 +594,46 @@ __global__ __launch_bounds__(kPairsThreads, 1) void pairs_kernel(PairsTiling g, 
             const unsigned valid = valid_in(n);
             if (slot >= valid || !has_job) return;
             const Phases ph = phases_of(n);
+            if constexpr (MODE == 2) {
+                // entry_job's own arithmetic on what the lane reads of the point: the iterates at m, m + 1, m + 2
+                // and (c, s) at m - 2, m - 1, m
+                for (unsigned s = slot; s < valid; s += slots) {
+                    const T* rec = record(n, s);
+                    const T* it = iterates(s) + o_it;
+                    const T* cs = rec + 8u + 2u * static_cast<unsigned>(e_m);
+                    const P2 xy = *reinterpret_cast<const P2*>(rec);
+                    const P2 zi = *reinterpret_cast<const P2*>(rec + 2);
+                    const V4 q0 = *reinterpret_cast<const V4*>(it);
+                    const V4 q1 = *reinterpret_cast<const V4*>(it + IT);
+                    const V4 q2 = *reinterpret_cast<const V4*>(it + 2 * IT);
+                    const P2 p0 = *reinterpret_cast<const P2*>(cs);
+                    const P2 p1 = *reinterpret_cast<const P2*>(cs - 2);
+                    const P2 p2 = *reinterpret_cast<const P2*>(cs - 4); // (for m = 1: two spare numbers, not used)
+                    Point<T> p;
+                    p.x = xy[0];
+                    p.y = xy[1];
+                    p.z = zi[0];
+                    p.ir = zi[1];
+                    p.x2 = p.y2 = p.z2 = 0;
+                    EntryWindow<T> in;
+                    in.pk_ = pkm;
+                    in.c_[0] = p2[0];
+                    in.c_[1] = p1[0];
+                    in.c_[2] = p0[0];
+                    in.s_[0] = p2[1];
+                    in.s_[1] = p1[1];
+                    in.s_[2] = p0[1];
+                    in.A_[0] = q0[0];
+                    in.A_[1] = q1[0];
+                    in.B_[0] = q0[1];
+                    in.B_[1] = q1[1];
+                    in.C_[0] = q0[2];
+                    in.C_[1] = q1[2];
+                    in.C_[2] = q2[2];
+                    entry_job_from<T, MODE, NORM, false>(e_l, e_m, e_tri, 0, p, in, staged_rows(ph, s));
+                }
+                return;
+            }
             O* rows_v = row_lds + ph.sph;
             O* rows_g = row_lds + g.off_dsph + ph.dsph;
             unsigned s = slot; // the same for the whole wave: the point's addresses are scalars
@@ -596,6 +716,7 @@ __global__ __launch_bounds__(kPairsThreads, 1) void pairs_kernel(PairsTiling g, 
             };
             flush_run(0, sph, first * ny, valid * ny);
             flush_run(g.off_dsph, dsph, first * 3 * ny, valid * 3 * ny);
+            if constexpr (MODE == 2) flush_run(g.off_ddsph, ddsph, first * 9 * ny, valid * 9 * ny);
         };
 
         __syncthreads();

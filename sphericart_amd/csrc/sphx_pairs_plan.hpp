@@ -21,27 +21,75 @@ struct PairsLaunch {
     unsigned lds_bytes = 0, threads = 0, workgroups = 0;
 };
 
-// The lane table: the pairs (l, m >= 1) of one point in a row, l and m descending, over as few waves as
-// hold them. (A table that kept the lanes of a half-wave on different LDS banks, at the price of one more
-// wave, measured 1-3 % slower: the stage is bound by instruction issue, not by LDS.) Returns the number
-// of waves, 0 if `waves` do not hold the pairs.
+// The lane table of values and gradients: the pairs (l, m >= 1) of one point in a row, l and m descending,
+// over as few waves as hold them; the waves of one such group share a point. (A table that kept the lanes of a
+// half-wave on different LDS banks, at the price of one more wave, measured 1-3 % slower: the stage is
+// bound by instruction issue, not by LDS.) Returns the number of waves, 0 if `waves` do not hold the pairs.
+inline unsigned short pairs_job(unsigned slot, int l, int m) {
+    return static_cast<unsigned short>((slot << 14) | (static_cast<unsigned>(l) << 7) | static_cast<unsigned>(m));
+}
 inline unsigned pairs_lane_table(int l_max, int hard, unsigned waves, unsigned short* table) {
     for (unsigned i = 0; i < kPairsThreads; ++i) table[i] = static_cast<unsigned short>(kPairsNoJob);
     if (waves > kPairsThreads / 64u) waves = kPairsThreads / 64u;
     unsigned at = 0;
     for (int l = l_max; l > hard; --l) {
         if (at + static_cast<unsigned>(l) > waves * 64u) return 0;
-        for (int m = l; m >= 1; --m) table[at++] = static_cast<unsigned short>((l << 8) | m);
+        for (int m = l; m >= 1; --m) table[at++] = pairs_job(0, l, m);
     }
     return (at + 63u) / 64u;
 }
 
+// The lane table with second derivatives. The entries with |m| = l, |m| = l - 1 and 1 <= |m| <= l - 2 are three
+// different pieces of code, and a wave runs every piece that one of its lanes needs: the table is ordered by
+// kind (the bulk of all points side by side, then |m| = l, then |m| = l - 1), the bulk filled up to a whole
+// wave where the lanes allow. As many points side by side (four at most) as `waves` waves hold. Returns that
+// number, 0 if not even one point fits.
+inline unsigned pairs_lane_table_by_kind(int l_max, int hard, unsigned waves, unsigned most_slots,
+                                         unsigned short* table) {
+    for (unsigned i = 0; i < kPairsThreads; ++i) table[i] = static_cast<unsigned short>(kPairsNoJob);
+    if (waves > kPairsThreads / 64u) waves = kPairsThreads / 64u;
+    const unsigned lanes = waves * 64u;
+    unsigned bulk = 0, levels = 0;
+    for (int l = hard + 1; l <= l_max; ++l) {
+        bulk += l >= 2 ? static_cast<unsigned>(l - 2) : 0u;
+        ++levels;
+    }
+    if (most_slots > 4u) most_slots = 4u;
+    for (unsigned slots = most_slots; slots >= 1u; --slots) {
+        if (slots * (bulk + 2u * levels) > lanes) continue;
+        unsigned at = 0;
+        for (unsigned s = 0; s < slots; ++s) {
+            for (int l = l_max; l > hard; --l) {
+                for (int m = l - 2; m >= 1; --m) table[at++] = pairs_job(s, l, m);
+            }
+        }
+        const unsigned padded = (at + 63u) & ~63u;
+        if (padded + slots * 2u * levels <= lanes) at = padded; // the other kinds start a wave of their own
+        for (unsigned s = 0; s < slots; ++s) {
+            for (int l = l_max; l > hard; --l) table[at++] = pairs_job(s, l, l);
+        }
+        for (unsigned s = 0; s < slots; ++s) {
+            for (int l = l_max; l > hard; --l) {
+                if (l >= 2) table[at++] = pairs_job(s, l, l - 1);
+            }
+        }
+        return slots;
+    }
+    return 0;
+}
+
 // false: this shape is not for pairs_kernel (the pairs of a point do not fit the waves, or the rows of
 // a tile and the tables do not fit LDS).
-inline bool plan_pairs(size_t n_samples, int l_max, size_t elem, size_t out_elem, int lds_limit, int cus,
+// `mode`: 1 values and gradients, 2 second derivatives too (in float64 in workgroups of 512 threads: the
+// entries need more than the 128 registers that sixteen waves leave a lane).
+inline bool plan_pairs(size_t n_samples, int l_max, int mode, size_t elem, size_t out_elem, int lds_limit, int cus,
                        const PairsChoice& want, PairsLaunch* out) {
-    constexpr int H = 6;
-    constexpr unsigned NYH = 49, COMP = 4, IT = 2, ITEMS = 9, WAVES = kPairsThreads / 64u;
+    if (mode != 1 && mode != 2) return false;
+    const int H = mode == 2 ? 1 : 6;
+    const unsigned NYH = static_cast<unsigned>((H + 1) * (H + 1));
+    const unsigned COMP = mode == 2 ? 13u : 4u, SEQS = static_cast<unsigned>(mode) + 1u, IT = mode == 2 ? 4u : 2u;
+    const unsigned ITEMS = mode == 2 ? 1u : 9u;
+    const unsigned WAVES = (mode == 2 && elem == 8 ? 512u : kPairsThreads) / 64u;
     if (l_max <= H || l_max > 64 || n_samples == 0) return false;
     PairsTiling& g = out->g;
     std::memset(&g, 0, sizeof(g));
@@ -60,10 +108,11 @@ inline bool plan_pairs(size_t n_samples, int l_max, size_t elem, size_t out_elem
     const unsigned q_stride = align4(L + 1);
     const unsigned q_elems = (L + 1) * q_stride;
     const unsigned f0_elems = align4(L + 1);
-    const unsigned park_stride = COMP * NYH + 1u; // odd: the lanes of a prep wave, one point each, spread over the banks
-    const unsigned iter_stride = align4(IT * tri_all + IT); // one group past the end is read, never used
+    // (with second derivatives nothing is parked)
+    const unsigned park_stride = mode == 2 ? 0u : COMP * NYH + 1u; // odd: the lanes of a prep wave, one point each, spread over the banks
+    const unsigned iter_stride = align4(IT * tri_all + 2u * IT); // up to two groups past the end are read, never used
     auto bytes_for = [&](unsigned S, unsigned tpb) {
-        const unsigned rows = align4(S * ny + line) + align4(S * 3 * ny + line);
+        const unsigned rows = align4(S * ny + line) + align4(S * 3 * ny + line) + (mode == 2 ? align4(S * 9 * ny + line) : 0u);
         const unsigned tables = q_elems + f0_elems + 2 * tpb * S * (point_stride + park_stride) + 4u + S * iter_stride;
         return rows * osize + tables * esize;
     };
@@ -74,25 +123,37 @@ inline bool plan_pairs(size_t n_samples, int l_max, size_t elem, size_t out_elem
     if (S > 16) S = 16;
     while (S > 1 && bytes_for(S, 3) > static_cast<unsigned>(lds_limit)) --S;
     // batches: as many tiles as a wave has lanes for and LDS holds; at least three, so that the nine work
-    // items of a batch fit its tile rounds with the prep waves there are
-    unsigned tpb = want.batch_tiles ? want.batch_tiles : 64u / S;
+    // items of a batch fit its tile rounds with the prep waves there are (with second derivatives a batch is
+    // only the records, and eight points are enough to share their chain of dependent operations)
+    unsigned tpb = want.batch_tiles ? want.batch_tiles : (mode == 2 ? (8u + S - 1u) / S : 64u / S);
+    if (tpb < 3) tpb = 3;
     if (tpb * S > 64u) tpb = 64u / S;
     while (tpb > 3 && bytes_for(S, tpb) > static_cast<unsigned>(lds_limit)) --tpb;
     if (tpb < 3 || bytes_for(S, tpb) > static_cast<unsigned>(lds_limit)) return false;
     unsigned P = want.prep_waves ? want.prep_waves : (ITEMS + tpb - 1u) / tpb;
     if (P * tpb < ITEMS) P = (ITEMS + tpb - 1u) / tpb;
     // one recursion per lane and tile where four waves suffice for that
-    unsigned NSEQ = want.sequence_waves ? want.sequence_waves : (S * 2u * levels + 63u) / 64u;
+    unsigned NSEQ = want.sequence_waves ? want.sequence_waves : (S * SEQS * levels + 63u) / 64u;
     if (NSEQ < 1) NSEQ = 1;
-    if (NSEQ > 4) NSEQ = 4;
+    if (NSEQ > WAVES / 4u) NSEQ = WAVES / 4u;
     if (P + NSEQ >= WAVES) return false;
     const unsigned room = WAVES - P - NSEQ;
     // the waves that hold a point's pairs, and as many points side by side as the entry waves allow
-    const unsigned slot_waves = pairs_lane_table(l_max, H, room, g.lane_job);
-    if (slot_waves == 0) return false;
-    unsigned slots = room / slot_waves;
-    if (slots > S) slots = S;
-    const unsigned E = slots * slot_waves;
+    unsigned slot_waves = 0, lane_slots = 0, E = 0;
+    if (mode == 1) {
+        slot_waves = pairs_lane_table(l_max, H, room, g.lane_job);
+        if (slot_waves == 0) return false;
+        unsigned slots = room / slot_waves;
+        if (slots > S) slots = S;
+        E = slots * slot_waves;
+    } else {
+        lane_slots = pairs_lane_table_by_kind(l_max, H, room, S, g.lane_job);
+        if (lane_slots == 0) return false;
+        for (unsigned i = 0; i < room * 64u; ++i) {
+            if (g.lane_job[i] != kPairsNoJob) E = i / 64u + 1u;
+        }
+        slot_waves = E;
+    }
 
     g.n_samples = n_samples;
     g.l_max = l_max;
@@ -104,9 +165,12 @@ inline bool plan_pairs(size_t n_samples, int l_max, size_t elem, size_t out_elem
     g.sequence_waves = NSEQ;
     g.entry_waves = E;
     g.slot_waves = slot_waves;
+    g.lane_slots = lane_slots;
     unsigned at = align4(S * ny + line);
     g.off_dsph = at;
     at = align4(at + S * 3 * ny + line);
+    g.off_ddsph = at;
+    if (mode == 2) at = align4(at + S * 9 * ny + line);
     g.tables_at = at * osize;
     at = 0;
     g.off_Q = at;

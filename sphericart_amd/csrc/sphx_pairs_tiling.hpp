@@ -19,14 +19,16 @@ struct PairsTiling {
     unsigned batch_tiles;    // tiles per batch of point records and parked closed forms
     unsigned magic_batch;    // ceil(2^32 / batch_tiles)
     unsigned prep_waves, sequence_waves, entry_waves;
-    unsigned slot_waves;     // entry waves that share one point; entry_waves / slot_waves points side by side
-    unsigned off_dsph;       // staged gradient rows, in elements of the output type
+    unsigned slot_waves;     // MODE 1: entry waves that share one point; entry_waves / slot_waves points side by side
+    unsigned lane_slots;     // MODE 2: points side by side in the entry lanes (the lane table says which lane takes which)
+    unsigned off_dsph, off_ddsph; // staged gradient and second-derivative rows, in elements of the output type
     unsigned tables_at;      // bytes: where the part of LDS in the arithmetic type starts
     unsigned off_Q, off_F0, off_pts, off_park, off_iter; // in numbers of the arithmetic type, from tables_at
     unsigned point_stride, park_stride, iter_stride;
     unsigned tmz_at;         // where 2(m+1)z starts in a point's record (a multiple of four numbers)
     unsigned q_stride;       // distance between the rows of the Q constants in LDS (a multiple of four)
-    // the pair (l << 8 | m) of every lane of the slot_waves waves that share a point
+    // the pair of every entry lane, slot << 14 | l << 7 | m (MODE 1: of the slot_waves waves that share a
+    // point, slot 0)
     unsigned short lane_job[kPairsThreads];
 };
 

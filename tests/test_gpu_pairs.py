@@ -1,8 +1,8 @@
-"""pairs_kernel (values and gradients, every entry lane bound to one (l, m) pair) against the oracle,
-number for number.
+"""pairs_kernel (derivatives, every entry lane bound to one (l, m) pair) against the oracle, number for number.
 
-The planner gives it float32 from l_max = 20 and float64 from l_max = 16 when a call has 32 768 points or
-more; here SPHX_PAIRS = 2 sends every shape it can hold through it, with the tile, batch and wave counts
+The planner gives it gradients in float32 from l_max = 20 and in float64 from l_max = 16, and second derivatives
+in float64 from l_max = 20, when a call has 32 768 points or more; here SPHX_PAIRS = 2 sends every shape it can
+hold through it, with the tile, batch and wave counts
 the planner would pick and with forced ones, so that every path of the kernel runs at sizes the oracle
 finishes in seconds: partial last tiles, fewer tiles than workgroups, several points side by side in the
 entry waves, several rounds of recursions per tile, outputs that start anywhere inside a 128-byte line.
@@ -20,28 +20,29 @@ from helpers import same_numbers, special_points
 pytestmark = pytest.mark.gpu
 
 
-def _evaluate(library, xyz, l_max, normalized, shift=0):
-    """sphx_forward_* with gradients into buffers with NaN guard bands; returns (sph, dsph, guards intact)."""
+def _evaluate(library, xyz, l_max, normalized, shift=0, mode=1):
+    """sphx_forward_* with derivatives into buffers with NaN guard bands; returns (sph, dsph[, ddsph], guards intact)."""
     n = xyz.shape[0]
     ny = (l_max + 1) ** 2
     tdtype = torch.float32 if xyz.dtype == np.float32 else torch.float64
-    sizes = (n * ny, 3 * n * ny)
+    sizes = (n * ny, 3 * n * ny, 9 * n * ny)[:mode + 1]
+    shapes = ((n, ny), (n, 3, ny), (n, 3, 3, ny))
     raw = [torch.full((size + 64,), float("nan"), dtype=tdtype, device="cuda") for size in sizes]
-    out = [raw[0][shift:shift + sizes[0]].view(n, ny), raw[1][shift:shift + sizes[1]].view(n, 3, ny)]
+    out = [raw[i][shift:shift + sizes[i]].view(shapes[i]) for i in range(mode + 1)]
     forward = library.sphx_forward_f32 if xyz.dtype == np.float32 else library.sphx_forward_f64
     xyz_dev = torch.from_numpy(xyz).cuda()
-    status = forward(xyz_dev.data_ptr(), n, l_max, int(normalized), 1, out[0].data_ptr(), out[1].data_ptr(), None,
-                     torch.cuda.current_stream().cuda_stream)
+    status = forward(xyz_dev.data_ptr(), n, l_max, int(normalized), mode, out[0].data_ptr(), out[1].data_ptr(),
+                     out[2].data_ptr() if mode == 2 else None, torch.cuda.current_stream().cuda_stream)
     assert status == 0, library.sphx_last_error()
     torch.cuda.synchronize()
     guards = all(bool(torch.isnan(raw[i][:shift]).all() and torch.isnan(raw[i][shift + sizes[i]:]).all())
-                 for i in range(2))
-    return out[0].cpu().numpy(), out[1].cpu().numpy(), guards
+                 for i in range(mode + 1))
+    return tuple(o.cpu().numpy() for o in out) + (guards,)
 
 
-def _plan_text(library, n, l_max, f64, normalized):
+def _plan_text(library, n, l_max, f64, normalized, mode=1):
     text = ctypes.create_string_buffer(512)
-    assert library.sphx_describe_plan(n, l_max, 1, int(f64), int(normalized), text, 512) == 0
+    assert library.sphx_describe_plan(n, l_max, mode, int(f64), int(normalized), text, 512) == 0
     return text.value.decode()
 
 
@@ -119,15 +120,49 @@ def test_few_points_and_shifted_outputs(oracle, library, switches):
             assert guards, (l_max, n)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("normalized", [True, False])
+def test_second_derivatives(oracle, library, switches, dtype, normalized):
+    """The same kernel with second derivatives (closed forms only to l = 1, three recursions per l, thirteen rows
+    per point, the lane table ordered by kind): l_max 2 .. 24, planned and forced tiles."""
+    rng = np.random.default_rng(17)
+    ran = 0
+    for l_max, overrides in ((2, {}), (3, {"SPHX_PAIRS_TILE": 1}), (4, {}), (5, {"SPHX_PAIRS_TILE": 7}), (8, {}),
+                             (9, {"SPHX_PAIRS_SEQUENCE_WAVES": 1, "SPHX_PAIRS_TILE": 5}), (12, {}),
+                             (16, {"SPHX_PAIRS_TILE": 2, "SPHX_PAIRS_CHUNK": 0}), (16, {}), (20, {}),
+                             (24, {"SPHX_PAIRS_BATCH": 9})):
+        library.sphx_reset_switches()
+        switches("SPHX_PAIRS", 2)
+        switches("SPHX_HESSIAN_LANES", 0)
+        for name, value in overrides.items():
+            switches(name, value)
+        n = 301 if l_max <= 12 else 83
+        text = _plan_text(library, n, l_max, dtype == np.float64, normalized, mode=2)
+        announce("pairs second derivatives", np.dtype(dtype).name, "normalized", normalized, "l_max", l_max, overrides,
+                 "n", n, text)
+        if not text.startswith("pairs_kernel"):
+            continue
+        ran += 1
+        xyz = special_points(dtype, rng, n)
+        want = oracle.compute(xyz, l_max, normalized, "hessians")
+        sph, dsph, ddsph, guards = _evaluate(library, xyz, l_max, normalized, shift=int(rng.integers(0, 17)), mode=2)
+        assert same_numbers(sph, want[0]).all(), (l_max, "values")
+        assert same_numbers(dsph, want[1]).all(), (l_max, "gradients")
+        assert same_numbers(ddsph, want[2]).all(), (l_max, "second derivatives")
+        assert guards
+    assert ran >= 8
+
+
 def test_planned_by_shape(library):
     """What the planner picks without overrides."""
-    assert _plan_text(library, 200_000, 32, False, True).startswith("pairs_kernel<float, true>")
-    assert _plan_text(library, 100_000, 20, False, False).startswith("pairs_kernel<float, false>")
-    assert _plan_text(library, 100_000, 16, True, True).startswith("pairs_kernel<double, true>")
+    assert _plan_text(library, 200_000, 32, False, True).startswith("pairs_kernel<float, 1, true>")
+    assert _plan_text(library, 100_000, 20, False, False).startswith("pairs_kernel<float, 1, false>")
+    assert _plan_text(library, 100_000, 16, True, True).startswith("pairs_kernel<double, 1, true>")
+    assert _plan_text(library, 50_000, 20, True, True, mode=2).startswith("pairs_kernel<double, 2, true>")
+    assert _plan_text(library, 100_000, 16, True, False, mode=2).startswith("recursion_kernel")  # cfg4
     assert _plan_text(library, 100_000, 19, False, True).startswith("recursion_kernel")
     assert _plan_text(library, 100_000, 15, True, True).startswith("recursion_kernel")
     assert _plan_text(library, 20_000, 32, False, True).startswith("recursion_kernel")  # few points
-    # second derivatives and values alone stay where they were
-    text = ctypes.create_string_buffer(512)
-    assert library.sphx_describe_plan(200_000, 32, 0, 0, 1, text, 512) == 0 and not text.value.startswith(b"pairs")
-    assert library.sphx_describe_plan(200_000, 24, 2, 0, 1, text, 512) == 0 and not text.value.startswith(b"pairs")
+    # second derivatives in float32 and values alone stay where they were
+    assert not _plan_text(library, 200_000, 32, False, True, mode=0).startswith("pairs")
+    assert not _plan_text(library, 200_000, 24, False, True, mode=2).startswith("pairs")
