@@ -602,11 +602,20 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
 // 377, 376, float64 l_max = 24, 28, 32 317, 322, 335 against 292, 305, 297. With few points
 // (below 4 096) 512 threads stay: more workgroups have a tile then.
 // SPHX_GROUP_THREADS = 512 or 1024 overrides the rule.
-static unsigned group_threads(size_t n_samples, int mode, size_t elem, bool forward) {
-    const bool exists = forward && (mode <= 1 || (mode == 2 && elem == 4));
+static unsigned group_threads(size_t n_samples, int mode, size_t elem, bool forward, bool normalized = true,
+                              int l_max = -1) {
+    // Second derivatives in float64: the entries (l, +m) and (l, -m) as one job need 169-237 registers per lane.
+    // As two jobs, solid harmonics need 121, which sixteen waves allow (normalised 181: those keep eight waves).
+    // 1.2 GB of output, us, 512 threads against 1024 with the two sides as two jobs in one list: l_max = 4, 5, 6, 8,
+    // 10, 12, 14, 16, 18, 20, 22 251, 244, 247, 259, 253, 216, 225, 227, 220, 226, 231 against 201, 204, 205, 204,
+    // 208, 211, 205, 215, 206, 221, 216; cfg4 538 against 507; l_max = 3 305 against 243. At l_max = 2 the list is
+    // three jobs a point: 219 against 227.
+    const bool solid_f64_hessians = mode == 2 && elem == 8 && !normalized;
+    const bool exists = forward && (mode <= 1 || (mode == 2 && elem == 4) || solid_f64_hessians);
     if (!exists) return kRecursionThreads;
     const int want = switch_or(SW_GROUP_THREADS, 0);
     if (want == 512 || want == 1024) return static_cast<unsigned>(want);
+    if (solid_f64_hessians && l_max < 3) return kRecursionThreads;
     return n_samples >= 4096 ? 2 * kRecursionThreads : kRecursionThreads;
 }
 
@@ -765,6 +774,8 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         // 121 -> 104, 100, 96, 113; solid l_max = 6, 12 94, 92 -> 83, 83; with one point per tile
         // splitting stays, l_max = 24, 28 117, 104 against 184, 166)
         *split = may_split && S < 2 && one_side_costs * rounds(jobs_split) < 10 * rounds(jobs);
+        // (float64 in workgroups of 1024 threads: only the one-sided job fits a lane's 128 registers)
+        if (may_split && mode == 2 && elem == 8 && threads > kRecursionThreads) *split = true;
         return *split ? one_side_costs * rounds(jobs_split) : 10 * rounds(jobs);
     };
     // A second sequence wave takes a wave from the entries. One is enough where it saves the
@@ -855,7 +866,8 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     const bool by_shape = mode == 0   ? (threads > kRecursionThreads ? S >= 2 : saves_a_round && S >= 3 && g.points_per_pass <= 2)
                           : mode == 1 ? S >= 3 || (saves_a_round && S >= 2)
                                       : (S >= 3 && !(cheap_jobs && fill >= 90u)) || (S == 2 && !*split_sides) ||
-                                            (saves_a_round && S >= 2);
+                                            (saves_a_round && S >= 2) ||
+                                            (cheap_jobs && threads > kRecursionThreads && S >= 2);
     if (want_list == 2 || (want_list == 1 && saves_a_round) || (want_list < 0 && by_shape)) {
         g.points_per_pass = 0;
     }
@@ -1018,7 +1030,8 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // l_max = 3 104, 108 (solid 89, 100), l_max = 4 147, 107 (solid 113, 87), l_max = 5 130, 112
     // (solid 99, 86); float64 l_max = 3 129, 114 (solid 91, 102), l_max = 5 163, 107; 20 000 points
     // float32 l_max = 3 9.0, 11.2, l_max = 4 17.9, 13.5.)
-    const bool hessian_lanes_pay = elem == 4 ? l_max <= 3 : (l_max == 3 && !normalized);
+    // (Solid harmonics in float64, l_max = 3, 1.2 GB of output: 259 us against 243 in workgroups of 1024 threads.)
+    const bool hessian_lanes_pay = elem == 4 ? l_max <= 3 : (l_max == 3 && !normalized && n_samples < 32768);
     if (lane_kernels && mode == 2 && (hessian_lanes == 2 || (hessian_lanes == 1 && hessian_lanes_pay)) &&
         plan_hessian_lanes(n_samples, l_max, elem, lds_limit, &plan->closed, normalized)) {
         plan->lanes = true;
@@ -1074,7 +1087,7 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     // the tile takes all of it (1.5 GB of output, l_max = 6: 694 -> 473 us, l_max = 10: 582 ->
     // 479, l_max = 12: 545 -> 468; solid harmonics l_max = 4-12: 10-20 % less, l_max = 16, 100k
     // points: 580 -> 560).
-    const unsigned threads = group_threads(n_samples, mode, elem, lane_kernels);
+    const unsigned threads = group_threads(n_samples, mode, elem, lane_kernels, normalized, l_max);
     const int whole_cu = (mode == 2 && elem == 8) || threads > kRecursionThreads ? lds_limit : 80 * 1024;
     const unsigned budget = static_cast<unsigned>(switch_or(SW_TILE_LDS_BUDGET, whole_cu));
     bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
@@ -1201,8 +1214,8 @@ template <typename X> struct AsGiven {
 
 // Workgroups of 1024 threads (one per CU, all of its LDS) exist for all but second derivatives
 // in float64, which need more registers than sixteen waves leave a lane, and the fused product.
-template <typename T, int MODE, bool VJP>
-constexpr bool kLargeGroups = !VJP && (MODE <= 1 || (MODE == 2 && sizeof(T) == 4));
+template <typename T, int MODE, bool VJP, bool NORM = true, bool SPLIT = false>
+constexpr bool kLargeGroups = !VJP && (MODE <= 1 || (MODE == 2 && sizeof(T) == 4) || (MODE == 2 && !NORM && SPLIT));
 
 template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false,
           typename O = T, unsigned NT = kRecursionThreads>
@@ -1215,7 +1228,7 @@ static hipError_t launch_recursion(const Launch& l, const typename AsGiven<O>::t
             return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, false, true, O, NT>(l, xyz, sph, dsph, ddsph, stream);
         }
     }
-    if constexpr (NT == kRecursionThreads && kLargeGroups<T, MODE, VJP>) {
+    if constexpr (NT == kRecursionThreads && kLargeGroups<T, MODE, VJP, NORM, SPLIT>) {
         if (l.threads == 2 * kRecursionThreads) {
             return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O, 2 * kRecursionThreads>(
                 l, xyz, sph, dsph, ddsph, stream);

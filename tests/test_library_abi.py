@@ -89,8 +89,14 @@ def test_launch_plans(library):
     assert status == 0 and (tile, threads, groups) == (5, 960, 256) and 140_000 < lds <= 160 * 1024
     status, (tile, threads, lds, groups) = _plan(library, 2_000, 32, 1, False)
     assert status == 0 and threads == 512 and lds <= 80 * 1024
-    # second derivatives in float64 keep 512 threads (more than 128 registers per lane)
+    # second derivatives in float64 keep 512 threads (more than 128 registers per lane); solid harmonics, whose
+    # entries (l, +m) and (l, -m) fit 128 registers as two jobs, take 1024 (cfg4)
     assert _plan(library, 100_000, 16, 2, True)[1][1] == 512
+    text = ctypes.create_string_buffer(512)
+    assert library.sphx_describe_plan(100_000, 16, 2, 1, 0, text, 512) == 0
+    assert text.value.decode().startswith("recursion_kernel<double, 2, false, true, true, false, true> [4 points per tile, 1024 threads")
+    assert library.sphx_describe_plan(100_000, 16, 2, 1, 1, text, 512) == 0
+    assert "512 threads" in text.value.decode()
     # values: as many points per workgroup as fit in half a CU's LDS, in steps of four; in float32
     # one workgroup with all of LDS while 40 points fit, then the recursion kernel
     status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 16, 0, False)
