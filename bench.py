@@ -109,7 +109,42 @@ def parse():
         help="instead of the hot path, launch plain device-to-device copies of as many bytes as "
         "the workload writes per launch: the yardstick for the FETCH_SIZE / WRITE_SIZE counters",
     )
+    p.add_argument(
+        "--sweep",
+        action="store_true",
+        help="instead of one workload, the table of achieved bandwidth over l_max x derivatives x precision x "
+        "kind of harmonics at 20 000 points, at 1.2 GB of output and at 2 000 000 points (sphericart_amd/sweep.py), "
+        "as one JSON document on stdout; progress goes to stderr",
+    )
+    p.add_argument("--sweep-sizes", default="20k,1.2GB,2M", help="with --sweep: which of the three sizes")
+    p.add_argument("--sweep-markdown", action="store_true", help="with --sweep: print the tables as Markdown instead")
     return p.parse_args()
+
+
+def sweep(lib, args):
+    import subprocess
+
+    from sphericart_amd import sweep as table
+
+    sizes = tuple(s for s in args.sweep_sizes.split(",") if s)
+
+    def progress(row):
+        print(f"{table.key_of(row):48s} {row['us']:9.1f} us {100 * row['frac']:5.1f} %  {row['kernel']}",
+              file=sys.stderr, flush=True)
+
+    rows = table.run(lib, sizes=sizes, progress=progress)
+    if args.sweep_markdown:
+        for size in sizes:
+            print(f"\n{size}\n\n{table.as_markdown(rows, size)}")
+        return 0
+    try:
+        commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True,
+                                timeout=10).stdout.strip() or None
+    except (OSError, subprocess.SubprocessError):
+        commit = None
+    print(json.dumps({"command": "python bench.py --sweep --sweep-sizes " + ",".join(sizes), "commit": commit,
+                      "peak_GBps": table.PEAK_HBM_GBPS, "rows": rows}, indent=0))
+    return 0
 
 
 def cpu_baseline(workload, xyz):
@@ -375,6 +410,8 @@ def main():
     w = WORKLOADS[args.workload]
     lib = sphericart_amd.get_library()
     torch.cuda.set_device(0)
+    if args.sweep:
+        return sweep(lib, args)
 
     prepared = Prepared(lib, w, args.rotate_mb if args.op == "forward" else 0)
     xyz_host, xyz = prepared.xyz_host, prepared.xyz

@@ -147,11 +147,14 @@ SPHX_EXPORT size_t sphx_forward_f32_via_f64_workspace(size_t n_samples, int l_ma
 
 /* sphx_forward_f32_via_f64 for callers that cannot allocate device memory: code
  * under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc. No counterpart in the reference. The float64 rows are staged in a
- * scratch array of 32 MiB that is part of the library's device code (every GPU
- * the library runs on holds its own copy until the process ends); the call
- * allocates and frees nothing and only enqueues on `stream`. The whole call
- * must fit into the scratch: more than
+ * hipMalloc. No counterpart in the reference. The call allocates and frees
+ * nothing and only enqueues on `stream`. Beyond the closed forms (l_max > 6,
+ * or > 1 with second derivatives) it is the one launch of the kernel that
+ * computes in float64 and stores float rows, as in sphx_forward_f32_via_f64:
+ * no workspace is needed and any number of points goes. Up to there the
+ * float64 rows are staged in a scratch array of 32 MiB that is part of the
+ * library's device code (every GPU the library runs on holds its own copy
+ * until the process ends), and the whole call must fit into it: more than
  * sphx_forward_f32_via_f64_static_capacity(l_max, derivatives) points
  * (32 MiB / (8 * (3 + (l_max+1)^2 * {1, 4, 13})); 0 for invalid arguments)
  * return SPHX_ERR_UNSUPPORTED with a message that names the limit; larger

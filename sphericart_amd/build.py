@@ -18,7 +18,14 @@ LIBRARY = os.path.join(HERE, "libsphericart_amd.so")
 
 OBJECTS = os.path.join(HERE, "build")
 
-SOURCES = ["sphx_kernels.hip", "sphx_pairs.hip", "sphx_backward.hip", "sphx_tables.cpp", "device_api.cpp", "capi.cpp"]
+# the translation units with the most kernels first: they take longest
+SOURCES = [
+    "sphx_forward_f64_hessians.hip", "sphx_forward_f32_hessians.hip", "sphx_wide_hessians.hip",
+    "sphx_forward_f64_gradients.hip", "sphx_forward_f32_gradients.hip", "sphx_wide_gradients.hip",
+    "sphx_forward_f64_values.hip", "sphx_forward_f32_values.hip", "sphx_wide_values.hip",
+    "sphx_vjp_f64.hip", "sphx_vjp_f32.hip", "sphx_pairs.hip", "sphx_backward.hip", "sphx_via_f64.hip",
+    "sphx_runtime.cpp", "sphx_plan.cpp", "sphx_tables.cpp", "device_api.cpp", "capi.cpp",
+]
 
 # -ffp-contract=off: one rounding per source-level operation, on device and
 #   host alike; results then match the reference CPU evaluator built the same

@@ -26,32 +26,8 @@ namespace sphx {
 // row are produced here (the recursion kernel fills in the rest), so the runs
 // are (H+1)^2 long and ny apart.
 // ---------------------------------------------------------------------------
-// Bytes of LDS one pass may use: 52 KB lets three workgroups share a CU. Measured on MI355X,
-// l_max = 6 float32 with gradients runs fastest with a single pass (50 KB).
-#ifndef SPHX_PHASE_LDS_BUDGET
-#define SPHX_PHASE_LDS_BUDGET (52 * 1024)
-#endif
-
-__host__ __device__ constexpr unsigned components_of(int mode) {
-    return mode == 0 ? 1u : (mode == 1 ? 4u : 13u);
-}
-
-// LDS elements per point in the closed-form kernel: the rows of all arrays, each array padded
-// by one element when (H+1)^2 is even so that the per-point stride is odd (lanes staging the
-// same entry of different points then hit different banks).
-__host__ __device__ constexpr unsigned closed_form_pad(int H) {
-    return ((H + 1) * (H + 1)) % 2 == 0 ? 1u : 0u;
-}
-
-__host__ __device__ constexpr unsigned closed_form_phases(unsigned elem, int mode, int H) {
-    const unsigned ny = (H + 1) * (H + 1);
-    const unsigned per_point = (components_of(mode) * ny + (mode + 1) * closed_form_pad(H)) * elem;
-    unsigned phases = 1;
-    while (phases < 16 && (64 / phases) * per_point > SPHX_PHASE_LDS_BUDGET) {
-        phases *= 2;
-    }
-    return phases;
-}
+// (The LDS one pass may use, SPHX_PHASE_LDS_BUDGET, and the padding of the rows: sphx_geometry.hpp. 52 KB lets
+// three workgroups share a CU.)
 
 template <typename T, int MODE, bool NORM, int H, bool PREFIX>
 __global__ __launch_bounds__(64) void closed_form_kernel(Tiling g, const T* __restrict__ xyz,

@@ -507,13 +507,6 @@ __global__ __launch_bounds__(NT) void gradients_lanes_kernel(Tiling g, const T* 
 // g.off_jobs, g.jobs_per_point: the waves' scratch [A | B | C] and a lane's share of it.
 // g.sequence_waves (1, 2 or 4): the waves that share one channel, each taking a part of its m.
 // ---------------------------------------------------------------------------
-constexpr unsigned kHessianLaneThreads = 256; // float64 entries need more than 128 registers
-template <typename T> constexpr unsigned hessian_lane_threads() {
-    // (float32 with 512 threads, 128 registers per lane: l_max = 2-5 5-15 % slower with the
-    // same number of waves)
-    return kHessianLaneThreads;
-}
-
 template <typename T, bool NORM>
 __global__ __launch_bounds__(hessian_lane_threads<T>()) void hessians_lanes_kernel(Tiling g, const T* __restrict__ xyz,
                                                                             T* __restrict__ sph,

@@ -1,151 +1,23 @@
-// The C-ABI launch layer declared in include/sphx_launch.h: plans, dispatch and
-// entry points. The kernels (gfx950) are in sphx_closed_form_kernel.hpp,
-// sphx_lane_kernels.hpp, sphx_vjp_kernels.hpp and sphx_recursion_kernel.hpp.
-//
-// Work decomposition. The outputs of consecutive points are consecutive in
-// every output array, so a workgroup takes a *tile* of S consecutive points,
-// builds the tile's slice of sph / dsph / ddsph in LDS in exactly the HBM
-// layout, and then streams the three slices out with contiguous 16-byte
-// stores: every 128-byte line of the outputs is written once, in full, by
-// neighbouring lanes. Inside a tile
-//
-//   * l <= H (H = 6, or 1 when second derivatives are asked for: the split of
-//     the reference CPU classes, sphericart/src/sphericart.cpp:45-92) is
-//     evaluated in closed form, one point per lane, in registers;
-//   * every l > H is one independent job per (point, l) pair
-//     (the reference makes channels independent on purpose,
-//     sphericart/include/templates_core.hpp:77-80), so the lanes of the
-//     workgroup run the Q_l^m recursions of different l side by side.
-//
-// `closed_form_kernel` is the all-closed-form case (l_max <= 6 without second
-// derivatives, l_max <= 1 with): one wave, one point per lane, 64 points per
-// tile. `recursion_kernel` is the general case; its workgroups are persistent
-// and walk over tiles so that the prefactor tables are fetched once.
-//
-// The prefactor tables are computed on the host (sphx_tables.cpp) with the
-// reference's recurrences and kept in constant memory; they depend on (l, m)
-// only, so one table up to SPHX_TABLE_LMAX serves every l_max.
+// The planner: from the shape of a call to kernels, tiles and LDS layouts. Plain host C++.
 
-#include <hip/hip_runtime.h>
+#include "sphx_plan.hpp"
 
-#include <cstdint>
-#include <cstdio>
-#include <cstdlib>
 #include <atomic>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
-#include <string>
-#include <type_traits>
-#include <vector>
 
 #include "../../include/sphx_launch.h"
-#include "sphx_device.hpp"
-#include "sphx_tables.hpp"
-
-#include "sphx_tiling.hpp"
-#include "sphx_closed_form_kernel.hpp"
-#include "sphx_lane_kernels.hpp"
-#include "sphx_vjp_kernels.hpp"
-#include "sphx_recursion_kernel.hpp"
-#include "sphx_pairs.hpp"
 
 namespace sphx {
 
-// ---------------------------------------------------------------------------
-// Host side of the launch layer
-// ---------------------------------------------------------------------------
-
 thread_local std::string t_error;
 
-static int fail(int code, const std::string& what) {
+int fail(int code, const std::string& what) {
     t_error = what;
     return code;
 }
 
-#define SPHX_HIP(call)                                                                            \
-    do {                                                                                          \
-        hipError_t status_ = (call);                                                              \
-        if (status_ != hipSuccess) {                                                              \
-            return fail(SPHX_ERR_HIP, std::string(#call) + ": " + hipGetErrorString(status_));    \
-        }                                                                                         \
-    } while (0)
-
-constexpr int kMaxDevices = 64;
-static std::mutex g_init_mutex;
-static bool g_tables_ready[kMaxDevices] = {};
-static int g_lds_limit[kMaxDevices] = {};
-static int g_compute_units[kMaxDevices] = {};
-// where the constant tables of a device live, for kernels of other translation units
-struct TableAddresses {
-    const float *F32, *Q32;
-    const double *F64, *Q64;
-};
-static TableAddresses g_table_addresses[kMaxDevices] = {};
-
-static int find_scratch(int device);
-
-// Upload the tables to the constant memory of `device` (current) once.
-static int ensure_device_ready(int device) {
-    if (device < 0 || device >= kMaxDevices) {
-        return fail(SPHX_ERR_ARGUMENT, "device ordinal out of range");
-    }
-    std::lock_guard<std::mutex> lock(g_init_mutex);
-    if (g_tables_ready[device]) {
-        return SPHX_OK;
-    }
-    const HostTables& t = host_tables();
-    const size_t n = kTableEntries;
-    SPHX_HIP(hipMemcpyToSymbol(HIP_SYMBOL(kF32), t.f32.data(), n * sizeof(float)));
-    SPHX_HIP(hipMemcpyToSymbol(HIP_SYMBOL(kQ32), t.f32.data() + n, n * sizeof(float)));
-    SPHX_HIP(hipMemcpyToSymbol(HIP_SYMBOL(kF64), t.f64.data(), n * sizeof(double)));
-    SPHX_HIP(hipMemcpyToSymbol(HIP_SYMBOL(kQ64), t.f64.data() + n, n * sizeof(double)));
-    {
-        void *f32 = nullptr, *q32 = nullptr, *f64 = nullptr, *q64 = nullptr;
-        SPHX_HIP(hipGetSymbolAddress(&f32, HIP_SYMBOL(kF32)));
-        SPHX_HIP(hipGetSymbolAddress(&q32, HIP_SYMBOL(kQ32)));
-        SPHX_HIP(hipGetSymbolAddress(&f64, HIP_SYMBOL(kF64)));
-        SPHX_HIP(hipGetSymbolAddress(&q64, HIP_SYMBOL(kQ64)));
-        g_table_addresses[device] = TableAddresses{static_cast<const float*>(f32), static_cast<const float*>(q32),
-                                                   static_cast<const double*>(f64), static_cast<const double*>(q64)};
-    }
-    int lds = 0, cus = 0;
-    SPHX_HIP(hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device));
-    SPHX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
-    // The kernels deal their workgroups to eight XCDs (`blockIdx.x & 7`): on a device partitioned
-    // otherwise the results would still be right but every XCD would write all over the outputs.
-    // Said once, not enforced; a runtime that does not know the attribute is left alone.
-    int xcds = 0;
-    if (hipDeviceGetAttribute(&xcds, hipDeviceAttributeNumberOfXccs, device) != hipSuccess) {
-        (void)hipGetLastError();
-    } else if (xcds != 8 && xcds > 0) {
-        std::fprintf(stderr,
-                     "sphericart_amd: device %d reports %d XCDs; the kernels' workgroup order is laid out "
-                     "for the 8 XCDs of an MI355X in SPX mode and will be slower here\n",
-                     device, xcds);
-    }
-    {
-        const int status = find_scratch(device);
-        if (status != SPHX_OK) return status;
-    }
-    g_lds_limit[device] = lds;
-    g_compute_units[device] = cus;
-    g_tables_ready[device] = true;
-    return SPHX_OK;
-}
-
-// Overrides of single planning decisions, for measurements and tests (sphx_set_switch). None is
-// set in normal use: a call is then planned from its shape alone and no environment variable is
-// looked at. The variables of the same names are read once, when the library is first used, and
-// only if SPHX_DEBUG_SWITCHES is set to something other than 0.
-enum Switch : int {
-    SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_GRADIENT_LANES, SW_GRADIENT_LANES_PARTS,
-    SW_GRADIENT_LANES_TILE, SW_GRADIENT_LANES_WAVES, SW_GROUP_THREADS, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST,
-    SW_PAIRS, SW_PAIRS_BATCH, SW_PAIRS_CHUNK, SW_PAIRS_PREP_WAVES, SW_PAIRS_SEQUENCE_WAVES, SW_PAIRS_TILE,
-    SW_PREFIX_INSIDE,
-    SW_SEQUENCE_WAVES, SW_SLICE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
-    SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_ALONE, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
-    SW_VALUES_PACK, SW_VALUES_TILE_STEP, SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_VJP_STEP_FLOOR, SW_VJP_TILE_STEP, SW_COUNT
-};
 static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_GRADIENT_LANES",
     "SPHX_GRADIENT_LANES_PARTS", "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_GROUP_THREADS",
@@ -180,30 +52,48 @@ static void read_switches_from_environment() {
     g_switch_generation.fetch_add(1);
 }
 
-// The overrides as a planning call sees them: a copy taken once per plan.
+// The overrides as a planning call sees them: this thread's copy, taken again when they change.
 static thread_local Switches t_switches;
-static int switch_or(Switch which, int fallback) {
+static thread_local unsigned t_switches_generation = 0;
+
+int switch_or(Switch which, int fallback) {
     return t_switches.set[which] ? t_switches.value[which] : fallback;
 }
 
-struct Launch {
-    Tiling g;
-    unsigned workgroups;
-    unsigned threads;
-    unsigned lds_bytes;
-};
+unsigned refresh_switches() {
+    std::call_once(g_switch_env_once, read_switches_from_environment);
+    const unsigned generation = g_switch_generation.load(std::memory_order_acquire);
+    if (t_switches_generation != generation) {
+        std::lock_guard<std::mutex> lock(g_switch_mutex);
+        t_switches = g_switches;
+        t_switches_generation = g_switch_generation.load();
+    }
+    return t_switches_generation;
+}
 
-struct Plan {
-    bool lanes;       // values only, short rows: one launch of values_kernel (uses `closed`)
-    bool closed_only; // l_max within the closed forms: one launch of closed_form_kernel
-    bool whole;       // recursion_kernel evaluates the closed forms too: one launch
-                      // otherwise closed_form_kernel<PREFIX> + recursion_kernel: two launches
-    bool split_sides; // recursion_kernel takes the entries (l, +m) and (l, -m) as two jobs
-    bool pairs;       // values and gradients at large l_max: one launch of pairs_kernel (uses `pairs_launch`)
-    Launch closed;
-    Launch rec;
-    PairsLaunch pairs_launch;
-};
+int set_switch(const char* name, int value) {
+    // the environment first, so that what is set here wins over it
+    std::call_once(g_switch_env_once, read_switches_from_environment);
+    if (name != nullptr) {
+        for (int i = 0; i < SW_COUNT; ++i) {
+            if (std::strcmp(name, kSwitchNames[i]) == 0) {
+                std::lock_guard<std::mutex> lock(g_switch_mutex);
+                g_switches.set[i] = true;
+                g_switches.value[i] = value;
+                g_switch_generation.fetch_add(1);
+                return SPHX_OK;
+            }
+        }
+    }
+    return fail(SPHX_ERR_ARGUMENT, std::string("unknown switch: ") + (name ? name : "(null)"));
+}
+
+void reset_switches() {
+    std::call_once(g_switch_env_once, read_switches_from_environment);
+    std::lock_guard<std::mutex> lock(g_switch_mutex);
+    g_switches = Switches();
+    g_switch_generation.fetch_add(1);
+}
 
 static unsigned pow2_floor(unsigned v) {
     unsigned p = 1;
@@ -981,8 +871,8 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
 }
 
 // Choose kernels, tile sizes and LDS layouts. `lds_limit` / `cus` describe the device.
-static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit, int cus,
-                     Plan* plan, bool lane_kernels = true, bool normalized = true) {
+int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit, int cus, Plan* plan,
+              bool lane_kernels, bool normalized) {
     if (l_max < 0) return fail(SPHX_ERR_ARGUMENT, "l_max must be non-negative");
     if (mode < 0 || mode > 2) return fail(SPHX_ERR_ARGUMENT, "unknown derivative selector");
     if (l_max > SPHX_TABLE_LMAX) {
@@ -1142,312 +1032,10 @@ static int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds
     return SPHX_OK;
 }
 
-// What a launch needs to know about a kernel on a device, asked from the runtime once per
-// (device, kernel, LDS size) instead of on every call: the calls take microseconds each, which
-// is the whole budget of a small evaluation.
-struct KernelFacts {
-    int device;
-    const void* kernel;
-    unsigned lds_bytes;
-    unsigned resident_workgroups; // on the whole device, a multiple of 8; 0 = unknown
-};
-static std::mutex g_facts_mutex;
-static std::vector<KernelFacts> g_facts;
-
-// Raises the kernel's dynamic LDS limit if needed and returns how many workgroups of `threads`
-// threads are resident on the device at once (0 if the runtime would not tell).
-static hipError_t kernel_facts(const void* kernel, unsigned threads, unsigned lds_bytes,
-                               unsigned* resident_workgroups) {
-    int device = 0;
-    hipError_t e = hipGetDevice(&device);
-    if (e != hipSuccess) return e;
-    {
-        std::lock_guard<std::mutex> lock(g_facts_mutex);
-        for (const KernelFacts& f : g_facts) {
-            if (f.device == device && f.kernel == kernel && f.lds_bytes == lds_bytes) {
-                *resident_workgroups = f.resident_workgroups;
-                return hipSuccess;
-            }
-        }
-    }
-    if (lds_bytes > 64u * 1024u) {
-        // the limit of the device, not of this launch: the attribute belongs to the kernel, and
-        // a later launch with less must not lower it for one with more that is already cached
-        int limit = device >= 0 && device < kMaxDevices ? g_lds_limit[device] : 0;
-        if (limit < static_cast<int>(lds_bytes)) limit = static_cast<int>(lds_bytes);
-        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, limit);
-        if (e != hipSuccess) return e;
-    }
-    KernelFacts fresh{device, kernel, lds_bytes, 0u};
-    int per_cu = 0;
-    const int cus = device >= 0 && device < kMaxDevices ? g_compute_units[device] : 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, static_cast<int>(threads),
-                                                     lds_bytes) == hipSuccess &&
-        per_cu > 0 && cus > 0) {
-        fresh.resident_workgroups = (static_cast<unsigned>(per_cu) * static_cast<unsigned>(cus)) & ~7u;
-    } else {
-        (void)hipGetLastError();
-    }
-    std::lock_guard<std::mutex> lock(g_facts_mutex);
-    g_facts.push_back(fresh);
-    *resident_workgroups = fresh.resident_workgroups;
-    return hipSuccess;
-}
-
-template <typename T, int MODE, bool NORM, int H, bool PREFIX>
-static hipError_t launch_closed(const Launch& l, const T* xyz, T* sph, T* dsph, T* ddsph,
-                                hipStream_t stream) {
-    auto kernel = closed_form_kernel<T, MODE, NORM, H, PREFIX>;
-    if (l.lds_bytes > 64u * 1024u) {
-        unsigned unused = 0;
-        hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &unused);
-        if (e != hipSuccess) return e;
-    }
-    hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz,
-                       sph, dsph, ddsph);
-    return hipGetLastError();
-}
-
-template <typename X> struct AsGiven {
-    using type = X; // a parameter of this type takes no part in template argument deduction
-};
-
-// Workgroups of 1024 threads (one per CU, all of its LDS) exist for all but second derivatives
-// in float64, which need more registers than sixteen waves leave a lane, and the fused product.
-template <typename T, int MODE, bool VJP, bool NORM = true, bool SPLIT = false>
-constexpr bool kLargeGroups = !VJP && (MODE <= 1 || (MODE == 2 && sizeof(T) == 4) || (MODE == 2 && !NORM && SPLIT));
-
-template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false,
-          typename O = T, unsigned NT = kRecursionThreads>
-static hipError_t launch_recursion(const Launch& l, const typename AsGiven<O>::type* xyz,
-                                   typename AsGiven<O>::type* sph, typename AsGiven<O>::type* dsph,
-                                   typename AsGiven<O>::type* ddsph, hipStream_t stream) {
-    if constexpr (!VJP && !LIST) {
-        // the variant whose entry lanes take the jobs of a tile as one list
-        if (l.g.points_per_pass == 0) {
-            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, false, true, O, NT>(l, xyz, sph, dsph, ddsph, stream);
-        }
-    }
-    if constexpr (NT == kRecursionThreads && kLargeGroups<T, MODE, VJP, NORM, SPLIT>) {
-        if (l.threads == 2 * kRecursionThreads) {
-            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O, 2 * kRecursionThreads>(
-                l, xyz, sph, dsph, ddsph, stream);
-        }
-    }
-    if (l.threads != NT) return hipErrorInvalidValue; // never planned
-    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O, NT>;
-    // The workgroups are persistent: launch exactly as many as are resident at once (registers
-    // may allow fewer per CU than LDS does), or the last ones would run alone after the rest.
-    unsigned workgroups = l.workgroups;
-    unsigned cap = 0;
-    hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &cap);
-    if (e != hipSuccess) return e;
-    if (cap >= 8 && cap < workgroups) workgroups = cap;
-    hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz,
-                       sph, dsph, ddsph);
-    return hipGetLastError();
-}
-
-template <typename T> static const T* table_address(int device, bool q);
-template <> const float* table_address<float>(int device, bool q) {
-    return q ? g_table_addresses[device].Q32 : g_table_addresses[device].F32;
-}
-template <> const double* table_address<double>(int device, bool q) {
-    return q ? g_table_addresses[device].Q64 : g_table_addresses[device].F64;
-}
-
-template <typename T, int MODE, bool NORM>
-static hipError_t dispatch(const Plan& plan, int device, const T* xyz, T* sph, T* dsph, T* ddsph,
-                           hipStream_t stream) {
-    if (plan.pairs) {
-        if constexpr (MODE >= 1) {
-            return launch_pairs(plan.pairs_launch, MODE, NORM, table_address<T>(device, false),
-                                table_address<T>(device, true), xyz, sph, dsph, ddsph, stream);
-        }
-        return hipErrorInvalidValue; // never planned
-    }
-    if (plan.lanes) {
-        if constexpr (MODE == 0) {
-            const Launch& l = plan.closed;
-            auto kernel = l.g.points_per_pass == 4   ? values_kernel<T, NORM, 4>
-                          : l.g.points_per_pass == 2 ? (l.threads > 512 ? values_kernel<T, NORM, 2, 1024> : values_kernel<T, NORM, 2>)
-                          : l.threads > 512          ? values_kernel<T, NORM, 1, 1024>
-                                                     : values_kernel<T, NORM, 1>;
-            if (l.lds_bytes > 64u * 1024u) {
-                unsigned unused = 0;
-                hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &unused);
-                if (e != hipSuccess) return e;
-            }
-            hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz, sph);
-            return hipGetLastError();
-        }
-        if constexpr (MODE == 1) {
-            const Launch& l = plan.closed;
-            if (l.g.l_max < 4) return hipErrorInvalidValue; // never planned
-            auto kernel = l.g.l_max >= 6   ? (l.threads > 512 ? gradients_lanes_kernel<T, NORM, 6, 1024>
-                                                              : gradients_lanes_kernel<T, NORM, 6>)
-                          : l.g.l_max == 5 ? gradients_lanes_kernel<T, NORM, 5>
-                                           : gradients_lanes_kernel<T, NORM, 4>;
-            if (l.lds_bytes > 64u * 1024u) {
-                unsigned unused = 0;
-                hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &unused);
-                if (e != hipSuccess) return e;
-            }
-            hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz, sph,
-                               dsph);
-            return hipGetLastError();
-        }
-        if constexpr (MODE == 2) {
-            const Launch& l = plan.closed;
-            auto kernel = hessians_lanes_kernel<T, NORM>;
-            if (l.lds_bytes > 64u * 1024u) {
-                unsigned unused = 0;
-                hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &unused);
-                if (e != hipSuccess) return e;
-            }
-            hipLaunchKernelGGL(kernel, dim3(l.workgroups), dim3(l.threads), l.lds_bytes, stream, l.g, xyz, sph,
-                               dsph, ddsph);
-            return hipGetLastError();
-        }
-        return hipErrorInvalidValue;
-    }
-    if (!plan.closed_only) {
-        if constexpr (MODE == 2) {
-            if (plan.split_sides) {
-                return launch_recursion<T, MODE, NORM, true, true>(plan.rec, xyz, sph, dsph, ddsph, stream);
-            }
-            return launch_recursion<T, MODE, NORM, true, false>(plan.rec, xyz, sph, dsph, ddsph, stream);
-        } else {
-            if (plan.whole) {
-                return launch_recursion<T, MODE, NORM, true, false>(plan.rec, xyz, sph, dsph, ddsph, stream);
-            }
-            if (plan.rec.g.prefix_inside != 0) {
-                return launch_recursion<T, MODE, NORM, false, false>(plan.rec, xyz, sph, dsph, ddsph, stream);
-            }
-            // the two kernels write disjoint parts of every row
-            hipError_t e = launch_closed<T, MODE, NORM, 6, true>(plan.closed, xyz, sph, dsph, ddsph, stream);
-            if (e != hipSuccess) return e;
-            return launch_recursion<T, MODE, NORM, false, false>(plan.rec, xyz, sph, dsph, ddsph, stream);
-        }
-    }
-    const Launch& l = plan.closed;
-    switch (l.g.l_max) {
-    case 0:
-        return launch_closed<T, MODE, NORM, 0, false>(l, xyz, sph, dsph, ddsph, stream);
-    case 1:
-        return launch_closed<T, MODE, NORM, 1, false>(l, xyz, sph, dsph, ddsph, stream);
-    default:
-        break;
-    }
-    if constexpr (MODE < 2) {
-        switch (l.g.l_max) {
-        case 2:
-            return launch_closed<T, MODE, NORM, 2, false>(l, xyz, sph, dsph, ddsph, stream);
-        case 3:
-            return launch_closed<T, MODE, NORM, 3, false>(l, xyz, sph, dsph, ddsph, stream);
-        case 4:
-            return launch_closed<T, MODE, NORM, 4, false>(l, xyz, sph, dsph, ddsph, stream);
-        case 5:
-            return launch_closed<T, MODE, NORM, 5, false>(l, xyz, sph, dsph, ddsph, stream);
-        case 6:
-            return launch_closed<T, MODE, NORM, 6, false>(l, xyz, sph, dsph, ddsph, stream);
-        default:
-            break;
-        }
-    }
-    return hipErrorInvalidValue;
-}
-
-// What a call of a given shape launches, kept per thread so that a steady stream of equal calls
-// plans once: planning is a few hundred host instructions and, with overrides, a lock.
-struct PlannedCall {
-    // key
-    unsigned generation = 0; // of the overrides; 0 = empty slot
-    int kind = 0;            // 0: forward, 1: fused product, 2: float arrays evaluated in float64
-    size_t n_samples = 0;
-    int l_max = 0, mode = 0, elem = 0, normalized = 0, device = 0;
-    // what was planned
-    Plan plan;
-    Launch lanes;         // fused product beyond l_max = 6: the lane kernels' launch
-    bool use_lanes = false;
-    bool lane_groups = false;
-    bool wide = false;    // kind 2: the recursion kernel covers this shape
-};
-constexpr int kPlannedCalls = 16;
-static thread_local PlannedCall t_planned[kPlannedCalls];
-static thread_local unsigned t_planned_next = 0;
-static thread_local unsigned t_switches_generation = 0;
-
-// The slot for this shape; `*fresh` says that it has yet to be planned (by the caller, who then
-// sets `generation`; a failed plan leaves the slot empty).
-static PlannedCall* planned_call(int kind, size_t n_samples, int l_max, int mode, int elem,
-                                 int normalized, int device, bool* fresh) {
-    std::call_once(g_switch_env_once, read_switches_from_environment);
-    const unsigned generation = g_switch_generation.load(std::memory_order_acquire);
-    if (t_switches_generation != generation) {
-        std::lock_guard<std::mutex> lock(g_switch_mutex);
-        t_switches = g_switches;
-        t_switches_generation = g_switch_generation.load();
-    }
-    for (PlannedCall& c : t_planned) {
-        if (c.generation == t_switches_generation && c.kind == kind && c.n_samples == n_samples &&
-            c.l_max == l_max && c.mode == mode && c.elem == elem && c.normalized == normalized &&
-            c.device == device) {
-            *fresh = false;
-            return &c;
-        }
-    }
-    PlannedCall* c = &t_planned[t_planned_next++ % kPlannedCalls];
-    c->generation = 0;
-    c->kind = kind;
-    c->n_samples = n_samples;
-    c->l_max = l_max;
-    c->mode = mode;
-    c->elem = elem;
-    c->normalized = normalized;
-    c->device = device;
-    c->use_lanes = c->lane_groups = false;
-    *fresh = true;
-    return c;
-}
-
-// The evaluation proper, on `device`, which is the current one.
-template <typename T>
-static int forward_on(int device, const T* xyz, size_t n_samples, int l_max, int normalized, int mode,
-                      T* sph, T* dsph, T* ddsph, void* stream) {
-    int status = ensure_device_ready(device);
-    if (status != SPHX_OK) return status;
-    bool fresh = false;
-    PlannedCall* call = planned_call(0, n_samples, l_max, mode, sizeof(T), normalized != 0, device, &fresh);
-    if (fresh) {
-        status = make_plan(n_samples, l_max, mode, sizeof(T), g_lds_limit[device],
-                           g_compute_units[device], &call->plan, true, normalized != 0);
-        if (status != SPHX_OK) return status;
-        call->generation = t_switches_generation;
-    }
-    const Plan& plan = call->plan;
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    hipError_t e;
-    if (normalized) {
-        e = mode == 0   ? dispatch<T, 0, true>(plan, device, xyz, sph, dsph, ddsph, s)
-            : mode == 1 ? dispatch<T, 1, true>(plan, device, xyz, sph, dsph, ddsph, s)
-                        : dispatch<T, 2, true>(plan, device, xyz, sph, dsph, ddsph, s);
-    } else {
-        e = mode == 0   ? dispatch<T, 0, false>(plan, device, xyz, sph, dsph, ddsph, s)
-            : mode == 1 ? dispatch<T, 1, false>(plan, device, xyz, sph, dsph, ddsph, s)
-                        : dispatch<T, 2, false>(plan, device, xyz, sph, dsph, ddsph, s);
-    }
-    if (e != hipSuccess) {
-        return fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
-    }
-    return SPHX_OK;
-}
-
 // float arrays evaluated in float64 inside the recursion kernel (its O = float, T = double
 // variants): which shapes that covers, and the launch. Below the closed-form limit there is no
 // recursion kernel to run; the caller then evaluates into a float64 workspace and narrows.
-static bool make_wide_plan(size_t n_samples, int l_max, int mode, int lds_limit, int cus, Plan* plan,
-                           bool normalized) {
+bool make_wide_plan(size_t n_samples, int l_max, int mode, int lds_limit, int cus, Plan* plan, bool normalized) {
     const int hard = mode == 2 ? 1 : 6;
     if (l_max <= hard || l_max > SPHX_TABLE_LMAX || (n_samples + 63) / 64 > 0x7fffffffull) return false;
     plan->lanes = false;
@@ -1475,581 +1063,40 @@ static bool make_wide_plan(size_t n_samples, int l_max, int mode, int lds_limit,
     return fits;
 }
 
-template <int MODE, bool NORM>
-static hipError_t dispatch_wide(const Plan& plan, const float* xyz, float* sph, float* dsph, float* ddsph,
-                                hipStream_t stream) {
-    if constexpr (MODE == 2) {
-        if (plan.split_sides) {
-            return launch_recursion<double, 2, NORM, true, true, false, false, float>(plan.rec, xyz, sph, dsph, ddsph, stream);
-        }
-        return launch_recursion<double, 2, NORM, true, false, false, false, float>(plan.rec, xyz, sph, dsph, ddsph, stream);
-    } else {
-        if (plan.whole) {
-            return launch_recursion<double, MODE, NORM, true, false, false, false, float>(plan.rec, xyz, sph, dsph, ddsph, stream);
-        }
-        return launch_recursion<double, MODE, NORM, false, false, false, false, float>(plan.rec, xyz, sph, dsph, ddsph, stream);
+int make_vjp_plan(size_t n_samples, int l_max, size_t elem, int lds_limit, int cus, VjpPlan* out) {
+    out->use_lanes = out->lane_groups = false;
+    if (l_max > 6 && switch_or(SW_VJP_LANES, 1) != 0) {
+        out->use_lanes = plan_values(n_samples, l_max, elem, lds_limit, &out->lanes, true);
+        // groups of lanes with channels of their own pay off from tiles of 16 points down
+        // (200k points, float32 l_max = 24: 225 against 279 us; float64 l_max = 24: 665
+        // against 866; with tiles of 32 the scalar-unit kernel is ahead, float64 l_max = 12:
+        // 329 against 397)
+        out->lane_groups = out->use_lanes && out->lanes.g.tile <= switch_or(SW_VJP_GROUPS_BELOW, 16);
     }
+    if (out->use_lanes) return SPHX_OK;
+    // the closed-form or the recursion kernels with the contraction in place of the flush
+    return make_plan(n_samples, l_max, 1, elem, lds_limit, cus, &out->plan, false, true);
 }
 
-// `device` is current. *taken = false: not a shape for this path, nothing was enqueued.
-static int forward_wide_on(int device, const float* xyz, size_t n_samples, int l_max, int normalized,
-                           int mode, float* sph, float* dsph, float* ddsph, void* stream, bool* taken) {
-    *taken = false;
-    int status = ensure_device_ready(device);
-    if (status != SPHX_OK) return status;
-    bool fresh = false;
-    PlannedCall* call = planned_call(2, n_samples, l_max, mode, 8, normalized != 0, device, &fresh);
-    if (fresh) {
-        call->wide = make_wide_plan(n_samples, l_max, mode, g_lds_limit[device], g_compute_units[device],
-                                    &call->plan, normalized != 0);
-        call->generation = t_switches_generation;
-    }
-    if (!call->wide) return SPHX_OK;
-    const Plan& plan = call->plan;
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    hipError_t e;
-    if (normalized) {
-        e = mode == 0   ? dispatch_wide<0, true>(plan, xyz, sph, dsph, ddsph, s)
-            : mode == 1 ? dispatch_wide<1, true>(plan, xyz, sph, dsph, ddsph, s)
-                        : dispatch_wide<2, true>(plan, xyz, sph, dsph, ddsph, s);
-    } else {
-        e = mode == 0   ? dispatch_wide<0, false>(plan, xyz, sph, dsph, ddsph, s)
-            : mode == 1 ? dispatch_wide<1, false>(plan, xyz, sph, dsph, ddsph, s)
-                        : dispatch_wide<2, false>(plan, xyz, sph, dsph, ddsph, s);
-    }
-    if (e != hipSuccess) {
-        return fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
-    }
-    *taken = true;
-    return SPHX_OK;
-}
-
-template <typename T>
-static int forward(const T* xyz, size_t n_samples, int l_max, int normalized, int mode, T* sph,
-                   T* dsph, T* ddsph, void* stream) {
-    t_error.clear();
-    if (n_samples == 0) {
-        return SPHX_OK;
-    }
-    if (mode < 0 || mode > 2) return fail(SPHX_ERR_ARGUMENT, "unknown derivative selector");
-    if (xyz == nullptr) return fail(SPHX_ERR_ARGUMENT, "xyz is a null pointer");
-    if (sph == nullptr) return fail(SPHX_ERR_ARGUMENT, "sph is a null pointer");
-    if (mode >= 1 && dsph == nullptr) return fail(SPHX_ERR_ARGUMENT, "dsph is a null pointer");
-    if (mode >= 2 && ddsph == nullptr) return fail(SPHX_ERR_ARGUMENT, "ddsph is a null pointer");
-
-    hipPointerAttribute_t attr;
-    SPHX_HIP(hipPointerGetAttributes(&attr, xyz));
-    int current = 0;
-    SPHX_HIP(hipGetDevice(&current));
-    const int device = attr.device;
-    if (device != current) {
-        SPHX_HIP(hipSetDevice(device));
-    }
-
-    int status = forward_on<T>(device, xyz, n_samples, l_max, normalized, mode, sph, dsph, ddsph, stream);
-
-    if (device != current) {
-        hipError_t e = hipSetDevice(current);
-        if (e != hipSuccess && status == SPHX_OK) {
-            status = fail(SPHX_ERR_HIP, std::string("hipSetDevice: ") + hipGetErrorString(e));
-        }
-    }
-    return status;
-}
-
-// l_max > 6: the gradient kernels with the contraction in place of the flush; the closed forms
-// either inside the recursion kernel or, when its tiles are small, in a launch of their own that
-// stores the sum over l <= 6, to which the recursion kernel then adds the rest.
-template <typename T, bool NORM>
-static hipError_t launch_vjp_recursion(const Plan& plan, const T* xyz, const T* sph_grad, T* xyz_grad,
-                                       int accumulate, hipStream_t stream);
-
-template <typename T, bool NORM, int H>
-static hipError_t launch_vjp(const Launch& l, const T* xyz, const T* sph_grad, T* xyz_grad,
-                             int accumulate, hipStream_t stream) {
-    constexpr unsigned NY = (H + 1) * (H + 1);
-    const unsigned lds_bytes = 64u * (NY + closed_form_pad(H)) * static_cast<unsigned>(sizeof(T));
-    hipLaunchKernelGGL((closed_form_vjp_kernel<T, NORM, H>), dim3(l.workgroups), dim3(64), lds_bytes,
-                       stream, l.g, xyz, sph_grad, xyz_grad, accumulate);
-    return hipGetLastError();
-}
-
-template <typename T, bool NORM>
-static hipError_t dispatch_vjp(const Launch& l, int l_max, const T* xyz, const T* sph_grad,
-                               T* xyz_grad, int accumulate, hipStream_t stream) {
-    switch (l_max) {
-    case 0: return launch_vjp<T, NORM, 0>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
-    case 1: return launch_vjp<T, NORM, 1>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
-    case 2: return launch_vjp<T, NORM, 2>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
-    case 3: return launch_vjp<T, NORM, 3>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
-    case 4: return launch_vjp<T, NORM, 4>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
-    case 5: return launch_vjp<T, NORM, 5>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
-    case 6: return launch_vjp<T, NORM, 6>(l, xyz, sph_grad, xyz_grad, accumulate, stream);
-    default: return hipErrorInvalidValue;
-    }
-}
-
-template <typename T, bool NORM>
-static hipError_t launch_vjp_recursion(const Plan& plan, const T* xyz, const T* sph_grad, T* xyz_grad,
-                                       int accumulate, hipStream_t stream) {
-    Launch rec = plan.rec;
-    rec.g.vjp_accumulate = accumulate != 0;
-    // the kernel reads its `sph` argument and writes three numbers per point through `dsph`
-    T* upstream = const_cast<T*>(sph_grad);
-    if (plan.whole) {
-        return launch_recursion<T, 1, NORM, true, false, true>(rec, xyz, upstream, xyz_grad, nullptr, stream);
-    }
-    hipError_t e = launch_vjp<T, NORM, 6>(plan.closed, xyz, sph_grad, xyz_grad, accumulate, stream);
-    if (e != hipSuccess) return e;
-    return launch_recursion<T, 1, NORM, false, false, true>(rec, xyz, upstream, xyz_grad, nullptr, stream);
-}
-
-template <typename T>
-static int vjp(const T* xyz, const T* sph_grad, size_t n_samples, int l_max, int normalized,
-               T* xyz_grad, int accumulate, void* stream) {
-    t_error.clear();
-    if (n_samples == 0) return SPHX_OK;
-    if (l_max < 0) return fail(SPHX_ERR_ARGUMENT, "l_max must be non-negative");
-    if (xyz == nullptr || sph_grad == nullptr || xyz_grad == nullptr) {
-        return fail(SPHX_ERR_ARGUMENT, "null pointer passed to the vector-Jacobian product");
-    }
-    if ((n_samples + 63) / 64 > 0x7fffffffull) {
-        return fail(SPHX_ERR_UNSUPPORTED, "too many samples for one launch");
-    }
-    hipPointerAttribute_t attr;
-    SPHX_HIP(hipPointerGetAttributes(&attr, xyz));
-    int current = 0;
-    SPHX_HIP(hipGetDevice(&current));
-    const int device = attr.device;
-    if (device != current) {
-        SPHX_HIP(hipSetDevice(device));
-    }
-    int status = ensure_device_ready(device);
-    if (status == SPHX_OK && l_max > SPHX_TABLE_LMAX) {
-        status = fail(SPHX_ERR_UNSUPPORTED, "l_max = " + std::to_string(l_max) +
-                                                " exceeds the device prefactor tables (" +
-                                                std::to_string(SPHX_TABLE_LMAX) + ")");
-    }
-    const PlannedCall* planned = nullptr;
-    if (status == SPHX_OK) {
-        bool fresh = false;
-        PlannedCall* call = planned_call(1, n_samples, l_max, 1, sizeof(T), normalized != 0, device, &fresh);
-        if (fresh) {
-            if (l_max > 6 && switch_or(SW_VJP_LANES, 1) != 0) {
-                call->use_lanes = plan_values(n_samples, l_max, sizeof(T), g_lds_limit[device], &call->lanes, true);
-                // groups of lanes with channels of their own pay off from tiles of 16 points down
-                // (200k points, float32 l_max = 24: 225 against 279 us; float64 l_max = 24: 665
-                // against 866; with tiles of 32 the scalar-unit kernel is ahead, float64 l_max = 12:
-                // 329 against 397)
-                call->lane_groups = call->use_lanes && call->lanes.g.tile <= switch_or(SW_VJP_GROUPS_BELOW, 16);
-            }
-            if (!call->use_lanes) {
-                // the closed-form or the recursion kernels with the contraction in place of the flush
-                status = make_plan(n_samples, l_max, 1, sizeof(T), g_lds_limit[device], g_compute_units[device],
-                                   &call->plan, false);
-            }
-            if (status == SPHX_OK) call->generation = t_switches_generation;
-        }
-        planned = call;
-    }
-    if (status == SPHX_OK) {
-        const Plan& plan = planned->plan;
-        const Launch& lanes = planned->lanes;
-        const bool use_lanes = planned->use_lanes;
-        hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-        hipError_t e;
-        if (use_lanes) {
-            auto launch = [&](auto kernel) -> hipError_t {
-                if (lanes.lds_bytes > 64u * 1024u) {
-                    unsigned unused = 0;
-                    hipError_t err = kernel_facts(reinterpret_cast<const void*>(kernel), lanes.threads,
-                                                  lanes.lds_bytes, &unused);
-                    if (err != hipSuccess) return err;
-                }
-                hipLaunchKernelGGL(kernel, dim3(lanes.workgroups), dim3(lanes.threads), lanes.lds_bytes, s,
-                                   lanes.g, xyz, sph_grad, xyz_grad, accumulate);
-                return hipGetLastError();
-            };
-            if (!planned->lane_groups) {
-                if (lanes.threads > 512) {
-                    e = normalized ? launch(vjp_lanes_kernel<T, true, 1024>) : launch(vjp_lanes_kernel<T, false, 1024>);
-                } else {
-                    e = normalized ? launch(vjp_lanes_kernel<T, true>) : launch(vjp_lanes_kernel<T, false>);
-                }
-            } else {
-                e = normalized ? launch(vjp_groups_kernel<T, true>) : launch(vjp_groups_kernel<T, false>);
-            }
-        } else if (plan.closed_only) {
-            e = normalized ? dispatch_vjp<T, true>(plan.closed, l_max, xyz, sph_grad, xyz_grad, accumulate, s)
-                           : dispatch_vjp<T, false>(plan.closed, l_max, xyz, sph_grad, xyz_grad, accumulate, s);
-        } else {
-            e = normalized ? launch_vjp_recursion<T, true>(plan, xyz, sph_grad, xyz_grad, accumulate, s)
-                           : launch_vjp_recursion<T, false>(plan, xyz, sph_grad, xyz_grad, accumulate, s);
-        }
-        if (e != hipSuccess) {
-            status = fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
-        }
-    }
-    if (device != current) {
-        hipError_t e = hipSetDevice(current);
-        if (e != hipSuccess && status == SPHX_OK) {
-            status = fail(SPHX_ERR_HIP, std::string("hipSetDevice: ") + hipGetErrorString(e));
-        }
-    }
-    return status;
-}
-
-// ---------------------------------------------------------------------------
-// float32 arrays evaluated in float64. In float32 the reference's prefactors
-// and Q_l^l = (2l-1)!! leave the range of the type from l = 29 (NaN and inf in
-// the outputs) and high-|m| entries come out as exact zeros from l of about 20
-// (sphericart/include/templates.hpp:54-97 evaluated in float). This path, which
-// a caller must ask for, evaluates in float64 and rounds every result once:
-// beyond the closed forms in one launch of the recursion kernel's mixed variant
-// (forward_wide_on), else by widening xyz, running the float64 kernels into a
-// workspace and narrowing the rows (below).
-// ---------------------------------------------------------------------------
-constexpr unsigned kConvertThreads = 256;
-
-__global__ __launch_bounds__(kConvertThreads) void widen_kernel(const float* __restrict__ in,
-                                                               double* __restrict__ out,
-                                                               unsigned long long count) {
-    const unsigned long long stride = static_cast<unsigned long long>(gridDim.x) * kConvertThreads;
-    for (unsigned long long i = static_cast<unsigned long long>(blockIdx.x) * kConvertThreads + threadIdx.x;
-         i < count; i += stride) {
-        out[i] = static_cast<double>(in[i]);
-    }
-}
-
-__global__ __launch_bounds__(kConvertThreads) void narrow_kernel(const double* __restrict__ in,
-                                                                float* __restrict__ out,
-                                                                unsigned long long count) {
-    const unsigned long long stride = static_cast<unsigned long long>(gridDim.x) * kConvertThreads;
-    for (unsigned long long i = static_cast<unsigned long long>(blockIdx.x) * kConvertThreads + threadIdx.x;
-         i < count; i += stride) {
-        out[i] = static_cast<float>(in[i]); // round to nearest even, overflow to infinity
-    }
-}
-
-static unsigned convert_blocks(unsigned long long count) {
-    const unsigned long long want = (count + kConvertThreads - 1) / kConvertThreads;
-    return static_cast<unsigned>(want < 16384ull ? (want ? want : 1ull) : 16384ull);
-}
-
-// float64 bytes one point needs in the workspace: its coordinates and its rows
-static size_t via_f64_bytes_per_point(int l_max, int mode) {
-    const size_t ny = static_cast<size_t>(l_max + 1) * (l_max + 1);
-    return sizeof(double) * (3 + ny * components_of(mode));
-}
-
-// The library's own scratch memory for sphx_forward_f32_via_f64_static: callers that must not
-// allocate (HIP graph capture, serving loops, harnesses that forbid it) get the float64 rows of one
-// call staged here. Every device the library runs on holds its own copy of the array, at its own
-// address, until the process ends; g_scratch[device] is that address, asked from the runtime once
-// per device (ensure_device_ready). In host code the array's name is only a handle for that
-// question, never an address to hand to a kernel.
-constexpr size_t kScratchBytes = size_t(32) << 20;
-static __device__ __align__(256) unsigned char scratch[kScratchBytes];
-static void* g_scratch[kMaxDevices] = {};
-
-// with `device` current; called under g_init_mutex by ensure_device_ready
-static int find_scratch(int device) {
-    void* ptr = nullptr;
-    SPHX_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
-    if (ptr == nullptr) return fail(SPHX_ERR_HIP, "hipGetSymbolAddress returned no address for the scratch array");
-    g_scratch[device] = ptr;
-    return SPHX_OK;
-}
-
-static int check_via_f64_arguments(const float* xyz, int l_max, int mode, const float* sph,
-                                   const float* dsph, const float* ddsph) {
-    if (l_max < 0) return fail(SPHX_ERR_ARGUMENT, "l_max must be non-negative");
-    if (mode < 0 || mode > 2) return fail(SPHX_ERR_ARGUMENT, "unknown derivative selector");
-    if (l_max > SPHX_TABLE_LMAX) {
-        return fail(SPHX_ERR_UNSUPPORTED, "l_max = " + std::to_string(l_max) +
-                                              " exceeds the device prefactor tables (" +
-                                              std::to_string(SPHX_TABLE_LMAX) + ")");
-    }
-    if (xyz == nullptr) return fail(SPHX_ERR_ARGUMENT, "xyz is a null pointer");
-    if (sph == nullptr) return fail(SPHX_ERR_ARGUMENT, "sph is a null pointer");
-    if (mode >= 1 && dsph == nullptr) return fail(SPHX_ERR_ARGUMENT, "dsph is a null pointer");
-    if (mode >= 2 && ddsph == nullptr) return fail(SPHX_ERR_ARGUMENT, "ddsph is a null pointer");
-    return SPHX_OK;
-}
-
-// The points in chunks of as many as the workspace holds: widen, evaluate in float64, narrow.
-// `device` is current. Enqueues only.
-static int via_f64_chunks(int device, const float* xyz, size_t n_samples, int l_max, int normalized,
-                          int mode, float* sph, float* dsph, float* ddsph, void* workspace,
-                          size_t workspace_bytes, void* stream) {
-    const size_t per_point = via_f64_bytes_per_point(l_max, mode);
-    const size_t ny = static_cast<size_t>(l_max + 1) * (l_max + 1);
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    size_t chunk = workspace_bytes / per_point;
-    if (chunk == 0) {
-        return fail(SPHX_ERR_ARGUMENT, "the workspace holds no point: " + std::to_string(per_point) +
-                                           " bytes are needed per point");
-    }
-    if ((reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) {
-        return fail(SPHX_ERR_ARGUMENT, "the workspace must be aligned to 16 bytes");
-    }
-    if (chunk > n_samples) chunk = n_samples;
-    if (chunk >= 64) chunk &= ~size_t(63); // whole tiles of the closed-form kernels
-    // workspace layout for a chunk of c points: sph[c][ny], dsph[c][3][ny], ddsph[c][9][ny], xyz[c][3]
-    double* w_sph = static_cast<double*>(workspace);
-    double* w_dsph = w_sph + chunk * ny;
-    double* w_ddsph = w_dsph + (mode >= 1 ? chunk * 3 * ny : 0);
-    double* w_xyz = w_ddsph + (mode >= 2 ? chunk * 9 * ny : 0);
-    for (size_t first = 0; first < n_samples; first += chunk) {
-        const size_t count = n_samples - first < chunk ? n_samples - first : chunk;
-        hipLaunchKernelGGL(widen_kernel, dim3(convert_blocks(count * 3)), dim3(kConvertThreads), 0, s,
-                           xyz + first * 3, w_xyz, static_cast<unsigned long long>(count * 3));
-        const int status = forward_on<double>(device, w_xyz, count, l_max, normalized, mode, w_sph,
-                                              mode >= 1 ? w_dsph : nullptr, mode >= 2 ? w_ddsph : nullptr,
-                                              stream);
-        if (status != SPHX_OK) return status;
-        hipLaunchKernelGGL(narrow_kernel, dim3(convert_blocks(count * ny)), dim3(kConvertThreads), 0, s,
-                           w_sph, sph + first * ny, static_cast<unsigned long long>(count * ny));
-        if (mode >= 1) {
-            hipLaunchKernelGGL(narrow_kernel, dim3(convert_blocks(count * 3 * ny)), dim3(kConvertThreads), 0,
-                               s, w_dsph, dsph + first * 3 * ny, static_cast<unsigned long long>(count * 3 * ny));
-        }
-        if (mode >= 2) {
-            hipLaunchKernelGGL(narrow_kernel, dim3(convert_blocks(count * 9 * ny)), dim3(kConvertThreads), 0,
-                               s, w_ddsph, ddsph + first * 9 * ny, static_cast<unsigned long long>(count * 9 * ny));
-        }
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) {
-            return fail(SPHX_ERR_HIP, std::string("kernel launch: ") + hipGetErrorString(e));
-        }
-    }
-    return SPHX_OK;
-}
-
-static int forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, int normalized, int mode,
-                               float* sph, float* dsph, float* ddsph, void* workspace,
-                               size_t workspace_bytes, void* stream) {
-    t_error.clear();
-    if (n_samples == 0) return SPHX_OK;
-    int status = check_via_f64_arguments(xyz, l_max, mode, sph, dsph, ddsph);
-    if (status != SPHX_OK) return status;
-
-    hipPointerAttribute_t attr;
-    SPHX_HIP(hipPointerGetAttributes(&attr, xyz));
-    int current = 0;
-    SPHX_HIP(hipGetDevice(&current));
-    const int device = attr.device;
-    if (device != current) SPHX_HIP(hipSetDevice(device));
-
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    void* owned = nullptr;
-    // Beyond the closed forms the recursion kernel does it all in one launch: it reads the float
-    // coordinates, computes in float64 and stages float rows. No workspace is touched then.
-    bool fused = false;
-    status = forward_wide_on(device, xyz, n_samples, l_max, normalized, mode, sph, dsph, ddsph, stream, &fused);
-    if (status == SPHX_OK && !fused && workspace == nullptr) {
-        // No workspace given: one of our own for at most 256 MiB worth of points at a time, taken
-        // from and returned to the device's memory pool in stream order, so that the call still
-        // only enqueues (an allocation that waits for the device would stall the caller).
-        const size_t per_point = via_f64_bytes_per_point(l_max, mode);
-        size_t points = (size_t(256) << 20) / per_point;
-        if (points < 64) points = 64;
-        if (points > n_samples) points = n_samples;
-        workspace_bytes = points * per_point;
-        hipError_t e = hipMallocAsync(&owned, workspace_bytes, s);
-        if (e != hipSuccess) {
-            status = fail(SPHX_ERR_HIP, std::string("hipMallocAsync of the float64 workspace: ") + hipGetErrorString(e));
-        }
-        workspace = owned;
-    }
-    if (status == SPHX_OK && !fused) {
-        status = via_f64_chunks(device, xyz, n_samples, l_max, normalized, mode, sph, dsph, ddsph, workspace,
-                                workspace_bytes, stream);
-    }
-    if (owned != nullptr) {
-        hipError_t e = hipFreeAsync(owned, s); // after the work enqueued above, in stream order
-        if (e != hipSuccess && status == SPHX_OK) {
-            status = fail(SPHX_ERR_HIP, std::string("hipFreeAsync: ") + hipGetErrorString(e));
-        }
-    }
-    if (device != current) {
-        hipError_t e = hipSetDevice(current);
-        if (e != hipSuccess && status == SPHX_OK) {
-            status = fail(SPHX_ERR_HIP, std::string("hipSetDevice: ") + hipGetErrorString(e));
-        }
-    }
-    return status;
-}
-
-// The same with the library's scratch array as the workspace: nothing is allocated. One chunk
-// only, so a call is a fixed, short sequence of launches; more points than fit are refused.
-static int forward_f32_via_f64_static(const float* xyz, size_t n_samples, int l_max, int normalized,
-                                      int mode, float* sph, float* dsph, float* ddsph, void* stream) {
-    t_error.clear();
-    if (n_samples == 0) return SPHX_OK;
-    int status = check_via_f64_arguments(xyz, l_max, mode, sph, dsph, ddsph);
-    if (status != SPHX_OK) return status;
-    const size_t per_point = via_f64_bytes_per_point(l_max, mode);
-    if (n_samples > kScratchBytes / per_point) {
-        return fail(SPHX_ERR_UNSUPPORTED,
-                    std::to_string(n_samples) + " points of " + std::to_string(per_point) +
-                        " bytes each exceed the library's scratch memory of " + std::to_string(kScratchBytes) +
-                        " bytes: at most " + std::to_string(kScratchBytes / per_point) +
-                        " points of this shape per call");
-    }
-    hipPointerAttribute_t attr;
-    SPHX_HIP(hipPointerGetAttributes(&attr, xyz));
-    int current = 0;
-    SPHX_HIP(hipGetDevice(&current));
-    const int device = attr.device;
-    if (device != current) SPHX_HIP(hipSetDevice(device));
-    status = ensure_device_ready(device); // finds this device's copy of the scratch array
-    if (status == SPHX_OK) {
-        // Every number of the part of the scratch this call uses is written (widen_kernel, the
-        // float64 kernels) before it is read (the kernels, narrow_kernel), whatever the last
-        // call left there: nothing has to be cleared.
-        status = via_f64_chunks(device, xyz, n_samples, l_max, normalized, mode, sph, dsph, ddsph,
-                                g_scratch[device], kScratchBytes, stream);
-    }
-    if (device != current) {
-        hipError_t e = hipSetDevice(current);
-        if (e != hipSuccess && status == SPHX_OK) {
-            status = fail(SPHX_ERR_HIP, std::string("hipSetDevice: ") + hipGetErrorString(e));
-        }
-    }
-    return status;
-}
-
-} // namespace sphx
-
-extern "C" {
-
-int sphx_forward_f32(const float* xyz, size_t n_samples, int l_max, int normalized,
-                     int derivatives, float* sph, float* dsph, float* ddsph, void* stream) {
-    return sphx::forward<float>(xyz, n_samples, l_max, normalized, derivatives, sph, dsph, ddsph,
-                                stream);
-}
-
-int sphx_forward_f64(const double* xyz, size_t n_samples, int l_max, int normalized,
-                     int derivatives, double* sph, double* dsph, double* ddsph, void* stream) {
-    return sphx::forward<double>(xyz, n_samples, l_max, normalized, derivatives, sph, dsph, ddsph,
-                                 stream);
-}
-
-int sphx_forward_f32_via_f64(const float* xyz, size_t n_samples, int l_max, int normalized,
-                             int derivatives, float* sph, float* dsph, float* ddsph, void* workspace,
-                             size_t workspace_bytes, void* stream) {
-    return sphx::forward_f32_via_f64(xyz, n_samples, l_max, normalized, derivatives, sph, dsph, ddsph,
-                                     workspace, workspace_bytes, stream);
-}
-
-int sphx_forward_f32_via_f64_static(const float* xyz, size_t n_samples, int l_max, int normalized,
-                                    int derivatives, float* sph, float* dsph, float* ddsph, void* stream) {
-    return sphx::forward_f32_via_f64_static(xyz, n_samples, l_max, normalized, derivatives, sph, dsph, ddsph,
-                                            stream);
-}
-
-size_t sphx_forward_f32_via_f64_static_capacity(int l_max, int derivatives) {
-    if (l_max < 0 || l_max > SPHX_TABLE_LMAX || derivatives < 0 || derivatives > 2) return 0;
-    return sphx::kScratchBytes / sphx::via_f64_bytes_per_point(l_max, derivatives);
-}
-
-size_t sphx_forward_f32_via_f64_workspace(size_t n_samples, int l_max, int derivatives) {
-    if (l_max < 0 || derivatives < 0 || derivatives > 2) return 0;
-    return n_samples * sphx::via_f64_bytes_per_point(l_max, derivatives);
-}
-
-int sphx_vjp_f32(const float* xyz, const float* sph_grad, size_t n_samples, int l_max, int normalized,
-                 float* xyz_grad, int accumulate, void* stream) {
-    return sphx::vjp<float>(xyz, sph_grad, n_samples, l_max, normalized, xyz_grad, accumulate, stream);
-}
-
-int sphx_vjp_f64(const double* xyz, const double* sph_grad, size_t n_samples, int l_max,
-                 int normalized, double* xyz_grad, int accumulate, void* stream) {
-    return sphx::vjp<double>(xyz, sph_grad, n_samples, l_max, normalized, xyz_grad, accumulate, stream);
-}
-
-int sphx_device_count(void) {
-    int n = 0;
-    hipError_t e = hipGetDeviceCount(&n);
-    if (e != hipSuccess) {
-        sphx::t_error = std::string("hipGetDeviceCount: ") + hipGetErrorString(e);
-        return -1;
-    }
-    return n;
-}
-
-const char* sphx_last_error(void) { return sphx::t_error.c_str(); }
-
-int sphx_plan(size_t n_samples, int l_max, int derivatives, int is_f64, int* tile_samples,
-              int* threads, int* lds_bytes, int* workgroups) {
-    sphx::t_error.clear();
-    int device = 0, lds = 160 * 1024, cus = 256;
-    if (hipGetDevice(&device) == hipSuccess) {
-        int v = 0;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, device) == hipSuccess && v > 0) lds = v;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
-    } else {
-        (void)hipGetLastError();
-    }
-    sphx::Plan plan;
-    bool fresh = false; // only for the side effect: the overrides as this thread's plans see them
-    (void)sphx::planned_call(-1, 0, 0, 0, 0, 0, -1, &fresh);
-    int status = sphx::make_plan(n_samples ? n_samples : 1, l_max, derivatives,
-                                 is_f64 ? sizeof(double) : sizeof(float), lds, cus, &plan);
-    if (status != SPHX_OK) return status;
-    if (plan.pairs) {
-        if (tile_samples) *tile_samples = static_cast<int>(plan.pairs_launch.g.tile);
-        if (threads) *threads = static_cast<int>(plan.pairs_launch.threads);
-        if (lds_bytes) *lds_bytes = static_cast<int>(plan.pairs_launch.lds_bytes);
-        if (workgroups) *workgroups = static_cast<int>(plan.pairs_launch.workgroups);
-        return SPHX_OK;
-    }
-    const sphx::Launch& main = plan.closed_only || plan.lanes ? plan.closed : plan.rec;
-    if (tile_samples) *tile_samples = main.g.tile;
-    if (threads) *threads = static_cast<int>(main.threads);
-    if (lds_bytes) *lds_bytes = static_cast<int>(main.lds_bytes);
-    if (workgroups) *workgroups = static_cast<int>(main.workgroups);
-    return SPHX_OK;
-}
-
-int sphx_describe_plan(size_t n_samples, int l_max, int derivatives, int is_f64, int normalized,
-                       char* out, size_t capacity) {
-    sphx::t_error.clear();
-    if (out == nullptr || capacity == 0) return sphx::fail(SPHX_ERR_ARGUMENT, "no room for the description");
-    int device = 0, lds = 160 * 1024, cus = 256;
-    if (hipGetDevice(&device) == hipSuccess) {
-        int v = 0;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, device) == hipSuccess && v > 0) lds = v;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
-    } else {
-        (void)hipGetLastError();
-    }
-    sphx::Plan plan;
-    bool fresh = false;
-    (void)sphx::planned_call(-1, 0, 0, 0, 0, 0, -1, &fresh);
-    const int status = sphx::make_plan(n_samples ? n_samples : 1, l_max, derivatives,
-                                       is_f64 ? sizeof(double) : sizeof(float), lds, cus, &plan, true,
-                                       normalized != 0);
-    if (status != SPHX_OK) return status;
+std::string describe(const Plan& plan, int l_max, int mode, bool is_f64, bool normalized) {
     const std::string t = is_f64 ? "double" : "float";
-    const std::string head = t + ", " + std::to_string(derivatives) + ", " + (normalized ? "true" : "false");
-    auto geometry = [](const sphx::Launch& l) {
+    const std::string head = t + ", " + std::to_string(mode) + ", " + (normalized ? "true" : "false");
+    auto geometry = [](const Launch& l) {
         return " [" + std::to_string(l.g.tile) + " points per tile, " + std::to_string(l.threads) + " threads, " +
                std::to_string(l.lds_bytes) + " B LDS, " + std::to_string(l.workgroups) + " workgroups]";
     };
     std::string text;
     if (plan.pairs) {
-        const sphx::PairsLaunch& l = plan.pairs_launch;
-        text = "pairs_kernel<" + head + "> [" + std::to_string(l.g.tile) +
-               " points per tile, " + std::to_string(l.threads) + " threads, " + std::to_string(l.lds_bytes) +
-               " B LDS, " + std::to_string(l.workgroups) + " workgroups]";
+        const PairsLaunch& l = plan.pairs_launch;
+        text = "pairs_kernel<" + head + "> [" + std::to_string(l.g.tile) + " points per tile, " +
+               std::to_string(l.threads) + " threads, " + std::to_string(l.lds_bytes) + " B LDS, " +
+               std::to_string(l.workgroups) + " workgroups]";
     } else if (plan.closed_only) {
         text = "closed_form_kernel<" + head + ", " + std::to_string(l_max) + ", false>" + geometry(plan.closed);
     } else if (plan.lanes) {
         const char* names[3] = {"values_kernel", "gradients_lanes_kernel", "hessians_lanes_kernel"};
-        text = std::string(names[derivatives]) + "<" + t + ", " + (normalized ? "true" : "false") +
-               (derivatives == 0 ? ", " + std::to_string(plan.closed.g.points_per_pass) : std::string()) + ">" +
+        text = std::string(names[mode]) + "<" + t + ", " + (normalized ? "true" : "false") +
+               (mode == 0 ? ", " + std::to_string(plan.closed.g.points_per_pass) : std::string()) + ">" +
                geometry(plan.closed);
     } else {
         if (!plan.whole && plan.rec.g.prefix_inside == 0) {
@@ -2059,30 +1106,7 @@ int sphx_describe_plan(size_t n_samples, int l_max, int derivatives, int is_f64,
                 (plan.split_sides ? "true" : "false") + ", false, " +
                 (plan.rec.g.points_per_pass == 0 ? "true" : "false") + ">" + geometry(plan.rec);
     }
-    std::snprintf(out, capacity, "%s", text.c_str());
-    return SPHX_OK;
+    return text;
 }
 
-int sphx_set_switch(const char* name, int value) {
-    sphx::t_error.clear();
-    if (name != nullptr) {
-        for (int i = 0; i < sphx::SW_COUNT; ++i) {
-            if (std::strcmp(name, sphx::kSwitchNames[i]) == 0) {
-                std::lock_guard<std::mutex> lock(sphx::g_switch_mutex);
-                sphx::g_switches.set[i] = true;
-                sphx::g_switches.value[i] = value;
-                sphx::g_switch_generation.fetch_add(1);
-                return SPHX_OK;
-            }
-        }
-    }
-    return sphx::fail(SPHX_ERR_ARGUMENT, std::string("unknown switch: ") + (name ? name : "(null)"));
-}
-
-void sphx_reset_switches(void) {
-    std::lock_guard<std::mutex> lock(sphx::g_switch_mutex);
-    sphx::g_switches = sphx::Switches();
-    sphx::g_switch_generation.fetch_add(1);
-}
-
-} // extern "C"
+} // namespace sphx

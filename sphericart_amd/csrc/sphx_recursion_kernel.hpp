@@ -52,7 +52,7 @@ namespace sphx {
 // WHOLE == false: the rows start at l = H + 1 (closed_form_kernel<PREFIX>
 // writes the part below); every (point, component) row is its own run.
 // ---------------------------------------------------------------------------
-constexpr unsigned kRecursionThreads = 512;
+// (kRecursionThreads, the threads of a workgroup that shares its CU with a second one: sphx_geometry.hpp)
 
 // Values and gradients: at most 128 registers, so that two workgroups of 512 threads or one of
 // 1024 fit on a CU (four waves per SIMD) wherever their LDS allows. Only the float64 closed forms exceed that on their own

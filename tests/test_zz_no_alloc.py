@@ -1,6 +1,6 @@
-"""``sphx_forward_f32_via_f64_static``: the variant of ``sphx_forward_f32_via_f64`` that stages its
-float64 rows in the library's own scratch array instead of a workspace, for callers that cannot
-allocate device memory. Checked number for number against the existing entry point (which
+"""``sphx_forward_f32_via_f64_static``: the variant of ``sphx_forward_f32_via_f64`` for callers that cannot
+allocate device memory. Within the closed forms (l_max <= 6, or <= 1 with second derivatives) it stages its
+float64 rows in the library's own scratch array instead of a workspace; beyond, it is the same single launch. Checked number for number against the existing entry point (which
 ``tests/test_gpu_via_float64.py`` pins against the rounded float64 oracle) on consecutive calls
 that share the scratch, the later ones smaller, and against the oracle directly.
 """
@@ -57,13 +57,15 @@ def test_consecutive_calls_share_the_scratch(oracle, library):
     calls nothing is allocated and nothing waits."""
     rng = np.random.default_rng(77)
     cases = [(6, True, "gradients", 5000), (6, True, "gradients", 1201), (33, True, "gradients", 700),
-             (33, False, "gradients", 64), (12, False, "hessians", 300), (12, True, "hessians", 7),
-             (40, True, "values", 2049), (3, False, "values", 1)]
+             (33, False, "gradients", 64), (12, False, "hessians", 300), (1, True, "hessians", 3000),
+             (1, False, "hessians", 100), (12, True, "hessians", 7), (40, True, "values", 2049),
+             (5, True, "values", 4097), (3, False, "values", 1)]
     prepared = []
     for l_max, normalized, mode, n in cases:
         xyz = special_points(np.float32, rng, n)
         xyz_dev = torch.from_numpy(xyz).cuda()
-        assert n <= library.sphx_forward_f32_via_f64_static_capacity(l_max, MODE_INDEX[mode])
+        hard = 1 if mode == "hessians" else 6
+        assert l_max > hard or n <= library.sphx_forward_f32_via_f64_static_capacity(l_max, MODE_INDEX[mode])
         prepared.append((xyz, xyz_dev, with_workspace(library, xyz_dev, l_max, normalized, mode),
                          outputs(n, l_max, MODE_INDEX[mode])))
     torch.cuda.synchronize()
@@ -81,7 +83,7 @@ def test_consecutive_calls_share_the_scratch(oracle, library):
 
 
 def test_more_points_than_the_scratch_holds_are_refused(library):
-    l_max, k = 20, 1
+    l_max, k = 6, 1
     capacity = library.sphx_forward_f32_via_f64_static_capacity(l_max, k)
     n = capacity + 1
     xyz_dev = torch.ones((n, 3), dtype=torch.float32, device="cuda")
@@ -99,3 +101,17 @@ def test_more_points_than_the_scratch_holds_are_refused(library):
     assert status == 0, library.sphx_last_error()
     torch.cuda.synchronize()
     assert torch.isfinite(out[0][:capacity]).all() and (out[0][capacity:] == -7.0).all()
+
+
+def test_beyond_the_closed_forms_no_scratch_is_needed(oracle, library):
+    """More points than the scratch would hold, at an l_max that the one-launch kernel covers."""
+    l_max, k = 20, 1
+    n = library.sphx_forward_f32_via_f64_static_capacity(l_max, k) + 77
+    xyz = special_points(np.float32, np.random.default_rng(78), n)
+    xyz_dev = torch.from_numpy(xyz).cuda()
+    got = outputs(n, l_max, k)
+    without_allocation(library, xyz_dev, l_max, True, "gradients", got)
+    torch.cuda.synchronize()
+    reference = oracle.compute(xyz.astype(np.float64), l_max, True, "gradients")
+    for g, r in zip(got[:2], reference[:2]):
+        assert same_numbers(g.cpu().numpy(), r.astype(np.float32)).all()
