@@ -48,26 +48,24 @@ sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBPS = 8000.0
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script (summaries under profiles/), each counter scaled by what it reads for a
-# plain device-to-device copy of known size (`--calibrate-copy`: WRITE_SIZE
-# reads the copied bytes exactly, FETCH_SIZE half of them, so fetches are
-# doubled). KiB per dispatch * 1024 * factor, fetch + write, all kernels of one
-# call added up; the five configurations as in profiles/*_cfgN.md.
-MEASURED_TRAFFIC_BYTES = {
-    "cfg1": 26804978,
-    "cfg2": 76110936,
-    "cfg3": 796269808,
-    "cfg4": 3008426691,
-    "cfg5": 3487699849,
-    "cfg3:backward": int((394551.2 * 2.0 + 11719.3) * 1024),
-    "cfg3:vjp": int((101629.1 * 2.0 + 11718.8) * 1024),
-    "cfg5:vjp": int((426714.7 * 2.0 + 2343.8) * 1024),
-    "val10": 496336405,
-    "val22": 1064214171,
-    "grad10": 1948445144,
-    "hess5": 942427644,
-}
+def measured_traffic(key, kernels):
+    """HBM bytes per launch of a workload from profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+    of this script (the summaries under profiles/ that each entry names), each counter scaled by what it reads
+    for a plain device-to-device copy of known size (`--calibrate-copy`: WRITE_SIZE reads the copied bytes
+    exactly, FETCH_SIZE half of them, so fetches are doubled), fetch + write, all kernels of one call added up.
+    None when the entry was measured on another kernel than the one the library now launches for the shape."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as fd:
+            entry = json.load(fd)["workloads"].get(key)
+    except (OSError, ValueError, KeyError):
+        return None
+    if entry is None:
+        return None
+    if kernels is not None:
+        launched = "+".join(part.split("<")[0].strip() for part in kernels.split(" + "))
+        if launched != entry["kernel"]:
+            return None
+    return entry["bytes"]
 
 
 def parse():
@@ -142,8 +140,8 @@ def sweep(lib, args):
                                 timeout=10).stdout.strip() or None
     except (OSError, subprocess.SubprocessError):
         commit = None
-    print(json.dumps({"command": "python bench.py --sweep --sweep-sizes " + ",".join(sizes), "commit": commit,
-                      "peak_GBps": table.PEAK_HBM_GBPS, "rows": rows}, indent=0))
+    print(table.dump(rows, command="python bench.py --sweep --sweep-sizes " + ",".join(sizes), commit=commit,
+                     peak_GBps=table.PEAK_HBM_GBPS))
     return 0
 
 
@@ -179,6 +177,15 @@ def cpu_baseline(workload, xyz):
     timed = times[2:] if len(times) > 4 else times
     best = min(timed)
     cores = oracle.max_threads(flavour)
+    model = "unknown CPU"
+    try:
+        with open("/proc/cpuinfo") as fd:
+            for line in fd:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
     return {
         "value": n / best,
         "unit": "points/s",
@@ -186,8 +193,8 @@ def cpu_baseline(workload, xyz):
         "kind": kind,
         "sample": f"{passes} passes over all {n} points of the workload, best pass "
         f"{best * 1e3:.2f} ms, median {statistics.median(timed) * 1e3:.2f} ms; "
-        f"{'compiled reference sources (-O3, AVX2/FMA)' if kind == 'reference' else 'restatement (-O2, no FMA)'}, "
-        f"OpenMP over {cores} threads",
+        f"{'compiled reference sources (g++ -O3 -march=x86-64-v3 -ffp-contract=fast)' if kind == 'reference' else 'restatement (g++ -O2 -ffp-contract=off)'}, "
+        f"OpenMP over {cores} threads of {model}",
         "GBps": workload.bytes_per_point * n / best / 1e9,
     }
 
@@ -351,6 +358,106 @@ def roofline_of(device_ms, steps, launch_ms, bytes_per_launch):
     }
 
 
+def measure_yardsticks(lib, stream):
+    """What bounds a launch from below on this device, measured here: the duration of a kernel that does nothing,
+    enqueued back to back (what the GPU needs to start and retire any kernel), and the rate at which plain
+    streaming stores fill 1 GB of HBM (the evaluator's store pattern with nothing to compute)."""
+    import torch
+
+    def timed(step, steps):
+        for _ in range(steps // 4):
+            step()
+        best = None
+        for _ in range(3):
+            _, ms = time_back_to_back(step, steps, stream)
+            best = ms if best is None else min(best, ms)
+        return best / steps * 1e-3
+
+    def empty():
+        if lib.sphx_probe_empty_launch(stream.cuda_stream) != 0:
+            raise RuntimeError(lib.sphx_last_error().decode())
+
+    nbytes = 1 << 30
+    buffer = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+
+    def fill():
+        if lib.sphx_probe_fill(buffer.data_ptr(), nbytes, stream.cuda_stream) != 0:
+            raise RuntimeError(lib.sphx_last_error().decode())
+
+    empty_s = timed(empty, 2000)
+    fill_s = timed(fill, 40)
+    del buffer
+    torch.cuda.empty_cache()
+    return {"empty_launch_us": empty_s * 1e6, "fill_GBps": nbytes / fill_s / 1e9}
+
+
+def with_floor(entry, yardsticks, nbytes):
+    """latency_floor_us: an empty launch plus the algorithmic bytes at the measured fill rate; frac_of_floor: that
+    over the measured launch (1 = nothing left to gain for a kernel that computes nothing)."""
+    floor_us = yardsticks["empty_launch_us"] + nbytes / (yardsticks["fill_GBps"] * 1e9) * 1e6
+    entry["latency_floor_us"] = floor_us
+    entry["frac_of_floor"] = floor_us / entry["avg_launch_us"]
+    return entry
+
+
+def host_cost(lib, stream):
+    """Host microseconds per call of calls in a row that nobody waits for, the shape of cfg1 (10 000 points,
+    l_max = 8, float64, values and gradients): through sphx_forward_f64 and through the sphericart_cuda_* C API
+    from a loop in C (sphx_probe_host_cost_f64), through sphx_forward_f64 from Python (ctypes), and through the
+    torch operator. The host enqueues faster than the GPU evaluates, and once some 1 500 launches wait in the
+    queue a further call blocks until one has run: `burst` is ten bursts of 1 000 calls, each started with the
+    queue empty (what a call costs the host), `sustained` 10 000 calls in one go (what it costs once the queue is
+    full: the kernel's time), `gpu` the same with the wait at the end included."""
+    import torch
+
+    import sphericart_amd.torch as sphericart_torch
+    from sphericart_amd.workloads import WORKLOADS
+
+    w = WORKLOADS["cfg1"]
+    prepared = Prepared(lib, w)
+    sph, dsph, _ = prepared.outputs[0]
+    result = {"shape": "cfg1", "burst_calls": 1000, "sustained_calls": 10_000}
+    seconds = ctypes.c_double()
+
+    def in_c(through, calls):
+        status = lib.sphx_probe_host_cost_f64(through, prepared.xyz.data_ptr(), prepared.n, w.l_max, sph.data_ptr(),
+                                              dsph.data_ptr(), stream.cuda_stream, calls, ctypes.byref(seconds))
+        if status != 0:
+            raise RuntimeError(lib.sphx_last_error().decode())
+        return seconds.value
+
+    def from_python(step, calls):
+        t0 = time.perf_counter()
+        for _ in range(calls):
+            step()
+        return (time.perf_counter() - t0) / calls
+
+    calculator = sphericart_torch.SphericalHarmonics(w.l_max)
+    routes = {
+        "sphx_forward_f64": lambda calls: in_c(0, calls),
+        "sphericart_cuda_c_api": lambda calls: in_c(1, calls),
+        "sphx_forward_f64_from_python": lambda calls: from_python(prepared.step, calls),
+        "torch_op": lambda calls: from_python(lambda: calculator.compute_with_gradients(prepared.xyz), calls),
+    }
+    with torch.no_grad():
+        for name, route in routes.items():
+            route(200)
+            bursts = []
+            for _ in range(10):
+                torch.cuda.synchronize()
+                bursts.append(route(1000))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            sustained = route(10_000)
+            torch.cuda.synchronize()
+            with_wait = (time.perf_counter() - t0) / 10_000
+            result[name] = {"burst": statistics.median(bursts) * 1e6, "sustained": sustained * 1e6,
+                            "gpu": with_wait * 1e6}
+    del prepared
+    torch.cuda.empty_cache()
+    return result
+
+
 def measure(prepared, steps, settle_seconds, warmup):
     settle(prepared.step, settle_seconds, warmup)
     wall, device_ms = time_back_to_back(prepared.step, steps, prepared.stream)
@@ -358,7 +465,7 @@ def measure(prepared, steps, settle_seconds, warmup):
     return wall, roofline_of(device_ms, steps, launch_ms, prepared.bytes_per_launch)
 
 
-def measure_config(lib, name, steps, settle_seconds, with_cold):
+def measure_config(lib, name, steps, settle_seconds, with_cold, yardsticks):
     """One of the benchmark configurations next to the headline: per-launch event times with the
     outputs in place and, for the small ones, rotating through 1 GB of output buffers."""
     import torch
@@ -375,8 +482,9 @@ def measure_config(lib, name, steps, settle_seconds, with_cold):
         "kernels": prepared.kernels(),
         "launches_timed": steps,
         "points_per_s": w.n_samples * steps / wall,
-        "traffic": MEASURED_TRAFFIC_BYTES.get(name),
+        "traffic": measured_traffic(name, prepared.kernels()),
     })
+    with_floor(entry, yardsticks, prepared.bytes_per_launch)
     del prepared
     torch.cuda.empty_cache()
     if with_cold:
@@ -482,8 +590,8 @@ def main():
     wall, device_ms = time_back_to_back(step, args.steps, stream)
     # the single launch: K more steps, an event pair around each
     roofline = roofline_of(device_ms, args.steps, time_each_launch(step, args.steps, stream), bytes_per_launch)
-    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(
-        args.workload if args.op == "forward" else f"{args.workload}:{args.op}")
+    roofline["traffic"] = measured_traffic(args.workload if args.op == "forward" else f"{args.workload}:{args.op}",
+                                           prepared.kernels() if args.op == "forward" else None)
     headline = args.workload == "cfg3" and args.op == "forward" and args.rotate_mb == 0
 
     result = {
@@ -531,10 +639,14 @@ def main():
         }
         del cold, prepared, sph, dsph, ddsph
         torch.cuda.empty_cache()
+        yardsticks = measure_yardsticks(lib, stream)
+        result["yardsticks"] = yardsticks
+        with_floor(result["roofline"], yardsticks, bytes_per_launch)
         result["roofline_by_config"] = {
-            name: measure_config(lib, name, args.steps, args.settle_seconds, with_cold=name in ("cfg1", "cfg2"))
+            name: measure_config(lib, name, args.steps, args.settle_seconds, name in ("cfg1", "cfg2"), yardsticks)
             for name in ("cfg1", "cfg2", "cfg4", "cfg5")
         }
+        result["host_us_per_call"] = host_cost(lib, stream)
     print(json.dumps(result))
     return 0
 

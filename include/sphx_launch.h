@@ -184,6 +184,18 @@ SPHX_EXPORT int sphx_device_count(void);
  * message into the same std::runtime_error. */
 SPHX_EXPORT const char* sphx_last_error(void);
 
+/* Yardsticks for benchmarks; none of them has a counterpart in the reference and none is on the path of an
+ * evaluation. sphx_probe_empty_launch enqueues a kernel that does nothing (what a launch costs whatever it
+ * computes); sphx_probe_fill writes `bytes` bytes (a multiple of 16, `out` aligned to 16) with the store pattern
+ * of the evaluator's flush and nothing to compute (how fast plain stores fill HBM); sphx_probe_host_cost_f64
+ * makes `calls` calls in a row without waiting for the GPU, values and gradients of normalised harmonics in
+ * float64, through sphx_forward_f64 (`through` = 0) or through a calculator of the sphericart_cuda_* C API
+ * (1), and reports the host seconds per call. */
+SPHX_EXPORT int sphx_probe_empty_launch(void* stream);
+SPHX_EXPORT int sphx_probe_fill(void* out, size_t bytes, void* stream);
+SPHX_EXPORT int sphx_probe_host_cost_f64(int through, const double* xyz, size_t n_samples, int l_max, double* sph,
+                                         double* dsph, void* stream, int calls, double* seconds_per_call);
+
 /* Launch geometry chosen for a call of this shape (for benchmarks and tests):
  * samples per workgroup tile, threads per workgroup, LDS bytes per workgroup,
  * number of workgroups. Returns a status code. No counterpart in the reference

@@ -42,6 +42,9 @@ LAUNCH_SYMBOLS = [
     "sphx_describe_plan",
     "sphx_set_switch",
     "sphx_reset_switches",
+    "sphx_probe_empty_launch",
+    "sphx_probe_fill",
+    "sphx_probe_host_cost_f64",
 ]
 
 
@@ -101,6 +104,13 @@ def _declare(lib):
     lib.sphx_last_error.argtypes = []
     lib.sphx_plan.restype = c_int
     lib.sphx_plan.argtypes = [c_size_t, c_int, c_int, c_int] + [ctypes.POINTER(c_int)] * 4
+    lib.sphx_probe_empty_launch.restype = c_int
+    lib.sphx_probe_empty_launch.argtypes = [c_void_p]
+    lib.sphx_probe_fill.restype = c_int
+    lib.sphx_probe_fill.argtypes = [c_void_p, c_size_t, c_void_p]
+    lib.sphx_probe_host_cost_f64.restype = c_int
+    lib.sphx_probe_host_cost_f64.argtypes = [c_int, c_void_p, c_size_t, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                             ctypes.POINTER(ctypes.c_double)]
 
 
 def get_library():

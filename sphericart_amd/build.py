@@ -24,6 +24,7 @@ SOURCES = [
     "sphx_forward_f64_gradients.hip", "sphx_forward_f32_gradients.hip", "sphx_wide_gradients.hip",
     "sphx_forward_f64_values.hip", "sphx_forward_f32_values.hip", "sphx_wide_values.hip",
     "sphx_vjp_f64.hip", "sphx_vjp_f32.hip", "sphx_pairs.hip", "sphx_backward.hip", "sphx_via_f64.hip",
+    "sphx_probe.hip",
     "sphx_runtime.cpp", "sphx_plan.cpp", "sphx_tables.cpp", "device_api.cpp", "capi.cpp",
 ]
 

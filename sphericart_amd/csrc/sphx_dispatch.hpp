@@ -95,6 +95,7 @@ static hipError_t dispatch(const Plan& plan, const DeviceState& device, const T*
                           : l.g.points_per_pass == 2 ? (l.threads > 512 ? values_kernel<T, NORM, 2, 1024> : values_kernel<T, NORM, 2>)
                           : l.threads > 512          ? values_kernel<T, NORM, 1, 1024>
                                                      : values_kernel<T, NORM, 1>;
+            if (l.threads > (l.g.points_per_pass == 4 ? 512u : 1024u)) return hipErrorInvalidValue; // never planned
             if (l.lds_bytes > 64u * 1024u) {
                 unsigned unused = 0;
                 hipError_t e = kernel_facts(reinterpret_cast<const void*>(kernel), l.threads, l.lds_bytes, &unused);
@@ -106,6 +107,7 @@ static hipError_t dispatch(const Plan& plan, const DeviceState& device, const T*
         if constexpr (MODE == 1) {
             const Launch& l = plan.closed;
             if (l.g.l_max < 4) return hipErrorInvalidValue; // never planned
+            if (l.threads > (l.g.l_max >= 6 ? 1024u : 512u)) return hipErrorInvalidValue; // never planned
             auto kernel = l.g.l_max >= 6   ? (l.threads > 512 ? gradients_lanes_kernel<T, NORM, 6, 1024>
                                                               : gradients_lanes_kernel<T, NORM, 6>)
                           : l.g.l_max == 5 ? gradients_lanes_kernel<T, NORM, 5>
@@ -121,6 +123,7 @@ static hipError_t dispatch(const Plan& plan, const DeviceState& device, const T*
         }
         if constexpr (MODE == 2) {
             const Launch& l = plan.closed;
+            if (l.threads > hessian_lane_threads<T>()) return hipErrorInvalidValue; // never planned
             auto kernel = hessians_lanes_kernel<T, NORM>;
             if (l.lds_bytes > 64u * 1024u) {
                 unsigned unused = 0;

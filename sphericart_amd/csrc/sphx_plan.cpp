@@ -284,8 +284,9 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     out->workgroups = g.tiles_per_xcd * 8u;
     // one wave per l channel above the closed forms, eight at most
     // (alone on its CU: up to sixteen; twelve for one channel per wave in float32)
+    // (four channels side by side: that kernel exists for up to eight waves only)
     const int most = with_sums ? (sums_elems > 8u * 3u * 64u ? 16 : 8)
-                               : (bytes > half ? (elem == 4 && pack == 1 ? 12 : 16) : 8);
+                               : (bytes > half && pack != 4 ? (elem == 4 && pack == 1 ? 12 : 16) : 8);
     int waves = switch_or(SW_VALUES_WAVES, waves_by_shape != 0 && alone ? waves_by_shape : most);
     waves = waves < 1 ? 1 : (waves > most ? most : waves);
     // (the product's closed-form slices want at least four; values: one for the tables, one for

@@ -6,8 +6,9 @@ those stay below 6 GB).
 tests/test_zy_sweep_guard.py measures the 1.2 GB column again and fails where a shape has fallen more than a
 tenth below it. A row is
 
-    {"derivatives": "gradients", "dtype": "f32", "harmonics": "spherical", "l_max": 20, "size": "1.2GB",
-     "n_samples": 169779, "us": 274.1, "frac": 0.547, "kernel": "pairs_kernel"}
+    ["gradients", "f32", "spherical", 20, "1.2GB", 169779, 274.1, 0.547, "pairs_kernel"]
+
+(derivatives, dtype, harmonics, l_max, size, n_samples, us, frac, kernel; `load` gives the rows as dictionaries).
 
 `us` is the best of three series of launches enqueued back to back after a warm-up, between two events on the
 launch stream; `frac` the algorithmic bytes of a launch, sizeof(T) * (3 + (l_max + 1)^2 * {1, 4, 13}) per point,
@@ -101,6 +102,27 @@ def measure_row(lib, derivatives, dtype, harmonics, l_max, size, n, launches=30,
     return {"derivatives": derivatives, "dtype": dtype, "harmonics": harmonics, "l_max": l_max, "size": size,
             "n_samples": n, "us": round(best, 2), "frac": round(nbytes / best / 1e3 / PEAK_HBM_GBPS, 4),
             "kernel": kernel}
+
+
+COLUMNS = ("derivatives", "dtype", "harmonics", "l_max", "size", "n_samples", "us", "frac", "kernel")
+
+
+def dump(rows, **header):
+    """The table as JSON text: the header's fields, the column names once, one row per line."""
+    import json
+
+    head = json.dumps(dict(header, columns=list(COLUMNS)))[:-1]
+    lines = ",\n".join(json.dumps([row[c] for c in COLUMNS]) for row in rows)
+    return head + ', "rows": [\n' + lines + "\n]}"
+
+
+def load(path):
+    """The rows of a table written by dump, as dictionaries."""
+    import json
+
+    with open(path) as fd:
+        table = json.load(fd)
+    return [dict(zip(table["columns"], row)) for row in table["rows"]]
 
 
 def key_of(row):

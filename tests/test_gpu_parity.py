@@ -259,6 +259,61 @@ def test_benchmark_configurations_at_full_size(oracle, library, name):
         check(got, want, (name, first))
 
 
+def test_literal_clouds_of_the_reference_at_full_size(oracle, library):
+    """The first and the last benchmark configuration with their clouds drawn the way the reference's own scripts
+    draw them, at full size: cfg1 as i.i.d. N(0, 1) components from numpy's generator, cfg5 with radii exp(u), u
+    uniform in [ln 1e-2, ln 1e2), on directions uniform on the sphere (normalised normal deviates), 0.5 % of the
+    points put on the +-z axis. The array is drawn here and handed to the GPU and to the oracle alike, so the
+    C library's exp and numpy's generator need not agree between machines. (The seeded clouds of
+    sphericart_amd.workloads stay the fixtures' and the benchmark's: those are the same bits everywhere.)"""
+    rng = np.random.default_rng(20240521)
+    clouds = {"cfg1": rng.standard_normal((10_000, 3))}
+    n = 200_000
+    directions = rng.standard_normal((n, 3))
+    directions /= np.linalg.norm(directions, axis=1, keepdims=True)
+    radii = np.exp(rng.uniform(np.log(1e-2), np.log(1e2), size=n))
+    cloud = directions * radii[:, None]
+    on_axis = np.arange(n) % 200 == 0
+    cloud[on_axis, 0] = 0.0
+    cloud[on_axis, 1] = 0.0
+    cloud[on_axis, 2] = np.where(np.arange(n)[on_axis] % 400 == 0, 1.0, -1.0) * radii[on_axis]
+    clouds["cfg5"] = cloud
+    for name, xyz in clouds.items():
+        w = WORKLOADS[name]
+        xyz = np.ascontiguousarray(xyz.astype(w.numpy_dtype))
+        assert xyz.shape == (w.n_samples, 3)
+        announce("literal cloud", name, w.description)
+        xyz_dev = torch.from_numpy(xyz).cuda()
+        status, out = run_launch_layer(library, xyz_dev, w.l_max, w.normalized, w.derivatives)
+        assert status == 0, library.sphx_last_error()
+        torch.cuda.synchronize()
+        slab = max(1, min(w.n_samples, (256 << 20) // w.bytes_per_point))
+        for first in range(0, w.n_samples, slab):
+            last = min(w.n_samples, first + slab)
+            want = oracle.compute(xyz[first:last], w.l_max, w.normalized, w.derivatives)
+            got = tuple(o[first:last].cpu().numpy() if o is not None else None for o in out)
+            check(got, want, (name, first))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_values_with_fewer_points_than_a_channel_has_prefactors(oracle, library, dtype):
+    """values_kernel hands a channel's prefactors from lane to lane: with one, two or five points in a tile (or a
+    last tile that holds so few) most of the lanes that hold a prefactor have no point. Every l_max the kernel
+    takes, to the largest of the tables."""
+    rng = np.random.default_rng(53)
+    for l_max in (7, 10, 20, 33, 40, 63):
+        for n in (1, 2, 5, 25, 45, 64 + 3):
+            for normalized in (True, False):
+                announce("values, few points", np.dtype(dtype).name, normalized, l_max, n)
+                xyz = special_points(dtype, rng, n)
+                want = oracle.compute(xyz, l_max, normalized, "values")
+                status, got = run_launch_layer(library, torch.from_numpy(xyz).cuda(), l_max, normalized, "values")
+                torch.cuda.synchronize()
+                assert status == 0, library.sphx_last_error()
+                got = tuple(None if g is None else g.cpu().numpy() for g in got)
+                check(got, want, (l_max, normalized, n))
+
+
 @pytest.mark.parametrize("name", ["cfg3", "cfg4", "cfg5"])
 def test_size_independent_properties_at_full_size(library, name):
     """Identities that need no reference at all, evaluated on the device over the whole output:

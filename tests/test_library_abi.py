@@ -140,9 +140,36 @@ def test_planner_overrides(library, switches):
     assert _plan(library, 50_000, 20, 1, False)[1][1] in (512, 1024)  # recursion_kernel again
     library.sphx_reset_switches()
     assert _plan(library, 50_000, 20, 1, False) == default
+    # four channels side by side in a wave: that kernel exists for up to eight waves, whatever the shape asks
+    switches("SPHX_VALUES_PACK", 4)
+    for l_max in (25, 33, 39, 40):
+        status, (tile, threads, _, _) = _plan(library, 100_000, l_max, 0, False)
+        assert status == 0 and threads <= 512, (l_max, tile, threads)
+    library.sphx_reset_switches()
     assert library.sphx_set_switch(b"SPHX_NO_SUCH_SWITCH", 1) == 1
     assert b"unknown switch" in library.sphx_last_error()
     assert library.sphx_set_switch(None, 1) == 1
+
+
+def test_asking_for_plans_keeps_the_plans_of_recent_calls_and_set_switch_wins_over_the_environment():
+    """A process of its own with SPHX_DEBUG_SWITCHES: a switch set by the program before anything else still holds
+    after the environment has been read."""
+    code = (
+        "import sys, ctypes; sys.path.insert(0, %r)\n"
+        "from sphericart_amd import _c_lib\n"
+        "lib = _c_lib.get_library()\n"
+        "assert lib.sphx_set_switch(b'SPHX_TILE', 3) == 0\n"
+        "out = [ctypes.c_int() for _ in range(4)]\n"
+        "assert lib.sphx_plan(50000, 14, 1, 0, *[ctypes.byref(v) for v in out]) == 0\n"
+        "print(out[0].value)\n"
+    ) % ROOT
+    env = dict(os.environ, SPHX_DEBUG_SWITCHES="1", SPHX_TILE="5")
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, check=True, env=env).stdout
+    assert out.strip() == "3"
+    del env["SPHX_TILE"]
+    env["SPHX_SEQUENCE_WAVES"] = "1"  # (another switch from the environment is still read)
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, check=True, env=env).stdout
+    assert out.strip() == "3"
 
 
 def test_static_scratch_capacity(library):

@@ -1,0 +1,47 @@
+"""The planner's choices, guarded by what they achieve: the 1.2 GB column of the table of achieved bandwidth
+(``python bench.py --sweep``, kept as ``profiles/sweep.json``) is measured again, and a shape that has fallen
+more than a tenth below the fraction of the HBM peak recorded there fails. A slow shape is measured a second
+time before it counts (another process's burst on the box, clocks that have not come up yet).
+
+Collected next to last, so that a timing that fails hides no parity test.
+"""
+
+import os
+
+import pytest
+
+from gpu_utils import announce
+from sphericart_amd import sweep
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_no_shape_has_fallen_a_tenth_below_the_recorded_table(library):
+    recorded = {sweep.key_of(row): row for row in sweep.load(os.path.join(ROOT, "profiles", "sweep.json"))}
+    fallen = []
+    measured = 0
+    for shape in sweep.shapes(sizes=("1.2GB",)):
+        key = sweep.key_of(dict(zip(("derivatives", "dtype", "harmonics", "l_max", "size"), shape[:5])))
+        want = recorded.get(key)
+        if want is None:
+            continue
+        announce("sweep guard", key)
+        row = sweep.measure_row(library, *shape, launches=20, series=3)
+        if row["frac"] < 0.9 * want["frac"]:
+            row = sweep.measure_row(library, *shape, launches=40, series=4)
+        measured += 1
+        if row["frac"] < 0.9 * want["frac"]:
+            fallen.append((key, row["kernel"], row["frac"], "recorded", want["kernel"], want["frac"]))
+    assert measured >= 150, "profiles/sweep.json holds too few rows of the 1.2 GB column"
+    assert not fallen, fallen
+
+
+def test_recorded_table_meets_the_bars_it_was_made_for():
+    """What the table says of itself, no GPU involved in the check: the rows at 1.2 GB that the kernels were
+    tuned for."""
+    rows = [r for r in sweep.load(os.path.join(ROOT, "profiles", "sweep.json")) if r["size"] == "1.2GB"]
+    assert len(rows) >= 150
+    for r in rows:
+        assert 0.3 < r["frac"] < 1.0, r
