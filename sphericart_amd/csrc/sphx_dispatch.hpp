@@ -75,7 +75,7 @@ template <typename T, int MODE, bool NORM>
 static hipError_t dispatch(const Plan& plan, const DeviceState& device, const T* xyz, T* sph, T* dsph, T* ddsph,
                            hipStream_t stream) {
     if (plan.pairs) {
-        if constexpr (MODE >= 1) {
+        {
             const T *F, *Q;
             if constexpr (sizeof(T) == 4) {
                 F = device.F32;
@@ -86,7 +86,6 @@ static hipError_t dispatch(const Plan& plan, const DeviceState& device, const T*
             }
             return launch_pairs(plan.pairs_launch, MODE, NORM, F, Q, xyz, sph, dsph, ddsph, stream);
         }
-        return hipErrorInvalidValue; // never planned
     }
     if (plan.lanes) {
         if constexpr (MODE == 0) {

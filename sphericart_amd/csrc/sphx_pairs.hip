@@ -1,4 +1,4 @@
-// pairs_kernel (sphx_pairs_kernel.hpp) and its launch: values and gradients at large l_max, where the rows
+// pairs_kernel (sphx_pairs_kernel.hpp) and its launch: values and derivatives at large l_max, where the rows
 // of few points fill LDS. A translation unit of its own, so that it compiles next to the other kernels.
 
 #include <hip/hip_runtime.h>
@@ -52,6 +52,10 @@ hipError_t launch(const PairsLaunch& plan, const T* table_F, const T* table_Q, c
 template <typename T>
 hipError_t launch_any(const PairsLaunch& plan, int mode, bool normalized, const T* table_F, const T* table_Q,
                       const T* xyz, T* sph, T* dsph, T* ddsph, hipStream_t stream) {
+    if (mode == 0) {
+        return normalized ? launch<T, 0, true>(plan, table_F, table_Q, xyz, sph, dsph, ddsph, stream)
+                          : launch<T, 0, false>(plan, table_F, table_Q, xyz, sph, dsph, ddsph, stream);
+    }
     if (mode == 1) {
         return normalized ? launch<T, 1, true>(plan, table_F, table_Q, xyz, sph, dsph, ddsph, stream)
                           : launch<T, 1, false>(plan, table_F, table_Q, xyz, sph, dsph, ddsph, stream);

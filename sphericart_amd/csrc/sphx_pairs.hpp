@@ -10,7 +10,7 @@ namespace sphx {
 
 // Enqueue the launch `plan` describes on `stream`, on the current device. `table_F` / `table_Q` are the
 // device's prefactor tables (triangular, entry (l, m) at l (l + 1) / 2 + m) in the type of the arithmetic.
-// `mode`: 1 values and gradients, 2 second derivatives too (what the plan was made for).
+// `mode`: 0 values alone, 1 with gradients, 2 with second derivatives too (what the plan was made for).
 hipError_t launch_pairs(const PairsLaunch& plan, int mode, bool normalized, const float* table_F,
                         const float* table_Q, const float* xyz, float* sph, float* dsph, float* ddsph,
                         hipStream_t stream);

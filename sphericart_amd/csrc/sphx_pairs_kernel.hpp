@@ -101,13 +101,15 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
                                                                 unsigned long long* clocks
 #endif
 ) {
-    static_assert(MODE == 1 || MODE == 2, "values alone have kernels of their own");
+    static_assert(MODE >= 0 && MODE <= 2, "values alone, with gradients, with second derivatives too");
     constexpr int H = MODE == 2 ? 1 : 6;
     constexpr unsigned NYH = (H + 1) * (H + 1);
-    constexpr unsigned COMP = MODE == 2 ? 13 : 4;  // component rows per point
+    constexpr unsigned COMP = MODE == 2 ? 13 : (MODE == 1 ? 4 : 1); // component rows per point
     constexpr unsigned SEQS = MODE + 1;            // recursions per (point, l): Q_l^m, the Q_{l-1} and Q_{l-2} sequences
-    constexpr unsigned IT = MODE == 2 ? 4 : 2;     // ... interleaved in LDS: (A_m, B_m) pairs, (A_m, B_m, C_m, -) fours
-    constexpr unsigned ITEMS = MODE == 2 ? 1 : 9;  // work items of a batch: the records, eight slices of closed forms
+    // ... interleaved in LDS: A_m alone, (A_m, B_m) pairs, (A_m, B_m, C_m, -) fours
+    constexpr unsigned IT = MODE == 2 ? 4 : (MODE == 1 ? 2 : 1);
+    // work items of a batch: the records; the closed forms in eight slices, or their values in one
+    constexpr unsigned ITEMS = MODE == 2 ? 1 : (MODE == 1 ? 9 : 2);
     using P2 = typename Pair2<T>::type;
     using V4 = T __attribute__((ext_vector_type(4)));
 
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
     // records and parked closed forms: two buffers of one batch each
     const unsigned tpb = g.batch_tiles;
     auto batch_slot = [&](unsigned n) -> unsigned { // tile n's place in the two batch buffers
-        const unsigned b = __umulhi(n, g.magic_batch);
+        const unsigned b = tpb == 1u ? n : __umulhi(n, g.magic_batch); // (2^32 / 1 is no 32-bit number)
         return (b & 1u) * tpb + (n - b * tpb);
     };
     auto record = [&](unsigned n, unsigned s) -> T* {
@@ -184,7 +186,7 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
         const unsigned long long first_point = static_cast<unsigned long long>(tile_of(n)) * S;
         Phases ph;
         ph.sph = phase_of(sph, first_point * ny);
-        ph.dsph = phase_of(dsph, first_point * 3 * ny);
+        ph.dsph = MODE >= 1 ? phase_of(dsph, first_point * 3 * ny) : 0u;
         ph.ddsph = MODE == 2 ? phase_of(ddsph, first_point * 9 * ny) : 0u;
         return ph;
     };
@@ -192,7 +194,7 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
         Rows<O> rows;
         rows.ny = static_cast<int>(ny);
         rows.sph = row_lds + ph.sph + s * ny;
-        rows.dsph = row_lds + g.off_dsph + ph.dsph + s * 3 * ny;
+        rows.dsph = MODE >= 1 ? row_lds + g.off_dsph + ph.dsph + s * 3 * ny : nullptr;
         rows.ddsph = MODE == 2 ? row_lds + g.off_ddsph + ph.ddsph + s * 9 * ny : nullptr;
         return rows;
     };
@@ -250,6 +252,13 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
                 azimuth_pairs_job<T>(p, L, rec + 8, rec + g.tmz_at);
                 return;
             }
+            if constexpr (MODE == 0) {
+                Rows<T> rows;
+                rows.ny = static_cast<int>(NYH);
+                rows.sph = parked(n, s);
+                rows.dsph = rows.ddsph = nullptr;
+                closed_form_job<T, MODE, NORM, H>(p, rows);
+            }
             if constexpr (MODE == 1) {
                 Rows<T> rows;
                 rows.ny = static_cast<int>(NYH);
@@ -269,7 +278,7 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
             }
         };
         const unsigned prep_lanes = 64u * P;
-        // MODE 1: the closed forms of tile n from the parking area into its rows: point after point, a lane
+        // MODE 0, 1: the closed forms of tile n from the parking area into its rows: point after point, a lane
         // takes the same entries of every point
         [[maybe_unused]] auto unpark_stage = [&](unsigned n, unsigned valid, O* rows_v, O* rows_g) {
             for (unsigned r = tid; r < COMP * NYH; r += prep_lanes) {
@@ -316,7 +325,10 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
                 p.ir = zi[1];
                 p.x2 = p.y2 = p.z2 = 0;
                 const T pk = F0[l];
-                if constexpr (MODE == 1) {
+                if constexpr (MODE == 0) {
+                    // templates_core.hpp:393-395
+                    row_lds[ph.sph + s * ny + static_cast<unsigned>(l * (l + 1))] = static_cast<O>(it[0] * pk);
+                } else if constexpr (MODE == 1) {
                     const P2 it0 = *reinterpret_cast<const P2*>(it);      // Q_l^0 and the Q_{l-1} sequence at 0
                     const P2 it1 = *reinterpret_cast<const P2*>(it + IT); // ... at 1
                     Entry<T> e;
@@ -353,10 +365,13 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
             }
         };
 
-        // batch 0 in full, then one batch ahead: one work item per tile round
-        fetch(0);
-        for (unsigned item = wave; item < ITEMS; item += P) prep_item(0, item);
-        fetch(1);
+        // the first batch (or two) in full, then one batch (or two) ahead: one work item per tile round
+        const unsigned ahead = g.lookahead;
+        for (unsigned b = 0; b < ahead; ++b) {
+            fetch(b);
+            for (unsigned item = wave; item < ITEMS; item += P) prep_item(b, item);
+        }
+        fetch(ahead);
         __syncthreads();
         unsigned step = 0, batch = 0;
         SPHX_MARK(c_wait_b);
@@ -367,7 +382,7 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
             SPHX_MARK(c_wait_a);
             {
                 const Phases ph = phases_of(n);
-                if constexpr (MODE == 1) {
+                if constexpr (MODE <= 1) {
                     unpark_stage(n, valid, row_lds + ph.sph, row_lds + g.off_dsph + ph.dsph);
                 } else {
                     low_stage(n, valid, ph);
@@ -378,11 +393,11 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
             __syncthreads(); // rows of tile n complete
             SPHX_MARK(c_wait_b);
             const unsigned item = step * P + wave;
-            if (item < ITEMS) prep_item(batch + 1, item);
+            if (item < ITEMS) prep_item(batch + ahead, item);
             if (++step == tpb) {
                 step = 0;
                 ++batch;
-                fetch(batch + 1);
+                fetch(batch + ahead);
             }
             SPHX_MARK(c_flush);
         }
@@ -505,11 +520,11 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
         // MODE 1: the waves of a slot share a point, which is then the same for a whole wave (its addresses are
         // scalars). MODE 2: the table deals the lanes to the points lane by lane.
         const unsigned ew = wave - entry_first;
-        const unsigned wave_slot = MODE == 1 ? ew / g.slot_waves : 0u;
+        const unsigned wave_slot = MODE <= 1 ? ew / g.slot_waves : 0u;
         const unsigned job = g.lane_job[(ew - wave_slot * g.slot_waves) * 64u + lane];
         const bool has_job = job != kPairsNoJob;
-        const unsigned slot = MODE == 1 ? wave_slot : (has_job ? job >> 14 : 0u);
-        const unsigned slots = MODE == 1 ? g.entry_waves / g.slot_waves : g.lane_slots;
+        const unsigned slot = MODE <= 1 ? wave_slot : (has_job ? job >> 14 : 0u);
+        const unsigned slots = MODE <= 1 ? g.entry_waves / g.slot_waves : g.lane_slots;
         const int e_l = has_job ? static_cast<int>((job >> 7) & 127u) : H + 1;
         const int e_m = has_job ? static_cast<int>(job & 127u) : 1;
         const bool no_pdq = e_m >= e_l - 1; // |m| = l and l - 1: no Q_{l-1}^{m+1} term in d/dx, d/dy
@@ -594,6 +609,35 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
             const unsigned valid = valid_in(n);
             if (slot >= valid || !has_job) return;
             const Phases ph = phases_of(n);
+            if constexpr (MODE == 0) {
+                // values alone, templates_core.hpp:214-218 (:127-128 and :160-162 for |m| = l and l - 1): the
+                // iterate, its prefactor, c_m and s_m. Four points per turn: their reads are in flight together.
+                O* vp = row_lds + ph.sph + slot * ny + k_plus;
+                O* vm = row_lds + ph.sph + slot * ny + k_minus;
+                const unsigned step = slots * ny;
+                for (unsigned s = slot; s < valid; s += 4u * slots) {
+                    T a[4];
+                    P2 cs[4];
+#pragma unroll
+                    for (unsigned u = 0; u < 4u; ++u) {
+                        // (past the tile's last point: the last point once more, nothing stored)
+                        const unsigned su = s + u * slots < valid ? s + u * slots : s;
+                        a[u] = iterates(su)[o_it];
+                        cs[u] = *reinterpret_cast<const P2*>(record(n, su) + o_cs + 2);
+                    }
+#pragma unroll
+                    for (unsigned u = 0; u < 4u; ++u) {
+                        if (s + u * slots < valid) {
+                            const T pq = a[u] * pkm;
+                            vp[u * step] = static_cast<O>(pq * cs[u][0]);
+                            vm[u * step] = static_cast<O>(pq * cs[u][1]);
+                        }
+                    }
+                    vp += 4u * step;
+                    vm += 4u * step;
+                }
+                return;
+            }
             if constexpr (MODE == 2) {
                 // entry_job's own arithmetic on what the lane reads of the point: the iterates at m, m + 1, m + 2
                 // and (c, s) at m - 2, m - 1, m
@@ -715,7 +759,7 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
                 }
             };
             flush_run(0, sph, first * ny, valid * ny);
-            flush_run(g.off_dsph, dsph, first * 3 * ny, valid * 3 * ny);
+            if constexpr (MODE >= 1) flush_run(g.off_dsph, dsph, first * 3 * ny, valid * 3 * ny);
             if constexpr (MODE == 2) flush_run(g.off_ddsph, ddsph, first * 9 * ny, valid * 9 * ny);
         };
 

@@ -84,11 +84,12 @@ inline unsigned pairs_lane_table_by_kind(int l_max, int hard, unsigned waves, un
 // entries need more than the 128 registers that sixteen waves leave a lane).
 inline bool plan_pairs(size_t n_samples, int l_max, int mode, size_t elem, size_t out_elem, int lds_limit, int cus,
                        const PairsChoice& want, PairsLaunch* out) {
-    if (mode != 1 && mode != 2) return false;
+    if (mode < 0 || mode > 2) return false;
     const int H = mode == 2 ? 1 : 6;
     const unsigned NYH = static_cast<unsigned>((H + 1) * (H + 1));
-    const unsigned COMP = mode == 2 ? 13u : 4u, SEQS = static_cast<unsigned>(mode) + 1u, IT = mode == 2 ? 4u : 2u;
-    const unsigned ITEMS = mode == 2 ? 1u : 9u;
+    const unsigned COMP = mode == 2 ? 13u : (mode == 1 ? 4u : 1u), SEQS = static_cast<unsigned>(mode) + 1u;
+    const unsigned IT = mode == 2 ? 4u : (mode == 1 ? 2u : 1u);
+    const unsigned ITEMS = mode == 2 ? 1u : (mode == 1 ? 9u : 2u);
     const unsigned WAVES = (mode == 2 && elem == 8 ? 512u : kPairsThreads) / 64u;
     if (l_max <= H || l_max > 64 || n_samples == 0) return false;
     PairsTiling& g = out->g;
@@ -109,38 +110,79 @@ inline bool plan_pairs(size_t n_samples, int l_max, int mode, size_t elem, size_
     const unsigned q_elems = (L + 1) * q_stride;
     const unsigned f0_elems = align4(L + 1);
     // (with second derivatives nothing is parked)
-    const unsigned park_stride = mode == 2 ? 0u : COMP * NYH + 1u; // odd: the lanes of a prep wave, one point each, spread over the banks
+    const unsigned park_stride = mode == 2 ? 0u : (COMP * NYH) | 1u; // odd: the lanes of a prep wave, one point each, spread over the banks
     const unsigned iter_stride = align4(IT * tri_all + 2u * IT); // up to two groups past the end are read, never used
     auto bytes_for = [&](unsigned S, unsigned tpb) {
-        const unsigned rows = align4(S * ny + line) + align4(S * 3 * ny + line) + (mode == 2 ? align4(S * 9 * ny + line) : 0u);
+        const unsigned rows = align4(S * ny + line) + (mode >= 1 ? align4(S * 3 * ny + line) : 0u) +
+                              (mode == 2 ? align4(S * 9 * ny + line) : 0u);
         const unsigned tables = q_elems + f0_elems + 2 * tpb * S * (point_stride + park_stride) + 4u + S * iter_stride;
         return rows * osize + tables * esize;
     };
 
     // as many points per tile as LDS holds next to a batch of three tiles, twelve at most (1.2 GB of
     // output, l_max = 20 - 36: within 3 % of the best tile size on every shape)
-    unsigned S = want.tile ? want.tile : 12u;
-    if (S > 16) S = 16;
-    while (S > 1 && bytes_for(S, 3) > static_cast<unsigned>(lds_limit)) --S;
+    unsigned S = want.tile ? want.tile : (mode == 0 ? 64u : 12u);
+    // (values alone: two work items a batch, so a batch is a single tile, of up to a wave's lanes of points)
+    const unsigned least_batch = mode == 0 ? 1u : 3u;
+    if (S > (mode == 0 ? 64u : 16u)) S = mode == 0 ? 64u : 16u;
+    while (S > 1 && bytes_for(S, least_batch) > static_cast<unsigned>(lds_limit)) --S;
+    // Values alone: an entry is three multiplications, and what a tile costs is the entry waves going through
+    // its points one after the other, then the longer of the flush and the recursions of the next tile, which
+    // run side by side. More sequence waves shorten the recursions and leave fewer entry waves, which then take
+    // fewer points side by side. The largest tile that fits (smaller ones measured slower throughout) with the
+    // number of sequence waves of the least estimated cycles: 140 per point an entry wave goes through, 80 per
+    // step of a round of recursions, stores that drain at 11 bytes per cycle after the first 19 KB, and a
+    // quarter of the shorter of the two that run side by side for what they take from each other (measured on
+    // this kernel, MI355X; the choice is within 2 % of the best number of waves on every shape tried).
+    unsigned model_sequence_waves = 0;
+    if (mode == 0 && want.tile == 0) {
+        const unsigned pairs = (L * (L + 1u)) / 2u - static_cast<unsigned>(H * (H + 1)) / 2u;
+        const unsigned pair_waves = (pairs + 63u) / 64u;
+        const unsigned most = S;
+        unsigned long long best = ~0ull;
+        for (unsigned s_try = most; s_try == most; --s_try) {
+            for (unsigned q = 2u; q <= WAVES / 2u; ++q) {
+                if (2u + q + pair_waves > WAVES) break;
+                unsigned slots = (WAVES - 2u - q) / pair_waves;
+                if (slots > s_try) slots = s_try;
+                const unsigned long long entry = (s_try + slots - 1u) / slots * 140ull;
+                const unsigned long long rounds = (s_try * levels + 64u * q - 1u) / (64u * q);
+                const unsigned long long recursions = rounds * (L + 1u) * 80ull;
+                const unsigned long long bytes = static_cast<unsigned long long>(s_try) * ny * osize;
+                const unsigned long long flush = bytes > 19000ull ? (bytes - 19000ull) / 11ull : 0ull;
+                const unsigned long long longer = recursions > flush ? recursions : flush;
+                const unsigned long long shorter = recursions > flush ? flush : recursions;
+                const unsigned long long per_point = (entry + longer + shorter / 4ull + 600ull) * 1000ull / s_try;
+                if (per_point <= best) {
+                    best = per_point;
+                    S = s_try;
+                    model_sequence_waves = q;
+                }
+            }
+        }
+    }
     // batches: as many tiles as a wave has lanes for and LDS holds; at least three, so that the nine work
     // items of a batch fit its tile rounds with the prep waves there are (with second derivatives a batch is
     // only the records, and eight points are enough to share their chain of dependent operations)
     unsigned tpb = want.batch_tiles ? want.batch_tiles : (mode == 2 ? (8u + S - 1u) / S : 64u / S);
-    if (tpb < 3) tpb = 3;
+    if (tpb < least_batch) tpb = least_batch;
     if (tpb * S > 64u) tpb = 64u / S;
-    while (tpb > 3 && bytes_for(S, tpb) > static_cast<unsigned>(lds_limit)) --tpb;
-    if (tpb < 3 || bytes_for(S, tpb) > static_cast<unsigned>(lds_limit)) return false;
+    while (tpb > least_batch && bytes_for(S, tpb) > static_cast<unsigned>(lds_limit)) --tpb;
+    if (tpb < least_batch || bytes_for(S, tpb) > static_cast<unsigned>(lds_limit)) return false;
+    if (mode == 0 && want.batch_tiles == 0) tpb = 1u;
     unsigned P = want.prep_waves ? want.prep_waves : (ITEMS + tpb - 1u) / tpb;
     if (P * tpb < ITEMS) P = (ITEMS + tpb - 1u) / tpb;
     // one recursion per lane and tile where four waves suffice for that
-    unsigned NSEQ = want.sequence_waves ? want.sequence_waves : (S * SEQS * levels + 63u) / 64u;
+    unsigned NSEQ = want.sequence_waves      ? want.sequence_waves
+                    : model_sequence_waves != 0 ? model_sequence_waves
+                                                : (S * SEQS * levels + 63u) / 64u;
     if (NSEQ < 1) NSEQ = 1;
-    if (NSEQ > WAVES / 4u) NSEQ = WAVES / 4u;
+    if (NSEQ > (mode == 0 ? WAVES / 2u : WAVES / 4u)) NSEQ = mode == 0 ? WAVES / 2u : WAVES / 4u;
     if (P + NSEQ >= WAVES) return false;
     const unsigned room = WAVES - P - NSEQ;
     // the waves that hold a point's pairs, and as many points side by side as the entry waves allow
     unsigned slot_waves = 0, lane_slots = 0, E = 0;
-    if (mode == 1) {
+    if (mode <= 1) {
         slot_waves = pairs_lane_table(l_max, H, room, g.lane_job);
         if (slot_waves == 0) return false;
         unsigned slots = room / slot_waves;
@@ -168,7 +210,7 @@ inline bool plan_pairs(size_t n_samples, int l_max, int mode, size_t elem, size_
     g.lane_slots = lane_slots;
     unsigned at = align4(S * ny + line);
     g.off_dsph = at;
-    at = align4(at + S * 3 * ny + line);
+    if (mode >= 1) at = align4(at + S * 3 * ny + line);
     g.off_ddsph = at;
     if (mode == 2) at = align4(at + S * 9 * ny + line);
     g.tables_at = at * osize;
@@ -178,6 +220,7 @@ inline bool plan_pairs(size_t n_samples, int l_max, int mode, size_t elem, size_
     g.off_F0 = at;
     at += f0_elems;
     g.off_pts = at;
+    g.lookahead = tpb == 1u ? 2u : 1u;
     at += 2 * tpb * S * point_stride;
     g.off_park = at;
     at += 2 * tpb * S * park_stride;

@@ -18,6 +18,11 @@ struct PairsTiling {
     unsigned chunk_shift;    // a workgroup takes 2^chunk_shift consecutive tiles at a time
     unsigned batch_tiles;    // tiles per batch of point records and parked closed forms
     unsigned magic_batch;    // ceil(2^32 / batch_tiles)
+    // How many batches ahead of the tile being staged the records are prepared: 1, or 2 where a batch is a
+    // single tile (the recursions of tile n + 1 run while tile n is flushed, when its records must be complete;
+    // the records of tile n + 2 then take the place of those of tile n, which is staged by then). Two buffers of
+    // one batch each either way.
+    unsigned lookahead;
     unsigned prep_waves, sequence_waves, entry_waves;
     unsigned slot_waves;     // MODE 1: entry waves that share one point; entry_waves / slot_waves points side by side
     unsigned lane_slots;     // MODE 2: points side by side in the entry lanes (the lane table says which lane takes which)

@@ -909,6 +909,28 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
         plan_closed(n_samples, l_max, l_max, mode, elem, &plan->closed);
         return SPHX_OK;
     }
+    // Values alone where the rows of few points fill LDS: pairs_kernel (below, with the derivatives), which keeps
+    // the recursions of the next tile and the flush of this one side by side. 1.2 GB of output, us, against
+    // values_kernel (the recursion kernel from l_max = 34): float32 l_max = 22, 24, 26, 28, 30, 32, 34, 36 262,
+    // 254, 242, 252, 231, 219, 236, 243 against 262, 296, 293, 319, 318, 306, 379, 381; float64 l_max = 20, 24,
+    // 28, 32, 36 220, 222, 224, 215, 223 against 266, 301, 312, 298, 303; below (float32 l_max = 20 264 against
+    // 257, float64 l_max = 18 293 against 247) a point's pairs leave the entry lanes idle.
+    if (lane_kernels && mode == 0 && l_max > hard) {
+        const int pairs = switch_or(SW_PAIRS, 1);
+        const bool pairs_by_shape = n_samples >= 32768 && (elem == 4 ? l_max >= 23 : l_max >= 20);
+        if (pairs == 2 || (pairs == 1 && pairs_by_shape)) {
+            PairsChoice want;
+            want.tile = static_cast<unsigned>(switch_or(SW_PAIRS_TILE, 0));
+            want.batch_tiles = static_cast<unsigned>(switch_or(SW_PAIRS_BATCH, 0));
+            want.prep_waves = static_cast<unsigned>(switch_or(SW_PAIRS_PREP_WAVES, 0));
+            want.sequence_waves = static_cast<unsigned>(switch_or(SW_PAIRS_SEQUENCE_WAVES, 0));
+            want.chunk_shift_plus_one = static_cast<unsigned>(switch_or(SW_PAIRS_CHUNK, -1) + 1);
+            if (plan_pairs(n_samples, l_max, mode, elem, elem, lds_limit, cus, want, &plan->pairs_launch)) {
+                plan->pairs = true;
+                return SPHX_OK;
+            }
+        }
+    }
     if (lane_kernels && mode == 0 && plan_values(n_samples, l_max, elem, lds_limit, &plan->closed)) {
         plan->lanes = true;
         return SPHX_OK;

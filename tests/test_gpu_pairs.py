@@ -1,8 +1,8 @@
-"""pairs_kernel (derivatives, every entry lane bound to one (l, m) pair) against the oracle, number for number.
+"""pairs_kernel (every entry lane bound to one (l, m) pair) against the oracle, number for number.
 
-The planner gives it gradients in float32 from l_max = 20 and in float64 from l_max = 16, and second derivatives
-in float64 from l_max = 20, when a call has 32 768 points or more; here SPHX_PAIRS = 2 sends every shape it can
-hold through it, with the tile, batch and wave counts
+The planner gives it values alone in float32 from l_max = 23 and in float64 from l_max = 20, gradients in float32
+from l_max = 20 and in float64 from l_max = 16, and second derivatives in float64 from l_max = 20, when a call
+has 32 768 points or more; here SPHX_PAIRS = 2 sends every shape it can hold through it, with the tile, batch and wave counts
 the planner would pick and with forced ones, so that every path of the kernel runs at sizes the oracle
 finishes in seconds: partial last tiles, fewer tiles than workgroups, several points side by side in the
 entry waves, several rounds of recursions per tile, outputs that start anywhere inside a 128-byte line.
@@ -31,8 +31,9 @@ def _evaluate(library, xyz, l_max, normalized, shift=0, mode=1):
     out = [raw[i][shift:shift + sizes[i]].view(shapes[i]) for i in range(mode + 1)]
     forward = library.sphx_forward_f32 if xyz.dtype == np.float32 else library.sphx_forward_f64
     xyz_dev = torch.from_numpy(xyz).cuda()
-    status = forward(xyz_dev.data_ptr(), n, l_max, int(normalized), mode, out[0].data_ptr(), out[1].data_ptr(),
-                     out[2].data_ptr() if mode == 2 else None, torch.cuda.current_stream().cuda_stream)
+    status = forward(xyz_dev.data_ptr(), n, l_max, int(normalized), mode, out[0].data_ptr(),
+                     out[1].data_ptr() if mode >= 1 else None, out[2].data_ptr() if mode == 2 else None,
+                     torch.cuda.current_stream().cuda_stream)
     assert status == 0, library.sphx_last_error()
     torch.cuda.synchronize()
     guards = all(bool(torch.isnan(raw[i][:shift]).all() and torch.isnan(raw[i][shift + sizes[i]:]).all())
@@ -153,6 +154,37 @@ def test_second_derivatives(oracle, library, switches, dtype, normalized):
     assert ran >= 8
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("normalized", [True, False])
+def test_values_alone(oracle, library, switches, dtype, normalized):
+    """The same kernel without derivatives (one row per point, a batch is a single tile of up to 64 points, the
+    entry lanes take four points per turn): l_max 7 .. 36, planned and forced tiles, batches of several tiles,
+    few points, outputs that start anywhere inside a line."""
+    rng = np.random.default_rng(19)
+    ran = 0
+    for l_max, overrides in ((7, {}), (8, {"SPHX_PAIRS_TILE": 1}), (9, {"SPHX_PAIRS_TILE": 3, "SPHX_PAIRS_BATCH": 3}),
+                             (12, {}), (16, {"SPHX_PAIRS_TILE": 5, "SPHX_PAIRS_SEQUENCE_WAVES": 1}), (20, {}),
+                             (23, {"SPHX_PAIRS_TILE": 6, "SPHX_PAIRS_BATCH": 2, "SPHX_PAIRS_PREP_WAVES": 1}), (24, {}),
+                             (27, {"SPHX_PAIRS_SEQUENCE_WAVES": 8}), (28, {}), (31, {"SPHX_PAIRS_TILE": 7}), (32, {}),
+                             (33, {"SPHX_PAIRS_CHUNK": 2, "SPHX_PAIRS_TILE": 2}), (36, {})):
+        library.sphx_reset_switches()
+        switches("SPHX_PAIRS", 2)
+        for name, value in overrides.items():
+            switches(name, value)
+        for n in (1, 5, 70, 333):
+            text = _plan_text(library, n, l_max, dtype == np.float64, normalized, mode=0)
+            announce("pairs values", np.dtype(dtype).name, "normalized", normalized, "l_max", l_max, overrides, "n", n, text)
+            if not text.startswith("pairs_kernel"):
+                continue
+            ran += 1
+            xyz = special_points(dtype, rng, n)
+            want = oracle.compute(xyz, l_max, normalized, "values")
+            (sph, guards) = _evaluate(library, xyz, l_max, normalized, shift=int(rng.integers(0, 33)), mode=0)
+            assert same_numbers(sph, want[0]).all(), (l_max, overrides, n, "values")
+            assert guards, (l_max, overrides, n)
+    assert ran >= 40
+
+
 def test_planned_by_shape(library):
     """What the planner picks without overrides."""
     assert _plan_text(library, 200_000, 32, False, True).startswith("pairs_kernel<float, 1, true>")
@@ -163,6 +195,10 @@ def test_planned_by_shape(library):
     assert _plan_text(library, 100_000, 19, False, True).startswith("recursion_kernel")
     assert _plan_text(library, 100_000, 15, True, True).startswith("recursion_kernel")
     assert _plan_text(library, 20_000, 32, False, True).startswith("recursion_kernel")  # few points
-    # second derivatives in float32 and values alone stay where they were
-    assert not _plan_text(library, 200_000, 32, False, True, mode=0).startswith("pairs")
+    assert _plan_text(library, 200_000, 32, False, True, mode=0).startswith("pairs_kernel<float, 0, true>")
+    assert _plan_text(library, 200_000, 20, True, False, mode=0).startswith("pairs_kernel<double, 0, false>")
+    assert _plan_text(library, 200_000, 22, False, True, mode=0).startswith("values_kernel")
+    assert _plan_text(library, 200_000, 19, True, True, mode=0).startswith("values_kernel")
+    assert _plan_text(library, 20_000, 32, False, True, mode=0).startswith("values_kernel")  # few points
+    # second derivatives in float32 stay where they were
     assert not _plan_text(library, 200_000, 24, False, True, mode=2).startswith("pairs")

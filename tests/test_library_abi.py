@@ -98,18 +98,23 @@ def test_launch_plans(library):
     assert library.sphx_describe_plan(100_000, 16, 2, 1, 1, text, 512) == 0
     assert "512 threads" in text.value.decode()
     # values: as many points per workgroup as fit in half a CU's LDS, in steps of four; in float32
-    # one workgroup with all of LDS while 40 points fit, then the recursion kernel
+    # one workgroup with all of LDS while 40 points fit; from l_max = 23 (float64: 20) pairs_kernel with as
+    # many points per tile as fit (and the lanes kernel again where there are few points)
     status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 16, 0, False)
     assert status == 0 and (tile, threads) == (60, 512) and lds == 60 * (289 + 51) * 4
     status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 28, 0, False)
+    assert status == 0 and (tile, threads, groups) == (25, 1024, 256) and 150_000 < lds <= 160 * 1024
+    status, (tile, threads, lds, groups) = _plan(library, 20_000, 28, 0, False)
     assert status == 0 and (tile, threads) == (44, 768) and 80 * 1024 < lds <= 160 * 1024
     # tiles of 32 and 16 points: two and four channels side by side in a wave
     assert _plan(library, 1_000_000, 22, 0, False)[1][:2] == [32, 512]
-    assert _plan(library, 1_000_000, 26, 0, False)[1][:2] == [16, 320]
-    assert _plan(library, 1_000_000, 32, 0, False)[1][:2] == [32, 832]
-    assert _plan(library, 1_000_000, 34, 0, False)[1][1] == 1024
-    assert _plan(library, 1_000_000, 22, 0, True)[1][:2] == [32, 1024]
-    assert _plan(library, 1_000_000, 23, 0, True)[1][1] == 1024
+    assert _plan(library, 20_000, 26, 0, False)[1][:2] == [16, 320]
+    assert _plan(library, 20_000, 32, 0, False)[1][:2] == [32, 832]
+    assert _plan(library, 20_000, 34, 0, False)[1][1] == 1024
+    assert _plan(library, 20_000, 22, 0, True)[1][:2] == [32, 1024]
+    assert _plan(library, 20_000, 23, 0, True)[1][1] == 1024
+    assert _plan(library, 1_000_000, 32, 0, False)[1][:2] == [20, 1024]
+    assert _plan(library, 1_000_000, 24, 0, True)[1][0] == 16
     assert _plan(library, 10, 65, 0, False)[0] == 2       # beyond the tables
     assert _plan(library, 10, 64, 2, True)[0] == 2        # one point's rows no longer fit in LDS
     assert b"LDS" in library.sphx_last_error()
@@ -142,6 +147,7 @@ def test_planner_overrides(library, switches):
     assert _plan(library, 50_000, 20, 1, False) == default
     # four channels side by side in a wave: that kernel exists for up to eight waves, whatever the shape asks
     switches("SPHX_VALUES_PACK", 4)
+    switches("SPHX_PAIRS", 0)
     for l_max in (25, 33, 39, 40):
         status, (tile, threads, _, _) = _plan(library, 100_000, l_max, 0, False)
         assert status == 0 and threads <= 512, (l_max, tile, threads)
