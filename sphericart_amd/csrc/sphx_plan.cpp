@@ -8,6 +8,7 @@
 #include <mutex>
 
 #include "../../include/sphx_launch.h"
+#include "sphx_plan_shapes.hpp"
 
 namespace sphx {
 
@@ -123,8 +124,9 @@ static void plan_closed(size_t n_samples, int l_max, int hard, int mode, size_t 
     out->lds_bytes = at * static_cast<unsigned>(elem);
 }
 
-// values_kernel: up to 64 points per workgroup, their rows and tables in LDS. Returns false
-// when that does not fit, and the recursion kernel takes over.
+// values_kernel: up to 64 points per workgroup, their rows and tables in LDS. Returns false when that does not
+// fit, and the recursion kernel takes over. `with_sums`: the same layout for the lane kernels of the fused
+// product, which keep no rows for HBM but the sums of their waves.
 static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit, Launch* out,
                         bool with_sums = false) {
     Tiling& g = out->g;
@@ -139,100 +141,25 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     const unsigned tri_all = static_cast<unsigned>(l_max + 1) * (l_max + 2) / 2;
     unsigned allowed = static_cast<unsigned>(switch_or(SW_VALUES_LDS, 160 * 1024));
     if (allowed > static_cast<unsigned>(lds_limit)) allowed = static_cast<unsigned>(lds_limit);
-    // Fewer than 64 points per workgroup leave lanes idle, and from some tile on the recursion
-    // kernel with its job list is faster. Values, 1 GB of output, us, values kernel against
-    // recursion kernel: float32 with two workgroups per CU l_max = 24 (28 points) 306 against 397,
-    // l_max = 26 (24 points) 338 against 392; with one workgroup per CU l_max = 28 (44 points) 355
-    // against 393, l_max = 29 (40) 370 against 390, l_max = 30 (38) 419 against 391; float64
-    // l_max = 22 (32 points) 297 against 305, l_max = 23 (30) 319 against 302.
-    // The product keeps no rows for HBM in LDS and has far more arithmetic per point to win:
-    // it goes down to 8 points (l_max = 24 float64, 200k points: 830 us with 16 points per
-    // workgroup against 1 456 us through the recursion kernel).
+    // Fewer than 64 points per workgroup leave lanes idle, and from some tile on the recursion kernel with its
+    // job list is faster: values stop at 24 points in float32 and 32 in float64. The product has far more
+    // arithmetic per point to win and goes down to 8 points.
     const unsigned smallest = static_cast<unsigned>(
         with_sums ? switch_or(SW_VJP_MIN_TILE, 8) : switch_or(SW_VALUES_MIN_TILE, elem == 4 ? 24 : 32));
-    // Between tiles of 24-44 points, with lanes idle, and the recursion kernel lie two more forms
-    // of the values kernel: one workgroup per CU with all of its LDS, up to 64 points and up to
-    // sixteen waves, and tiles of 32 or 16 points whose waves evaluate two or four channels side
-    // by side, all lanes at work. Which is fastest goes by the shape, not by a rule (row lengths,
-    // channels per wave and workgroups per CU all change with l_max). 1 GB of values, us, in the
-    // order: tile that fits half of LDS / one workgroup with all of LDS / two channels, 32 points,
-    // in half of LDS / the same with all of LDS / four channels, 16 points / recursion kernel.
-    // float32:
-    //   l_max 18 216 263 216 224 249 412    l_max 19 248 285 291 290 289 418    l_max 20 238 270 250 250 279 403
-    //   l_max 21 254 262 248 252 268 397    l_max 22 271 260 238 239 260 389    l_max 23 319 288   - 427 341 425
-    //   l_max 24 285 287   - 373 296 398    l_max 25 319 295   - 366 286 397    l_max 26 317 300   - 350 275 393
-    //   l_max 27   - 333   - 359 393 419    l_max 28   - 317   - 334 354 393    l_max 29   - 329   - 326 342 389
-    //   l_max 30   - 357   - 317 332 391    l_max 31   - 360   - 324 348 389    l_max 32   - 368   - 300 313 378
-    //   l_max 33   - 365   - 297 305 386    l_max 34   - 404   - 418   - 383
-    // float64:
-    //   l_max 13 220 243   - 282 310 313    l_max 14 224 212   - 239 309 310    l_max 15 258 225   - 257 326 347
-    //   l_max 16   - 228   - 360 335 322    l_max 20   - 252   - 299 363 313    l_max 21   - 273   - 303 365 296
-    //   l_max 22   - 273   - 281 328 303    l_max 23   - 326   -   - 582 301
-    // (Sixteen waves for a workgroup alone on its CU: float64 l_max = 16-21 239, 255, 248, 268, 272, 291 us
-    // with eight, 228, 236, 228, 259, 252, 273 with up to sixteen; float32 l_max = 27, 28 340, 327 with
-    // eight, 337, 326 with sixteen, 333, 317 with twelve.)
-    unsigned pack_by_shape = 1;
-    bool alone_by_shape = false;
-    if (!with_sums && elem == 4) {
-        if (l_max == 21 || l_max == 22 || (l_max >= 29 && l_max <= 33)) pack_by_shape = 2;
-        if (l_max == 25 || l_max == 26) pack_by_shape = 4;
-        alone_by_shape = l_max == 23;
-    } else if (!with_sums) {
-        alone_by_shape = l_max == 14 || l_max == 15;
-    }
-    // The product: tiles go down in steps of four points to 32 and halve from there, to 16 and 8
-    // points with groups of lanes (vjp_groups_kernel). One workgroup with all of LDS is faster on
-    // some shapes, with a number of waves that goes by the shape as well (the channels and the
-    // eight closed-form slices share the waves; more than eight waves need twice the room for
-    // their sums, which can cost points). 200k points (400k to l_max = 16), us, tiles in half of LDS /
-    // one workgroup per CU with 8 / with up to 12 waves, float64:
-    //   l_max 13 257 261 261    l_max 14 498 287 286    l_max 15 519 328 324    l_max 16 538 383 360
-    //   l_max 17 289 228 214    l_max 18 299 261 240    l_max 19 315 290 272    l_max 20 330 336 316
-    //   l_max 21 588 375 620    l_max 22 613 556 557    l_max 23 627 588 589    l_max 24 640 610 610
-    //   l_max 25 660 649 650    l_max 26 675 689 690    l_max 29 804 804 804
-    // float32 (l_max = 21, 31 with 16 waves 162, 423):
-    //   l_max 19 144 153 135    l_max 20 155 168 154    l_max 21 181 178 172    l_max 22 211 168 185
-    //   l_max 23 216 212 201    l_max 24 222 244 224    l_max 25 335 274 255    l_max 26 340 294 276
-    //   l_max 27 348 289 313    l_max 28 356 318 342    l_max 29 385 404 370    l_max 30 397 381 422
-    //   l_max 31 477 436 442    l_max 32 500 470 645    l_max 33 510 675 676    l_max 34 518 694 695
-    //   l_max 35 789 725 726    l_max 36 807 748 748    l_max 37 820 773 773    l_max 40 874 852 851
-    // (Tiles that halved all the way: float64 l_max = 10, 15, 16, 17 153, 405, 459, 259 us against 139, 340,
-    // 393, 230 with the same number of waves; float32 l_max = 15, 17, 18 166, 118, 135 against 153, 97, 114.)
-    // (On some shapes the steps of four go on below 32 points, to tiles of 28, 24 and 20 for the
-    // lanes kernel, before the groups of lanes take over. With that, one workgroup per CU with 8 /
-    // 12 waves against the best of the above: float64 l_max = 21 375 364 against 375, l_max = 22 444
-    // 405 against 559, l_max = 23 468 464 against 589, l_max = 24 565 564 against 611, l_max = 25 598
-    // 602 against 649, l_max = 26 719 661 against 677; float32 l_max = 35 692 642 against 725,
-    // l_max = 36 678 667 against 749, l_max = 37 718 792 against 773, l_max = 43 866 868 against 909.)
-    int waves_by_shape = 0;
-    unsigned floor_by_shape = 32;
-    if (with_sums && elem == 8) {
-        if (l_max >= 14 && l_max <= 26) waves_by_shape = l_max == 25 ? 8 : 12;
-        if (l_max >= 21 && l_max <= 26) floor_by_shape = 16;
-    } else if (with_sums) {
-        if (l_max == 19 || l_max == 23 || l_max == 25 || l_max == 26 || l_max == 29 || l_max == 35 || l_max == 36) {
-            waves_by_shape = 12;
-        }
-        if (l_max == 21 || l_max == 31) waves_by_shape = 16;
-        if (l_max == 22 || l_max == 27 || l_max == 28 || l_max == 30 || l_max == 32 || (l_max >= 37 && l_max <= 40) ||
-            l_max == 43) {
-            waves_by_shape = 8;
-        }
-        if ((l_max >= 35 && l_max <= 37) || l_max == 43) floor_by_shape = 16;
-    }
-    if (waves_by_shape != 0) alone_by_shape = true;
-    const bool alone = switch_or(SW_VALUES_ALONE, alone_by_shape ? 1 : 0) != 0;
+    // Which form of the kernel goes by the shape (sphx_plan_shapes.hpp): tiles of 64 / pack points whose waves
+    // evaluate `pack` channels side by side, all lanes at work; one workgroup per CU with all of its LDS and up
+    // to sixteen waves, or two with half of it each.
+    const ShapeRow* shape = shape_row(with_sums ? 1 : 0, static_cast<int>(elem), l_max);
+    const unsigned pack_by_shape = shape ? shape->pack : 1u;
+    const int waves_by_shape = shape ? shape->waves : 0;
+    const unsigned floor_by_shape = shape ? shape->floor : 32u;
+    const bool alone = switch_or(SW_VALUES_ALONE, shape && shape->alone ? 1 : 0) != 0;
     const unsigned smallest_alone = !with_sums && elem == 4 && smallest < 40 && !alone ? 40 : smallest;
-    // Values: the tile goes down in steps of 4 points, so that as many lanes work as rows fit
-    // (l_max = 16: 60 points where halving leaves 32, 202 against 278 us in float32, 240 against
-    // 352 in float64; steps of 1 or 2 gain nothing more and some odd sizes lose). The product halves.
-    // (the product: the same above 32 points, halves from there down, for the groups of lanes of
-    // vjp_groups_kernel)
+    // The tile goes down in steps of four points, so that as many lanes work as rows fit; the product's halves
+    // from `floor` on, for the groups of lanes of vjp_groups_kernel.
     const unsigned step = static_cast<unsigned>(with_sums ? switch_or(SW_VJP_TILE_STEP, 4) : switch_or(SW_VALUES_TILE_STEP, 4));
-    // Two workgroups per CU (80 KB each) overlap one's tables and flush with the other's
-    // arithmetic: preferred, also with fewer lanes at work, over one workgroup with all of LDS
-    // (l_max = 16 float32, 500k points, 32 points against 64: 142 against 164 us; l_max = 12
-    // float64: 115 against 146).
+    // Two workgroups per CU (80 KB each) overlap one's tables and flush with the other's arithmetic: preferred,
+    // also with fewer lanes at work, over one workgroup with all of LDS unless the shape says otherwise.
     const unsigned half = 80u * 1024u;
     unsigned tile = 0, rows = 0, bytes = 0, sums_elems = 0;
     const unsigned step_floor = static_cast<unsigned>(switch_or(SW_VJP_STEP_FLOOR, static_cast<int>(floor_by_shape)));
@@ -292,9 +219,8 @@ static bool plan_values(size_t n_samples, int l_max, size_t elem, int lds_limit,
     // (the product's closed-form slices want at least four; values: one for the tables, one for
     // the closed forms)
     int want = (l_max - 6 + static_cast<int>(pack) - 1) / static_cast<int>(pack);
-    // the product, 0.8 GB of sph_grad, us: l_max = 9, 10 (three and four channels) 266, 310 with
-    // four waves, 207, 282 with three (float64 279, 333 against 233, 304); l_max = 12 350 with six,
-    // 316 with four (float64 385 against 321); one or two channels are best with four
+    // (the product: one or two channels are best with four waves, three or four channels with three, five or
+    // six with four)
     if (with_sums) want = want <= 2 ? 4 : (want <= 4 ? 3 : (want <= 6 ? 4 : want));
     if (!with_sums && want < 2) want = switch_or(SW_VALUES_MIN_WAVES, 2);
     out->threads = 64u * static_cast<unsigned>(want < waves ? want : waves);
@@ -316,19 +242,13 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     // (closed forms only, l_max <= 6: no tables)
     const unsigned table_stride = l_max <= 6 ? 0u : (3u * static_cast<unsigned>(l_max + 1)) | 1u;
     const unsigned limit = static_cast<unsigned>(lds_limit);
-    // Which tile: the one that keeps most points resident on a CU (tile times the workgroups
-    // that fit), a tile of 16 counted at three quarters because it leaves three lanes in four
-    // idle; between equals the larger tile, unless its workgroup would be alone on the CU (two
-    // overlap one another's phases). Measured, 500k points, float32: l_max = 7 105 us with
-    // 2 x 64 points against 119 with 4 x 32; l_max = 9 173 us with 2 x 32 against 186 with 64;
-    // l_max = 13 357 us with 3 x 16 against 433 with 32; l_max = 15 579 us with 32 against 651
-    // with 2 x 16. Below 32 resident points (or 3 x 16) the recursion kernel is the faster one
-    // (l_max = 18: 1 038 us against 1 236).
-    // Few points (one workgroup per CU can take them all): the time of the call is the time of
-    // one workgroup, and every workgroup beyond one per CU makes the waves of a CU queue for its
-    // vector ALUs with most of their lanes idle. Then the tile is N / CUs, rounded up to a
-    // multiple of four: cfg1 (10 000 points, float64 l_max = 8) 11.8 us with 632 tiles of 16,
-    // 16.1 us with 320 tiles of 32 (one per CU at a time: two rounds), see below for tiles of 40.
+    // Which tile: the one that keeps most points resident on a CU (tile times the workgroups that fit), a tile of
+    // 16 counted at three quarters because it leaves three lanes in four idle; between equals the larger tile,
+    // unless its workgroup would be alone on the CU (two overlap one another's phases). Below 32 resident points
+    // (or 3 x 16) the recursion kernel is the faster one.
+    // Few points (one workgroup per CU can take them all): the time of the call is the time of one workgroup, and
+    // every workgroup beyond one per CU makes the waves of a CU queue for its vector ALUs with most of their lanes
+    // idle. Then the tile is N / CUs, rounded up to a multiple of four.
     unsigned few = 0;
     const unsigned forced_tile = static_cast<unsigned>(switch_or(SW_GRADIENT_LANES_TILE, 0));
     if (cus > 0 && n_samples <= static_cast<size_t>(cus) * 64u) {
@@ -345,10 +265,9 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
         const unsigned b = (ot + t * table_stride) * esize;
         if (b > limit) continue;
         unsigned score = (limit / b) * t * (t >= 32 ? 4u : 3u);
-        // l_max = 6, closed forms only: 32 points per workgroup, half the lanes idle, but twice as
-        // many workgroups in different phases on a CU (1M points, float32: 127 us against 140 us
-        // with 64 points; a tile of 32 rows of 49 numbers is a whole number of 128-byte lines,
-        // tiles of 24, 28, 36, 40, 48 points took 143-164 us)
+        // l_max = 6, closed forms only: 32 points per workgroup, half the lanes idle, but twice as many workgroups in
+        // different phases on a CU, and a tile of 32 rows of 49 numbers is a whole number of 128-byte lines (1M points,
+        // float32: 127 us against 140 us with 64 points)
         if (l_max == 6 && t == 32) score = 1u << 28;
         if (t == few) score = 1u << 29;
         if (forced_tile == t) score = 1u << 30;
@@ -375,19 +294,11 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     g.off_pts = off_t;
     g.off_iter = table_stride;
     out->workgroups = g.tiles_per_xcd * 8u;
-    // Eight waves share the closed-form slices and the channels; with one or two channels four
-    // are enough and leave room for more workgroups (1.5 GB of output: float64 l_max = 8 469 us
-    // with eight waves, 345 with four; float32 l_max = 7, 8 286, 274 against 273, 261; from three
-    // channels on eight waves are faster, l_max = 12: 357 against 411).
-    // (few points: one workgroup per CU, occupancy is no concern and eight waves shorten the
-    // longest chain of work in the workgroup)
-    // (closed forms only, l_max <= 6: eight; six for normalised float32 at l_max = 6, 127 us
-    // against 130 us with eight and 136-138 us with four or five)
-    // (few points, three channels or more, or float64 tiles of up to 16 points: sixteen waves, two
-    // to a channel where that leaves four for the closed forms; 10 000 points, us, eight waves
-    // against sixteen: float32 l_max = 10 9.5 against 8.6, l_max = 12 11.8 against 10.9; float64
-    // l_max = 8 with 2 000 points 8.0 against 6.2; one or two channels at 40 points per tile gain
-    // nothing, float64 l_max = 8 9.2 against 9.1, l_max = 7 7.9 against 8.3)
+    // Eight waves share the closed-form slices and the channels; with one or two channels four are enough and
+    // leave room for more workgroups. Closed forms only (l_max <= 6): eight, six for normalised float32 at
+    // l_max = 6. Few points (one workgroup per CU, occupancy is no concern): eight waves shorten the longest chain
+    // of work in the workgroup, and with three channels or more, or float64 tiles of up to 16 points, sixteen do,
+    // two to a channel where that leaves four for the closed forms.
     const bool many = tile == few && l_max > 6 && (l_max >= 9 || (elem == 8 && tile <= 16));
     const int by_shape = l_max <= 6 ? (l_max == 6 && elem == 4 && normalized && tile != few ? 6 : 8)
                                     : (l_max <= 8 && tile != few ? 4 : (many ? 16 : 8));
@@ -396,13 +307,9 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     waves = waves < 1 ? 1 : (waves > most ? most : waves);
     out->threads = 64u * static_cast<unsigned>(waves);
     out->lds_bytes = bytes;
-    // Few points, one or two channels: two waves per channel, each with half of its m (the longest
-    // chain of the one workgroup a CU has is then half a channel or two slices of the closed
-    // forms, not a whole channel). Measured on one device, one wave per channel against two, us:
-    // float64 10 000 points l_max = 8 10.0 against 9.0, l_max = 7 8.7 against 7.8; float32
-    // l_max = 8 7.6 against 6.7, 2 000 points 7.0 against 5.6. With three channels two waves are
-    // left for the eight slices and nothing is gained (float64 l_max = 9 10.2 against 10.5), with
-    // four channels none (l_max = 10: 9.5 against 9.1 in float32, 9.9 against 10.2 in float64).
+    // Few points, one or two channels: two waves per channel, each with half of its m (the longest chain of the
+    // one workgroup a CU has is then half a channel or two slices of the closed forms, not a whole channel; cfg1
+    // 10.0 -> 9.0 us). With three channels or more too few waves are left for the slices and nothing is gained.
     const unsigned channels = l_max > 6 ? static_cast<unsigned>(l_max - 6) : 0u;
     const bool halves = tile == few && channels >= 1 && (channels <= 2 ? waves >= 8 : 2u * channels + 4u <= static_cast<unsigned>(waves));
     const int parts = switch_or(SW_GRADIENT_LANES_PARTS, halves ? 2 : 1);
@@ -424,10 +331,9 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
     const unsigned table_stride = (3u * static_cast<unsigned>(l_max + 1)) | 1u;
     const unsigned channels = static_cast<unsigned>(l_max - 1);
     const unsigned most = (elem == 4 ? hessian_lane_threads<float>() : hessian_lane_threads<double>()) / 64u;
-    // Waves per channel, each with a part of its m: two where one or two channels would leave the
-    // workgroup with one or two waves (80 MB of output, us, one against two: float32 l_max = 3
-    // 99 against 83, solid 80 against 70, 20 000 points 10.9 against 9.1; l_max = 2 74 against 70,
-    // solid 58 against 61; float64 l_max = 3 solid 85 against 73, normalised 105 against 151).
+    // Waves per channel, each with a part of its m: two where one or two channels would leave the workgroup with
+    // one or two waves and that measured faster (l_max = 3 in float32 and for solid harmonics in float64, l_max = 2
+    // for normalised float32: 10-20 %).
     const bool shared = (l_max == 3 && (elem == 4 || !normalized)) || (l_max == 2 && elem == 4 && normalized);
     unsigned parts = static_cast<unsigned>(switch_or(SW_HESSIAN_LANES_PARTS, shared ? 2 : 1));
     if (parts != 1 && parts != 2 && parts != 4) parts = 1;
@@ -478,29 +384,19 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
     return true;
 }
 
-// Threads per workgroup of the recursion kernel: 512, two workgroups to a CU, or 1024, one
-// workgroup with all of the CU's LDS and tiles of twice as many points (not the fused product,
-// and not second derivatives in float64, whose entry jobs need more than the 128 registers a
-// lane of sixteen waves has). Two workgroups of 512 on a CU run their stages and
-// their flushes against each other as chance has it, and a tile of one or two points leaves the
-// entry lanes and the sequence lanes half idle in their last rounds; one workgroup of 1024
-// measured, 1.2 GB of output, us, 512 against 1024: gradients float32 l_max = 14, 20, 24, 28,
-// 32, 36 283, 306, 323, 329, 331, 342 against 245, 249, 259, 253, 267, 268 (l_max = 40 288
-// against 290); float64 l_max = 12, 16, 20, 24, 32 303, 307, 320, 271, 266 against 239, 233,
-// 252, 248, 249; second derivatives float32 l_max = 4, 8, 12, 16, 20, 24 252, 262, 271, 258,
-// 334, 361 against 231, 239, 238, 238, 245, 266; solid harmonics alike; values, whose entries
-// are three multiplications, gain less: float32 l_max = 24, 32, 40 405, 383, 378 against 396,
-// 377, 376, float64 l_max = 24, 28, 32 317, 322, 335 against 292, 305, 297. With few points
-// (below 4 096) 512 threads stay: more workgroups have a tile then.
+// Threads per workgroup of the recursion kernel: 512, two workgroups to a CU, or 1024, one workgroup with all of
+// the CU's LDS and tiles of twice as many points. Two workgroups of 512 on a CU run their stages and their
+// flushes against each other as chance has it, and a tile of one or two points leaves the entry lanes and the
+// sequence lanes half idle in their last rounds: one workgroup of 1024 is 10-25 % faster with derivatives and
+// up to 8 % with values alone (profiles/sweep.json was made with this rule). With few points (below 4 096) 512
+// threads stay: more workgroups have a tile then. Not the fused product, which has no such kernel.
 // SPHX_GROUP_THREADS = 512 or 1024 overrides the rule.
 static unsigned group_threads(size_t n_samples, int mode, size_t elem, bool forward, bool normalized = true,
                               int l_max = -1) {
-    // Second derivatives in float64: the entries (l, +m) and (l, -m) as one job need 169-237 registers per lane.
-    // As two jobs, solid harmonics need 121, which sixteen waves allow (normalised 181: those keep eight waves).
-    // 1.2 GB of output, us, 512 threads against 1024 with the two sides as two jobs in one list: l_max = 4, 5, 6, 8,
-    // 10, 12, 14, 16, 18, 20, 22 251, 244, 247, 259, 253, 216, 225, 227, 220, 226, 231 against 201, 204, 205, 204,
-    // 208, 211, 205, 215, 206, 221, 216; cfg4 538 against 507; l_max = 3 305 against 243. At l_max = 2 the list is
-    // three jobs a point: 219 against 227.
+    // Second derivatives in float64: the entries (l, +m) and (l, -m) as one job need 169-237 registers per lane,
+    // more than the 128 that sixteen waves leave. As two jobs solid harmonics need 121 (normalised 181: those keep
+    // eight waves) and gain 5-20 % from l_max = 3 on (cfg4 538 -> 507 us); at l_max = 2 the list is three jobs a
+    // point and eight waves are as fast.
     const bool solid_f64_hessians = mode == 2 && elem == 8 && !normalized;
     const bool exists = forward && (mode <= 1 || (mode == 2 && elem == 4) || solid_f64_hessians);
     if (!exists) return kRecursionThreads;
@@ -551,31 +447,21 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         if (bytes_for(1) <= limit || !may_split) break;
         may_split = false; // the longer job table is what does not fit
     }
-    // (One row buffer. A second one, flushed by a wave of its own while the next tile is computed,
-    // was built and measured: it once paid where a single buffer holds one or two points (second
-    // derivatives l_max = 16, float64: 770 us against 810 us), but a wave that flushes alone waits
-    // for its own LDS loads most of the time and the entry waves lose a wave and half the points
-    // per tile. 400 MB of output, us, two buffers against one: second derivatives float32
-    // l_max = 20, 22, 28 157, 122, 167 against 121, 100, 105 (solid 109, 96 against 88, 79);
-    // float64 l_max = 20, 22 149, 134 against 126, 105. Its loop is no longer in the kernel,
-    // which is 1-4 % faster without it.)
+    // (One row buffer. A second one, flushed by a wave of its own while the next tile is computed, measured 20-60 %
+    // slower from l_max = 20 on: a wave that flushes alone waits for its own LDS loads most of the time, and the
+    // entry waves lose a wave and half the points per tile.)
     if (bytes_for(1) > limit) return false;
     unsigned S = 1;
     if (bytes_for(1) <= budget) {
-        // as many points as the budget holds, a power of two or not: fewer barrier rounds per
-        // point (2 GB of output, gradients, float64 l_max = 13: 824 us with 4 points per tile,
-        // 611 with 7; l_max = 14: 705 with 4, 602 with 6; float32 l_max = 21: 639 with 4, 603
-        // with 6; second derivatives, float64 l_max = 12: 783 with 2, 547 with 3; never more
-        // than 4 % slower than the power of two below)
+        // as many points as the budget holds, a power of two or not: fewer barrier rounds per point (up to 30 %
+        // faster, never more than 4 % slower than the power of two below)
         S = (budget - fixed) / point_bytes;
         if (switch_or(SW_TILE_POW2, 0) != 0) S = pow2_floor(S);
         if (S > 64) S = 64;
     }
-    // Few points: with the largest tile there would be fewer tiles than workgroups that a launch
-    // keeps resident. Then the tile is just large enough to give every one of them a tile (for
-    // values and gradients four points at least: below that the closed forms of l <= 6 weigh
-    // too much). 500 points, us: second derivatives float64 l_max = 6 16.1 -> 10.2, l_max = 16
-    // 16.6 -> 12.6, float32 l_max = 12 17.5 -> 11.2; gradients float32 l_max = 20 23.9 -> 12.7.
+    // Few points: with the largest tile there would be fewer tiles than workgroups that a launch keeps resident.
+    // Then the tile is just large enough to give every one of them a tile (for values and gradients four points
+    // at least: below that the closed forms of l <= 6 weigh too much). 500 points: 16-24 us -> 10-13 us.
     if (S > 1 && switch_or(SW_TILE_SMALL_N, 1) != 0) {
         unsigned per_cu = limit / bytes_for(S);
         per_cu = per_cu < 1 ? 1u : (per_cu > 2 ? 2u : per_cu);
@@ -618,15 +504,10 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.ny = static_cast<int>(ny);
     g.tile = static_cast<int>(S);
     g.az_shift = az_shift;
-    // Waves of their own for the closed forms of l <= 6 (whole rows): with sixteen waves and
-    // float32 gradients, where the tile otherwise waits for the entry waves that carry a slice on
-    // top of their jobs; one of them up to eight points per tile, two from nine on, three from 28
-    // on (l_max = 8, 9, 10, 12, 13 with two 224, 226, 226, 233, 244 us, with three 209, 216, 222,
-    // 231, 241). 1.2 GB of
-    // output, us, three sequence waves and the slices on all waves against two sequence waves and
-    // one / two slice waves: l_max = 14, 18, 24, 28, 32, 36, 40 252, 253, 263, 256, 270, 270, 296
-    // against 250, 241, 253, 248, 254, 260, 275 / 237, 237, 248, 254, 255, 262, 271. In float64 the
-    // closed forms are too much for two or three waves (l_max = 16: 258 against 340 / 300 us).
+    // Waves of their own for the closed forms of l <= 6 (whole rows): with sixteen waves and float32 gradients, where
+    // the tile otherwise waits for the entry waves that carry a slice on top of their jobs; one of them up to eight
+    // points per tile, two from nine on, three from 28 on (3-6 % at l_max = 8 .. 40). In float64 the closed forms are
+    // too much for two or three waves.
     g.slice_waves = 0;
     const bool slices_apart = threads > kRecursionThreads && mode == 1 && elem == 4;
     if (whole && mode < 2) {
@@ -634,15 +515,11 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         g.slice_waves = want < 0 ? 0u : (want > 4 ? 4u : static_cast<unsigned>(want));
     }
     g.sequence_waves = S * arrays * static_cast<unsigned>(l_max - hard) > 64 ? 2u : 1u;
-    // Split the sides when that lets the entries of a tile go through the entry waves in fewer
-    // rounds than it costs, a one-sided job being about 0.6 of a two-sided one. Normalised
-    // float32 is the exception: always split, because the two-sided kernel needs 152 registers
-    // per lane, so that only one workgroup fits on a CU, and the one-sided 116 (1.5 GB of
-    // output, l_max = 5, 16 points per tile: 895 against 652 us; l_max = 10, 8 points: 826
-    // against 598; l_max = 12, 4 points: 1 005 against 642; l_max = 15, 4 points: 780 against
-    // 460). For solid harmonics in float32 both fit twice (119 and 88 registers) and the rule
-    // holds (l_max = 10: 319 us by the rule, 404 always split; l_max = 12: 327 against 399);
-    // float64 with the sides always split loses 10-20 % at most l_max.
+    // Split the sides when that lets the entries of a tile go through the entry waves in fewer rounds than it
+    // costs, a one-sided job being about 0.6 of a two-sided one. Normalised float32 is the exception: always split,
+    // because the two-sided kernel needs 152 registers per lane, so that only one workgroup of 512 threads fits on
+    // a CU, and the one-sided 116. For solid harmonics in float32 both fit twice (119 and 88 registers) and the
+    // rule holds; float64 with the sides always split loses 10-20 % at most l_max.
     const unsigned one_side_costs = static_cast<unsigned>(switch_or(SW_SPLIT_RATIO, elem == 4 && normalized ? 1 : 6));
     unsigned wide = 0;
     auto per_pass = [&](unsigned j) { return j >= wide ? 1u : wide / j; };
@@ -659,34 +536,22 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // rounds of the entry waves per tile, in tenths of two-sided jobs, with `waves` sequence waves
     auto entry_cost = [&](unsigned waves, bool* split) {
         wide = threads - 64 * (1 + waves + g.slice_waves);
-        // (with two or more points per tile the jobs go as a list ordered by kind, which fills the
-        // lanes without splitting, and the two-sided job shares the common factors: 400 MB of
-        // output, us, split against not, normalised float32 l_max = 4, 8, 16, 20 110, 115, 108,
-        // 121 -> 104, 100, 96, 113; solid l_max = 6, 12 94, 92 -> 83, 83; with one point per tile
-        // splitting stays, l_max = 24, 28 117, 104 against 184, 166)
+        // (with two or more points per tile the jobs go as a list ordered by kind, which fills the lanes without
+        // splitting, and the two-sided job shares the common factors: 5-15 % faster; with one point per tile
+        // splitting stays)
         *split = may_split && S < 2 && one_side_costs * rounds(jobs_split) < 10 * rounds(jobs);
         // (float64 in workgroups of 1024 threads: only the one-sided job fits a lane's 128 registers)
         if (may_split && mode == 2 && elem == 8 && threads > kRecursionThreads) *split = true;
         return *split ? one_side_costs * rounds(jobs_split) : 10 * rounds(jobs);
     };
-    // A second sequence wave takes a wave from the entries. One is enough where it saves the
-    // entry waves a round per tile, and for values alone, whose recursions are a third of the
-    // work (1.5 GB of output, one against two: gradients float32 l_max = 18, 19 437, 449 against
-    // 545, 595 us; float64 l_max = 15, 16, 18 475, 423, 428 against 522, 460, 494; second
-    // derivatives float32 l_max = 10, 13 496, 490 against 637, 637; values float32 l_max = 40,
-    // 48 468, 428 against 527, 477; with equal rounds two are faster by 2-3 % with derivatives).
-    // Second derivatives in float64 follow no such rule (l_max = 6, 8, 10: 555, 437, 505 against
-    // 449, 558, 445) and keep two.
+    // A second sequence wave takes a wave from the entries. One is enough where it saves the entry waves a round
+    // per tile, and for values alone, whose recursions are a third of the work; with equal rounds two are faster by
+    // 2-3 % with derivatives. Second derivatives in float64 follow no such rule and keep two.
     if (threads > kRecursionThreads) {
-        // Sixteen waves: the tile is larger, the recursions of a tile more, and the tile waits for
-        // them if they need many rounds. Measured with two, three and four sequence waves (1.2 GB
-        // of output, us): gradients float32 l_max = 12, 16, 20, 24, 28, 32 249, 257, 252, 265, 255,
-        // 272 / 238, 245, 249, 259, 253, 267 / 244, 248, 264, 272, 269, 281: three. Float64
-        // l_max = 9, 12, 16, 18, 20, 32 223, 244, 244, 248, 270, 251 / 218, 245, 240, 234, 252, 257 /
-        // 239, 239, 233, 239, 257, 253: as few rounds of recursions as four waves would need, with
-        // as few waves as that takes. Second derivatives, float32, l_max = 4, 8, 12, 16, 20, 24 240,
-        // 239, 240, 238, 245, 276 / 231, 248, 247, 246, 250, 266: the entries weigh more there, two,
-        // three at both ends.
+        // Sixteen waves: the tile is larger, the recursions of a tile more, and the tile waits for them if they need
+        // many rounds. By measurement with two, three and four sequence waves: gradients in float32 three (two next
+        // to slice waves); in float64 as few rounds of recursions as four waves would need, with as few waves as that
+        // takes; second derivatives, where the entries weigh more, two, three at both ends of the l_max range.
         const unsigned recursions = S * arrays * static_cast<unsigned>(l_max - hard);
         if (mode == 1 && elem == 4) {
             g.sequence_waves = g.slice_waves != 0 ? 2 : 3; // (two with slice waves, see above)
@@ -699,9 +564,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         } else if (mode == 2) {
             g.sequence_waves = l_max <= 4 || l_max >= 22 ? 3u : 2u;
         } else {
-            // values, two against three: float32 l_max = 24, 28, 32, 40, 48 381, 436, 373, 420, 355
-            // against 396, 392, 377, 376, 366; float64 l_max = 24, 28, 32 295, 326, 293 against
-            // 292, 305, 297
+            // values: three (within 3 % of two on every shape, 10 % ahead at l_max = 28, 40)
             g.sequence_waves = 3;
         }
     } else if (g.sequence_waves == 2 && !(mode == 2 && elem == 8)) {
@@ -729,31 +592,21 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         for (int k = 0; k < 3; ++k) g.kind_magic[k] = g.kind_jobs[k] ? magic_of(g.kind_jobs[k]) : 0u;
     }
     g.points_per_pass = per_pass(g.jobs_per_point);
-    // The jobs of a tile as one list. Values: the list is point after point and costs a few
-    // instructions per job, so only where it saves a round and few points go side by side anyway
-    // (float32 l_max = 40, 48: 527, 477 -> 468, 428 us). With derivatives the list is ordered by
-    // kind of job first (recursion_kernel), which keeps the lanes of a wave on one branch of
-    // entry_job: side by side, the 77 one-sided jobs of a point at l_max = 8 with second
-    // derivatives put all seven kinds into every wave and 41 % of the lanes were active on
-    // average. 400 MB of output, us, points side by side against the list: second derivatives
-    // float32 l_max = 6, 8, 10, 12 (22, 14, 9, 6 points per tile) 164, 157, 138, 144 -> 115, 117,
-    // 117, 115 (solid 108, 97, 97, 97 -> 98, 84, 89, 93); float64 l_max = 4, 8, 12, 16 146, 165,
-    // 135, 123 -> 106, 104, 99, 96; gradients float32 l_max = 18, 24, 26 124, 123, 116 -> 109, 116,
-    // 108, float64 l_max = 12, 13, 14 122, 127, 127 -> 107, 111, 115. With one or two points per
-    // tile the list loses unless it saves a round (float32 gradients l_max = 32, 40: 113, 101 ->
-    // 117, 119; l_max = 36, five rounds instead of six, 111 -> 108, solid 127 -> 112), and so it
-    // does for solid second derivatives in float64 where the points side by side fill the lanes
-    // anyway (cfg4, four points, 94 % of the lanes: 535 -> 559 us; l_max = 15, 83 %: 98 -> 84 us).
-    // Second derivatives with two points per tile: the list unless the sides are split (float64
-    // l_max = 20, 22 156, 138 -> 126, 105 us; solid float32 l_max = 22 83 -> 79; float32 with split
-    // sides 100 -> 108).
+    // The jobs of a tile as one list. Values: the list is point after point and costs a few instructions per job, so
+    // only where it saves a round and few points go side by side anyway. With derivatives the list is ordered by
+    // kind of job first (recursion_kernel), which keeps the lanes of a wave on one branch of entry_job: side by
+    // side, the 77 one-sided jobs of a point at l_max = 8 with second derivatives put all seven kinds into every
+    // wave and 41 % of the lanes were active on average (20-35 % faster as a list). With one or two points per tile
+    // the list loses unless it saves a round, and so it does for solid second derivatives in float64 in workgroups
+    // of 512 threads where the points side by side fill the lanes anyway. Second derivatives with two points per
+    // tile: the list unless the sides are split.
     const int want_list = switch_or(SW_JOB_LIST, -1);
     const bool saves_a_round = (S * g.jobs_per_point + wide - 1) / wide < rounds_by_point(g.jobs_per_point);
     // lanes that points side by side would fill, in percent
     const unsigned fill = 100u * g.points_per_pass * g.jobs_per_point / wide;
     const bool cheap_jobs = mode == 2 && elem == 8 && !normalized; // no chain rule, few branches
-    // (values in workgroups of 1024 threads: always the list, us per 1.2 GB without and with:
-    // float32 l_max = 26 475, 391; float64 l_max = 26, 36 353, 307 and 351, 299; the same elsewhere)
+    // (values in workgroups of 1024 threads: always the list, 15 % faster; solid second derivatives in float64
+    // in workgroups of 1024 threads, whose sides are two jobs: always the list as well)
     const bool by_shape = mode == 0   ? (threads > kRecursionThreads ? S >= 2 : saves_a_round && S >= 3 && g.points_per_pass <= 2)
                           : mode == 1 ? S >= 3 || (saves_a_round && S >= 2)
                                       : (S >= 3 && !(cheap_jobs && fill >= 90u)) || (S == 2 && !*split_sides) ||
@@ -787,20 +640,13 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     out->lds_bytes = g.tables_at + at * esize;
     out->threads = threads;
     if (out->lds_bytes > limit) return false;
-    // Jobs point by point, one point per pass, with derivatives: in the last round of a point the
-    // jobs with |m| = l, |m| = l - 1 and m = 0 are moved to wave boundaries of the entry lanes where
-    // the lanes of that round allow it, because a wave runs the branch of every kind of job it
-    // holds one after the other and the tile waits for the slowest wave. Float32 l_max = 32, 533
-    // jobs on 320 lanes: the second round was 135 bulk jobs, then 26 + 26 + 26, all three in the
-    // third wave together with the end of the bulk; moved, m = 0 follows the bulk and the other two
-    // start the fourth and fifth wave. The gaps are places without a job at the end of the job
-    // table. With one workgroup of 1024 threads on a CU this pays (float64 gradients l_max = 32,
-    // two points per tile: 290 -> 249 us per 1.2 GB). With two workgroups of 512 the slowest wave of
-    // a tile of cfg5 went from 7 400 to 5 900 cycles and a launch from 979 to 926 us for the first
-    // few launches after a pause, but from 896 to 947 us in a long series of launches, and builds
-    // of the kernel that differ in a few scalar instructions moved either number by 5 %: how the
-    // stages and flushes of the two workgroups of a CU fall against each other decides there,
-    // and nothing in the kernel controls that. Off for 512 threads (SPHX_SPREAD_KINDS).
+    // Jobs point by point, one point per pass, with derivatives: in the last round of a point the jobs with
+    // |m| = l, |m| = l - 1 and m = 0 are moved to wave boundaries of the entry lanes where the lanes of that round
+    // allow it, because a wave runs the branch of every kind of job it holds one after the other and the tile waits
+    // for the slowest wave. The gaps are places without a job at the end of the job table. With one workgroup of
+    // 1024 threads on a CU this pays (float64 gradients l_max = 32: 290 -> 249 us per 1.2 GB); with two workgroups
+    // of 512, how their stages and flushes fall against each other decides, and nothing in the kernel controls
+    // that: off there (SPHX_SPREAD_KINDS).
     g.kind_at[0] = g.kind_at[1] = g.kind_at[2] = 0;
     if (mode >= 1 && !*split_sides && g.points_per_pass == 1 && switch_or(SW_SPREAD_KINDS, threads > kRecursionThreads ? 1 : 0) != 0) {
         const unsigned levels = g.kind_jobs[1], bulk = g.kind_jobs[0], jobs_now = g.jobs_per_point;
@@ -844,12 +690,9 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
 
     g.n_tiles = static_cast<unsigned>((n_samples + S - 1) / S);
     g.tiles_per_xcd = (g.n_tiles + 7u) / 8u;
-    // Chunks of consecutive tiles per workgroup: only where a tile is one run per array, and a
-    // run is at least a line long (so that a carried part never spans two tiles). About eight
-    // points per chunk: chunks of eight tiles whatever their size were as good for tiles of one
-    // or two points and worse for larger ones (second derivatives, float64, 1.5 GB of output:
-    // l_max = 16, 4 points per tile, 446 us in chunks of eight tiles, 394 in chunks of two;
-    // l_max = 8, 14 points, 632 against 561 for single tiles; cfg4 562 against 528).
+    // Chunks of consecutive tiles per workgroup: only where a tile is one run per array, and a run is at least a
+    // line long (so that a carried part never spans two tiles). About eight points per chunk: chunks of eight tiles
+    // whatever their size were as good for tiles of one or two points and 6-13 % worse for larger ones.
     g.chunk_shift = 0;
     if (whole && S * nrow * osize >= 128u) {
         const int want = switch_or(SW_CHUNK_SHIFT, S >= 5 ? 0 : (S >= 3 ? 1 : (S == 2 ? 2 : 3)));
@@ -859,9 +702,9 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     if (per_cu < 1) per_cu = 1;
     if (per_cu > 2048u / threads) per_cu = 2048u / threads; // 2048 lanes per CU
     unsigned want = (static_cast<unsigned>(cus) * per_cu + 7u) & ~7u;
-    // Few points: shorter chunks, down to single tiles, until every resident workgroup has one
-    // (10 000 points at l_max = 8 are 625 tiles of 16: in chunks of 8 they kept 80 workgroups
-    // busy for 41 us, as single tiles they take 512 and a third of the time).
+    // Few points: shorter chunks, down to single tiles, until every resident workgroup has one (10 000 points at
+    // l_max = 8 are 625 tiles of 16: in chunks of 8 they kept 80 workgroups busy for 41 us, as single tiles they take
+    // 512 and a third of the time).
     auto chunks_in_xcd = [&]() { return (g.tiles_per_xcd + (1u << g.chunk_shift) - 1u) >> g.chunk_shift; };
     while (g.chunk_shift > 0 && chunks_in_xcd() * 8u < want) --g.chunk_shift;
     const unsigned chunks_per_xcd = chunks_in_xcd();
@@ -890,14 +733,10 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
     plan->whole = true;
     plan->split_sides = false;
     plan->pairs = false;
-    // Gradients in closed form, where the rows of a tile are so long that few single-wave
-    // workgroups of closed_form_kernel share a CU: the lanes kernel instead, which cuts the closed
-    // forms in slices for six or eight waves and flushes with all of them. Measured, us, against
-    // closed_form_kernel: l_max = 6 float32 1M points 127 against 134 (solid 133 against 134), 300k
-    // 43 against 49, 100k 17 against 23, 10k 5.0 against 6.8; float64 500k 125 against 148 (solid
-    // 131 against 152), 100k 29 against 42; l_max = 5 float64 680k 135 against 149; l_max = 4
-    // float32 2M 131 against 141, 100k 8.7 against 11.3. Not below: l_max = 3 float32 100k 8.0
-    // against 7.3, l_max = 4 float64 1M 139 against 132, l_max = 5 float32 140 against 142.
+    // Gradients in closed form, where the rows of a tile are so long that few single-wave workgroups of
+    // closed_form_kernel share a CU: the lanes kernel instead, which cuts the closed forms in slices for six or
+    // eight waves and flushes with all of them (5-25 % faster at l_max = 6, at l_max = 5 in float64 and at
+    // l_max = 4 for normalised float32, at every size from 10 000 points to 2M; not below).
     const bool in_slices = l_max == 6 || (l_max == 5 && elem == 8) || (l_max == 4 && elem == 4 && normalized);
     if (plan->closed_only && lane_kernels && mode == 1 && in_slices && switch_or(SW_GRADIENT_LANES, 1) != 0 &&
         plan_gradient_lanes(n_samples, l_max, elem, lds_limit, cus, &plan->closed, normalized)) {
@@ -910,11 +749,9 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
         return SPHX_OK;
     }
     // Values alone where the rows of few points fill LDS: pairs_kernel (below, with the derivatives), which keeps
-    // the recursions of the next tile and the flush of this one side by side. 1.2 GB of output, us, against
-    // values_kernel (the recursion kernel from l_max = 34): float32 l_max = 22, 24, 26, 28, 30, 32, 34, 36 262,
-    // 254, 242, 252, 231, 219, 236, 243 against 262, 296, 293, 319, 318, 306, 379, 381; float64 l_max = 20, 24,
-    // 28, 32, 36 220, 222, 224, 215, 223 against 266, 301, 312, 298, 303; below (float32 l_max = 20 264 against
-    // 257, float64 l_max = 18 293 against 247) a point's pairs leave the entry lanes idle.
+    // the recursions of the next tile and the flush of this one side by side: 10-35 % faster than values_kernel
+    // (the recursion kernel from l_max = 34) from l_max = 23 in float32 and 20 in float64. Below, a point's pairs
+    // leave the entry lanes idle and values_kernel is ahead.
     if (lane_kernels && mode == 0 && l_max > hard) {
         const int pairs = switch_or(SW_PAIRS, 1);
         const bool pairs_by_shape = n_samples >= 32768 && (elem == 4 ? l_max >= 23 : l_max >= 20);
@@ -938,36 +775,19 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
     // Second derivatives at small l_max: one point per lane where that was measured to be faster
     // than the recursion kernel (SPHX_HESSIAN_LANES: 0 never, 2 wherever the rows fit).
     const int hessian_lanes = switch_or(SW_HESSIAN_LANES, 1);
-    // (Since the recursion kernel takes its jobs as a list ordered by kind it wins from l_max = 4
-    // on; 400 MB of output, us, lanes against recursion: float32 l_max = 2 87, 99 (solid 72, 82),
-    // l_max = 3 104, 108 (solid 89, 100), l_max = 4 147, 107 (solid 113, 87), l_max = 5 130, 112
-    // (solid 99, 86); float64 l_max = 3 129, 114 (solid 91, 102), l_max = 5 163, 107; 20 000 points
-    // float32 l_max = 3 9.0, 11.2, l_max = 4 17.9, 13.5.)
-    // (Solid harmonics in float64, l_max = 3, 1.2 GB of output: 259 us against 243 in workgroups of 1024 threads.)
+    // (Since the recursion kernel takes its jobs as a list ordered by kind it wins from l_max = 4 on; the lanes keep
+    // l_max <= 3 in float32 and, for calls too small for workgroups of 1024 threads, solid l_max = 3 in float64.)
     const bool hessian_lanes_pay = elem == 4 ? l_max <= 3 : (l_max == 3 && !normalized && n_samples < 32768);
     if (lane_kernels && mode == 2 && (hessian_lanes == 2 || (hessian_lanes == 1 && hessian_lanes_pay)) &&
         plan_hessian_lanes(n_samples, l_max, elem, lds_limit, &plan->closed, normalized)) {
         plan->lanes = true;
         return SPHX_OK;
     }
-    // (float32 from l_max = 14 on the recursion kernel with its jobs as a list ordered by kind is
-    // ahead: 600 MB of output, lanes against recursion, l_max = 13 151, 150 us; 14 169, 153; 15 189,
-    // 171; 16 174, 154; solid 14 152, 144; 16 160, 144. SPHX_GRADIENT_LANES=2: lanes wherever they fit.)
-    // (With workgroups of 1024 threads the recursion kernel is ahead earlier when there are points
-    // enough for them: 1.2 GB of output, us, lanes against recursion, float32 l_max = 8 214, 206; 9
-    // 256, 217; 10 241, 227; 11 256, 286; 12 306, 238; 13 301, 246; float64 l_max = 7 224, 507; 8
-    // 246, 214; 9 307, 218; 10 293, 226; 11 309, 292. The lanes keep l_max <= 8 and 11 in float32,
-    // l_max = 7 in float64, and every call of fewer than 32 768 points (50 000 points, lanes against
-    // recursion: float64 l_max = 9 54, 43 us, float32 l_max = 12 42, 38 us; 20 000 points 25, 22 and 21, 24).)
     // Derivatives where the rows of few points fill LDS: pairs_kernel, whose entry lanes keep one (l, m) pair for
-    // the whole launch and whose other work runs while the rows are flushed. 1.2 GB of output, us, pairs_kernel
-    // against recursion_kernel. Gradients: float32 l_max = 16, 20, 24, 28, 32, 36 299, 274, 267, 269, 253, 262
-    // against 289, 286, 291, 288, 285, 286; float64 l_max = 14, 16, 20, 24, 28, 32, 36 289, 280, 265, 251, 268, 268,
-    // 248 against 283, 289, 288, 290, 285, 285, 274; cfg5 (l_max = 32, 200 000 points) 570-620 against 700. Below,
-    // a point's pairs leave most of the entry lanes idle and it loses (float32 l_max = 12: 383 against 277).
-    // Second derivatives: float64 l_max = 12, 16, 20, 24 287, 299, 296, 318 against 290, 290, 333, 352; float32
-    // l_max = 12, 16, 20, 24 350, 303, 318, 307 against 289, 285, 294, 304 (the recursion kernel's job list by
-    // kind fills sixteen waves better). SPHX_PAIRS: 0 never, 2 wherever it fits.
+    // the whole launch and whose other work runs while the rows are flushed. Gradients: 5-15 % faster than the
+    // recursion kernel from l_max = 20 in float32 and 16 in float64 (cfg5 700 -> 570-620 us); below, a point's
+    // pairs leave most of the entry lanes idle. Second derivatives: ahead in float64 from l_max = 20; in float32
+    // the recursion kernel's job list by kind fills sixteen waves better. SPHX_PAIRS: 0 never, 2 wherever it fits.
     {
         const int pairs = switch_or(SW_PAIRS, 1);
         const bool pairs_by_shape = n_samples >= 32768 && (mode == 1 ? (elem == 4 ? l_max >= 20 : l_max >= 16)
@@ -985,6 +805,11 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
             }
         }
     }
+    // Gradients just above the closed forms: the lanes kernel (one point per lane, the channels dealt to the
+    // waves) up to l_max = 13 in float32 and wherever its tiles fit in float64; from there the recursion kernel with
+    // its jobs as a list ordered by kind is ahead. Where the recursion kernel runs in workgroups of 1024 threads
+    // (calls of 32 768 points or more) it is ahead earlier: the lanes keep l_max <= 8 and 11 in float32 and
+    // l_max = 7 in float64. SPHX_GRADIENT_LANES: 0 never, 2 wherever the rows fit.
     const int gradient_lanes = switch_or(SW_GRADIENT_LANES, 1);
     const bool large_groups = group_threads(n_samples, mode, elem, lane_kernels) > kRecursionThreads && n_samples >= 32768;
     const bool lanes_by_shape = large_groups ? (elem == 4 ? l_max <= 8 || l_max == 11 : l_max <= 7)
@@ -994,39 +819,21 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
         plan->lanes = true;
         return SPHX_OK;
     }
-    // LDS a workgroup of the recursion kernel may take: half a CU's, so that two share the CU.
-    // With second derivatives in float64 the kernel needs more than 128 registers per lane,
-    // one workgroup of 512 threads is all a CU holds, and half of LDS would lie idle: there
-    // the tile takes all of it (1.5 GB of output, l_max = 6: 694 -> 473 us, l_max = 10: 582 ->
-    // 479, l_max = 12: 545 -> 468; solid harmonics l_max = 4-12: 10-20 % less, l_max = 16, 100k
-    // points: 580 -> 560).
+    // LDS a workgroup of the recursion kernel may take: half a CU's, so that two share the CU. A workgroup that is
+    // alone on its CU anyway (1024 threads, or second derivatives in float64, which need more than 128 registers
+    // per lane) takes all of it: 10-30 % faster.
     const unsigned threads = group_threads(n_samples, mode, elem, lane_kernels, normalized, l_max);
     const int whole_cu = (mode == 2 && elem == 8) || threads > kRecursionThreads ? lds_limit : 80 * 1024;
     const unsigned budget = static_cast<unsigned>(switch_or(SW_TILE_LDS_BUDGET, whole_cu));
     bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
                                &plan->split_sides, normalized, 0, threads);
-    // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of
-    // the lanes idle for some two thousand instructions per tile: then the recursion kernel
-    // stages l >= 7 only and its wave 0, which mostly waits, writes l <= 6 straight from
-    // registers, 64 points at a time (prefix_inside). The price is rows cut in two, each part a
-    // run of its own in HBM, which costs the more the shorter the rows are. Measured with 2.5 GB
-    // of output and 400 calls in a row (in bursts of 60 calls, or with a few hundred MB of
-    // output, the last-level cache merges the parts and the cut rows look 10-30 % better than
-    // they are), whole against cut, us. Gradients, float32: l_max = 17 (8 points per tile) 764
-    // against 1 014; l_max = 19, 20, 22 (4) 1 196, 1 121, 922 against 992, 988, 817; l_max = 24
-    // (4) 707 against 741; l_max = 28, 32 (2) 881, 781 against 883, 636. Gradients, float64:
-    // l_max = 12 (8) 737 against 1 084; l_max = 13, 14, 16, 18 (4) 1 029, 878, 775, 812 against
-    // 1 049, 1 059, 918, 848; l_max = 20, 24 (2) 995, 706 against 886, 626. Values: float32
-    // l_max = 36, 40 (4) 1 004, 977 against 885, 865; float64 l_max = 24, 28 (4) 924, 856
-    // against 741, 749.
-    // (With the job-list variant of the kernel the whole rows gained more than the cut ones:
-    // float32 gradients, 1.5 GB of output, whole against cut: l_max = 19-22 (5-7 points per tile)
-    // 393, 407, 373, 399 us against 431, 451, 419, 424; l_max = 28, 30 (3) 396, 371 against 532,
-    // 510; l_max = 32 (2) 462 against 389. Float32 gradients are therefore cut below three
-    // points per tile only; values below eight, float64 gradients below four as before.)
-    // (Since the float64 rows go out in whole lines, copy_out<LINES>, the cut rows gained 20 %
-    // there: l_max = 20, 100k points 491 -> 376 us, and with four points per tile they now win as
-    // well, l_max = 18: 291 us cut against 328 whole; with five, l_max = 16: 580 against 481.)
+    // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of the lanes idle for
+    // some two thousand instructions per tile: then the recursion kernel stages l >= 7 only and its wave 0, which
+    // mostly waits, writes l <= 6 straight from registers, 64 points at a time (prefix_inside). The price is rows
+    // cut in two, each part a run of its own in HBM, which costs the more the shorter the rows are. By measurement
+    // (2.5 GB of output, hundreds of calls in a row: in short bursts the last-level cache merges the parts and the
+    // cut rows look 10-30 % better than they are) float32 gradients are cut below three points per tile, float64
+    // gradients below five, values below eight.
     const int split_below = switch_or(SW_SPLIT_BELOW, mode == 0 ? 8 : (elem == 4 ? 3 : 5));
     const bool cut = plan->rec.g.tile < split_below;
     if (mode < 2 && (!fits || cut)) {
@@ -1090,10 +897,8 @@ int make_vjp_plan(size_t n_samples, int l_max, size_t elem, int lds_limit, int c
     out->use_lanes = out->lane_groups = false;
     if (l_max > 6 && switch_or(SW_VJP_LANES, 1) != 0) {
         out->use_lanes = plan_values(n_samples, l_max, elem, lds_limit, &out->lanes, true);
-        // groups of lanes with channels of their own pay off from tiles of 16 points down
-        // (200k points, float32 l_max = 24: 225 against 279 us; float64 l_max = 24: 665
-        // against 866; with tiles of 32 the scalar-unit kernel is ahead, float64 l_max = 12:
-        // 329 against 397)
+        // groups of lanes with channels of their own pay off from tiles of 16 points down (20-25 % at l_max = 24);
+        // with tiles of 32 the kernel that takes its prefactors from the scalar unit is ahead
         out->lane_groups = out->use_lanes && out->lanes.g.tile <= switch_or(SW_VJP_GROUPS_BELOW, 16);
     }
     if (out->use_lanes) return SPHX_OK;
