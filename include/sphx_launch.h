@@ -212,7 +212,7 @@ SPHX_EXPORT int sphx_describe_plan(size_t n_samples, int l_max, int derivatives,
 
 /* Override one decision of the launch planner, for measurements and for tests
  * that want both sides of a choice exercised: `name` is one of the SPHX_*
- * names listed in sphx_kernels.hip (SPHX_TILE, SPHX_JOB_LIST, ...), unknown
+ * names listed in sphx_plan.hpp (SPHX_TILE, SPHX_JOB_LIST, ...), unknown
  * names return SPHX_ERR_ARGUMENT. Process-wide; takes effect with the next
  * call on any thread. sphx_reset_switches() drops all overrides. Without
  * overrides a call is planned from its shape alone. The environment variables

@@ -35,10 +35,13 @@ template <typename X> struct AsGiven {
     using type = X; // a parameter of this type takes no part in template argument deduction
 };
 
-// Workgroups of 1024 threads (one per CU, all of its LDS) exist for all but second derivatives
-// in float64, which need more registers than sixteen waves leave a lane, and the fused product.
-template <typename T, int MODE, bool VJP, bool NORM = true, bool SPLIT = false>
-constexpr bool kLargeGroups = !VJP && (MODE <= 1 || (MODE == 2 && sizeof(T) == 4) || (MODE == 2 && !NORM && SPLIT));
+// Workgroups of 1024 threads (one per CU, all of its LDS) exist for all but the fused product and those
+// second derivatives in float64 whose entry jobs need more registers than sixteen waves leave a lane (128): the
+// two sides of an (l, m) pair as one job (163-231), and for normalised harmonics the sides as two jobs taken
+// point by point (173; as one list ordered by kind 129, which the compiler brings down to 128).
+template <typename T, int MODE, bool VJP, bool NORM = true, bool SPLIT = false, bool LIST = false>
+constexpr bool kLargeGroups =
+    !VJP && (MODE <= 1 || (MODE == 2 && sizeof(T) == 4) || (MODE == 2 && SPLIT && (!NORM || LIST)));
 
 template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false,
           typename O = T, unsigned NT = kRecursionThreads>
@@ -51,7 +54,7 @@ static hipError_t launch_recursion(const Launch& l, const typename AsGiven<O>::t
             return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, false, true, O, NT>(l, xyz, sph, dsph, ddsph, stream);
         }
     }
-    if constexpr (NT == kRecursionThreads && kLargeGroups<T, MODE, VJP, NORM, SPLIT>) {
+    if constexpr (NT == kRecursionThreads && kLargeGroups<T, MODE, VJP, NORM, SPLIT, LIST>) {
         if (l.threads == 2 * kRecursionThreads) {
             return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O, 2 * kRecursionThreads>(
                 l, xyz, sph, dsph, ddsph, stream);

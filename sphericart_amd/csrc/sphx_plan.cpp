@@ -393,16 +393,19 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
 // SPHX_GROUP_THREADS = 512 or 1024 overrides the rule.
 static unsigned group_threads(size_t n_samples, int mode, size_t elem, bool forward, bool normalized = true,
                               int l_max = -1) {
-    // Second derivatives in float64: the entries (l, +m) and (l, -m) as one job need 169-237 registers per lane,
-    // more than the 128 that sixteen waves leave. As two jobs solid harmonics need 121 (normalised 181: those keep
-    // eight waves) and gain 5-20 % from l_max = 3 on (cfg4 538 -> 507 us); at l_max = 2 the list is three jobs a
-    // point and eight waves are as fast.
-    const bool solid_f64_hessians = mode == 2 && elem == 8 && !normalized;
-    const bool exists = forward && (mode <= 1 || (mode == 2 && elem == 4) || solid_f64_hessians);
-    if (!exists) return kRecursionThreads;
+    // Second derivatives in float64: the entries (l, +m) and (l, -m) as one job need 163-231 registers per lane,
+    // more than the 128 that sixteen waves leave. As two jobs solid harmonics need 103-113, normalised ones 128
+    // when the jobs of a tile go as one list ordered by kind (plan_recursion sees to both), and sixteen waves gain
+    // 5-20 % from l_max = 3 on (cfg4 538 -> 507 us); at l_max = 2 the list is three jobs a point and eight waves
+    // are as fast. (A caller that passes no l_max, the path that evaluates float arrays in float64, keeps eight.)
+    const bool f64_hessians = mode == 2 && elem == 8;
+    if (!forward || (f64_hessians && l_max < 0)) return kRecursionThreads;
     const int want = switch_or(SW_GROUP_THREADS, 0);
     if (want == 512 || want == 1024) return static_cast<unsigned>(want);
-    if (solid_f64_hessians && l_max < 3) return kRecursionThreads;
+    if (f64_hessians && l_max < 3) return kRecursionThreads;
+    // (normalised: one-sided jobs are 20 % more work, which sixteen waves make up for only at l_max = 3 and, with
+    // two or three points per tile, at l_max = 18 .. 23: 2-12 %)
+    if (f64_hessians && normalized && !(l_max == 3 || (l_max >= 18 && l_max <= 23))) return kRecursionThreads;
     return n_samples >= 4096 ? 2 * kRecursionThreads : kRecursionThreads;
 }
 
@@ -605,6 +608,8 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // lanes that points side by side would fill, in percent
     const unsigned fill = 100u * g.points_per_pass * g.jobs_per_point / wide;
     const bool cheap_jobs = mode == 2 && elem == 8 && !normalized; // no chain rule, few branches
+    // (normalised second derivatives in float64 in workgroups of 1024 threads exist as a list only)
+    const bool must_list = mode == 2 && elem == 8 && normalized && threads > kRecursionThreads;
     // (values in workgroups of 1024 threads: always the list, 15 % faster; solid second derivatives in float64
     // in workgroups of 1024 threads, whose sides are two jobs: always the list as well)
     const bool by_shape = mode == 0   ? (threads > kRecursionThreads ? S >= 2 : saves_a_round && S >= 3 && g.points_per_pass <= 2)
@@ -612,7 +617,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
                                       : (S >= 3 && !(cheap_jobs && fill >= 90u)) || (S == 2 && !*split_sides) ||
                                             (saves_a_round && S >= 2) ||
                                             (cheap_jobs && threads > kRecursionThreads && S >= 2);
-    if (want_list == 2 || (want_list == 1 && saves_a_round) || (want_list < 0 && by_shape)) {
+    if (must_list || want_list == 2 || (want_list == 1 && saves_a_round) || (want_list < 0 && by_shape)) {
         g.points_per_pass = 0;
     }
 
@@ -822,11 +827,17 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
     // LDS a workgroup of the recursion kernel may take: half a CU's, so that two share the CU. A workgroup that is
     // alone on its CU anyway (1024 threads, or second derivatives in float64, which need more than 128 registers
     // per lane) takes all of it: 10-30 % faster.
-    const unsigned threads = group_threads(n_samples, mode, elem, lane_kernels, normalized, l_max);
+    unsigned threads = group_threads(n_samples, mode, elem, lane_kernels, normalized, l_max);
     const int whole_cu = (mode == 2 && elem == 8) || threads > kRecursionThreads ? lds_limit : 80 * 1024;
     const unsigned budget = static_cast<unsigned>(switch_or(SW_TILE_LDS_BUDGET, whole_cu));
     bool fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
                                &plan->split_sides, normalized, 0, threads);
+    if (fits && mode == 2 && elem == 8 && threads > kRecursionThreads && !plan->split_sides) {
+        // (the sides could not be split, an override or a job table that does not fit: eight waves then)
+        threads = kRecursionThreads;
+        fits = plan_recursion(n_samples, l_max, mode, true, elem, budget, lds_limit, cus, &plan->rec,
+                              &plan->split_sides, normalized, 0, threads);
+    }
     // With few points per tile the one-lane-per-point closed forms of l <= 6 would leave most of the lanes idle for
     // some two thousand instructions per tile: then the recursion kernel stages l >= 7 only and its wave 0, which
     // mostly waits, writes l <= 6 straight from registers, 64 points at a time (prefix_inside). The price is rows
