@@ -432,13 +432,13 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     const unsigned jobs_split = 2 * jobs - static_cast<unsigned>(l_max - hard);
     bool may_split = mode == 2 && switch_or(SW_SPLIT_SIDES, 1) != 0;
     auto table_elems_for = [&](bool split) { return ((split ? jobs_split : jobs) * 4 + esize - 1) / esize; };
-    // per point: the rows in every row buffer, point tables three times, iterates twice
+    // per point: the rows, point tables twice, iterates once
     // staged rows are `row_stride` apart (recursion_kernel): nrow, or a little more when the rows
     // are cut so that they keep their position within 16 bytes
     const unsigned row_stride = nrow + (whole ? 0u : nyh % (16u / osize));
     const unsigned rows_per_point = components_of(mode) * row_stride;
     // (the records of a point and its sequences of iterates are an odd number of words apart)
-    const unsigned rest_per_point = 3 * ((8 + 3 * (l_max + 1)) | 1u) + 2 * arrays * (tri_all | 1u);
+    const unsigned rest_per_point = 2 * ((8 + 3 * (l_max + 1)) | 1u) + arrays * (tri_all | 1u);
     unsigned fixed = 0; // bytes
     const unsigned point_bytes = rows_per_point * osize + rest_per_point * esize;
     auto bytes_for = [&](unsigned S) { return S * point_bytes + fixed; };
@@ -493,14 +493,14 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         for (unsigned shift = cap < 0 ? 0u : (cap > 6 ? 6u : static_cast<unsigned>(cap)); shift >= 1; --shift) {
             const unsigned tiles = 1u << shift;
             if (tiles * S > 64) continue;
-            const unsigned extra = (2 * tiles - 3) * S * point_record * esize;
+            const unsigned extra = (2 * tiles - 2) * S * point_record * esize;
             if (bytes_for(S) + extra <= allowed || bytes_for(S) + extra <= budget) {
                 az_shift = shift;
                 break;
             }
         }
     }
-    const unsigned table_slots = az_shift == 0 ? 3u : 2u << az_shift;
+    const unsigned table_slots = 2u << az_shift;
 
     g.n_samples = n_samples;
     g.l_max = l_max;
@@ -508,13 +508,13 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.tile = static_cast<int>(S);
     g.az_shift = az_shift;
     // Waves of their own for the closed forms of l <= 6 (whole rows): with sixteen waves and float32 gradients, where
-    // the tile otherwise waits for the entry waves that carry a slice on top of their jobs; one of them up to eight
-    // points per tile, two from nine on, three from 28 on (3-6 % at l_max = 8 .. 40). In float64 the closed forms are
-    // too much for two or three waves.
+    // the tile otherwise waits for the entry waves that carry a slice on top of their jobs: three of them (l_max =
+    // 9 .. 18: 1-4 % over none, one or two are 5-20 % behind). In float64 the closed forms are too much for three or
+    // four waves (3-10 % behind none).
     g.slice_waves = 0;
     const bool slices_apart = threads > kRecursionThreads && mode == 1 && elem == 4;
     if (whole && mode < 2) {
-        const int want = switch_or(SW_SLICE_WAVES, slices_apart ? (S >= 28 ? 3 : (S >= 9 ? 2 : 1)) : 0);
+        const int want = switch_or(SW_SLICE_WAVES, slices_apart && S >= 9 ? 3 : 0);
         g.slice_waves = want < 0 ? 0u : (want > 4 ? 4u : static_cast<unsigned>(want));
     }
     g.sequence_waves = S * arrays * static_cast<unsigned>(l_max - hard) > 64 ? 2u : 1u;
@@ -538,7 +538,8 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     };
     // rounds of the entry waves per tile, in tenths of two-sided jobs, with `waves` sequence waves
     auto entry_cost = [&](unsigned waves, bool* split) {
-        wide = threads - 64 * (1 + waves + g.slice_waves);
+        (void)waves; // (the sequence waves work while the others flush and compute entries like the rest)
+        wide = threads - 64 * g.slice_waves;
         // (with two or more points per tile the jobs go as a list ordered by kind, which fills the lanes without
         // splitting, and the two-sided job shares the common factors: 5-15 % faster; with one point per tile
         // splitting stays)
@@ -547,38 +548,31 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         if (may_split && mode == 2 && elem == 8 && threads > kRecursionThreads) *split = true;
         return *split ? one_side_costs * rounds(jobs_split) : 10 * rounds(jobs);
     };
-    // A second sequence wave takes a wave from the entries. One is enough where it saves the entry waves a round
-    // per tile, and for values alone, whose recursions are a third of the work; with equal rounds two are faster by
-    // 2-3 % with derivatives. Second derivatives in float64 follow no such rule and keep two.
+    // The sequence waves run the recursions of the next tile while the other waves flush this one; the tile waits for
+    // whichever takes longer. More of them finish the recursions sooner and leave fewer waves to keep stores in
+    // flight. By measurement with two to eight of sixteen waves: gradients four in float32 (l_max = 10-16: 57-62 %
+    // with two, 66-69 % with four) and three in float64; second derivatives in float32 six for normalised harmonics
+    // and three for solid ones, whose entries are shorter and whose flush weighs more (l_max = 8: 72.6 % with three,
+    // 65 % with six; two from l_max = 16 on); in float64 two, three at both ends of the l_max range.
     if (threads > kRecursionThreads) {
-        // Sixteen waves: the tile is larger, the recursions of a tile more, and the tile waits for them if they need
-        // many rounds. By measurement with two, three and four sequence waves: gradients in float32 three (two next
-        // to slice waves); in float64 as few rounds of recursions as four waves would need, with as few waves as that
-        // takes; second derivatives, where the entries weigh more, two, three at both ends of the l_max range.
-        const unsigned recursions = S * arrays * static_cast<unsigned>(l_max - hard);
-        if (mode == 1 && elem == 4) {
-            g.sequence_waves = g.slice_waves != 0 ? 2 : 3; // (two with slice waves, see above)
-        } else if (mode == 1) {
-            const unsigned least = (recursions + 255u) / 256u;
-            g.sequence_waves = 2;
-            while (g.sequence_waves < 4 && (recursions + 64u * g.sequence_waves - 1u) / (64u * g.sequence_waves) > least) {
-                ++g.sequence_waves;
-            }
+        if (mode == 1) {
+            g.sequence_waves = elem == 4 ? 4 : 3;
+        } else if (mode == 2 && elem == 4) {
+            g.sequence_waves = normalized ? 6 : (l_max <= 15 ? 3 : 2);
         } else if (mode == 2) {
             g.sequence_waves = l_max <= 4 || l_max >= 22 ? 3u : 2u;
         } else {
-            // values: three (within 3 % of two on every shape, 10 % ahead at l_max = 28, 40)
             g.sequence_waves = 3;
         }
-    } else if (g.sequence_waves == 2 && !(mode == 2 && elem == 8)) {
-        bool split_one = false, split_two = false;
-        const unsigned with_one = entry_cost(1, &split_one);
-        const unsigned with_two = entry_cost(2, &split_two);
-        if (mode == 0 || with_one < with_two) g.sequence_waves = 1;
+    } else if (mode == 0) {
+        g.sequence_waves = 1; // values alone: the recursions are a third of the work
     }
     {
+        // (at least four waves flush)
         const int forced_seq = switch_or(SW_SEQUENCE_WAVES, 0);
-        if (forced_seq >= 1 && forced_seq <= 4) g.sequence_waves = static_cast<unsigned>(forced_seq);
+        if (forced_seq >= 1) g.sequence_waves = static_cast<unsigned>(forced_seq);
+        const unsigned most = threads / 64u - 5u;
+        if (g.sequence_waves > most) g.sequence_waves = most;
     }
     entry_cost(g.sequence_waves, split_sides); // leaves `wide` as it will be
     g.jobs_per_point = *split_sides ? jobs_split : jobs;
@@ -639,7 +633,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.off_pts = at;
     at += table_slots * S * point_record;
     g.off_iter = at;
-    at += 2 * S * arrays * (tri_all | 1u);
+    at += S * arrays * (tri_all | 1u);
     g.off_jobs = at;
     at += table_elems_for(may_split);
     out->lds_bytes = g.tables_at + at * esize;
@@ -861,7 +855,7 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
     if (fits && !lane_kernels && plan->rec.g.points_per_pass == 0) {
         // the fused product has no job-list variant of the kernel: whole points side by side
         const Tiling& g = plan->rec.g;
-        const unsigned wide = plan->rec.threads - 64 * (1 + g.sequence_waves + g.slice_waves);
+        const unsigned wide = plan->rec.threads - 64 * g.slice_waves;
         plan->rec.g.points_per_pass = g.jobs_per_point >= wide ? 1u : wide / g.jobs_per_point;
     }
     if (!fits) {

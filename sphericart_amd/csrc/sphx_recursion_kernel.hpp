@@ -14,25 +14,29 @@ namespace sphx {
 
 // ---------------------------------------------------------------------------
 // l > H through the recursion. NT = 512 or 1024 threads, persistent workgroups
-// that walk over tiles of `tile` consecutive points, four tiles in flight per
-// workgroup, every wave with a role of its own and one barrier per tile:
+// that walk over tiles of `tile` consecutive points. A tile has two phases with a
+// barrier in front of each:
 //
-//   wave 0       one batch of up to eight tiles ahead, one lane per point:
-//                normalised coordinates, c_m, s_m, 2(m+1)z into LDS (azimuth_job);
-//   waves 1 ..   tile i+1, one lane per (point, l, sequence): the bare Q recursions,
-//                every iterate into LDS (sequence_job); g.sequence_waves of them;
-//   entry waves  tile i, one job per (point, l, m >= 0): the entries (l, +-m) of
-//                every requested array, chain rule included, staged in LDS in
-//                HBM layout (entry_job). Neighbouring lanes take neighbouring m
-//                of one (point, l), so their LDS traffic falls on neighbouring
-//                banks;
-//   all waves    after a second barrier: stream the staged rows of tile i to HBM
-//                with 16-byte stores.
+//   entries      every wave (but the slice waves), one job per (point, l, m >= 0) of
+//                tile i: the entries (l, +-m) of every requested array, chain rule
+//                included, staged in LDS in HBM layout (entry_job). Neighbouring
+//                lanes take neighbouring m of one (point, l), so their LDS traffic
+//                falls on neighbouring banks;
+//   flush        most waves stream the staged rows of tile i to HBM with 16-byte
+//                stores, and meanwhile
+//     wave 0       one batch of up to eight tiles ahead, one lane per point:
+//                  normalised coordinates, c_m, s_m, 2(m+1)z into LDS (azimuth_job);
+//     waves 1 ..   tile i+1, one lane per (point, l, sequence): the bare Q
+//                  recursions, every iterate into LDS (sequence_job);
+//                  g.sequence_waves of them.
 //
-// The first two stages are short chains of dependent operations that only a
-// few lanes can share; running them one and two tiles ahead of the wide stage
-// takes them off the critical path. The point tables are kept in three
-// buffers, the iterates in two, the staged rows in one. (A second row buffer,
+// The entries keep the vector units of the CU busy; the flush waits for the
+// stores to drain and issues little. Tables and recursions are short chains of
+// dependent operations that only a few lanes can share: in the flush they cost
+// no time of their own, and the entries then have every wave. (Next to the
+// entries, as they were first, they took a fifth of the waves and of the issue
+// slots of the phase that bounds the tile.) The point tables are kept in two
+// buffers, the iterates and the staged rows in one. (A second row buffer,
 // flushed by waves of their own while the next tile is computed, was built and
 // measured slower on every shape: waves that only flush wait for their own LDS
 // loads most of the time, and the tile has to be half as large.)
@@ -153,17 +157,18 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
     const unsigned iterate_stride = tri_all | 1u;
     // The tables are made for 2^az_shift tiles at a time (a batch), one lane per point, so that
     // the recurrences, a chain of dependent operations that few lanes share, run once per batch
-    // instead of once per tile. Single tiles are made two rounds ahead and kept in three
-    // buffers; batches are made one batch ahead and kept in two.
+    // instead of once per tile. Single tiles are made two tiles ahead (the recursions of the
+    // next tile run in the same phase and read the one in between), batches one batch ahead;
+    // two buffers either way, since a tile's tables are done with when its entries are.
     const unsigned batch_tiles = 1u << g.az_shift;
     const unsigned batch_lead = batch_tiles == 1 ? 2u : 1u;
-    const unsigned batch_buffers = batch_tiles == 1 ? 3u : 2u;
+    const unsigned batch_buffers = 2u;
     auto point_data = [&](unsigned n, unsigned s) -> T* { // point s of this workgroup's n-th tile
         const unsigned slot = (((n >> g.az_shift) % batch_buffers) << g.az_shift) | (n & (batch_tiles - 1u));
         return lds + g.off_pts + (slot * S + s) * point_stride;
     };
-    auto iterates = [&](unsigned buffer, unsigned s, unsigned which, int l) -> T* {
-        return lds + g.off_iter + ((buffer * S + s) * ARRAYS + which) * iterate_stride + l * (l + 1) / 2;
+    auto iterates = [&](unsigned s, unsigned which, int l) -> T* {
+        return lds + g.off_iter + (s * ARRAYS + which) * iterate_stride + l * (l + 1) / 2;
     };
 
     // same XCD-contiguous walk as the closed-form kernel
@@ -286,7 +291,7 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
             azimuth_job<T>(p, L, rec + 8, rec + 8 + (L + 1), rec + 8 + 2 * (L + 1));
         }
     };
-    // stage two of tile n (waves 1 .. g.sequence_waves)
+    // the recursions of tile n (waves 1 .. g.sequence_waves)
     auto recursion_stage = [&](unsigned n) {
         const unsigned count = valid_in(n);
         const unsigned per_l = count * ARRAYS;
@@ -299,15 +304,15 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
             const unsigned which = rest - s * ARRAYS;
             const T* rec = point_data(n, s);
             sequence_job<T>(l, static_cast<int>(which), rec[2], rec[7], Q, rec + 8 + 2 * (L + 1),
-                            iterates(n & 1u, s, which, l));
+                            iterates(s, which, l));
         }
     };
 
-    // The waves between the sequence waves and the slice waves compute entries.
-    const unsigned entry_first_wave = 1 + g.sequence_waves;
+    // All waves but the slice waves, the last ones, compute entries.
     const unsigned entry_end_wave = NT / 64 - g.slice_waves;
-    const unsigned wide_first = 64 * entry_first_wave;
-    const unsigned wide_lanes = 64 * (entry_end_wave - entry_first_wave);
+    const unsigned wide_lanes = 64 * entry_end_wave;
+    // the waves that prepare the next tiles while the others flush
+    const unsigned apart_waves = 1 + g.sequence_waves;
 
     constexpr unsigned LINE = 128u / static_cast<unsigned>(sizeof(O)); // elements per 128-byte line
     // position within its 128-byte line of element `element` of an output array
@@ -370,17 +375,21 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
                     if (6 % among == who) closed_form_job<T, MODE, NORM, H, 41, 45>(p, rows);
                     if (7 % among == who) closed_form_job<T, MODE, NORM, H, 45, 49>(p, rows);
                 } else {
-                    if (who == 0) closed_form_job<T, MODE, NORM, H>(p, rows);
+                    // (l <= 1: four entries, the chain rule of each is most of its work)
+                    if (0 % among == who) closed_form_job<T, MODE, NORM, H, 0, 1>(p, rows);
+                    if (1 % among == who) closed_form_job<T, MODE, NORM, H, 1, 2>(p, rows);
+                    if (2 % among == who) closed_form_job<T, MODE, NORM, H, 2, 3>(p, rows);
+                    if (3 % among == who) closed_form_job<T, MODE, NORM, H, 3, 4>(p, rows);
                 }
             }
         }
     };
 
-    // stage three of tile n (the entry waves)
+    // the entries of tile n (the entry waves)
     auto entry_stage = [&](unsigned n) {
         const unsigned valid = valid_in(n);
         O* staged = row_lds;
-        const unsigned t = tid - wide_first;
+        const unsigned t = tid;
         const Phases ph = phases_of(n);
         const unsigned phase_sph = ph.sph, phase_dsph = ph.dsph, phase_ddsph = ph.ddsph;
         // what depends on the point only
@@ -405,9 +414,9 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
             p.ir = rec[6];
             c = rec + 8;
             sn = rec + 8 + (L + 1);
-            itA = iterates(n & 1u, s, 0, 0);
-            itB = iterates(n & 1u, s, MODE >= 1 ? 1 : 0, 0);
-            itC = iterates(n & 1u, s, MODE == 2 ? 2 : 0, 0);
+            itA = iterates(s, 0, 0);
+            itB = iterates(s, MODE >= 1 ? 1 : 0, 0);
+            itC = iterates(s, MODE == 2 ? 2 : 0, 0);
             // rows are addressed with the entry's index in the full row; shift the bases when
             // the staged rows start at l = H + 1
             rows.sph = staged + phase_sph + s * row_stride - skip;
@@ -530,6 +539,7 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
                     const unsigned nvec = (full_hi - full_lo) / W;
                     const V* in = reinterpret_cast<const V*>(region + full_lo);
                     V* out = reinterpret_cast<V*>(line0 + full_lo);
+                    // (two or four loads in flight per lane ahead of their stores: no faster on any shape)
                     for (unsigned v = ft; v < nvec; v += count) {
                         emit<O, SPHX_STREAMING_STORES>(in[v], out + v);
                     }
@@ -581,16 +591,15 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
     // component r % 3): its lanes multiply the staged entries with the point's row of sph_grad
     // and a butterfly adds the lanes' sums up. With WHOLE == false the staged rows begin at
     // l = H + 1 and closed_form_vjp_kernel has already stored the sum over l <= H, so the
-    // result is added to what xyz_grad holds. Wave 0 stays out: it has loads in flight.
-    auto contract_stage = [&](unsigned n) {
+    // result is added to what xyz_grad holds. By `among` waves of which this is number `who`.
+    auto contract_stage = [&](unsigned n, unsigned who, unsigned among) {
         if constexpr (VJP) {
             const unsigned valid = valid_in(n);
             const unsigned long long first = static_cast<unsigned long long>(tile_of(n)) * S;
             const T* staged = row_lds + g.off_dsph; // O is T here
             const T* upstream = sph;
             T* xyz_grad = dsph;
-            if (wave == 0) return;
-            for (unsigned r = wave - 1; r < valid * 3; r += NT / 64 - 1) {
+            for (unsigned r = who; r < valid * 3; r += among) {
                 const unsigned s = r / 3;
                 const T* row = staged + r * row_stride - skip; // indexed with the entry's index in the full row
                 const T* weight = upstream + (first + s) * ny;
@@ -623,37 +632,35 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
             azimuth_stage(1, rx, ry, rz);
             fetch(2, rx, ry, rz);
         }
-    } else if (wave < entry_first_wave) {
+    } else if (wave < apart_waves) {
         recursion_stage(0);
     }
 
-    // every wave takes part in the flush, after a second barrier
     for (unsigned n = 0; valid_in(n) != 0; ++n) {
-        __syncthreads(); // tables of tile n+1, iterates of tile n in place; rows of tile n-1 flushed
-        // the closed-form slices go round all waves: those that make tables and iterates
-        // have time to spare; or to wave 0 and the waves set aside for them, when the entry
-        // waves that had a slice on top of their jobs were what the tile waited for
+        __syncthreads(); // iterates of tile n in place; rows of tile n-1 flushed
+        // the closed-form slices go round all waves, the last wave first (the jobs are dealt from
+        // lane 0 up, so that the last waves are the ones a short last round leaves idle), or to the
+        // waves set aside for them when the waves that had a slice on top of their jobs were what
+        // the tile waited for
         if (g.slice_waves == 0) {
-            closed_stage(n, wave, NT / 64);
-        } else if (wave == 0 || wave >= entry_end_wave) {
-            closed_stage(n, wave == 0 ? 0u : wave - entry_end_wave + 1u, g.slice_waves + 1u);
+            closed_stage(n, NT / 64 - 1 - wave, NT / 64);
+        } else if (wave >= entry_end_wave) {
+            closed_stage(n, wave - entry_end_wave, g.slice_waves);
         }
+        if (wave < entry_end_wave) entry_stage(n);
+        __syncthreads(); // rows of tile n complete, its tables and iterates done with
         if (wave == 0) {
             if ((n & (batch_tiles - 1u)) == 0) {
                 azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
                 fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz);
             }
             if (prefix_wave) prefix_slice();
-        } else if (wave < entry_first_wave) {
+        } else if (wave < apart_waves) {
             recursion_stage(n + 1);
-        } else if (wave < entry_end_wave) {
-            entry_stage(n);
-        }
-        __syncthreads(); // rows of tile n complete
-        if constexpr (VJP) {
-            contract_stage(n);
+        } else if constexpr (VJP) {
+            contract_stage(n, wave - apart_waves, NT / 64 - apart_waves);
         } else {
-            flush_stage(n, tid, NT);
+            flush_stage(n, tid - 64 * apart_waves, NT - 64 * apart_waves);
         }
     }
     // what is left of this workgroup's share of the batches (no barrier follows)

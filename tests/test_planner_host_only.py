@@ -26,8 +26,9 @@ SHAPES = [
     (500_000, 3, 2, 0, 1, "hessians_lanes_kernel<float, true>"),
     (1_000_000, 10, 1, 0, 1, "recursion_kernel<float, 1, true, true, false, false, true>"),
     (50_000, 20, 2, 1, 1, "pairs_kernel<double, 2, true>"),
-    (2_000, 32, 1, 0, 1, "recursion_kernel<float, 1, true, false, false, false, false>"),
-    (5, 24, 2, 1, 1, "recursion_kernel<double, 2, true, true, true, false, false>"),
+    (2_000, 32, 1, 0, 1, "recursion_kernel<float, 1, true, true, false, false, true>"),
+    (2_000, 40, 1, 1, 1, "recursion_kernel<double, 1, true, false, false, false, false>"),
+    (5, 24, 2, 1, 1, "recursion_kernel<double, 2, true, true, false, false, false>"),
     (1, 0, 0, 0, 1, "closed_form_kernel<float, 0, true, 0, false>"),
 ]
 
