@@ -44,24 +44,31 @@ constexpr bool kLargeGroups =
     !VJP && (MODE <= 1 || (MODE == 2 && sizeof(T) == 4) || (MODE == 2 && SPLIT && (!NORM || LIST)));
 
 template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false,
-          typename O = T, unsigned NT = kRecursionThreads>
+          typename O = T, unsigned NT = kRecursionThreads, bool TOGETHER = false>
 static hipError_t launch_recursion(const Launch& l, const typename AsGiven<O>::type* xyz,
                                    typename AsGiven<O>::type* sph, typename AsGiven<O>::type* dsph,
                                    typename AsGiven<O>::type* ddsph, hipStream_t stream) {
     if constexpr (!VJP && !LIST) {
         // the variant whose entry lanes take the jobs of a tile as one list
         if (l.g.points_per_pass == 0) {
-            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, false, true, O, NT>(l, xyz, sph, dsph, ddsph, stream);
+            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, false, true, O, NT, TOGETHER>(l, xyz, sph, dsph, ddsph, stream);
         }
     }
     if constexpr (NT == kRecursionThreads && kLargeGroups<T, MODE, VJP, NORM, SPLIT, LIST>) {
         if (l.threads == 2 * kRecursionThreads) {
-            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O, 2 * kRecursionThreads>(
+            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O, 2 * kRecursionThreads, TOGETHER>(
                 l, xyz, sph, dsph, ddsph, stream);
         }
     }
+    if constexpr (sizeof(T) == 8 && !TOGETHER) {
+        // the variant whose recursions run next to the entries
+        if (l.g.together != 0) {
+            return launch_recursion<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O, NT, true>(l, xyz, sph, dsph, ddsph, stream);
+        }
+    }
+    if ((l.g.together != 0) != TOGETHER) return hipErrorInvalidValue; // never planned
     if (l.threads != NT) return hipErrorInvalidValue; // never planned
-    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O, NT>;
+    auto kernel = recursion_kernel<T, MODE, NORM, WHOLE, SPLIT, VJP, LIST, O, NT, TOGETHER>;
     // The workgroups are persistent: launch exactly as many as are resident at once (registers
     // may allow fewer per CU than LDS does), or the last ones would run alone after the rest.
     unsigned workgroups = l.workgroups;

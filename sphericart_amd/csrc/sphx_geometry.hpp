@@ -27,8 +27,9 @@ struct Tiling {
     unsigned az_shift;      // the point tables are made for 2^az_shift tiles at a time
     unsigned chunk_shift;   // a workgroup takes 2^chunk_shift consecutive tiles at a time
     unsigned prefix_inside; // rows that start at l = 7: the recursion kernel writes l <= 6 too
-    unsigned slice_waves;   // not 0: wave 0 and this many waves of their own evaluate the closed forms
-                            // of l <= 6 (whole rows, one row buffer); 0: the slices go round all waves
+    unsigned slice_waves;   // not 0: this many waves of their own (together: and wave 0) evaluate the closed
+                            // forms of l <= 6 (whole rows); 0: the slices go round all waves
+    unsigned together;      // recursion_kernel, float64: 1 = the recursions run next to the entries (TOGETHER)
     // LDS carve-up, in elements of T: the staged rows come first, rows_elems of them, with the
     // gradient and second-derivative rows at off_dsph and off_ddsph inside a buffer; the other
     // offsets count from the start of dynamic LDS. (recursion_kernel: the row offsets are in

@@ -25,7 +25,7 @@ static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_HESSIAN_LANES",
     "SPHX_HESSIAN_LANES_PARTS", "SPHX_JOB_LIST",
     "SPHX_PAIRS", "SPHX_PAIRS_BATCH", "SPHX_PAIRS_CHUNK", "SPHX_PAIRS_PREP_WAVES", "SPHX_PAIRS_SEQUENCE_WAVES", "SPHX_PAIRS_TILE",
-    "SPHX_PREFIX_INSIDE", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
+    "SPHX_PREFIX_INSIDE", "SPHX_RECURSIONS_TOGETHER", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_ALONE", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
     "SPHX_VALUES_PACK", "SPHX_VALUES_TILE_STEP", "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE", "SPHX_VJP_STEP_FLOOR", "SPHX_VJP_TILE_STEP",
@@ -432,13 +432,24 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     const unsigned jobs_split = 2 * jobs - static_cast<unsigned>(l_max - hard);
     bool may_split = mode == 2 && switch_or(SW_SPLIT_SIDES, 1) != 0;
     auto table_elems_for = [&](bool split) { return ((split ? jobs_split : jobs) * 4 + esize - 1) / esize; };
-    // per point: the rows, point tables twice, iterates once
+    // Which division of the work (recursion_kernel): the recursions of the next tile while this one is flushed, or
+    // next to its entries (TOGETHER, float64 only). Next to the entries they are ahead where the flush would wait
+    // for them: solid second derivatives at l_max = 4 .. 18 (5-11 %, cfg4 557 -> 513 us) and solid gradients up to
+    // l_max = 10 (0-11 %) in calls of 32 768 points or more, and gradients from l_max = 27 on, where a recursion is a
+    // long chain (10 %). Everywhere else in float64 the other division gains 2-14 %, as in all of float32.
+    const bool together_by_shape = elem == 8 && ((!normalized && n_samples >= 32768 &&
+                                         (mode == 2 ? l_max >= 4 && l_max <= 18 : mode == 1 && l_max <= 10)) ||
+                                        (mode == 1 && l_max >= 27));
+    const bool together = elem == 8 && switch_or(SW_RECURSIONS_TOGETHER, together_by_shape ? 1 : 0) != 0;
+    g.together = together ? 1u : 0u;
+    // per point: the rows, point tables twice and iterates once (together: three times, when a batch is a single tile,
+    // and twice)
     // staged rows are `row_stride` apart (recursion_kernel): nrow, or a little more when the rows
     // are cut so that they keep their position within 16 bytes
     const unsigned row_stride = nrow + (whole ? 0u : nyh % (16u / osize));
     const unsigned rows_per_point = components_of(mode) * row_stride;
     // (the records of a point and its sequences of iterates are an odd number of words apart)
-    const unsigned rest_per_point = 2 * ((8 + 3 * (l_max + 1)) | 1u) + arrays * (tri_all | 1u);
+    const unsigned rest_per_point = (together ? 3u : 2u) * ((8 + 3 * (l_max + 1)) | 1u) + (together ? 2u : 1u) * arrays * (tri_all | 1u);
     unsigned fixed = 0; // bytes
     const unsigned point_bytes = rows_per_point * osize + rest_per_point * esize;
     auto bytes_for = [&](unsigned S) { return S * point_bytes + fixed; };
@@ -493,14 +504,14 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         for (unsigned shift = cap < 0 ? 0u : (cap > 6 ? 6u : static_cast<unsigned>(cap)); shift >= 1; --shift) {
             const unsigned tiles = 1u << shift;
             if (tiles * S > 64) continue;
-            const unsigned extra = (2 * tiles - 2) * S * point_record * esize;
+            const unsigned extra = (2 * tiles - (together ? 3 : 2)) * S * point_record * esize;
             if (bytes_for(S) + extra <= allowed || bytes_for(S) + extra <= budget) {
                 az_shift = shift;
                 break;
             }
         }
     }
-    const unsigned table_slots = 2u << az_shift;
+    const unsigned table_slots = together && az_shift == 0 ? 3u : 2u << az_shift;
 
     g.n_samples = n_samples;
     g.l_max = l_max;
@@ -538,8 +549,8 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     };
     // rounds of the entry waves per tile, in tenths of two-sided jobs, with `waves` sequence waves
     auto entry_cost = [&](unsigned waves, bool* split) {
-        (void)waves; // (the sequence waves work while the others flush and compute entries like the rest)
-        wide = threads - 64 * g.slice_waves;
+        // (together: wave 0 and the sequence waves compute no entries)
+        wide = threads - 64 * ((together ? 1 + waves : 0) + g.slice_waves);
         // (with two or more points per tile the jobs go as a list ordered by kind, which fills the lanes without
         // splitting, and the two-sided job shares the common factors: 5-15 % faster; with one point per tile
         // splitting stays)
@@ -554,7 +565,32 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // with two, 66-69 % with four) and three in float64; second derivatives in float32 six for normalised harmonics
     // and three for solid ones, whose entries are shorter and whose flush weighs more (l_max = 8: 72.6 % with three,
     // 65 % with six; two from l_max = 16 on); in float64 two, three at both ends of the l_max range.
-    if (threads > kRecursionThreads) {
+    if (together) {
+        // Next to the entries a sequence wave takes a wave from them. Sixteen waves: gradients as few rounds of
+        // recursions as four waves would need, with as few waves as that takes; second derivatives, where the
+        // entries weigh more, two, three at both ends of the l_max range; values three. Eight waves: one where it
+        // saves the entry waves a round per tile and for values alone, whose recursions are a third of the work;
+        // second derivatives keep two.
+        const unsigned recursions = S * arrays * static_cast<unsigned>(l_max - hard);
+        if (threads > kRecursionThreads) {
+            if (mode == 1) {
+                const unsigned least = (recursions + 255u) / 256u;
+                g.sequence_waves = 2;
+                while (g.sequence_waves < 4 && (recursions + 64u * g.sequence_waves - 1u) / (64u * g.sequence_waves) > least) {
+                    ++g.sequence_waves;
+                }
+            } else if (mode == 2) {
+                g.sequence_waves = l_max <= 4 || l_max >= 22 ? 3u : 2u;
+            } else {
+                g.sequence_waves = 3;
+            }
+        } else if (g.sequence_waves == 2 && mode != 2) {
+            bool split_one = false, split_two = false;
+            const unsigned with_one = entry_cost(1, &split_one);
+            const unsigned with_two = entry_cost(2, &split_two);
+            if (mode == 0 || with_one < with_two) g.sequence_waves = 1;
+        }
+    } else if (threads > kRecursionThreads) {
         if (mode == 1) {
             g.sequence_waves = elem == 4 ? 4 : 3;
         } else if (mode == 2 && elem == 4) {
@@ -571,7 +607,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         // (at least four waves flush)
         const int forced_seq = switch_or(SW_SEQUENCE_WAVES, 0);
         if (forced_seq >= 1) g.sequence_waves = static_cast<unsigned>(forced_seq);
-        const unsigned most = threads / 64u - 5u;
+        const unsigned most = together ? 4u : threads / 64u - 5u;
         if (g.sequence_waves > most) g.sequence_waves = most;
     }
     entry_cost(g.sequence_waves, split_sides); // leaves `wide` as it will be
@@ -633,7 +669,7 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     g.off_pts = at;
     at += table_slots * S * point_record;
     g.off_iter = at;
-    at += S * arrays * (tri_all | 1u);
+    at += (together ? 2u : 1u) * S * arrays * (tri_all | 1u);
     g.off_jobs = at;
     at += table_elems_for(may_split);
     out->lds_bytes = g.tables_at + at * esize;
@@ -855,7 +891,7 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
     if (fits && !lane_kernels && plan->rec.g.points_per_pass == 0) {
         // the fused product has no job-list variant of the kernel: whole points side by side
         const Tiling& g = plan->rec.g;
-        const unsigned wide = plan->rec.threads - 64 * g.slice_waves;
+        const unsigned wide = plan->rec.threads - 64 * ((g.together ? 1 + g.sequence_waves : 0) + g.slice_waves);
         plan->rec.g.points_per_pass = g.jobs_per_point >= wide ? 1u : wide / g.jobs_per_point;
     }
     if (!fits) {
@@ -937,7 +973,8 @@ std::string describe(const Plan& plan, int l_max, int mode, bool is_f64, bool no
         }
         text += "recursion_kernel<" + head + ", " + (plan.whole ? "true" : "false") + ", " +
                 (plan.split_sides ? "true" : "false") + ", false, " +
-                (plan.rec.g.points_per_pass == 0 ? "true" : "false") + ">" + geometry(plan.rec);
+                (plan.rec.g.points_per_pass == 0 ? "true" : "false") + ">" + geometry(plan.rec) +
+                (plan.rec.g.together != 0 ? " (recursions next to the entries)" : "");
     }
     return text;
 }

@@ -33,13 +33,19 @@ namespace sphx {
 // The entries keep the vector units of the CU busy; the flush waits for the
 // stores to drain and issues little. Tables and recursions are short chains of
 // dependent operations that only a few lanes can share: in the flush they cost
-// no time of their own, and the entries then have every wave. (Next to the
-// entries, as they were first, they took a fifth of the waves and of the issue
-// slots of the phase that bounds the tile.) The point tables are kept in two
-// buffers, the iterates and the staged rows in one. (A second row buffer,
-// flushed by waves of their own while the next tile is computed, was built and
-// measured slower on every shape: waves that only flush wait for their own LDS
-// loads most of the time, and the tile has to be half as large.)
+// no time of their own, and the entries then have every wave. The point tables
+// are kept in two buffers, the iterates and the staged rows in one. (A second
+// row buffer, flushed by waves of their own while the next tile is computed,
+// was built and measured slower on every shape: waves that only flush wait for
+// their own LDS loads most of the time, and the tile has to be half as large.)
+//
+// TOGETHER == true (float64 only) is the other division of the same work: wave 0
+// and the sequence waves do their part next to the entries, a tile ahead of them
+// (tables in three buffers when a batch is a single tile, iterates in two), the
+// waves after them compute the entries, and every wave flushes. In float64 the
+// recursions are long enough to hold up a flush that they share, and for solid
+// harmonics, whose entries are short, and at high l_max this division is the
+// faster one by 5-14 %; the host says which one a launch takes.
 //
 // NT = 512: two workgroups share a CU, half of its LDS each. NT = 1024: one
 // workgroup has the CU and all of its LDS, its tiles are more than twice as
@@ -70,13 +76,14 @@ namespace sphx {
 // rows are rows of O, so a tile holds as many points as in the float kernel's and the flush is
 // that kernel's.
 template <typename T, int MODE, bool NORM, bool WHOLE, bool SPLIT, bool VJP = false, bool LIST = false,
-          typename O = T, unsigned NT = kRecursionThreads>
+          typename O = T, unsigned NT = kRecursionThreads, bool TOGETHER = false>
 __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling g, const O* __restrict__ xyz,
                                                                      O* __restrict__ sph,
                                                                      O* __restrict__ dsph,
                                                                      O* __restrict__ ddsph) {
     static_assert(!VJP || (MODE == 1 && !SPLIT), "the fused product is built on the gradient kernel");
     static_assert(!VJP || std::is_same<T, O>::value, "the fused product stages what it computes");
+    static_assert(!TOGETHER || sizeof(T) == 8, "float32 has the recursions in the flush only");
     constexpr int H = MODE == 2 ? 1 : 6;
     constexpr unsigned NYH = (H + 1) * (H + 1);
     constexpr unsigned ARRAYS = MODE + 1; // iterate arrays per point: A, B, C
@@ -159,16 +166,18 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
     // the recurrences, a chain of dependent operations that few lanes share, run once per batch
     // instead of once per tile. Single tiles are made two tiles ahead (the recursions of the
     // next tile run in the same phase and read the one in between), batches one batch ahead;
-    // two buffers either way, since a tile's tables are done with when its entries are.
+    // two buffers either way, since a tile's tables are done with when its entries are
+    // (TOGETHER: the entries of a tile run in that phase too, three buffers for single tiles).
     const unsigned batch_tiles = 1u << g.az_shift;
     const unsigned batch_lead = batch_tiles == 1 ? 2u : 1u;
-    const unsigned batch_buffers = 2u;
+    const unsigned batch_buffers = TOGETHER && batch_tiles == 1 ? 3u : 2u;
     auto point_data = [&](unsigned n, unsigned s) -> T* { // point s of this workgroup's n-th tile
         const unsigned slot = (((n >> g.az_shift) % batch_buffers) << g.az_shift) | (n & (batch_tiles - 1u));
         return lds + g.off_pts + (slot * S + s) * point_stride;
     };
-    auto iterates = [&](unsigned s, unsigned which, int l) -> T* {
-        return lds + g.off_iter + (s * ARRAYS + which) * iterate_stride + l * (l + 1) / 2;
+    auto iterates = [&](unsigned n, unsigned s, unsigned which, int l) -> T* { // of this workgroup's n-th tile
+        const unsigned buffer = TOGETHER ? n & 1u : 0u;
+        return lds + g.off_iter + ((buffer * S + s) * ARRAYS + which) * iterate_stride + l * (l + 1) / 2;
     };
 
     // same XCD-contiguous walk as the closed-form kernel
@@ -304,15 +313,17 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
             const unsigned which = rest - s * ARRAYS;
             const T* rec = point_data(n, s);
             sequence_job<T>(l, static_cast<int>(which), rec[2], rec[7], Q, rec + 8 + 2 * (L + 1),
-                            iterates(s, which, l));
+                            iterates(n, s, which, l));
         }
     };
 
-    // All waves but the slice waves, the last ones, compute entries.
-    const unsigned entry_end_wave = NT / 64 - g.slice_waves;
-    const unsigned wide_lanes = 64 * entry_end_wave;
-    // the waves that prepare the next tiles while the others flush
+    // wave 0 and the sequence waves prepare the next tiles
     const unsigned apart_waves = 1 + g.sequence_waves;
+    // All waves but the slice waves, the last ones, compute entries (TOGETHER: the waves in between).
+    const unsigned entry_first_wave = TOGETHER ? apart_waves : 0u;
+    const unsigned entry_end_wave = NT / 64 - g.slice_waves;
+    const unsigned wide_first = 64 * entry_first_wave;
+    const unsigned wide_lanes = 64 * (entry_end_wave - entry_first_wave);
 
     constexpr unsigned LINE = 128u / static_cast<unsigned>(sizeof(O)); // elements per 128-byte line
     // position within its 128-byte line of element `element` of an output array
@@ -389,7 +400,7 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
     auto entry_stage = [&](unsigned n) {
         const unsigned valid = valid_in(n);
         O* staged = row_lds;
-        const unsigned t = tid;
+        const unsigned t = tid - wide_first;
         const Phases ph = phases_of(n);
         const unsigned phase_sph = ph.sph, phase_dsph = ph.dsph, phase_ddsph = ph.ddsph;
         // what depends on the point only
@@ -414,9 +425,9 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
             p.ir = rec[6];
             c = rec + 8;
             sn = rec + 8 + (L + 1);
-            itA = iterates(s, 0, 0);
-            itB = iterates(s, MODE >= 1 ? 1 : 0, 0);
-            itC = iterates(s, MODE == 2 ? 2 : 0, 0);
+            itA = iterates(n, s, 0, 0);
+            itB = iterates(n, s, MODE >= 1 ? 1 : 0, 0);
+            itC = iterates(n, s, MODE == 2 ? 2 : 0, 0);
             // rows are addressed with the entry's index in the full row; shift the bases when
             // the staged rows start at l = H + 1
             rows.sph = staged + phase_sph + s * row_stride - skip;
@@ -636,25 +647,46 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
         recursion_stage(0);
     }
 
+    // wave 0's part of tile n: the tables of a batch ahead, a slice of the rows that start at l = 7
+    auto table_stage = [&](unsigned n) {
+        if ((n & (batch_tiles - 1u)) == 0) {
+            azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
+            fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz);
+        }
+        if (prefix_wave) prefix_slice();
+    };
     for (unsigned n = 0; valid_in(n) != 0; ++n) {
         __syncthreads(); // iterates of tile n in place; rows of tile n-1 flushed
-        // the closed-form slices go round all waves, the last wave first (the jobs are dealt from
-        // lane 0 up, so that the last waves are the ones a short last round leaves idle), or to the
-        // waves set aside for them when the waves that had a slice on top of their jobs were what
-        // the tile waited for
+        // The closed-form slices go round all waves, or to the waves set aside for them when the waves that had a
+        // slice on top of their jobs were what the tile waited for. Round all waves: the last wave first (the jobs
+        // are dealt from lane 0 up, so that the last waves are the ones a short last round leaves idle); TOGETHER:
+        // the first wave first, the waves that make tables and iterates have time to spare.
         if (g.slice_waves == 0) {
-            closed_stage(n, NT / 64 - 1 - wave, NT / 64);
+            closed_stage(n, TOGETHER ? wave : NT / 64 - 1 - wave, NT / 64);
+        } else if constexpr (TOGETHER) {
+            if (wave == 0 || wave >= entry_end_wave) {
+                closed_stage(n, wave == 0 ? 0u : wave - entry_end_wave + 1u, g.slice_waves + 1u);
+            }
         } else if (wave >= entry_end_wave) {
             closed_stage(n, wave - entry_end_wave, g.slice_waves);
         }
-        if (wave < entry_end_wave) entry_stage(n);
-        __syncthreads(); // rows of tile n complete, its tables and iterates done with
-        if (wave == 0) {
-            if ((n & (batch_tiles - 1u)) == 0) {
-                azimuth_stage((n >> g.az_shift) + batch_lead, rx, ry, rz);
-                fetch((n >> g.az_shift) + batch_lead + 1, rx, ry, rz);
+        if constexpr (TOGETHER) {
+            if (wave == 0) {
+                table_stage(n);
+            } else if (wave < apart_waves) {
+                recursion_stage(n + 1);
             }
-            if (prefix_wave) prefix_slice();
+        }
+        if (wave >= entry_first_wave && wave < entry_end_wave) entry_stage(n);
+        __syncthreads(); // rows of tile n complete, its tables and iterates done with
+        if constexpr (TOGETHER) {
+            if constexpr (VJP) {
+                if (wave != 0) contract_stage(n, wave - 1, NT / 64 - 1); // (wave 0 has loads in flight)
+            } else {
+                flush_stage(n, tid, NT);
+            }
+        } else if (wave == 0) {
+            table_stage(n);
         } else if (wave < apart_waves) {
             recursion_stage(n + 1);
         } else if constexpr (VJP) {
