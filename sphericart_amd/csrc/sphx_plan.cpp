@@ -785,11 +785,11 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
     }
     // Values alone where the rows of few points fill LDS: pairs_kernel (below, with the derivatives), which keeps
     // the recursions of the next tile and the flush of this one side by side: 10-35 % faster than values_kernel
-    // (the recursion kernel from l_max = 34) from l_max = 23 in float32 and 20 in float64. Below, a point's pairs
-    // leave the entry lanes idle and values_kernel is ahead.
+    // (the recursion kernel from l_max = 34) from l_max = 24 in float32 and 19 in float64. Below, a point's pairs
+    // leave the entry lanes idle and values_kernel is ahead (float32 l_max = 23: 50.7 % against 44.2 %).
     if (lane_kernels && mode == 0 && l_max > hard) {
         const int pairs = switch_or(SW_PAIRS, 1);
-        const bool pairs_by_shape = n_samples >= 32768 && (elem == 4 ? l_max >= 23 : l_max >= 20);
+        const bool pairs_by_shape = n_samples >= 32768 && (elem == 4 ? l_max >= 24 : l_max >= 19);
         if (pairs == 2 || (pairs == 1 && pairs_by_shape)) {
             PairsChoice want;
             want.tile = static_cast<unsigned>(switch_or(SW_PAIRS_TILE, 0));
@@ -819,14 +819,17 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
         return SPHX_OK;
     }
     // Derivatives where the rows of few points fill LDS: pairs_kernel, whose entry lanes keep one (l, m) pair for
-    // the whole launch and whose other work runs while the rows are flushed. Gradients: 5-15 % faster than the
-    // recursion kernel from l_max = 20 in float32 and 16 in float64 (cfg5 700 -> 570-620 us); below, a point's
-    // pairs leave most of the entry lanes idle. Second derivatives: ahead in float64 from l_max = 20; in float32
-    // the recursion kernel's job list by kind fills sixteen waves better. SPHX_PAIRS: 0 never, 2 wherever it fits.
+    // the whole launch and whose other work runs while the rows are flushed. Gradients: up to 15 % faster than the
+    // recursion kernel from l_max = 20 in float32 and 17 in float64 (cfg5 700 -> 570-620 us); below, a point's
+    // pairs leave most of the entry lanes idle. Second derivatives in float64: ahead by 3-7 % at l_max = 20 and 21
+    // (normalised) and at l_max = 20 and from 24 on (solid), behind by 2-25 % elsewhere; in float32 the recursion
+    // kernel's job list by kind fills sixteen waves better. SPHX_PAIRS: 0 never, 2 wherever it fits.
     {
         const int pairs = switch_or(SW_PAIRS, 1);
-        const bool pairs_by_shape = n_samples >= 32768 && (mode == 1 ? (elem == 4 ? l_max >= 20 : l_max >= 16)
-                                                                     : (elem == 8 && l_max >= 20));
+        const bool pairs_by_shape =
+            n_samples >= 32768 &&
+            (mode == 1 ? (elem == 4 ? l_max >= 20 : l_max >= 17)
+                       : elem == 8 && (l_max == 20 || (normalized ? l_max == 21 : l_max >= 24)));
         if (lane_kernels && mode >= 1 && l_max > hard && (pairs == 2 || (pairs == 1 && pairs_by_shape))) {
             PairsChoice want;
             want.tile = static_cast<unsigned>(switch_or(SW_PAIRS_TILE, 0));
@@ -843,12 +846,12 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
     // Gradients just above the closed forms: the lanes kernel (one point per lane, the channels dealt to the
     // waves) up to l_max = 13 in float32 and wherever its tiles fit in float64; from there the recursion kernel with
     // its jobs as a list ordered by kind is ahead. Where the recursion kernel runs in workgroups of 1024 threads
-    // (calls of 32 768 points or more) it is ahead earlier: the lanes keep l_max <= 8 and 11 in float32 and
-    // l_max = 7 in float64. SPHX_GRADIENT_LANES: 0 never, 2 wherever the rows fit.
+    // (calls of 32 768 points or more) it is ahead from l_max = 8 on (3-20 %): the lanes keep l_max = 7; at
+    // 20 000 points from l_max = 10 on (6-30 %).
+    // SPHX_GRADIENT_LANES: 0 never, 2 wherever the rows fit.
     const int gradient_lanes = switch_or(SW_GRADIENT_LANES, 1);
     const bool large_groups = group_threads(n_samples, mode, elem, lane_kernels) > kRecursionThreads && n_samples >= 32768;
-    const bool lanes_by_shape = large_groups ? (elem == 4 ? l_max <= 8 || l_max == 11 : l_max <= 7)
-                                             : elem == 8 || l_max <= 13;
+    const bool lanes_by_shape = large_groups ? l_max <= 7 : (n_samples >= 16384 ? l_max <= 9 : elem == 8 || l_max <= 13);
     if (lane_kernels && mode == 1 && gradient_lanes != 0 && (gradient_lanes == 2 || lanes_by_shape) &&
         plan_gradient_lanes(n_samples, l_max, elem, lds_limit, cus, &plan->closed)) {
         plan->lanes = true;
