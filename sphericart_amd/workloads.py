@@ -138,7 +138,7 @@ def _cfg5(seed, n, first):
 
 
 _GENERATORS = {"cfg1": _cfg1, "cfg2": _cfg2, "cfg3": _cfg3, "cfg4": _cfg4, "cfg5": _cfg5, "val10": _cfg2, "val22": _cfg2,
-               "grad10": _cfg3, "hess5": _cfg3}
+               "val28": _cfg2, "grad10": _cfg3, "hess5": _cfg3}
 
 WORKLOADS = {
     "cfg1": Workload(
@@ -176,6 +176,11 @@ WORKLOADS = {
     "val22": Workload(
         "val22", "spherical, l_max=22, f32, values, 500k points, uniform directions, r ~ U[0.5,5)",
         22, "f32", True, "values", 500_000, 1013,
+    ),
+    # and where the rows of few points fill LDS (pairs_kernel)
+    "val28": Workload(
+        "val28", "spherical, l_max=28, f32, values, 350k points, uniform directions, r ~ U[0.5,5)",
+        28, "f32", True, "values", 350_000, 1014,
     ),
     # likewise gradients at l_max just above the closed forms
     "grad10": Workload(

@@ -53,6 +53,6 @@ def test_clouds_are_the_same_bits_everywhere():
 
 
 def test_bytes_per_point():
-    want = {"cfg1": 2616, "cfg2": 76, "cfg3": 796, "cfg4": 30080, "cfg5": 17436, "val10": 496, "val22": 2128, "grad10": 1948, "hess5": 1884}
+    want = {"cfg1": 2616, "cfg2": 76, "cfg3": 796, "cfg4": 30080, "cfg5": 17436, "val10": 496, "val22": 2128, "val28": 3376, "grad10": 1948, "hess5": 1884}
     for name, w in WORKLOADS.items():
         assert w.bytes_per_point == want[name]
