@@ -403,9 +403,8 @@ static unsigned group_threads(size_t n_samples, int mode, size_t elem, bool forw
     const int want = switch_or(SW_GROUP_THREADS, 0);
     if (want == 512 || want == 1024) return static_cast<unsigned>(want);
     if (f64_hessians && l_max < 3) return kRecursionThreads;
-    // (normalised: one-sided jobs are 20 % more work, which sixteen waves make up for only at l_max = 3 and, with
-    // two or three points per tile, at l_max = 18 .. 23: 2-12 %)
-    if (f64_hessians && normalized && !(l_max == 3 || (l_max >= 18 && l_max <= 23))) return kRecursionThreads;
+    // (normalised: one-sided jobs are 20 % more work, which sixteen waves make up for only at l_max = 3: 12 %)
+    if (f64_hessians && normalized && l_max != 3) return kRecursionThreads;
     return n_samples >= 4096 ? 2 * kRecursionThreads : kRecursionThreads;
 }
 
@@ -821,15 +820,15 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
     // Derivatives where the rows of few points fill LDS: pairs_kernel, whose entry lanes keep one (l, m) pair for
     // the whole launch and whose other work runs while the rows are flushed. Gradients: up to 15 % faster than the
     // recursion kernel from l_max = 20 in float32 and 17 in float64 (cfg5 700 -> 570-620 us); below, a point's
-    // pairs leave most of the entry lanes idle. Second derivatives in float64: ahead by 3-7 % at l_max = 20 and 21
-    // (normalised) and at l_max = 20 and from 24 on (solid), behind by 2-25 % elsewhere; in float32 the recursion
+    // pairs leave most of the entry lanes idle. Second derivatives in float64: ahead by 3-9 % at l_max = 20 and,
+    // for solid harmonics, from 24 on, behind by 2-25 % elsewhere; in float32 the recursion
     // kernel's job list by kind fills sixteen waves better. SPHX_PAIRS: 0 never, 2 wherever it fits.
     {
         const int pairs = switch_or(SW_PAIRS, 1);
         const bool pairs_by_shape =
             n_samples >= 32768 &&
             (mode == 1 ? (elem == 4 ? l_max >= 20 : l_max >= 17)
-                       : elem == 8 && (l_max == 20 || (normalized ? l_max == 21 : l_max >= 24)));
+                       : elem == 8 && (l_max == 20 || (!normalized && l_max >= 24)));
         if (lane_kernels && mode >= 1 && l_max > hard && (pairs == 2 || (pairs == 1 && pairs_by_shape))) {
             PairsChoice want;
             want.tile = static_cast<unsigned>(switch_or(SW_PAIRS_TILE, 0));
