@@ -189,16 +189,18 @@ def test_planned_by_shape(library):
     """What the planner picks without overrides."""
     assert _plan_text(library, 200_000, 32, False, True).startswith("pairs_kernel<float, 1, true>")
     assert _plan_text(library, 100_000, 20, False, False).startswith("pairs_kernel<float, 1, false>")
-    assert _plan_text(library, 100_000, 16, True, True).startswith("pairs_kernel<double, 1, true>")
+    assert _plan_text(library, 100_000, 17, True, True).startswith("pairs_kernel<double, 1, true>")
     assert _plan_text(library, 50_000, 20, True, True, mode=2).startswith("pairs_kernel<double, 2, true>")
     assert _plan_text(library, 100_000, 16, True, False, mode=2).startswith("recursion_kernel")  # cfg4
     assert _plan_text(library, 100_000, 19, False, True).startswith("recursion_kernel")
-    assert _plan_text(library, 100_000, 15, True, True).startswith("recursion_kernel")
+    assert _plan_text(library, 100_000, 16, True, True).startswith("recursion_kernel")
+    assert _plan_text(library, 50_000, 22, True, True, mode=2).startswith("recursion_kernel")
     assert _plan_text(library, 20_000, 32, False, True).startswith("recursion_kernel")  # few points
     assert _plan_text(library, 200_000, 32, False, True, mode=0).startswith("pairs_kernel<float, 0, true>")
     assert _plan_text(library, 200_000, 20, True, False, mode=0).startswith("pairs_kernel<double, 0, false>")
     assert _plan_text(library, 200_000, 22, False, True, mode=0).startswith("values_kernel")
-    assert _plan_text(library, 200_000, 19, True, True, mode=0).startswith("values_kernel")
+    assert _plan_text(library, 200_000, 18, True, True, mode=0).startswith("values_kernel")
+    assert _plan_text(library, 200_000, 23, False, True, mode=0).startswith("values_kernel")
     assert _plan_text(library, 20_000, 32, False, True, mode=0).startswith("values_kernel")  # few points
     # second derivatives in float32 stay where they were
     assert not _plan_text(library, 200_000, 24, False, True, mode=2).startswith("pairs")

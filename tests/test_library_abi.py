@@ -98,7 +98,7 @@ def test_launch_plans(library):
     assert library.sphx_describe_plan(100_000, 16, 2, 1, 1, text, 512) == 0
     assert "512 threads" in text.value.decode()
     # values: as many points per workgroup as fit in half a CU's LDS, in steps of four; in float32
-    # one workgroup with all of LDS while 40 points fit; from l_max = 23 (float64: 20) pairs_kernel with as
+    # one workgroup with all of LDS while 40 points fit; from l_max = 24 (float64: 19) pairs_kernel with as
     # many points per tile as fit (and the lanes kernel again where there are few points)
     status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 16, 0, False)
     assert status == 0 and (tile, threads) == (60, 512) and lds == 60 * (289 + 51) * 4
