@@ -3,7 +3,9 @@
 ``hipcc`` compiles the kernels for gfx950 and the host-side C and C++ API, one
 translation unit per process, and links them into
 ``sphericart_amd/libsphericart_amd.so``. hipcc cross-compiles, so this works on a
-machine without a GPU.
+machine without a GPU. Where torch is importable, ``g++`` then compiles the
+torch operators' C++ side (``csrc/sphx_torch.cpp``, host code only) against its
+headers into ``sphericart_amd/libsphericart_amd_torch.so``.
 """
 
 import os
@@ -43,6 +45,9 @@ FLAGS = [
 ]
 
 
+TORCH_SOURCE = os.path.join(CSRC, "sphx_torch.cpp")
+TORCH_LIBRARY = os.path.join(HERE, "libsphericart_amd_torch.so")
+
 EXAMPLE_SOURCE = os.path.join(os.path.dirname(HERE), "examples", "device_example.cpp")
 EXAMPLE = os.path.join(HERE, "device_example")
 
@@ -78,7 +83,39 @@ def build(verbose=False, extra_flags=(), jobs=None):
     if done.returncode != 0:
         raise RuntimeError(f"hipcc failed to link ({done.returncode}):\n{done.stdout}\n{done.stderr}")
     build_example(verbose)
+    build_torch_operators(verbose)
     return LIBRARY
+
+
+def build_torch_operators(verbose=False):
+    """``libsphericart_amd_torch.so``: schemas and device implementations of the torch operators, against the
+    headers of the torch that is installed. Returns None (and builds nothing) where torch is not importable: the
+    operators are then implemented in Python (sphericart_amd/torch/ops.py)."""
+    # (run as a script from its own directory, the package's `torch` subpackage would shadow torch itself)
+    shadowed = [path for path in sys.path if os.path.abspath(path or ".") == HERE]
+    for path in shadowed:
+        sys.path.remove(path)
+    try:
+        import torch
+        from torch.utils import cpp_extension
+    except ImportError:
+        if verbose:
+            print("torch is not importable: libsphericart_amd_torch.so not built", flush=True)
+        return None
+    libraries = os.path.join(os.path.dirname(torch.__file__), "lib")
+    command = [
+        shutil.which("g++") or "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+        "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+        *["-I" + path for path in cpp_extension.include_paths()], "-I/opt/rocm/include",
+        TORCH_SOURCE, "-L" + HERE, "-lsphericart_amd", "-L" + libraries,
+        "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip", "-Wl,-rpath,$ORIGIN", "-o", TORCH_LIBRARY,
+    ]
+    if verbose:
+        print(" ".join(command), flush=True)
+    done = subprocess.run(command, capture_output=True, text=True)
+    if done.returncode != 0:
+        raise RuntimeError(f"g++ failed on sphx_torch.cpp ({done.returncode}):\n{done.stdout}\n{done.stderr}")
+    return TORCH_LIBRARY
 
 
 def build_example(verbose=False):

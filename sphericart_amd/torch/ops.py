@@ -23,22 +23,43 @@ double backward works as it does in the reference.
 """
 
 import ctypes
+import os
 
 import torch
 
-from .._c_lib import get_library
+from .._c_lib import LIBRARY_PATH, get_library
 
 NAMESPACE = "sphericart_amd"
 _MODES = {"": 0, "_with_gradients": 1, "_with_hessians": 2}
 
-_lib = torch.library.Library(NAMESPACE, "DEF")
-for _prefix in ("spherical_harmonics", "solid_harmonics"):
-    _lib.define(f"{_prefix}(Tensor xyz, int l_max) -> Tensor")
-    _lib.define(f"{_prefix}_with_gradients(Tensor xyz, int l_max) -> (Tensor, Tensor)")
-    _lib.define(f"{_prefix}_with_hessians(Tensor xyz, int l_max) -> (Tensor, Tensor, Tensor)")
-    _lib.define(f"{_prefix}_vjp(Tensor xyz, Tensor sph_grad, int l_max) -> Tensor")
-_lib.define("contract_gradients(Tensor dsph, Tensor sph_grad) -> Tensor")
-_lib.define("contract_hessians(Tensor ddsph, Tensor dsph_grad) -> Tensor")
+# The schemas and the device implementations live in C++ (csrc/sphx_torch.cpp ->
+# libsphericart_amd_torch.so, built next to the HIP library) where that library has been built: a call
+# then costs the host the dispatcher, its outputs and one C call. Without it, or with
+# SPHERICART_AMD_PYTHON_OPERATORS=1, the same operators are defined here and implemented over ctypes;
+# either way the work is done by the same entry points of libsphericart_amd.so.
+TORCH_LIBRARY_PATH = os.path.join(os.path.dirname(LIBRARY_PATH), "libsphericart_amd_torch.so")
+
+
+def _load_cpp_operators():
+    if os.environ.get("SPHERICART_AMD_PYTHON_OPERATORS", "0") not in ("", "0"):
+        return False
+    if not os.path.exists(TORCH_LIBRARY_PATH):
+        return False
+    get_library()  # fails loudly when the HIP library itself is missing
+    torch.ops.load_library(TORCH_LIBRARY_PATH)
+    return True
+
+
+cpp_operators = _load_cpp_operators()
+_lib = torch.library.Library(NAMESPACE, "FRAGMENT" if cpp_operators else "DEF")
+if not cpp_operators:
+    for _prefix in ("spherical_harmonics", "solid_harmonics"):
+        _lib.define(f"{_prefix}(Tensor xyz, int l_max) -> Tensor")
+        _lib.define(f"{_prefix}_with_gradients(Tensor xyz, int l_max) -> (Tensor, Tensor)")
+        _lib.define(f"{_prefix}_with_hessians(Tensor xyz, int l_max) -> (Tensor, Tensor, Tensor)")
+        _lib.define(f"{_prefix}_vjp(Tensor xyz, Tensor sph_grad, int l_max) -> Tensor")
+    _lib.define("contract_gradients(Tensor dsph, Tensor sph_grad) -> Tensor")
+    _lib.define("contract_hessians(Tensor ddsph, Tensor dsph_grad) -> Tensor")
 
 
 def _suffix(tensor):
@@ -150,12 +171,13 @@ def _register_forward(prefix, normalized):
         _lib.impl(name, _no_cpu, "CPU")
 
 
-_register_forward("spherical_harmonics", True)
-_register_forward("solid_harmonics", False)
-_lib.impl("contract_gradients", lambda d, g: _contract("sphx_backward", d, g), "CUDA")
-_lib.impl("contract_hessians", lambda d, g: _contract("sphx_backward_second", d, g), "CUDA")
-_lib.impl("contract_gradients", _no_cpu, "CPU")
-_lib.impl("contract_hessians", _no_cpu, "CPU")
+if not cpp_operators:
+    _register_forward("spherical_harmonics", True)
+    _register_forward("solid_harmonics", False)
+    _lib.impl("contract_gradients", lambda d, g: _contract("sphx_backward", d, g), "CUDA")
+    _lib.impl("contract_hessians", lambda d, g: _contract("sphx_backward_second", d, g), "CUDA")
+    _lib.impl("contract_gradients", _no_cpu, "CPU")
+    _lib.impl("contract_hessians", _no_cpu, "CPU")
 
 _ops = getattr(torch.ops, NAMESPACE)
 
@@ -360,6 +382,10 @@ reference_namespace_defined = False
 
 def _define_reference_namespace():
     global _reference_lib, reference_namespace_defined
+    if cpp_operators:
+        # libsphericart_amd_torch.so defined it when it was loaded, unless the namespace was taken
+        reference_namespace_defined = bool(_ops.owns_reference_namespace())
+        return
     try:
         _reference_lib = torch.library.Library(REFERENCE_NAMESPACE, "DEF")
     except RuntimeError:
