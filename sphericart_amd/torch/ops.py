@@ -5,7 +5,9 @@ The reference registers six operators in the ``sphericart_torch`` namespace
 and vmap rules from Python (sphericart-torch/python/sphericart/torch/register.py:60-185).
 The same six live here in the ``sphericart_amd`` namespace with the same
 schemas; their device implementation calls ``sphx_forward_*`` on the tensor's
-current stream. Only the GPU key has an implementation: CPU tensors raise.
+current stream, from C++ where ``libsphericart_amd_torch.so`` has been built
+(csrc/sphx_torch.cpp), otherwise from the functions below over ctypes. Only the
+GPU key has an implementation: CPU tensors raise.
 Unless the reference's own extension already owns it, the ``sphericart_torch``
 namespace is defined as well, with the reference's eight schemas (the six
 operators and the two ``*_omp_num_threads``), each forwarding to its

@@ -1,7 +1,9 @@
 """The planner's choices, guarded by what they achieve: the 1.2 GB column of the table of achieved bandwidth
 (``python bench.py --sweep``, kept as ``profiles/sweep.json``) is measured again, and a shape that has fallen
 more than a tenth below the fraction of the HBM peak recorded there fails. A slow shape is measured a second
-time before it counts (another process's burst on the box, clocks that have not come up yet).
+and a third time, with fresh buffers, before it counts (another process's burst on the box, clocks that have
+not come up yet, and the float64 kernels' two states a tenth apart, which the recorded table, the slower of
+two runs per row, has seen only by chance).
 
 Collected next to last, so that a timing that fails hides no parity test.
 """
@@ -29,7 +31,9 @@ def test_no_shape_has_fallen_a_tenth_below_the_recorded_table(library):
             continue
         announce("sweep guard", key)
         row = sweep.measure_row(library, *shape, launches=20, series=3)
-        if row["frac"] < 0.9 * want["frac"]:
+        for _ in range(2):
+            if row["frac"] >= 0.9 * want["frac"]:
+                break
             row = sweep.measure_row(library, *shape, launches=40, series=4)
         measured += 1
         if row["frac"] < 0.9 * want["frac"]:
