@@ -597,10 +597,12 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         } else if (mode == 2) {
             g.sequence_waves = l_max <= 4 || l_max >= 22 ? 3u : 2u;
         } else {
-            g.sequence_waves = 3;
+            // values alone (l_max from 34 on, where no other kernel holds the rows): the recursions are a third
+            // of the work and the flush is short: float32 l_max = 40 344 us with three, 310 with four, 281 with eight
+            g.sequence_waves = elem == 4 ? 8 : 4;
         }
     } else if (mode == 0) {
-        g.sequence_waves = 1; // values alone: the recursions are a third of the work
+        g.sequence_waves = 1;
     }
     {
         // (at least four waves flush)
