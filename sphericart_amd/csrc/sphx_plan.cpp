@@ -25,7 +25,7 @@ static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_HESSIAN_LANES",
     "SPHX_HESSIAN_LANES_PARTS", "SPHX_JOB_LIST",
     "SPHX_PAIRS", "SPHX_PAIRS_BATCH", "SPHX_PAIRS_CHUNK", "SPHX_PAIRS_PREP_WAVES", "SPHX_PAIRS_SEQUENCE_WAVES", "SPHX_PAIRS_TILE",
-    "SPHX_PREFIX_INSIDE", "SPHX_RECURSIONS_TOGETHER", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
+    "SPHX_PREFIX_INSIDE", "SPHX_RECURSIONS_TOGETHER", "SPHX_ROW_PAD", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_ALONE", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
     "SPHX_VALUES_PACK", "SPHX_VALUES_TILE_STEP", "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE", "SPHX_VJP_STEP_FLOOR", "SPHX_VJP_TILE_STEP",
@@ -445,7 +445,13 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // and twice)
     // staged rows are `row_stride` apart (recursion_kernel): nrow, or a little more when the rows
     // are cut so that they keep their position within 16 bytes
-    const unsigned row_stride = nrow + (whole ? 0u : nyh % (16u / osize));
+    // (whole rows a multiple of 64 bytes long, l_max = 3 mod 4, would all start on one LDS bank: 16 bytes are left
+    // free after each, which the flush skips; recursion_kernel, row_pad. Not below l_max = 7, where a tile can be
+    // shorter than the line its end is carried in.)
+    const unsigned row_pad = whole && l_max >= 7 && (ny * osize) % 64u == 0 && switch_or(SW_ROW_PAD, 1) != 0 ? 16u / osize : 0u;
+    const unsigned row_stride = nrow + (whole ? row_pad : nyh % (16u / osize));
+    g.row_pad = row_pad;
+    g.magic_ny = magic_of(ny);
     const unsigned rows_per_point = components_of(mode) * row_stride;
     // (the records of a point and its sequences of iterates are an odd number of words apart)
     const unsigned rest_per_point = (together ? 3u : 2u) * ((8 + 3 * (l_max + 1)) | 1u) + (together ? 2u : 1u) * arrays * (tri_all | 1u);

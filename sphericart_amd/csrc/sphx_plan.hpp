@@ -23,7 +23,7 @@ enum Switch : int {
     SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_GRADIENT_LANES, SW_GRADIENT_LANES_PARTS,
     SW_GRADIENT_LANES_TILE, SW_GRADIENT_LANES_WAVES, SW_GROUP_THREADS, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST,
     SW_PAIRS, SW_PAIRS_BATCH, SW_PAIRS_CHUNK, SW_PAIRS_PREP_WAVES, SW_PAIRS_SEQUENCE_WAVES, SW_PAIRS_TILE,
-    SW_PREFIX_INSIDE, SW_RECURSIONS_TOGETHER,
+    SW_PREFIX_INSIDE, SW_RECURSIONS_TOGETHER, SW_ROW_PAD,
     SW_SEQUENCE_WAVES, SW_SLICE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
     SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_ALONE, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
     SW_VALUES_PACK, SW_VALUES_TILE_STEP, SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_VJP_STEP_FLOOR, SW_VJP_TILE_STEP, SW_COUNT

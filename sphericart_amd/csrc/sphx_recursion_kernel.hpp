@@ -103,7 +103,18 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
     // address modulo 16 bytes, puts every staged row at the same position within 16 bytes as
     // its destination, so that the copy is 16-byte loads and stores on both sides.
     constexpr unsigned W16 = 16u / static_cast<unsigned>(sizeof(O));
-    const unsigned row_stride = nrow + skip % W16;
+    // WHOLE, rows a multiple of 64 bytes long (l_max = 3 mod 4): every row would start on the same LDS bank, and
+    // whatever takes one point per lane (the closed forms above all) would store all its lanes' numbers to one
+    // bank, one after the other (float32 gradients l_max = 11: 59 % of the HBM peak against 66 % at l_max = 10
+    // and 12). The host then asks for 16 bytes between the staged rows, g.row_pad elements; the flush skips them
+    // (flush_run). They keep a row's 16-byte vectors whole only where the arrays start at multiples of 16 bytes:
+    // for other pointers the rows stay back to back.
+    const unsigned row_pad =
+        WHOLE && !VJP && ((reinterpret_cast<uintptr_t>(sph) | reinterpret_cast<uintptr_t>(dsph) |
+                           reinterpret_cast<uintptr_t>(ddsph)) & 15u) == 0
+            ? g.row_pad
+            : 0u;
+    const unsigned row_stride = WHOLE ? nrow + row_pad : nrow + skip % W16;
     const unsigned tri_all = (L + 1) * (L + 2) / 2;
 
     T* F = lds + g.off_F;
@@ -366,10 +377,10 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
                 p.z2 = rec[5];
                 p.ir = rec[6];
                 Rows<O> rows;
-                rows.ny = static_cast<int>(ny);
-                rows.sph = staged + ph.sph + lane * ny;
-                rows.dsph = staged + g.off_dsph + ph.dsph + lane * 3 * ny;
-                rows.ddsph = staged + g.off_ddsph + ph.ddsph + lane * 9 * ny;
+                rows.ny = static_cast<int>(row_stride);
+                rows.sph = staged + ph.sph + lane * row_stride;
+                rows.dsph = staged + g.off_dsph + ph.dsph + lane * 3 * row_stride;
+                rows.ddsph = staged + g.off_ddsph + ph.ddsph + lane * 9 * row_stride;
                 if constexpr (H == 6) {
                     // (Rows a multiple of 32 words long, l_max = 7, 15, 23, ...: the stores of all
                     // lanes fall on one LDS bank. Storing in rotated fours, two selects per number,
@@ -545,14 +556,19 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
                 const unsigned hi = phase + len;
                 const unsigned full_lo = (lo + LINE - 1u) / LINE * LINE;
                 const unsigned full_hi = hi / LINE * LINE;
+                // where element e of the region (counted as it lies in HBM) is staged: past the carried part of
+                // the first line, row_pad elements further for every row before it (exact: e * ny < 2^32)
+                auto staged_at = [&](unsigned e) -> unsigned {
+                    return row_pad == 0 || e < phase ? e : e + row_pad * __umulhi(e - phase, g.magic_ny);
+                };
                 unsigned tail_from; // what follows the head and the whole lines
                 if (full_hi > full_lo) {
                     const unsigned nvec = (full_hi - full_lo) / W;
-                    const V* in = reinterpret_cast<const V*>(region + full_lo);
                     V* out = reinterpret_cast<V*>(line0 + full_lo);
                     // (two or four loads in flight per lane ahead of their stores: no faster on any shape)
                     for (unsigned v = ft; v < nvec; v += count) {
-                        emit<O, SPHX_STREAMING_STORES>(in[v], out + v);
+                        emit<O, SPHX_STREAMING_STORES>(*reinterpret_cast<const V*>(region + staged_at(full_lo + v * W)),
+                                                       out + v);
                     }
                     tail_from = full_hi;
                 } else {
@@ -560,14 +576,14 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
                 }
                 // head: the part of the first line that belongs to this chunk
                 const unsigned head_end = full_lo < hi ? full_lo : hi;
-                if (lo + ft < head_end) line0[lo + ft] = region[lo + ft];
+                if (lo + ft < head_end) line0[lo + ft] = region[staged_at(lo + ft)];
                 // tail: stored if the chunk ends here, else handed to the next tile
                 const unsigned tail = hi - tail_from;
                 if (ft < tail) {
-                    const O value = region[tail_from + ft];
+                    const O value = region[staged_at(tail_from + ft)];
                     if (ends) {
                         line0[tail_from + ft] = value;
-                    } else if (carry_to + region_offset != region || tail_from != 0) {
+                    } else if (carry_to + region_offset != region || staged_at(tail_from + ft) != ft) {
                         carry_to[region_offset + ft] = value;
                     }
                 }

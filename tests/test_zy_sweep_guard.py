@@ -1,9 +1,13 @@
 """The planner's choices, guarded by what they achieve: the 1.2 GB column of the table of achieved bandwidth
-(``python bench.py --sweep``, kept as ``profiles/sweep.json``) is measured again, and a shape that has fallen
-more than a tenth below the fraction of the HBM peak recorded there fails. A slow shape is measured a second
-and a third time, with fresh buffers, before it counts (another process's burst on the box, clocks that have
-not come up yet, and the float64 kernels' two states a tenth apart, which the recorded table, the slower of
-two runs per row, has seen only by chance).
+(``python bench.py --sweep``, kept as ``profiles/sweep.json``) is measured again and compared row by row with the
+fraction of the HBM peak recorded there.
+
+Boxes differ by some 5 % as a whole, and the float64 kernels run in one of two states a tenth apart from
+process to process with the same code, so a row is not judged against the recorded number alone: the test
+fails when the rows as a whole have fallen a tenth (the median of measured / recorded below 0.9), or when a
+single row has fallen more than 15 % below what that median makes of its recorded value. A slow row is measured
+up to three times, with fresh buffers, before it counts (another process's burst on the box, clocks that have
+not come up yet).
 
 Collected next to last, so that a timing that fails hides no parity test.
 """
@@ -22,24 +26,32 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def test_no_shape_has_fallen_a_tenth_below_the_recorded_table(library):
     recorded = {sweep.key_of(row): row for row in sweep.load(os.path.join(ROOT, "profiles", "sweep.json"))}
-    fallen = []
-    measured = 0
+    shapes = {}
     for shape in sweep.shapes(sizes=("1.2GB",)):
         key = sweep.key_of(dict(zip(("derivatives", "dtype", "harmonics", "l_max", "size"), shape[:5])))
-        want = recorded.get(key)
-        if want is None:
-            continue
+        if key in recorded:
+            shapes[key] = shape
+    assert len(shapes) >= 150, "profiles/sweep.json holds too few rows of the 1.2 GB column"
+    rows = {}
+    for key, shape in shapes.items():
         announce("sweep guard", key)
-        row = sweep.measure_row(library, *shape, launches=20, series=3)
+        rows[key] = sweep.measure_row(library, *shape, launches=20, series=3)
+    ratio = lambda key: rows[key]["frac"] / recorded[key]["frac"]
+    median = sorted(ratio(key) for key in rows)[len(rows) // 2]
+    print(f"median of measured / recorded over {len(rows)} rows: {median:.3f}")
+    floor = 0.85 * min(median, 1.0)
+    for key in [key for key in rows if ratio(key) < floor]:
         for _ in range(2):
-            if row["frac"] >= 0.9 * want["frac"]:
+            if ratio(key) >= floor:
                 break
-            row = sweep.measure_row(library, *shape, launches=40, series=4)
-        measured += 1
-        if row["frac"] < 0.9 * want["frac"]:
-            fallen.append((key, row["kernel"], row["frac"], "recorded", want["kernel"], want["frac"]))
-    assert measured >= 150, "profiles/sweep.json holds too few rows of the 1.2 GB column"
-    assert not fallen, fallen
+            announce("sweep guard, again", key)
+            rows[key] = sweep.measure_row(library, *shapes[key], launches=40, series=4)
+    fallen = [(key, rows[key]["kernel"], rows[key]["frac"], "recorded", recorded[key]["kernel"], recorded[key]["frac"])
+              for key in rows if ratio(key) < floor]
+    worst = sorted(rows, key=ratio)[:8]
+    print("lowest:", [(key, round(ratio(key), 3)) for key in worst])
+    assert median >= 0.9, f"the rows as a whole run at {median:.3f} of the recorded table"
+    assert not fallen, (f"median {median:.3f}", fallen)
 
 
 def test_recorded_table_meets_the_bars_it_was_made_for():
