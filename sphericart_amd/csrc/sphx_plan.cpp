@@ -833,10 +833,10 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
     // kernel's job list by kind fills sixteen waves better. SPHX_PAIRS: 0 never, 2 wherever it fits.
     {
         const int pairs = switch_or(SW_PAIRS, 1);
+        // (second derivatives: thirteen rows per point, 8 192 points are as many tiles as 32 768 with gradients)
         const bool pairs_by_shape =
-            n_samples >= 32768 &&
-            (mode == 1 ? (elem == 4 ? l_max >= 20 : l_max >= 17)
-                       : elem == 8 && (l_max == 20 || (!normalized && l_max >= 24)));
+            mode == 1 ? n_samples >= 32768 && (elem == 4 ? l_max >= 20 : l_max >= 17)
+                      : n_samples >= 8192 && elem == 8 && (l_max == 20 || (!normalized && l_max >= 24));
         if (lane_kernels && mode >= 1 && l_max > hard && (pairs == 2 || (pairs == 1 && pairs_by_shape))) {
             PairsChoice want;
             want.tile = static_cast<unsigned>(switch_or(SW_PAIRS_TILE, 0));
