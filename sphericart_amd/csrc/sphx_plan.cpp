@@ -295,13 +295,14 @@ static bool plan_gradient_lanes(size_t n_samples, int l_max, size_t elem, int ld
     g.off_iter = table_stride;
     out->workgroups = g.tiles_per_xcd * 8u;
     // Eight waves share the closed-form slices and the channels; with one or two channels four are enough and
-    // leave room for more workgroups. Closed forms only (l_max <= 6): eight, six for normalised float32 at
-    // l_max = 6. Few points (one workgroup per CU, occupancy is no concern): eight waves shorten the longest chain
+    // leave room for more workgroups. Closed forms only (l_max <= 6): eight, a slice each. (Six, two of them with
+    // two slices, were 1-2 % ahead for normalised float32 at l_max = 6 on boxes whose clocks settle high, 122 us on
+    // cfg3 either way, and are 140 us against 122 us on boxes whose clocks settle low: the wave with two slices is
+    // then what a workgroup waits for.) Few points (one workgroup per CU, occupancy is no concern): eight waves shorten the longest chain
     // of work in the workgroup, and with three channels or more, or float64 tiles of up to 16 points, sixteen do,
     // two to a channel where that leaves four for the closed forms.
     const bool many = tile == few && l_max > 6 && (l_max >= 9 || (elem == 8 && tile <= 16));
-    const int by_shape = l_max <= 6 ? (l_max == 6 && elem == 4 && normalized && tile != few ? 6 : 8)
-                                    : (l_max <= 8 && tile != few ? 4 : (many ? 16 : 8));
+    const int by_shape = l_max <= 6 ? 8 : (l_max <= 8 && tile != few ? 4 : (many ? 16 : 8));
     int waves = switch_or(SW_GRADIENT_LANES_WAVES, by_shape);
     const int most = l_max >= 6 ? 16 : 8; // (the kernels of l_max = 4, 5 exist for 512 threads)
     waves = waves < 1 ? 1 : (waves > most ? most : waves);

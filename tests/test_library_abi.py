@@ -69,9 +69,9 @@ def _plan(library, n, l_max, mode, f64):
 
 
 def test_launch_plans(library):
-    # gradients at l_max = 6: the closed forms in slices for six waves, 32 points per workgroup
+    # gradients at l_max = 6: the closed forms in slices for eight waves, 32 points per workgroup
     status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 6, 1, False)
-    assert status == 0 and tile == 32 and threads == 384
+    assert status == 0 and tile == 32 and threads == 512
     assert lds == 32 * 4 * 49 * 4 and groups == 31256  # 8 XCD stretches of 3907 tiles
     # values at l_max = 6: one wave per 64 points
     status, (tile, threads, lds, groups) = _plan(library, 1_000_000, 6, 0, False)
