@@ -45,12 +45,12 @@ namespace sphx {
 // waves after them compute the entries, and every wave flushes. In float64 the
 // recursions are long enough to hold up a flush that they share, and for solid
 // harmonics, whose entries are short, and at high l_max this division is the
-// faster one by 5-14 %; the host says which one a launch takes.
+// faster one by 5-14 %; the host says which one a launch takes (g.together).
 //
 // NT = 512: two workgroups share a CU, half of its LDS each. NT = 1024: one
 // workgroup has the CU and all of its LDS, its tiles are more than twice as
 // large, and with g.slice_waves the closed forms of l <= H have waves of their
-// own (the last ones) next to wave 0.
+// own (the last ones; TOGETHER: next to wave 0).
 //
 // SPLIT == true (second derivatives, so few points per tile that the (l, m)
 // pairs of a tile leave lanes idle): the entries (l, +m) and (l, -m) are two
