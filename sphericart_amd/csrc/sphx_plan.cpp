@@ -23,7 +23,7 @@ static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_AZ_SHIFT", "SPHX_CHUNK_SHIFT", "SPHX_GRADIENT_LANES",
     "SPHX_GRADIENT_LANES_PARTS", "SPHX_GRADIENT_LANES_TILE", "SPHX_GRADIENT_LANES_WAVES", "SPHX_GROUP_THREADS",
     "SPHX_HESSIAN_LANES",
-    "SPHX_HESSIAN_LANES_PARTS", "SPHX_JOB_LIST",
+    "SPHX_HESSIAN_LANES_PARTS", "SPHX_HESSIAN_LANES_TILE", "SPHX_JOB_LIST",
     "SPHX_PAIRS", "SPHX_PAIRS_BATCH", "SPHX_PAIRS_CHUNK", "SPHX_PAIRS_PREP_WAVES", "SPHX_PAIRS_SEQUENCE_WAVES", "SPHX_PAIRS_TILE",
     "SPHX_PREFIX_INSIDE", "SPHX_RECURSIONS_TOGETHER", "SPHX_ROW_PAD", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
@@ -334,8 +334,8 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
     const unsigned most = (elem == 4 ? hessian_lane_threads<float>() : hessian_lane_threads<double>()) / 64u;
     // Waves per channel, each with a part of its m: two where one or two channels would leave the workgroup with
     // one or two waves and that measured faster (l_max = 3 in float32 and for solid harmonics in float64, l_max = 2
-    // for normalised float32: 10-20 %).
-    const bool shared = (l_max == 3 && (elem == 4 || !normalized)) || (l_max == 2 && elem == 4 && normalized);
+    // in float32: 5-20 %).
+    const bool shared = (l_max == 3 && (elem == 4 || !normalized)) || (l_max == 2 && elem == 4);
     unsigned parts = static_cast<unsigned>(switch_or(SW_HESSIAN_LANES_PARTS, shared ? 2 : 1));
     if (parts != 1 && parts != 2 && parts != 4) parts = 1;
     while (parts > 1 && parts > most) parts /= 2;
@@ -343,6 +343,7 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
     const unsigned waves = slots * parts;
     const unsigned limit = static_cast<unsigned>(lds_limit);
     unsigned tile = 0, off_d = 0, off_dd = 0, off_t = 0, off_s = 0, bytes = 0, best = 0, best_groups = 0;
+    const unsigned forced_tile = static_cast<unsigned>(switch_or(SW_HESSIAN_LANES_TILE, 0));
     for (unsigned t = 64; t >= 32; t /= 2) {
         const unsigned od = (t * s_stride + vec - 1u) / vec * vec;
         const unsigned odd = od + (t * d_stride + vec - 1u) / vec * vec;
@@ -350,7 +351,7 @@ static bool plan_hessian_lanes(size_t n_samples, int l_max, size_t elem, int lds
         const unsigned os = ot + t * table_stride;
         const unsigned b = (os + waves * t * table_stride) * esize;
         if (b > limit) continue;
-        const unsigned score = (limit / b) * t;
+        const unsigned score = forced_tile == t ? 1u << 30 : (limit / b) * t;
         if (score > best || (score == best && best_groups < 2)) {
             best = score;
             best_groups = limit / b;

@@ -21,7 +21,7 @@ int fail(int code, const std::string& what);
 // only if SPHX_DEBUG_SWITCHES is set to something other than 0.
 enum Switch : int {
     SW_AZ_SHIFT, SW_CHUNK_SHIFT, SW_GRADIENT_LANES, SW_GRADIENT_LANES_PARTS,
-    SW_GRADIENT_LANES_TILE, SW_GRADIENT_LANES_WAVES, SW_GROUP_THREADS, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_JOB_LIST,
+    SW_GRADIENT_LANES_TILE, SW_GRADIENT_LANES_WAVES, SW_GROUP_THREADS, SW_HESSIAN_LANES, SW_HESSIAN_LANES_PARTS, SW_HESSIAN_LANES_TILE, SW_JOB_LIST,
     SW_PAIRS, SW_PAIRS_BATCH, SW_PAIRS_CHUNK, SW_PAIRS_PREP_WAVES, SW_PAIRS_SEQUENCE_WAVES, SW_PAIRS_TILE,
     SW_PREFIX_INSIDE, SW_RECURSIONS_TOGETHER, SW_ROW_PAD,
     SW_SEQUENCE_WAVES, SW_SLICE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
