@@ -32,6 +32,7 @@ struct Tiling {
     unsigned together;      // recursion_kernel, float64: 1 = the recursions run next to the entries (TOGETHER)
     unsigned row_pad;       // recursion_kernel, whole rows: elements left free after every staged row (0 or 16 bytes' worth)
     unsigned magic_ny;      // ceil(2^32 / ny)
+    unsigned priorities;    // recursion_kernel: 1 = the waves that flush run at raised priority, 2 = those that prepare the next tile
     // LDS carve-up, in elements of T: the staged rows come first, rows_elems of them, with the
     // gradient and second-derivative rows at off_dsph and off_ddsph inside a buffer; the other
     // offsets count from the start of dynamic LDS. (recursion_kernel: the row offsets are in

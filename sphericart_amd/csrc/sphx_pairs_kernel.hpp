@@ -392,6 +392,7 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
             SPHX_MARK(c_work);
             __syncthreads(); // rows of tile n complete
             SPHX_MARK(c_wait_b);
+            if (g.priorities & 2u) __builtin_amdgcn_s_setprio(2);
             const unsigned item = step * P + wave;
             if (item < ITEMS) prep_item(batch + ahead, item);
             if (++step == tpb) {
@@ -399,6 +400,7 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
                 ++batch;
                 fetch(batch + ahead);
             }
+            __builtin_amdgcn_s_setprio(0);
             SPHX_MARK(c_flush);
         }
     } else if (wave < entry_first) {
@@ -512,7 +514,9 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
             SPHX_MARK(c_wait_a);
             __syncthreads(); // rows of tile n complete, its iterates no longer needed
             SPHX_MARK(c_wait_b);
+            if (g.priorities & 2u) __builtin_amdgcn_s_setprio(2);
             sequence_stage(n + 1);
+            __builtin_amdgcn_s_setprio(0);
             SPHX_MARK(c_flush);
         }
     } else {
@@ -772,7 +776,9 @@ __global__ __launch_bounds__(NT, 1) void pairs_kernel(PairsTiling g, const T* __
             SPHX_MARK(c_work);
             __syncthreads();
             SPHX_MARK(c_wait_b);
+            if (g.priorities & 1u) __builtin_amdgcn_s_setprio(2);
             flush_stage(n);
+            __builtin_amdgcn_s_setprio(0);
             SPHX_MARK(c_flush);
 #ifdef SPHX_PAIRS_CLOCKS
             ++c_tiles;

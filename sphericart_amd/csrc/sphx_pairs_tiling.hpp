@@ -32,6 +32,7 @@ struct PairsTiling {
     unsigned point_stride, park_stride, iter_stride;
     unsigned tmz_at;         // where 2(m+1)z starts in a point's record (a multiple of four numbers)
     unsigned q_stride;       // distance between the rows of the Q constants in LDS (a multiple of four)
+    unsigned priorities;     // 1 = the waves that flush run at raised priority, 2 = those that prepare the next tiles
     // the pair of every entry lane, slot << 14 | l << 7 | m (MODE 1: of the slot_waves waves that share a
     // point, slot 0)
     unsigned short lane_job[kPairsThreads];

@@ -28,7 +28,7 @@ static const char* const kSwitchNames[SW_COUNT] = {
     "SPHX_PREFIX_INSIDE", "SPHX_RECURSIONS_TOGETHER", "SPHX_ROW_PAD", "SPHX_SEQUENCE_WAVES", "SPHX_SLICE_WAVES", "SPHX_SPLIT_BELOW",
     "SPHX_SPLIT_RATIO", "SPHX_SPLIT_SIDES", "SPHX_SPREAD_KINDS", "SPHX_TILE", "SPHX_TILE_LDS_BUDGET", "SPHX_TILE_POW2",
     "SPHX_TILE_SMALL_N", "SPHX_VALUES_ALONE", "SPHX_VALUES_LDS", "SPHX_VALUES_MIN_TILE", "SPHX_VALUES_MIN_WAVES",
-    "SPHX_VALUES_PACK", "SPHX_VALUES_TILE_STEP", "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE", "SPHX_VJP_STEP_FLOOR", "SPHX_VJP_TILE_STEP",
+    "SPHX_VALUES_PACK", "SPHX_VALUES_TILE_STEP", "SPHX_VALUES_WAVES", "SPHX_VJP_GROUPS_BELOW", "SPHX_VJP_LANES", "SPHX_VJP_MIN_TILE", "SPHX_VJP_STEP_FLOOR", "SPHX_VJP_TILE_STEP", "SPHX_WAVE_PRIORITIES",
 };
 struct Switches {
     bool set[SW_COUNT] = {};
@@ -758,6 +758,17 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     return true;
 }
 
+// Wave priorities of the persistent kernels (Tiling::priorities): 1 = the flushing waves run at raised priority,
+// by the table of shapes in sphx_plan_shapes.hpp, for launches of `least` tiles or more per workgroup; the kernel's
+// first division of its work (together) has no waves that only flush. SPHX_WAVE_PRIORITIES overrides (2, 3: the waves
+// that prepare the next tile, too).
+static unsigned wave_priorities(int mode, size_t elem, bool normalized, int l_max, unsigned n_tiles,
+                                unsigned workgroups, unsigned least, bool forward) {
+    const bool by_shape = forward && n_tiles / least >= workgroups &&
+                          flush_priority_by_shape(mode, static_cast<int>(elem), normalized, l_max);
+    return static_cast<unsigned>(switch_or(SW_WAVE_PRIORITIES, by_shape ? 1 : 0));
+}
+
 // Choose kernels, tile sizes and LDS layouts. `lds_limit` / `cus` describe the device.
 int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit, int cus, Plan* plan,
               bool lane_kernels, bool normalized) {
@@ -807,6 +818,8 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
             want.sequence_waves = static_cast<unsigned>(switch_or(SW_PAIRS_SEQUENCE_WAVES, 0));
             want.chunk_shift_plus_one = static_cast<unsigned>(switch_or(SW_PAIRS_CHUNK, -1) + 1);
             if (plan_pairs(n_samples, l_max, mode, elem, elem, lds_limit, cus, want, &plan->pairs_launch)) {
+                PairsLaunch& made = plan->pairs_launch;
+                made.g.priorities = wave_priorities(mode, elem, normalized, l_max, made.g.n_tiles, made.workgroups, 32u, true);
                 plan->pairs = true;
                 return SPHX_OK;
             }
@@ -847,6 +860,8 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
             want.sequence_waves = static_cast<unsigned>(switch_or(SW_PAIRS_SEQUENCE_WAVES, 0));
             want.chunk_shift_plus_one = static_cast<unsigned>(switch_or(SW_PAIRS_CHUNK, -1) + 1);
             if (plan_pairs(n_samples, l_max, mode, elem, elem, lds_limit, cus, want, &plan->pairs_launch)) {
+                PairsLaunch& made = plan->pairs_launch;
+                made.g.priorities = wave_priorities(mode, elem, normalized, l_max, made.g.n_tiles, made.workgroups, 32u, true);
                 plan->pairs = true;
                 return SPHX_OK;
             }
@@ -912,6 +927,8 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
                         " with this many derivatives needs more LDS for the rows of one point than "
                         "the device offers (" + std::to_string(lds_limit) + " bytes)");
     }
+    plan->rec.g.priorities = wave_priorities(mode, elem, normalized, l_max, plan->rec.g.n_tiles, plan->rec.workgroups, 4u,
+                                             lane_kernels && plan->whole && plan->rec.g.together == 0);
     return SPHX_OK;
 }
 
@@ -971,7 +988,8 @@ std::string describe(const Plan& plan, int l_max, int mode, bool is_f64, bool no
         const PairsLaunch& l = plan.pairs_launch;
         text = "pairs_kernel<" + head + "> [" + std::to_string(l.g.tile) + " points per tile, " +
                std::to_string(l.threads) + " threads, " + std::to_string(l.lds_bytes) + " B LDS, " +
-               std::to_string(l.workgroups) + " workgroups]";
+               std::to_string(l.workgroups) + " workgroups]" +
+               ((l.g.priorities & 1u) != 0 ? " (flush at raised priority)" : "");
     } else if (plan.closed_only) {
         text = "closed_form_kernel<" + head + ", " + std::to_string(l_max) + ", false>" + geometry(plan.closed);
     } else if (plan.lanes) {
@@ -986,7 +1004,8 @@ std::string describe(const Plan& plan, int l_max, int mode, bool is_f64, bool no
         text += "recursion_kernel<" + head + ", " + (plan.whole ? "true" : "false") + ", " +
                 (plan.split_sides ? "true" : "false") + ", false, " +
                 (plan.rec.g.points_per_pass == 0 ? "true" : "false") + ">" + geometry(plan.rec) +
-                (plan.rec.g.together != 0 ? " (recursions next to the entries)" : "");
+                (plan.rec.g.together != 0 ? " (recursions next to the entries)" : "") +
+                ((plan.rec.g.priorities & 1u) != 0 ? " (flush at raised priority)" : "");
     }
     return text;
 }

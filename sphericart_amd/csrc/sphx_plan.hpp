@@ -26,7 +26,7 @@ enum Switch : int {
     SW_PREFIX_INSIDE, SW_RECURSIONS_TOGETHER, SW_ROW_PAD,
     SW_SEQUENCE_WAVES, SW_SLICE_WAVES, SW_SPLIT_BELOW, SW_SPLIT_RATIO, SW_SPLIT_SIDES, SW_SPREAD_KINDS, SW_TILE, SW_TILE_LDS_BUDGET,
     SW_TILE_POW2, SW_TILE_SMALL_N, SW_VALUES_ALONE, SW_VALUES_LDS, SW_VALUES_MIN_TILE, SW_VALUES_MIN_WAVES,
-    SW_VALUES_PACK, SW_VALUES_TILE_STEP, SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_VJP_STEP_FLOOR, SW_VJP_TILE_STEP, SW_COUNT
+    SW_VALUES_PACK, SW_VALUES_TILE_STEP, SW_VALUES_WAVES, SW_VJP_GROUPS_BELOW, SW_VJP_LANES, SW_VJP_MIN_TILE, SW_VJP_STEP_FLOOR, SW_VJP_TILE_STEP, SW_WAVE_PRIORITIES, SW_COUNT
 };
 
 // The value of an override as the plan being made sees it, `fallback` where none is set.

@@ -702,13 +702,19 @@ __global__ __launch_bounds__(NT, MODE < 2 ? 4 : 1) void recursion_kernel(Tiling 
                 flush_stage(n, tid, NT);
             }
         } else if (wave == 0) {
+            if (g.priorities & 2u) __builtin_amdgcn_s_setprio(2);
             table_stage(n);
+            __builtin_amdgcn_s_setprio(0);
         } else if (wave < apart_waves) {
+            if (g.priorities & 2u) __builtin_amdgcn_s_setprio(2);
             recursion_stage(n + 1);
+            __builtin_amdgcn_s_setprio(0);
         } else if constexpr (VJP) {
             contract_stage(n, wave - apart_waves, NT / 64 - apart_waves);
         } else {
+            if (g.priorities & 1u) __builtin_amdgcn_s_setprio(2);
             flush_stage(n, tid - 64 * apart_waves, NT - 64 * apart_waves);
+            __builtin_amdgcn_s_setprio(0);
         }
     }
     // what is left of this workgroup's share of the batches (no barrier follows)

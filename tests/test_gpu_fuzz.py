@@ -27,6 +27,7 @@ OVERRIDES = (
     ("SPHX_GROUP_THREADS", (1024,)), ("SPHX_SPREAD_KINDS", (0, 1)), ("SPHX_SLICE_WAVES", (0, 1, 2, 3)),
     ("SPHX_VALUES_TILE_STEP", (0, 1, 2, 8)), ("SPHX_VALUES_MIN_TILE", (8, 16, 48)),
     ("SPHX_VALUES_PACK", (1, 2, 4)), ("SPHX_VALUES_ALONE", (0, 1)),
+    ("SPHX_WAVE_PRIORITIES", (1, 2, 3)),
 )
 
 

@@ -209,6 +209,29 @@ def test_job_list_by_kind_and_points_side_by_side(oracle, library, switches, dty
             library.sphx_reset_switches()
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_wave_priorities_change_no_number(oracle, library, switches, dtype):
+    """The waves that flush a tile, or the ones that prepare the next, may run at raised priority in the two
+    persistent kernels (the planner's choice by shape, SPHX_WAVE_PRIORITIES here): every setting against the
+    oracle, on shapes of the recursion kernel and of pairs_kernel, many tiles per workgroup."""
+    rng = np.random.default_rng(29)
+    for mode, l_max, normalized, n, pairs in (("gradients", 12, False, 40000, 0), ("hessians", 10, False, 30000, 0),
+                                              ("gradients", 21, True, 6000, 2), ("hessians", 20, False, 3000, 2)):
+        xyz = special_points(dtype, rng, n)
+        want = oracle.compute(xyz, l_max, normalized, mode)
+        xyz_dev = torch.from_numpy(xyz).cuda()
+        for priorities in (0, 1, 2, 3):
+            switches("SPHX_PAIRS", pairs)
+            switches("SPHX_WAVE_PRIORITIES", priorities)
+            announce("wave priorities", np.dtype(dtype).name, mode, normalized, l_max, n, priorities)
+            status, got = run_launch_layer(library, xyz_dev, l_max, normalized, mode)
+            torch.cuda.synchronize()
+            assert status == 0, library.sphx_last_error()
+            got = tuple(None if g is None else g.cpu().numpy() for g in got)
+            check(got, want, (l_max, normalized, mode, priorities))
+        library.sphx_reset_switches()
+
+
 @pytest.mark.parametrize("name", CONFIGS)
 def test_golden_benchmark_configurations(name):
     xyz, l_max, normalized, mode, want = config_case(name)

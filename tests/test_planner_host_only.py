@@ -30,7 +30,13 @@ SHAPES = [
     (2_000, 40, 1, 1, 1, "recursion_kernel<double, 1, true, false, false, false, false>"),
     (5, 24, 2, 1, 1, "recursion_kernel<double, 2, true, true, false, false, false>"),
     (1, 0, 0, 0, 1, "closed_form_kernel<float, 0, true, 0, false>"),
+    # the flush at raised priority: by the table of shapes, and only with many tiles per workgroup
+    (200_000, 33, 1, 0, 0, "pairs_kernel<float, 1, false>"),
+    (40_000, 33, 1, 0, 0, "pairs_kernel<float, 1, false>"),
+    (300_000, 10, 2, 0, 0, "recursion_kernel<float, 2, false, true, false, false, true>"),
+    (300_000, 9, 2, 0, 0, "recursion_kernel<float, 2, false, true, false, false, true>"),
 ]
+PRIORITY = {(200_000, 33): True, (40_000, 33): False, (300_000, 10): True, (300_000, 9): False}
 
 
 @pytest.fixture(scope="module")
@@ -51,6 +57,7 @@ def test_plans_without_a_device_match_the_library_and_name_the_intended_kernels(
         assert library.sphx_describe_plan(n, l_max, mode, is_f64, normalized, text, len(text)) == 0
         assert line == text.value.decode(), (n, l_max, mode, is_f64, normalized)
         assert line.split(" + ")[-1].startswith(kernel + " ["), (line, kernel)
+        assert line.endswith("(flush at raised priority)") == PRIORITY.get((n, l_max), False), line
 
 
 def test_shapes_beyond_the_tables_or_lds_are_refused_with_a_message(probe):
