@@ -84,11 +84,13 @@ inline const ShapeRow* shape_row(int kind, int elem, int l_max) {
 // recursion_kernel and pairs_kernel: the shapes at which the waves that flush a tile run at raised priority
 // (s_setprio) while other waves prepare the next tile. The flush and the preparation end at the same barrier;
 // whichever of them a tile waits for gains or loses by it, and which one that is changes from one l_max to the
-// next with the tile and the rounds of the sequence lanes. Measured at 1.2 GB of output, interleaved in one process,
-// on two boxes: percent gained on either box (the same sign on both at nearly every l_max; the rows are the
-// shapes that gained 3 % or more on both, elsewhere the priority costs up to 10 %). The gain holds from 50 000 points up
-// in pairs_kernel (2 to 13 % at 50 000, 100 000, 200 000 and 400 000 points) and from 50 000 down to 20 000 in
-// recursion_kernel (1 to 11 %); the planner asks for 32 and 4 tiles per workgroup.
+// next with the tile and the rounds of the sequence lanes. Measured at 1.2 GB of output after 0.4 s of the same
+// launches (settled clocks), the two settings interleaved in one process, on two boxes: percent gained on either
+// box (the same sign on both at nearly every l_max, and the same in short bursts on two other boxes; the rows are
+// the shapes that gained 3 % or more on both, elsewhere the priority costs up to 10 %). The gain holds from
+// 50 000 points up in pairs_kernel (2 to 13 % at 50 000, 100 000, 200 000 and 400 000 points) and from 50 000
+// down to 20 000 in recursion_kernel (1 to 11 %); the planner asks for 32 and 4 tiles per workgroup. Whether the
+// priority is 1, 2 or 3 makes no difference.
 struct PriorityRow {
     int mode, elem;
     bool normalized;
@@ -98,29 +100,29 @@ struct PriorityRow {
 
 constexpr PriorityRow kFlushPriorityRows[] = {
     // gradients, float32
-    {1, 4, true, 8, 8, "+3 / +5"},
-    {1, 4, true, 31, 31, "+5 / +8 (l_max = 32, cfg5: between -3 and +6 from run to run at 50 000 to 800 000 points, left alone)"},
-    {1, 4, true, 34, 35, "+9 / +6, +13 / +14"},
-    {1, 4, false, 11, 12, "+6 / +5, +8 / +7"},
-    {1, 4, false, 14, 14, "+3 / +3"},
-    {1, 4, false, 29, 30, "+9 / +10, +3 / +3"},
-    {1, 4, false, 32, 34, "+5 / +7, +14 / +14, +9 / +9"},
+    {1, 4, true, 31, 31, "+4 / +8 (l_max = 32, cfg5: between -3 and +6 from run to run at 50 000 to 800 000 points, left alone)"},
+    {1, 4, true, 34, 35, "+8 / +8, +14 / +14"},
+    {1, 4, false, 11, 14, "+10 / +8, +7 / +7, +5 / +5, +6 / +5"},
+    {1, 4, false, 16, 16, "+5 / +5"},
+    {1, 4, false, 23, 23, "+5 / +6"},
+    {1, 4, false, 29, 30, "+12 / +10, +4 / +5"},
+    {1, 4, false, 32, 34, "+5 / +4, +14 / +12, +10 / +9"},
     // gradients, float64
-    {1, 8, true, 23, 24, "+6 / +5, +9 / +7"},
-    {1, 8, true, 32, 32, "+9 / +12"},
-    {1, 8, false, 19, 21, "+13 / +12, +3 / +4, +12 / +12"},
-    {1, 8, false, 25, 25, "+6 / +7"},
-    {1, 8, false, 28, 28, "+5 / +3"},
-    {1, 8, false, 30, 31, "+12 / +13, +5 / +5"},
-    // second derivatives, float32, solid (normalised: +1 to +3.5 at l_max = 5-28 on both boxes, -1 to -2 on a third)
-    {2, 4, false, 5, 6, "+10 / +9, +8 / +8"},
-    {2, 4, false, 8, 8, "+9 / +9"},
-    {2, 4, false, 10, 13, "+11 / +14, +8 / +10, +7 / +7, +4 / +3"},
-    {2, 4, false, 27, 28, "+4 / +3, +11 / +11"},
+    {1, 8, true, 23, 24, "+5 / +7, +8 / +5"},
+    {1, 8, true, 31, 32, "+7 / +6, +9 / +10"},
+    {1, 8, false, 19, 21, "+11 / +11, +4 / +4, +13 / +12"},
+    {1, 8, false, 25, 26, "+8 / +8, +3 / +3"},
+    {1, 8, false, 28, 28, "+4 / +3"},
+    {1, 8, false, 30, 31, "+12 / +14, +6 / +4"},
+    // second derivatives, float32, solid (normalised: 0 to +3 at l_max = 5-28 on both boxes, -1 to -2 on a third)
+    {2, 4, false, 5, 6, "+13 / +13, +11 / +12"},
+    {2, 4, false, 8, 8, "+11 / +9"},
+    {2, 4, false, 10, 14, "+14 / +14, +10 / +12, +10 / +8, +4 / +3, +7 / +6"},
+    {2, 4, false, 27, 28, "+6 / +5, +12 / +12"},
     // second derivatives, float64, solid
-    {2, 8, false, 19, 19, "+4 / +4"},
-    {2, 8, false, 22, 22, "+4 / +5"},
-    {2, 8, false, 24, 24, "+4 / +5"},
+    {2, 8, false, 19, 19, "+5 / +5"},
+    {2, 8, false, 22, 22, "+5 / +5"},
+    {2, 8, false, 24, 24, "+6 / +5"},
 };
 
 inline bool flush_priority_by_shape(int mode, int elem, bool normalized, int l_max) {
