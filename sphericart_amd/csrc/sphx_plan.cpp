@@ -609,6 +609,9 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
             // of the work and the flush is short: float32 l_max = 40 344 us with three, 310 with four, 281 with eight
             g.sequence_waves = elem == 4 ? 8 : 4;
         }
+        // (the shapes at which another number was measured to be ahead, with or without the flush at raised priority)
+        const PriorityRow* row = priority_row(mode, static_cast<int>(elem), normalized, l_max);
+        if (row != nullptr && row->sequence_waves != 0 && n_samples >= 32768) g.sequence_waves = row->sequence_waves;
     } else if (mode == 0) {
         g.sequence_waves = 1;
     }
@@ -764,9 +767,9 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
 // that prepare the next tile, too).
 static unsigned wave_priorities(int mode, size_t elem, bool normalized, int l_max, unsigned n_tiles,
                                 unsigned workgroups, unsigned least, bool forward) {
-    const bool by_shape = forward && n_tiles / least >= workgroups &&
-                          flush_priority_by_shape(mode, static_cast<int>(elem), normalized, l_max);
-    return static_cast<unsigned>(switch_or(SW_WAVE_PRIORITIES, by_shape ? 1 : 0));
+    const PriorityRow* row = priority_row(mode, static_cast<int>(elem), normalized, l_max);
+    const bool by_shape = forward && n_tiles / least >= workgroups && row != nullptr;
+    return static_cast<unsigned>(switch_or(SW_WAVE_PRIORITIES, by_shape ? static_cast<int>(row->priorities) : 0));
 }
 
 // Choose kernels, tile sizes and LDS layouts. `lds_limit` / `cus` describe the device.

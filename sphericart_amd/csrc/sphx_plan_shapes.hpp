@@ -95,44 +95,58 @@ struct PriorityRow {
     int mode, elem;
     bool normalized;
     int l_from, l_to;
+    unsigned priorities;     // 1: the flushing waves at raised priority
+    unsigned sequence_waves; // recursion_kernel: this many instead of the planner's rule (0: the rule)
     const char* measured;
 };
 
 constexpr PriorityRow kFlushPriorityRows[] = {
     // gradients, float32
-    {1, 4, true, 31, 31, "+4 / +8 (l_max = 32, cfg5: between -3 and +6 from run to run at 50 000 to 800 000 points, left alone)"},
-    {1, 4, true, 34, 35, "+8 / +8, +14 / +14"},
-    {1, 4, false, 11, 14, "+10 / +8, +7 / +7, +5 / +5, +6 / +5"},
-    {1, 4, false, 16, 16, "+5 / +5"},
-    {1, 4, false, 23, 23, "+5 / +6"},
-    {1, 4, false, 29, 30, "+12 / +10, +4 / +5"},
-    {1, 4, false, 32, 34, "+5 / +4, +14 / +12, +10 / +9"},
+    {1, 4, true, 31, 31, 1, 0, "+4 / +8 (l_max = 32, cfg5: between -3 and +6 from run to run at 50 000 to 800 000 points, left alone)"},
+    {1, 4, true, 34, 35, 1, 0, "+8 / +8, +14 / +14"},
+    {1, 4, false, 11, 14, 1, 0, "+10 / +8, +7 / +7, +5 / +5, +6 / +5"},
+    {1, 4, false, 16, 16, 1, 0, "+5 / +5"},
+    {1, 4, false, 23, 23, 1, 0, "+5 / +6"},
+    {1, 4, false, 29, 30, 1, 0, "+12 / +10, +4 / +5"},
+    {1, 4, false, 32, 34, 1, 0, "+5 / +4, +14 / +12, +10 / +9"},
     // gradients, float64
-    {1, 8, true, 23, 24, "+5 / +7, +8 / +5"},
-    {1, 8, true, 31, 32, "+7 / +6, +9 / +10"},
-    {1, 8, false, 19, 21, "+11 / +11, +4 / +4, +13 / +12"},
-    {1, 8, false, 25, 26, "+8 / +8, +3 / +3"},
-    {1, 8, false, 28, 28, "+4 / +3"},
-    {1, 8, false, 30, 31, "+12 / +14, +6 / +4"},
+    {1, 8, true, 23, 24, 1, 0, "+5 / +7, +8 / +5"},
+    {1, 8, true, 31, 32, 1, 0, "+7 / +6, +9 / +10"},
+    {1, 8, false, 19, 21, 1, 0, "+11 / +11, +4 / +4, +13 / +12"},
+    {1, 8, false, 25, 26, 1, 0, "+8 / +8, +3 / +3"},
+    {1, 8, false, 28, 28, 1, 0, "+4 / +3"},
+    {1, 8, false, 30, 31, 1, 0, "+12 / +14, +6 / +4"},
     // second derivatives, float32, solid (normalised: 0 to +3 at l_max = 5-28 on both boxes, -1 to -2 on a third)
-    {2, 4, false, 5, 6, "+13 / +13, +11 / +12"},
-    {2, 4, false, 8, 8, "+11 / +9"},
-    {2, 4, false, 10, 14, "+14 / +14, +10 / +12, +10 / +8, +4 / +3, +7 / +6"},
-    {2, 4, false, 27, 28, "+6 / +5, +12 / +12"},
+    {2, 4, false, 5, 6, 1, 0, "+13 / +13, +11 / +12"},
+    {2, 4, false, 8, 8, 1, 0, "+11 / +9"},
+    {2, 4, false, 10, 14, 1, 0, "+14 / +14, +10 / +12, +10 / +8, +4 / +3, +7 / +6"},
+    {2, 4, false, 27, 28, 1, 0, "+6 / +5, +12 / +12"},
     // second derivatives, float64, solid
-    {2, 8, false, 19, 19, "+5 / +5"},
-    {2, 8, false, 22, 22, "+5 / +5"},
-    {2, 8, false, 24, 24, "+6 / +5"},
+    {2, 8, false, 19, 19, 1, 0, "+5 / +5"},
+    {2, 8, false, 22, 22, 1, 0, "+5 / +5"},
+    {2, 8, false, 24, 24, 1, 0, "+6 / +5"},
+    // With another number of sequence waves than the rule's (four for gradients in float32, three in float64, three or
+    // two for solid second derivatives in float32). Every setting measured after 0.4 s of its own launches, median
+    // of three turns, us per 1.2 GB: the rule without priority / this row, on one box, then on another.
+    {1, 4, false, 8, 8, 1, 3, "221 / 197, 222 / 195"},
+    {1, 4, false, 9, 9, 0, 2, "221 / 205, 222 / 205"},
+    {1, 4, false, 10, 10, 1, 3, "230 / 202, 231 / 200"},
+    {1, 8, false, 11, 11, 1, 4, "211 / 204, 210 / 203"},
+    {1, 8, false, 13, 13, 1, 4, "217 / 209, 216 / 207"},
+    {1, 8, false, 15, 16, 1, 4, "218 / 208 and 220 / 212, 216 / 205 and 219 / 213"},
+    {2, 4, false, 4, 4, 0, 8, "215 / 199, 217 / 199"},
+    {2, 4, false, 18, 19, 1, 4, "214 / 206 and 216 / 207, 211 / 205 and 215 / 206"},
+    {2, 4, false, 21, 21, 1, 4, "219 / 207, 218 / 206"},
 };
 
-inline bool flush_priority_by_shape(int mode, int elem, bool normalized, int l_max) {
+inline const PriorityRow* priority_row(int mode, int elem, bool normalized, int l_max) {
     for (const PriorityRow& row : kFlushPriorityRows) {
         if (row.mode == mode && row.elem == elem && row.normalized == normalized && l_max >= row.l_from &&
             l_max <= row.l_to) {
-            return true;
+            return &row;
         }
     }
-    return false;
+    return nullptr;
 }
 
 } // namespace sphx
