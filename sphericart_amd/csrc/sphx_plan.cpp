@@ -820,6 +820,10 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
             want.prep_waves = static_cast<unsigned>(switch_or(SW_PAIRS_PREP_WAVES, 0));
             want.sequence_waves = static_cast<unsigned>(switch_or(SW_PAIRS_SEQUENCE_WAVES, 0));
             want.chunk_shift_plus_one = static_cast<unsigned>(switch_or(SW_PAIRS_CHUNK, -1) + 1);
+            if (const PriorityRow* row = priority_row(mode, static_cast<int>(elem), normalized, l_max)) {
+                // (the shapes at which another number of sequence waves than the planner's estimate was measured ahead)
+                if (want.sequence_waves == 0) want.sequence_waves = row->sequence_waves;
+            }
             if (plan_pairs(n_samples, l_max, mode, elem, elem, lds_limit, cus, want, &plan->pairs_launch)) {
                 PairsLaunch& made = plan->pairs_launch;
                 made.g.priorities = wave_priorities(mode, elem, normalized, l_max, made.g.n_tiles, made.workgroups, 32u, true);
@@ -862,6 +866,10 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
             want.prep_waves = static_cast<unsigned>(switch_or(SW_PAIRS_PREP_WAVES, 0));
             want.sequence_waves = static_cast<unsigned>(switch_or(SW_PAIRS_SEQUENCE_WAVES, 0));
             want.chunk_shift_plus_one = static_cast<unsigned>(switch_or(SW_PAIRS_CHUNK, -1) + 1);
+            if (const PriorityRow* row = priority_row(mode, static_cast<int>(elem), normalized, l_max)) {
+                // (the shapes at which another number of sequence waves than the planner's estimate was measured ahead)
+                if (want.sequence_waves == 0) want.sequence_waves = row->sequence_waves;
+            }
             if (plan_pairs(n_samples, l_max, mode, elem, elem, lds_limit, cus, want, &plan->pairs_launch)) {
                 PairsLaunch& made = plan->pairs_launch;
                 made.g.priorities = wave_priorities(mode, elem, normalized, l_max, made.g.n_tiles, made.workgroups, 32u, true);

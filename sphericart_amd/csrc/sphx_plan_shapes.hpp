@@ -107,14 +107,14 @@ constexpr PriorityRow kFlushPriorityRows[] = {
     {1, 4, false, 11, 14, 1, 0, "+10 / +8, +7 / +7, +5 / +5, +6 / +5"},
     {1, 4, false, 16, 16, 1, 0, "+5 / +5"},
     {1, 4, false, 23, 23, 1, 0, "+5 / +6"},
-    {1, 4, false, 29, 30, 1, 0, "+12 / +10, +4 / +5"},
-    {1, 4, false, 32, 34, 1, 0, "+5 / +4, +14 / +12, +10 / +9"},
+    {1, 4, false, 29, 29, 1, 0, "+12 / +10"},
+    {1, 4, false, 33, 34, 1, 0, "+14 / +12, +10 / +9"},
     // gradients, float64
     {1, 8, true, 23, 24, 1, 0, "+5 / +7, +8 / +5"},
     {1, 8, true, 31, 32, 1, 0, "+7 / +6, +9 / +10"},
-    {1, 8, false, 19, 21, 1, 0, "+11 / +11, +4 / +4, +13 / +12"},
-    {1, 8, false, 25, 26, 1, 0, "+8 / +8, +3 / +3"},
-    {1, 8, false, 28, 28, 1, 0, "+4 / +3"},
+    {1, 8, false, 19, 19, 1, 0, "+11 / +11"},
+    {1, 8, false, 21, 21, 1, 0, "+13 / +12"},
+    {1, 8, false, 25, 25, 1, 0, "+8 / +8"},
     {1, 8, false, 30, 31, 1, 0, "+12 / +14, +6 / +4"},
     // second derivatives, float32, solid (normalised: 0 to +3 at l_max = 5-28 on both boxes, -1 to -2 on a third)
     {2, 4, false, 5, 6, 1, 0, "+13 / +13, +11 / +12"},
@@ -137,6 +137,16 @@ constexpr PriorityRow kFlushPriorityRows[] = {
     {2, 4, false, 4, 4, 0, 8, "215 / 199, 217 / 199"},
     {2, 4, false, 18, 19, 1, 4, "214 / 206 and 216 / 207, 211 / 205 and 215 / 206"},
     {2, 4, false, 21, 21, 1, 4, "219 / 207, 218 / 206"},
+    // pairs_kernel with gradients, where the planner's estimate gives four sequence waves in float32 and two or three in
+    // float64: the rule with the priority where a row above had it / this row; one turn, then the median of three
+    {1, 4, false, 30, 30, 0, 3, "223 / 214, 223 / 211"},
+    {1, 4, false, 31, 31, 0, 3, "233 / 205, 233 / 204"},
+    {1, 4, false, 32, 32, 1, 3, "220 / 204, 217 / 205"},
+    {1, 4, false, 35, 35, 0, 3, "240 / 210, 241 / 211"},
+    {1, 8, false, 20, 20, 1, 2, "225 / 204, 225 / 204"},
+    {1, 8, false, 23, 23, 1, 2, "239 / 221, 237 / 225"},
+    {1, 8, false, 26, 27, 1, 4, "228 / 205 and 239 / 230, 229 / 206 and 240 / 231"},
+    {1, 8, false, 28, 29, 1, 2, "227 / 208 and 244 / 225, 227 / 208 and 244 / 228"},
 };
 
 inline const PriorityRow* priority_row(int mode, int elem, bool normalized, int l_max) {
