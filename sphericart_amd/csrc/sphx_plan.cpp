@@ -528,11 +528,12 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // Waves of their own for the closed forms of l <= 6 (whole rows): with sixteen waves and float32 gradients, where
     // the tile otherwise waits for the entry waves that carry a slice on top of their jobs: three of them (l_max =
     // 9 .. 18: 1-4 % over none, one or two are 5-20 % behind). In float64 the closed forms are too much for three or
-    // four waves (3-10 % behind none).
+    // four waves (3-10 % behind none). At l_max = 8, where the closed forms are 49 of the 81 entries, normalised
+    // harmonics take four (213 -> 203 us per 1.2 GB, each setting after 0.4 s of its own launches).
     g.slice_waves = 0;
     const bool slices_apart = threads > kRecursionThreads && mode == 1 && elem == 4;
     if (whole && mode < 2) {
-        const int want = switch_or(SW_SLICE_WAVES, slices_apart && S >= 9 ? 3 : 0);
+        const int want = switch_or(SW_SLICE_WAVES, slices_apart && S >= 9 ? (l_max == 8 && normalized ? 4 : 3) : 0);
         g.slice_waves = want < 0 ? 0u : (want > 4 ? 4u : static_cast<unsigned>(want));
     }
     g.sequence_waves = S * arrays * static_cast<unsigned>(l_max - hard) > 64 ? 2u : 1u;
@@ -611,7 +612,9 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
         }
         // (the shapes at which another number was measured to be ahead, with or without the flush at raised priority)
         const PriorityRow* row = priority_row(mode, static_cast<int>(elem), normalized, l_max);
-        if (row != nullptr && row->sequence_waves != 0 && n_samples >= 32768) g.sequence_waves = row->sequence_waves;
+        if (row != nullptr && row->sequence_waves != 0 && n_samples >= (mode == 2 ? 8192u : 32768u)) {
+            g.sequence_waves = row->sequence_waves;
+        }
     } else if (mode == 0) {
         g.sequence_waves = 1;
     }

@@ -137,6 +137,7 @@ constexpr PriorityRow kFlushPriorityRows[] = {
     {2, 4, false, 4, 4, 0, 8, "215 / 199, 217 / 199"},
     {2, 4, false, 18, 19, 1, 4, "214 / 206 and 216 / 207, 211 / 205 and 215 / 206"},
     {2, 4, false, 21, 21, 1, 4, "219 / 207, 218 / 206"},
+    {2, 8, false, 23, 23, 1, 2, "240 / 217, 239 / 218 (the rule: three)"},
     // pairs_kernel with gradients, where the planner's estimate gives four sequence waves in float32 and two or three in
     // float64: the rule with the priority where a row above had it / this row; one turn, then the median of three
     {1, 4, false, 30, 30, 0, 3, "223 / 214, 223 / 211"},
