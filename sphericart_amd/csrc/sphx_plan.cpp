@@ -405,8 +405,9 @@ static unsigned group_threads(size_t n_samples, int mode, size_t elem, bool forw
     const int want = switch_or(SW_GROUP_THREADS, 0);
     if (want == 512 || want == 1024) return static_cast<unsigned>(want);
     if (f64_hessians && l_max < 3) return kRecursionThreads;
-    // (normalised: one-sided jobs are 20 % more work, which sixteen waves make up for only at l_max = 3: 12 %)
-    if (f64_hessians && normalized && l_max != 3) return kRecursionThreads;
+    // (normalised: one-sided jobs are 20 % more work, which sixteen waves make up for at l_max = 3 (12 %), 4, 7 and 8
+    // (7, 8, 5 %; every setting measured after 0.4 s of its own launches); nothing in it at 5, 6, 9, 10, behind from 12)
+    if (f64_hessians && normalized && !(l_max == 3 || l_max == 4 || l_max == 7 || l_max == 8)) return kRecursionThreads;
     return n_samples >= 4096 ? 2 * kRecursionThreads : kRecursionThreads;
 }
 
@@ -438,9 +439,14 @@ static bool plan_recursion(size_t n_samples, int l_max, int mode, bool whole, si
     // for them: solid second derivatives at l_max = 4 .. 18 (5-11 %, cfg4 557 -> 513 us) and solid gradients up to
     // l_max = 10 (0-11 %) in calls of 32 768 points or more, and gradients from l_max = 27 on, where a recursion is a
     // long chain (10 %). Everywhere else in float64 the other division gains 2-14 %, as in all of float32.
-    const bool together_by_shape = elem == 8 && ((!normalized && n_samples >= 32768 &&
-                                         (mode == 2 ? l_max >= 4 && l_max <= 18 : mode == 1 && l_max <= 10)) ||
-                                        (mode == 1 && l_max >= 27));
+    // (Each division measured after 0.4 s of its own launches: solid gradients l_max = 9, 10 are 6 and 15 % ahead with
+    // the recursions apart, solid second derivatives at l_max = 10, 12, 14 by 6, 5, 4 %, behind by 1-3 % at the odd
+    // l_max between them and at 16.)
+    const bool together_by_shape =
+        elem == 8 && ((!normalized && n_samples >= 32768 &&
+                       (mode == 2 ? l_max >= 4 && l_max <= 18 && !(l_max == 10 || l_max == 12 || l_max == 14)
+                                  : mode == 1 && l_max <= 8)) ||
+                      (mode == 1 && l_max >= 27));
     const bool together = elem == 8 && switch_or(SW_RECURSIONS_TOGETHER, together_by_shape ? 1 : 0) != 0;
     g.together = together ? 1u : 0u;
     // per point: the rows, point tables twice and iterates once (together: three times, when a batch is a single tile,
@@ -889,7 +895,9 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
     // SPHX_GRADIENT_LANES: 0 never, 2 wherever the rows fit.
     const int gradient_lanes = switch_or(SW_GRADIENT_LANES, 1);
     const bool large_groups = group_threads(n_samples, mode, elem, lane_kernels) > kRecursionThreads && n_samples >= 32768;
-    const bool lanes_by_shape = large_groups ? l_max <= 7 : (n_samples >= 16384 ? l_max <= 9 : elem == 8 || l_max <= 13);
+    // (float64, normalised, l_max = 7: the recursion kernel is 8 % ahead there, 203 against 219 us per 1.2 GB)
+    const bool lanes_by_shape = large_groups ? l_max <= (elem == 8 && normalized ? 6 : 7)
+                                             : (n_samples >= 16384 ? l_max <= 9 : elem == 8 || l_max <= 13);
     if (lane_kernels && mode == 1 && gradient_lanes != 0 && (gradient_lanes == 2 || lanes_by_shape) &&
         plan_gradient_lanes(n_samples, l_max, elem, lds_limit, cus, &plan->closed)) {
         plan->lanes = true;
