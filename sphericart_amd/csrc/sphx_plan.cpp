@@ -406,8 +406,12 @@ static unsigned group_threads(size_t n_samples, int mode, size_t elem, bool forw
     if (want == 512 || want == 1024) return static_cast<unsigned>(want);
     if (f64_hessians && l_max < 3) return kRecursionThreads;
     // (normalised: one-sided jobs are 20 % more work, which sixteen waves make up for at l_max = 3 (12 %), 4, 7 and 8
-    // (7, 8, 5 %; every setting measured after 0.4 s of its own launches); nothing in it at 5, 6, 9, 10, behind from 12)
-    if (f64_hessians && normalized && !(l_max == 3 || l_max == 4 || l_max == 7 || l_max == 8)) return kRecursionThreads;
+    // (7, 8, 5 %; every setting measured after 0.4 s of its own launches); nothing in it at 5, 6, 9, 10, behind from 12
+    // to 24. From l_max = 25 a tile is a single point and a CU holds one workgroup either way: sixteen waves then,
+    // 448 -> 345 us per 1.2 GB at l_max = 25, 368 -> 331 at 26, 360 -> 327 at 28, 319 -> 315 at 32.)
+    if (f64_hessians && normalized && !(l_max == 3 || l_max == 4 || l_max == 7 || l_max == 8 || l_max >= 25)) {
+        return kRecursionThreads;
+    }
     return n_samples >= 4096 ? 2 * kRecursionThreads : kRecursionThreads;
 }
 
@@ -860,14 +864,17 @@ int make_plan(size_t n_samples, int l_max, int mode, size_t elem, int lds_limit,
     // the whole launch and whose other work runs while the rows are flushed. Gradients: up to 15 % faster than the
     // recursion kernel from l_max = 20 in float32 and 17 in float64 (cfg5 700 -> 570-620 us); below, a point's
     // pairs leave most of the entry lanes idle. Second derivatives in float64: ahead by 3-9 % at l_max = 20 and,
-    // for solid harmonics, from 24 on, behind by 2-25 % elsewhere; in float32 the recursion
+    // for solid harmonics, from 24 on, for normalised ones by 4, 14 and 12 % at l_max = 19, 21, 23 (and level at 22,
+    // 8 % behind at 24), behind by 2-25 % elsewhere; in float32 the recursion
     // kernel's job list by kind fills sixteen waves better. SPHX_PAIRS: 0 never, 2 wherever it fits.
     {
         const int pairs = switch_or(SW_PAIRS, 1);
         // (second derivatives: thirteen rows per point, 8 192 points are as many tiles as 32 768 with gradients)
         const bool pairs_by_shape =
             mode == 1 ? n_samples >= 32768 && (elem == 4 ? l_max >= 20 : l_max >= 17)
-                      : n_samples >= 8192 && elem == 8 && (l_max == 20 || (!normalized && l_max >= 24));
+                      : n_samples >= 8192 && elem == 8 &&
+                            (l_max == 20 || (!normalized && l_max >= 24) ||
+                             (normalized && (l_max == 19 || l_max == 21 || l_max == 23)));
         if (lane_kernels && mode >= 1 && l_max > hard && (pairs == 2 || (pairs == 1 && pairs_by_shape))) {
             PairsChoice want;
             want.tile = static_cast<unsigned>(switch_or(SW_PAIRS_TILE, 0));
