@@ -116,6 +116,8 @@ def parse():
     )
     p.add_argument("--sweep-sizes", default="20k,1.2GB,2M", help="with --sweep: which of the three sizes")
     p.add_argument("--sweep-markdown", action="store_true", help="with --sweep: print the tables as Markdown instead")
+    p.add_argument("--sweep-settle-seconds", type=float, default=0.3,
+                   help="with --sweep: seconds of launches of a row before it is timed (the clocks settle)")
     return p.parse_args()
 
 
@@ -130,7 +132,7 @@ def sweep(lib, args):
         print(f"{table.key_of(row):48s} {row['us']:9.1f} us {100 * row['frac']:5.1f} %  {row['kernel']}",
               file=sys.stderr, flush=True)
 
-    rows = table.run(lib, sizes=sizes, progress=progress)
+    rows = table.run(lib, sizes=sizes, progress=progress, settle=args.sweep_settle_seconds)
     if args.sweep_markdown:
         for size in sizes:
             print(f"\n{size}\n\n{table.as_markdown(rows, size)}")

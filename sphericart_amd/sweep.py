@@ -10,13 +10,15 @@ tenth below it. A row is
 
 (derivatives, dtype, harmonics, l_max, size, n_samples, us, frac, kernel; `load` gives the rows as dictionaries).
 
-`us` is the best of three series of launches enqueued back to back after a warm-up, between two events on the
+`us` is the best of three series of launches enqueued back to back after a warm-up (`bench.py --sweep`: after 0.3 s
+of the same launches, so that the clocks have settled as they do under sustained load), between two events on the
 launch stream; `frac` the algorithmic bytes of a launch, sizeof(T) * (3 + (l_max + 1)^2 * {1, 4, 13}) per point,
 over `us` and the 8 TB/s peak. The points are uniform in a cube: no kernel here branches on the coordinates
 except for points on the z axis, which the five benchmark clouds cover.
 """
 
 import ctypes
+import time
 
 PEAK_HBM_GBPS = 8000.0
 L_MAX = (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16, 18, 20, 24, 28, 32)
@@ -55,8 +57,10 @@ def shapes(sizes=SIZES, l_values=L_MAX):
                             yield derivatives, dtype, harmonics, l_max, size, n
 
 
-def measure_row(lib, derivatives, dtype, harmonics, l_max, size, n, launches=30, series=3):
-    """One row, measured on the current device."""
+def measure_row(lib, derivatives, dtype, harmonics, l_max, size, n, launches=30, series=3, settle=0.0):
+    """One row, measured on the current device: the best of `series` runs of `launches` launches back to back,
+    after `settle` seconds of the same launches (under sustained load the device lowers its clocks, and some shapes
+    rank differently in a short burst and after it has done so)."""
     import numpy as np
     import torch
 
@@ -82,6 +86,11 @@ def measure_row(lib, derivatives, dtype, harmonics, l_max, size, n, launches=30,
     for _ in range(max(8, launches // 2)):
         launch()
     torch.cuda.synchronize()
+    began = time.monotonic()
+    while time.monotonic() - began < settle:
+        for _ in range(50):
+            launch()
+        torch.cuda.synchronize()
     best = None
     for _ in range(series):
         begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -129,10 +138,10 @@ def key_of(row):
     return f"{row['derivatives']}/{row['dtype']}/{row['harmonics']}/l{row['l_max']}/{row['size']}"
 
 
-def run(lib, sizes=SIZES, l_values=L_MAX, progress=None):
+def run(lib, sizes=SIZES, l_values=L_MAX, progress=None, settle=0.0):
     rows = []
     for shape in shapes(sizes, l_values):
-        row = measure_row(lib, *shape, launches=60 if shape[4] == "20k" else 30)
+        row = measure_row(lib, *shape, launches=60 if shape[4] == "20k" else 30, settle=settle)
         rows.append(row)
         if progress is not None:
             progress(row)

@@ -2,8 +2,10 @@
 (``python bench.py --sweep``, kept as ``profiles/sweep.json``) is measured again and compared row by row with the
 fraction of the HBM peak recorded there.
 
-Boxes differ by some 5 % as a whole, and the float64 kernels run in one of two states a tenth apart from
-process to process with the same code, so a row is not judged against the recorded number alone: the test
+The table is recorded with every row settled (0.3 s of its own launches before it is timed); the test measures
+short bursts, which run 2-10 % faster on a cool device and rank a few shapes differently, boxes differ by some 5 %
+as a whole, and the float64 kernels run in one of two states a tenth apart from process to process with the same
+code, so a row is not judged against the recorded number alone: the test
 fails when the rows as a whole have fallen a tenth (the median of measured / recorded below 0.9), or when a
 single row has fallen more than 15 % below what that median makes of its recorded value. A slow row is measured
 up to three times, with fresh buffers, before it counts (another process's burst on the box, clocks that have
