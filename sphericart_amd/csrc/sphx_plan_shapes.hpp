@@ -84,8 +84,8 @@ inline const ShapeRow* shape_row(int kind, int elem, int l_max) {
 // recursion_kernel and pairs_kernel: the shapes at which the waves that flush a tile run at raised priority
 // (s_setprio) while other waves prepare the next tile. The flush and the preparation end at the same barrier;
 // whichever of them a tile waits for gains or loses by it, and which one that is changes from one l_max to the
-// next with the tile and the rounds of the sequence lanes. Measured at 1.2 GB of output after 0.4 s of the same
-// launches (settled clocks), the two settings interleaved in one process, on two boxes: percent gained on either
+// next with the tile and the rounds of the sequence lanes. Measured at 1.2 GB of output after 0.3 s of the same
+// launches (settled clocks; `python -m sphericart_amd.tune` is the measurement), on two boxes: percent gained on either
 // box (the same sign on both at nearly every l_max, and the same in short bursts on two other boxes; the rows are
 // the shapes that gained 3 % or more on both, elsewhere the priority costs up to 10 %). The gain holds from
 // 50 000 points up in pairs_kernel (2 to 13 % at 50 000, 100 000, 200 000 and 400 000 points) and from 50 000
